@@ -1,0 +1,189 @@
+#!/usr/bin/env python3
+"""Benchmark of the bidirectional GLA forward on one MI355X.
+
+A step = one bidirectional GLA forward (both directions, one library call) over
+one batch of synthetic inputs of the named workload, inputs resident in HBM.
+Input sets are rotated (>= 3 sets, > 256 MB in total) so that timed launches read
+HBM rather than the 256 MB Infinity Cache.
+
+Prints ONE JSON line on stdout; everything else goes to stderr.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBPS = 8000.0      # MI355X HBM3E, published
+MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16 MFMA, published
+
+
+def log(*a):
+    print(*a, file=sys.stderr, flush=True)
+
+
+def cpu_baseline(shape, seed, budget_s=20.0):
+    """Times the float32 torch port of the reference's recurrent routine on the host cores.
+
+    The sample is the named workload with the batch cut so one run stays near `budget_s`.
+    """
+    import torch
+
+    from oracle import gla_oracle as O
+    from vig_amd.synthetic import make_gla_inputs
+
+    threads = torch.get_num_threads()
+    # probe at batch 4 to size the sample
+    probe_B = min(4, shape.B)
+    q, k, v, gf, gb = make_gla_inputs(probe_B, shape.H, shape.L, shape.Dk, shape.Dv, seed, torch.float32)
+    t0 = time.perf_counter()
+    O.bidir_naive_recurrent_gla_f32(q, k, v, gf, gb)
+    t_probe = time.perf_counter() - t0
+    per_b = t_probe / probe_B
+    B = int(max(1, min(shape.B, budget_s / 3 / max(per_b, 1e-9))))
+    q, k, v, gf, gb = make_gla_inputs(B, shape.H, shape.L, shape.Dk, shape.Dv, seed, torch.float32)
+    O.bidir_naive_recurrent_gla_f32(q, k, v, gf, gb)  # warm-up
+    ts = []
+    for _ in range(2):
+        t0 = time.perf_counter()
+        O.bidir_naive_recurrent_gla_f32(q, k, v, gf, gb)
+        ts.append(time.perf_counter() - t0)
+    t = sorted(ts)[0]
+    tokens = B * shape.H * shape.L
+    flops = tokens * 8 * shape.Dk * shape.Dv
+    return {
+        "value": flops / t / 1e12,
+        "unit": "TFLOP/s",
+        "cores": threads,
+        "kind": "port",
+        "sample": f"B={B} of {shape.B} (H={shape.H} L={shape.L} Dk={shape.Dk} Dv={shape.Dv}, fp32 torch recurrent port, "
+                  f"two sweeps summed), best of 2 runs, {t:.3f} s",
+        "tokens_per_s": tokens / t,
+    }
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--config", type=int, default=1, help="named workload index (1 = ViG-S shape, the headline)")
+    ap.add_argument("--sets", type=int, default=0, help="input sets to rotate (0 = enough to exceed 256 MB, >= 3)")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--exact", action="store_true", help="time the fp32-arithmetic recurrent kernel instead")
+    args = ap.parse_args()
+
+    if args.gpus != 1:
+        log("bench.py: this build runs on ONE GPU; (batch, head) pairs are independent, so more GPUs would only "
+            "shard the batch. --gpus must be 1.")
+        sys.exit(2)
+
+    import torch
+
+    import vig_amd
+    from vig_amd import _lib
+    from vig_amd.synthetic import CONFIGS, make_gla_inputs, torch_dtype
+
+    if not os.path.exists(_lib.LIB_PATH):
+        from vig_amd.build import build_library
+        build_library()
+    lib = _lib.load()
+    assert torch.cuda.is_available(), "bench.py needs a GPU"
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+
+    s = CONFIGS[args.config]
+    dt = torch_dtype(s.dtype)
+    alg_bytes = s.alg_bytes()
+    alg_flops = s.alg_flops()
+    nsets = args.sets or max(3, int(300e6 // alg_bytes) + 1)
+    log(f"workload {s.name}: tokens={s.tokens} alg_bytes={alg_bytes/1e6:.1f} MB alg_flops={alg_flops/1e9:.2f} GF, "
+        f"{nsets} input sets")
+
+    sets = []
+    for i in range(nsets):
+        q, k, v, gf, gb = make_gla_inputs(s.B, s.H, s.L, s.Dk, s.Dv, 1000 + args.config + 17 * i, dt)
+        sets.append(tuple(t.to(dev) for t in (q, k, v, gf, gb)) + (torch.empty(s.B, s.H, s.L, s.Dv, dtype=dt, device=dev),))
+    io_dt = _lib.VIG_F32 if s.dtype == "f32" else _lib.VIG_BF16
+    ws_bytes = lib.vig_gla_bidir_fwd_workspace(s.B, s.H, s.L, s.Dk, s.Dv, io_dt)
+    if args.exact and s.dtype != "f32":
+        ws_bytes = max(ws_bytes, s.B * s.H * s.L * s.Dv * 4)
+    ws = torch.empty(max(ws_bytes, 1), dtype=torch.uint8, device=dev)
+    stream = torch.cuda.current_stream(dev)
+    sp = stream.cuda_stream
+    fn = lib.vig_gla_bidir_fwd_exact if args.exact else lib.vig_gla_bidir_fwd
+    scale = s.Dk ** -0.5
+
+    def step(i):
+        q, k, v, gf, gb, o = sets[i % nsets]
+        rc = fn(q.data_ptr(), k.data_ptr(), v.data_ptr(), gf.data_ptr(), gb.data_ptr(), o.data_ptr(),
+                ws.data_ptr(), ws_bytes, s.B, s.H, s.L, s.Dk, s.Dv, scale, 1.0, io_dt, io_dt, sp)
+        if rc != 0:
+            raise RuntimeError(f"vig_gla_bidir_fwd rc={rc}")
+
+    for i in range(args.warmup):
+        step(i)
+    torch.cuda.synchronize()
+
+    # whole-loop wall clock: K steps between two synchronisations
+    t0 = time.perf_counter()
+    for i in range(args.steps):
+        step(i)
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    ms_per_step = wall / args.steps * 1e3
+
+    # per-launch device time: HIP events recorded on the launch stream around each launch
+    evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(args.steps)]
+    for i in range(args.steps):
+        evs[i][0].record(stream)
+        step(i)
+        evs[i][1].record(stream)
+    torch.cuda.synchronize()
+    durs = sorted(a.elapsed_time(b) for a, b in evs)  # ms
+    k_avg = sum(durs) / len(durs)
+    k_med = durs[len(durs) // 2]
+    k_min = durs[0]
+    log(f"wall {ms_per_step*1e3:.1f} us/step; event-bracketed launch avg {k_avg*1e3:.1f} us, median {k_med*1e3:.1f}, min {k_min*1e3:.1f}")
+
+    tflops = alg_flops / (ms_per_step * 1e-3) / 1e12
+    achieved_gbps = alg_bytes / (k_avg * 1e-3) / 1e9
+    exec_flops_tok = 2 * (2 * 64 * (s.Dk + s.Dv) + 4 * s.Dk * s.Dv)  # executed MFMA FLOPs/token at chunk 64
+
+    out = {
+        "metric": "bidir GLA fwd TFLOP/s (algorithmic 8*Dk*Dv FLOP/token, both directions, 1 GPU)",
+        "value": tflops,
+        "unit": "TFLOP/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": ms_per_step,
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": s.dtype,
+        "data": "synthetic",
+        "config": {"workload": s.name, "B": s.B, "H": s.H, "L": s.L, "Dk": s.Dk, "Dv": s.Dv,
+                   "input_sets_rotated": nsets, "kernel_path": "recurrent_fp32" if args.exact else "default"},
+        "tokens_per_s": s.tokens / (ms_per_step * 1e-3),
+        "mfma_frac_algorithmic": tflops / MFMA_BF16_PEAK_TFLOPS,
+        "executed_tflops_chunk64": s.tokens * exec_flops_tok / (ms_per_step * 1e-3) / 1e12,
+        "kernel_us": {"avg": k_avg * 1e3, "median": k_med * 1e3, "min": k_min * 1e3},
+        "roofline": {"bound": "hbm", "achieved": achieved_gbps, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                     "frac": achieved_gbps / HBM_PEAK_GBPS, "traffic": None},
+    }
+    if not args.no_cpu:
+        out["cpu_baseline"] = cpu_baseline(s, 1000 + args.config)
+    else:
+        out["cpu_baseline"] = None
+    print(json.dumps(out), flush=True)
+
+
+if __name__ == "__main__":
+    main()

@@ -1,0 +1,133 @@
+/*
+ * vig_gla.h -- C ABI of the MI355X (gfx950) bidirectional gated-linear-attention
+ * forward path of ViG and its two neighbours (direction-wise gate preparation,
+ * 2D locality gate).
+ *
+ * Conventions shared by every entry point
+ *   - every pointer is DEVICE memory owned by the caller; nothing is allocated,
+ *     freed or synchronised inside; work is enqueued on `stream`
+ *     (a hipStream_t passed as void*; NULL = the null stream);
+ *   - tensors are dense row-major with the innermost dimension contiguous;
+ *   - return value: 0 on success, a negative VIG_E* code otherwise
+ *     (vig_gla_strerror() gives the text); a failed call enqueues nothing;
+ *   - dtype codes: VIG_F32 = 0, VIG_BF16 = 1.
+ *
+ * Citations name the reference (hustvl/ViG) interface each entry point replaces.
+ */
+#ifndef VIG_GLA_H_
+#define VIG_GLA_H_
+
+#include <stddef.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define VIG_F32 0
+#define VIG_BF16 1
+
+#define VIG_OK 0
+#define VIG_EINVAL (-22)  /* bad argument (null pointer, non-positive size) */
+#define VIG_ENOTSUP (-95) /* shape / dtype combination not built */
+#define VIG_ENOSPC (-28)  /* workspace too small */
+#define VIG_ELAUNCH (-5)  /* HIP reported a launch error */
+
+/* Library identification: "vig_gla <version> gfx950". */
+const char* vig_gla_version(void);
+const char* vig_gla_strerror(int code);
+
+/*
+ * Bidirectional GLA forward, both directions in one call, natural token order.
+ *
+ *   S_i  = diag(exp(gf_i)) S_{i-1} + k_i v_i^T      (i = 0..L-1)
+ *   S'_i = diag(exp(gb_i)) S'_{i+1} + k_i v_i^T     (i = L-1..0)
+ *   o_i  = out_scale * (scale*q_i)^T (S_i + S'_i)
+ *
+ * q, k, g_fwd, g_bwd: [B, H, L, Dk]; v, o: [B, H, L, Dv].  g_* are natural-log
+ * decays (<= 0).  g_bwd == NULL computes the forward direction only (the causal
+ * op).  io_dtype is the type of q, k, v, o; gate_dtype the type of g_*.
+ * `workspace` must hold vig_gla_bidir_fwd_workspace(...) bytes (may be NULL when
+ * that is 0).
+ *
+ * Replaces: bid_fused_recurrent_gla (flash-linear-attention/fla/ops/gla/
+ * recurrent_fuse.py:659-676, kernel :19-148; out_scale 1/2 from :442),
+ * batch_bid_fused_chunk_gla (fla/ops/gla/chunk_fuse.py:574-596) and, with
+ * g_bwd == NULL, fused_chunk_gla (chunk_fuse.py:554-572).
+ *
+ * Built shapes: Dk in {16, 32, 64, 128}, Dv in {32, 64}, any L >= 1.
+ */
+int vig_gla_bidir_fwd(const void* q, const void* k, const void* v,
+                      const void* g_fwd, const void* g_bwd, void* o,
+                      void* workspace, size_t workspace_bytes,
+                      int B, int H, int L, int Dk, int Dv,
+                      float scale, float out_scale,
+                      int io_dtype, int gate_dtype, void* stream);
+
+size_t vig_gla_bidir_fwd_workspace(int B, int H, int L, int Dk, int Dv, int io_dtype);
+
+/*
+ * Same contract as vig_gla_bidir_fwd, but always runs the fp32-arithmetic
+ * token-recurrent kernel whatever the dtypes (bf16 tensors are widened on load,
+ * the state and all sums stay fp32).  This is the op-level counterpart of the
+ * reference's recurrent kernels (fla/ops/gla/recurrent_fuse.py:19-148,152-246),
+ * kept callable for callers that want fp32 state arithmetic on bf16 tensors.
+ * Workspace: B*H*L*Dv*4 bytes when io_dtype is bf16 and g_bwd != NULL, else 0.
+ */
+int vig_gla_bidir_fwd_exact(const void* q, const void* k, const void* v,
+                            const void* g_fwd, const void* g_bwd, void* o,
+                            void* workspace, size_t workspace_bytes,
+                            int B, int H, int L, int Dk, int Dv,
+                            float scale, float out_scale,
+                            int io_dtype, int gate_dtype, void* stream);
+
+/*
+ * Direction-wise gate preparation.
+ *   gk_lin [B, L, 2*H*Dk]  ->  g_out [2, B, H, L, Dk]
+ *   g_out[dir,b,h,l,d] = max(logsigmoid(gk_lin[b,l,dir*H*Dk + h*Dk + d]) * inv_normalizer, clamp_min)
+ * clamp_min = NaN disables the clamp.  g_out[0] / g_out[1] are the g_fwd / g_bwd
+ * arguments of vig_gla_bidir_fwd.
+ *
+ * Replaces: classification/models/vig.py:432-441 (chunk(2), cat, rearrange,
+ * logsigmoid / gate_logit_normalizer, clamp_min).
+ */
+int vig_dirgate_fwd(const void* gk_lin, void* g_out, int B, int L, int H, int Dk,
+                    float inv_normalizer, float clamp_min,
+                    int in_dtype, int out_dtype, void* stream);
+
+/*
+ * 3x3 depthwise convolution on the token grid, channels-last, zero padding 1.
+ *   x [B, L=h*w, C], weight [C, 3, 3] (f32), bias [C] (f32) or NULL -> y [B, L, C]
+ *   optional SiLU on the result.
+ *
+ * Replaces: the in_proj of GatedLinearAttention (classification/models/vig.py:
+ * 291-294 applied at :428-430 with the two permutes around it).
+ */
+int vig_dwconv3x3_fwd(const void* x, const float* weight, const float* bias, void* y,
+                      int B, int h, int w, int C, int silu, int io_dtype, void* stream);
+
+/*
+ * Synthetic locality gate of the ViG-B benchmark shape:
+ *   y[b,hd,l,d] = o[b,hd,l,d] * sigmoid( dwconv3x3(o on the h x w grid, channel c = hd*Dv+d) )
+ * o, y: [B, H, L=h*w, Dv]; weight [H*Dv, 3, 3] f32.  In-place (y == o) is NOT allowed.
+ */
+int vig_locality_gate_fwd(const void* o, const float* weight, void* y,
+                          int B, int H, int h, int w, int Dv, int io_dtype, void* stream);
+
+/*
+ * Block epilogue before o_proj:
+ *   y[b,l,hd*Dv+d] = rms(o[b,hd,l,:])*w_g * s + rms(local[b,l,hd,:])*w_l * (1-s),  s = sigmoid(g_lin[b,l,hd*Dv+d])
+ *   rms(x) = x * rsqrt(mean(x^2) + eps); optional SiLU on y.
+ * o [B,H,L,Dv]; local, g_lin, y [B, L, H*Dv]; w_g, w_l [Dv] f32.
+ *
+ * Replaces: classification/models/vig.py:444-457 (two RMSNorm launches
+ * fla/modules/rmsnorm.py:69-125, three rearranges, sigmoid blend, out_act).
+ */
+int vig_locality_blend_fwd(const void* o, const void* local, const void* g_lin,
+                           const float* w_g, const float* w_l, void* y,
+                           int B, int H, int L, int Dv, float eps, int silu_out,
+                           int io_dtype, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* VIG_GLA_H_ */

@@ -1,0 +1,96 @@
+"""GPU parity of the GLA op's neighbours: gate preparation, 3x3 stencil, locality gate, blend epilogue."""
+import numpy as np
+import pytest
+import torch
+
+import vig_amd
+from oracle import gla_oracle as O
+from vig_amd.synthetic import make_locality_weight
+
+from .util import announce, f64, max_abs, max_rel
+
+pytestmark = pytest.mark.gpu
+
+
+def _randn(shape, seed, dtype=torch.float32, scale=1.0):
+    g = torch.Generator(device="cpu").manual_seed(seed)
+    return (torch.randn(*shape, generator=g) * scale).to(dtype)
+
+
+@pytest.mark.parametrize("dtype,tol", [(torch.float32, 1e-6), (torch.bfloat16, 2e-3)])
+@pytest.mark.parametrize("B,L,H,Dk", [(2, 196, 6, 32), (1, 197, 3, 64), (3, 7, 2, 16)])
+def test_dirgate(dtype, tol, B, L, H, Dk):
+    announce(f"dirgate {dtype} B{B} L{L} H{H} Dk{Dk}")
+    x = _randn((B, L, 2 * H * Dk), 1, dtype, 3.0)
+    want = O.dirgate_reference(f64(x), H, 16.0)
+    got = f64(vig_amd.dirgate(x.cuda(), H, 16.0))
+    assert got.shape == want.shape
+    assert max_abs(got, want) <= tol
+    wantc = O.dirgate_reference(f64(x), H, 16.0, clamp_min=-0.03)
+    gotc = f64(vig_amd.dirgate(x.cuda(), H, 16.0, clamp_min=-0.03))
+    assert max_abs(gotc, wantc) <= tol
+
+
+def test_dirgate_feeds_gla_layout():
+    """g_out[0]/g_out[1] are directly the g_fwd/g_bwd operands (reference: cat([fw,bw],0) viewed as [2,B,...])."""
+    announce("dirgate -> gla layout")
+    B, L, H, Dk = 2, 30, 2, 32
+    x = _randn((B, L, 2 * H * Dk), 2)
+    g = vig_amd.dirgate(x.cuda(), H)
+    ref = torch.nn.functional.logsigmoid(x) / 16
+    fw, bw = ref.chunk(2, dim=2)
+    cat = torch.cat([fw, bw], dim=0).reshape(2 * B, L, H, Dk).permute(0, 2, 1, 3)
+    assert (g.reshape(2 * B, H, L, Dk).cpu() - cat).abs().max() < 1e-6
+
+
+@pytest.mark.parametrize("dtype,tol", [(torch.float32, 1e-5), (torch.bfloat16, 2e-2)])
+@pytest.mark.parametrize("silu", [False, True])
+def test_dwconv3x3(dtype, tol, silu):
+    announce(f"dwconv3x3 {dtype} silu={silu}")
+    B, h, w, C = 3, 14, 14, 384
+    x = _randn((B, h * w, C), 3, dtype)
+    wt = make_locality_weight(C, 4)
+    bias = _randn((C,), 5)
+    want = O.dwconv3x3_reference(f64(x), f64(wt), (h, w), bias=f64(bias), silu=silu)
+    got = f64(vig_amd.dwconv3x3(x.cuda(), wt.cuda(), (h, w), bias=bias.cuda(), silu=silu))
+    assert max_abs(got, want) <= tol
+    want_nb = O.dwconv3x3_reference(f64(x), f64(wt), (h, w), silu=silu)
+    got_nb = f64(vig_amd.dwconv3x3(x.cuda(), wt.cuda(), (h, w), silu=silu))
+    assert max_abs(got_nb, want_nb) <= tol
+
+
+def test_dwconv3x3_nonsquare_grid():
+    announce("dwconv3x3 5x9 grid")
+    B, h, w, C = 2, 5, 9, 16
+    x = _randn((B, h * w, C), 6)
+    wt = make_locality_weight(C, 7)
+    want = O.dwconv3x3_reference(f64(x), f64(wt), (h, w))
+    got = f64(vig_amd.dwconv3x3(x.cuda(), wt.cuda(), (h, w)))
+    assert max_abs(got, want) <= 1e-5
+
+
+@pytest.mark.parametrize("dtype,tol", [(torch.float32, 1e-5), (torch.bfloat16, 2e-2)])
+def test_locality_gate(dtype, tol):
+    announce(f"locality sigmoid gate {dtype}")
+    B, H, h, w, Dv = 2, 12, 14, 14, 64
+    o = _randn((B, H, h * w, Dv), 8, dtype)
+    wt = make_locality_weight(H * Dv, 9)
+    want = O.locality_sigmoid_gate_reference(f64(o), f64(wt), (h, w))
+    got = f64(vig_amd.locality_gate(o.cuda(), wt.cuda(), (h, w)))
+    assert max_abs(got, want) <= tol
+
+
+@pytest.mark.parametrize("dtype,tol", [(torch.float32, 2e-5), (torch.bfloat16, 3e-2)])
+@pytest.mark.parametrize("H,Dv,L", [(6, 64, 196), (3, 32, 49), (5, 64, 7)])
+def test_locality_blend(dtype, tol, H, Dv, L):
+    announce(f"blend epilogue {dtype} H{H} Dv{Dv} L{L}")
+    B = 2
+    o = _randn((B, H, L, Dv), 10, dtype)
+    loc = _randn((B, L, H * Dv), 11, dtype)
+    gl = _randn((B, L, H * Dv), 12, dtype)
+    wg = _randn((Dv,), 13) * 0.1 + 1
+    wl = _randn((Dv,), 14) * 0.1 + 1
+    for silu in (False, True):
+        want = O.locality_blend_reference(f64(o), f64(loc), f64(gl), f64(wg), f64(wl), 1e-6, silu)
+        got = f64(vig_amd.locality_blend(o.cuda(), loc.cuda(), gl.cuda(), wg.cuda(), wl.cuda(), 1e-6, silu))
+        assert max_abs(got, want) <= tol

@@ -1,0 +1,158 @@
+"""GPU parity: the HIP path (through the C ABI) against the fp64 CPU oracle.
+
+Tolerances (stated by the task): fp32 mode max|a-b|/max|b| <= 1e-4; bf16 mode
+max|a-b| <= 2e-2 against the oracle run on the same bf16-rounded inputs.
+"""
+import numpy as np
+import pytest
+import torch
+
+import vig_amd
+from vig_amd.synthetic import CONFIGS, make_config_inputs, make_gla_inputs
+
+from .util import announce, f64, max_abs, max_rel, oracle_bidir
+
+pytestmark = pytest.mark.gpu
+
+FP32_TOL = 1e-4
+BF16_TOL = 2e-2
+
+
+def dev(*ts):
+    return tuple(t.cuda() if t is not None else None for t in ts)
+
+
+def test_cfg0_fp32_bidirectional():
+    announce("cfg0 fp32 B2 H3 L197 D64 via vig_gla_bidir_fwd")
+    q, k, v, gf, gb = make_config_inputs(0)
+    want = oracle_bidir(q, k, v, gf, gb)
+    got = f64(vig_amd.gla_bidir_forward(*dev(q, k, v, gf, gb)))
+    assert max_rel(got, want) <= FP32_TOL
+
+
+@pytest.mark.parametrize("L", [1, 2, 15, 16, 17, 63, 64, 65, 196, 197, 300])
+def test_fp32_ragged_lengths(L):
+    announce(f"fp32 ragged L={L}")
+    q, k, v, gf, gb = make_gla_inputs(2, 2, L, 64, 64, seed=L)
+    want = oracle_bidir(q, k, v, gf, gb)
+    got = f64(vig_amd.gla_bidir_forward(*dev(q, k, v, gf, gb)))
+    assert max_rel(got, want) <= FP32_TOL
+
+
+@pytest.mark.parametrize("Dk,Dv", [(16, 32), (32, 64), (64, 32), (128, 64)])
+def test_fp32_head_dims(Dk, Dv):
+    announce(f"fp32 Dk={Dk} Dv={Dv}")
+    q, k, v, gf, gb = make_gla_inputs(1, 3, 50, Dk, Dv, seed=7)
+    want = oracle_bidir(q, k, v, gf, gb)
+    got = f64(vig_amd.gla_bidir_forward(*dev(q, k, v, gf, gb)))
+    assert max_rel(got, want) <= FP32_TOL
+
+
+def test_fp32_strong_gates():
+    """Gates as in the reference's op tests: logsigmoid(randn).clamp_min(-3), no /16 (tests/ops/test_gla.py)."""
+    announce("fp32 strong gates L=300")
+    q, k, v, gf, gb = make_gla_inputs(2, 2, 300, 64, 64, seed=3, gate_scale=1.0)
+    gf, gb = gf.clamp_min(-3), gb.clamp_min(-3)
+    want = oracle_bidir(q, k, v, gf, gb)
+    got = f64(vig_amd.gla_bidir_forward(*dev(q, k, v, gf, gb)))
+    assert max_rel(got, want) <= FP32_TOL
+
+
+def test_fp32_causal_only_and_wrappers():
+    announce("fp32 causal-only + wrapper conventions")
+    q, k, v, gf, gb = make_gla_inputs(2, 2, 70, 32, 64, seed=11)
+    dq, dk_, dv_, dgf, dgb = dev(q, k, v, gf, gb)
+    o, st = vig_amd.fused_chunk_gla(dq, dk_, dv_, dgf)
+    assert st is None
+    assert max_rel(f64(o), oracle_bidir(q, k, v, gf, None)) <= FP32_TOL
+    g2 = torch.cat([dgf, dgb], dim=0)
+    want_half = oracle_bidir(q, k, v, gf, gb, out_scale=0.5)
+    o1, _ = vig_amd.batch_bid_fused_chunk_gla(dq, dk_, dv_, g2)
+    o2, _ = vig_amd.bid_fused_recurrent_gla(dq, dk_, dv_, g2, None)
+    assert max_rel(f64(o1), want_half) <= FP32_TOL
+    assert max_rel(f64(o2), want_half) <= FP32_TOL
+    of, orv = vig_amd.fused_recurrent_gla(dq, dk_, dv_, dgf, causal=False)
+    # causal=False: the reverse sweep shares the forward gates (naive.py:46-58)
+    from oracle import gla_oracle as O
+    assert max_rel(f64(orv), O.gla_recurrent(f64(q), f64(k), f64(v), f64(gf), reverse=True)) <= FP32_TOL
+    assert max_rel(f64(of), O.gla_recurrent(f64(q), f64(k), f64(v), f64(gf))) <= FP32_TOL
+    with pytest.raises(NotImplementedError):
+        vig_amd.fused_chunk_gla(dq, dk_, dv_, dgf, output_final_state=True)
+
+
+def test_fp32_zero_gate_closed_form():
+    """g = 0: o = scale * (tril(QK^T) + triu(QK^T)) V -- library matmul, no oracle involved."""
+    announce("fp32 g=0 closed form")
+    q, k, v, _, _ = make_gla_inputs(1, 2, 100, 64, 64, seed=5)
+    z = torch.zeros_like(q)
+    got = f64(vig_amd.gla_bidir_forward(*dev(q, k, v, z, z)))
+    A = (q.double() @ k.double().transpose(-1, -2)) * (64 ** -0.5)
+    want = ((torch.tril(A) + torch.triu(A)) @ v.double()).numpy()
+    assert max_rel(got, want) <= FP32_TOL
+
+
+@pytest.mark.parametrize("L", [1, 17, 196, 197])
+def test_bf16_exact_path_small(L):
+    announce(f"bf16 io through the fp32-arithmetic kernel L={L}")
+    q, k, v, gf, gb = make_gla_inputs(2, 3, L, 64, 64, seed=100 + L, dtype=torch.bfloat16)
+    want = oracle_bidir(q, k, v, gf, gb)
+    got = f64(vig_amd.gla_bidir_forward(*dev(q, k, v, gf, gb), exact=True))
+    assert max_abs(got, want) <= BF16_TOL
+
+
+@pytest.mark.parametrize("L,Dk", [(1, 64), (5, 64), (16, 64), (49, 64), (64, 64), (65, 64), (196, 64), (197, 64),
+                                   (256, 64), (257, 64), (300, 64), (196, 32), (197, 32), (700, 32)])
+def test_bf16_default_path(L, Dk):
+    announce(f"bf16 default (MFMA) path L={L} Dk={Dk}")
+    q, k, v, gf, gb = make_gla_inputs(3, 2, L, Dk, 64, seed=200 + L, dtype=torch.bfloat16)
+    want = oracle_bidir(q, k, v, gf, gb)
+    got = f64(vig_amd.gla_bidir_forward(*dev(q, k, v, gf, gb)))
+    assert max_abs(got, want) <= BF16_TOL
+
+
+def test_bf16_causal_only():
+    announce("bf16 default path, forward direction only")
+    q, k, v, gf, _ = make_gla_inputs(2, 2, 196, 64, 64, seed=31, dtype=torch.bfloat16)
+    want = oracle_bidir(q, k, v, gf, None)
+    got = f64(vig_amd.gla_bidir_forward(*dev(q, k, v, gf, None)))
+    assert max_abs(got, want) <= BF16_TOL
+
+
+def test_bf16_zero_gate_closed_form():
+    announce("bf16 g=0 closed form")
+    q, k, v, _, _ = make_gla_inputs(1, 2, 196, 64, 64, seed=6, dtype=torch.bfloat16)
+    z = torch.zeros_like(q)
+    got = f64(vig_amd.gla_bidir_forward(*dev(q, k, v, z, z)))
+    A = (q.double() @ k.double().transpose(-1, -2)) * (64 ** -0.5)
+    want = ((torch.tril(A) + torch.triu(A)) @ v.double()).numpy()
+    assert max_abs(got, want) <= BF16_TOL
+
+
+@pytest.mark.parametrize("idx,batch", [(1, None), (2, None), (3, None), (4, 64)])
+def test_bf16_named_configs_full_size(idx, batch):
+    """Full-size named workloads against the oracle (the oracle finishes these in seconds)."""
+    s = CONFIGS[idx]
+    announce(f"bf16 {s.name} batch={batch or s.B}")
+    q, k, v, gf, gb = make_config_inputs(idx, batch=batch)
+    want = oracle_bidir(q, k, v, gf, gb)
+    o = vig_amd.gla_bidir_forward(*dev(q, k, v, gf, gb))
+    got = f64(o)
+    err = max_abs(got, want)
+    print(f"  max-abs err {err:.3e}  max|o| {np.abs(want).max():.3f}", flush=True)
+    assert err <= BF16_TOL
+    # size-independent properties at full size: linearity in v and determinism
+    o2 = vig_amd.gla_bidir_forward(*dev(q, k, v, gf, gb))
+    assert torch.equal(o, o2), "kernel is not deterministic"
+    o_neg = vig_amd.gla_bidir_forward(*dev(q, k, -v, gf, gb))
+    assert torch.equal(o_neg, -o), "sign symmetry in v violated"
+
+
+def test_bf16_flip_symmetry_full_size():
+    """bwd(x, g) == flip(fwd(flip x, flip g)) at the ViG-S shape, bit-exact is not required (<= 2 bf16 roundings)."""
+    announce("bf16 flip symmetry cfg1 quarter batch")
+    q, k, v, gf, gb = make_config_inputs(1, batch=32)
+    dq, dk_, dv_, dgf, dgb = dev(q, k, v, gf, gb)
+    a = vig_amd.gla_bidir_forward(dq, dk_, dv_, dgf, dgb)
+    fl = lambda x: x.flip(dims=[2]).contiguous()
+    b = fl(vig_amd.gla_bidir_forward(fl(dq), fl(dk_), fl(dv_), fl(dgb), fl(dgf)))
+    assert (a.float() - b.float()).abs().max().item() <= BF16_TOL

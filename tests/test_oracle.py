@@ -1,0 +1,190 @@
+"""Pins the CPU oracle by closed forms, invariants and brute force (no GPU).
+
+The reference ships no golden vectors for this path, so each check below is
+chosen so that a plausible slip (dropped scale, gate applied after instead of
+before the update, wrong decay window, transposed operand, wrong triangle)
+fails at least one of them.
+"""
+import numpy as np
+import pytest
+
+from oracle import gla_oracle as O
+
+
+def _rand(rng, B=1, H=2, L=9, Dk=4, Dv=3, gscale=1.0):
+    q = rng.standard_normal((B, H, L, Dk))
+    k = rng.standard_normal((B, H, L, Dk))
+    v = rng.standard_normal((B, H, L, Dv))
+    g = -np.log1p(np.exp(-rng.standard_normal((B, H, L, Dk)))) * gscale
+    return q, k, v, g
+
+
+@pytest.mark.parametrize("reverse", [False, True])
+def test_L1_closed_form(rng, reverse):
+    q, k, v, g = _rand(rng, L=1, Dk=8, Dv=5)
+    o = O.gla_recurrent(q, k, v, g, reverse=reverse)
+    want = (8 ** -0.5) * (q * k).sum(-1, keepdims=True) * v
+    np.testing.assert_allclose(o, want, rtol=1e-13, atol=1e-14)
+
+
+def test_zero_gate_is_plain_causal_matmul(rng):
+    q, k, v, g = _rand(rng, L=17, Dk=8, Dv=6)
+    g = np.zeros_like(g)
+    s = 8 ** -0.5
+    A = np.einsum("bhid,bhjd->bhij", q, k) * s
+    of = O.gla_recurrent(q, k, v, g)
+    ob = O.gla_recurrent(q, k, v, g, reverse=True)
+    np.testing.assert_allclose(of, np.einsum("bhij,bhjv->bhiv", np.tril(A), v), rtol=1e-12, atol=1e-12)
+    np.testing.assert_allclose(ob, np.einsum("bhij,bhjv->bhiv", np.triu(A), v), rtol=1e-12, atol=1e-12)
+    # the diagonal is counted in both directions
+    both = O.bidir_gla_recurrent(q, k, v, g, g)
+    np.testing.assert_allclose(both, np.einsum("bhij,bhjv->bhiv", np.tril(A) + np.triu(A), v), rtol=1e-12, atol=1e-12)
+
+
+@pytest.mark.parametrize("reverse", [False, True])
+def test_minus_infinity_gate_keeps_only_the_diagonal(rng, reverse):
+    q, k, v, g = _rand(rng, L=11, Dk=4, Dv=3)
+    g = np.full_like(g, -800.0)  # exp underflows to exactly 0 in float64
+    o = O.gla_recurrent(q, k, v, g, reverse=reverse)
+    want = 0.5 * (q * k).sum(-1, keepdims=True) * v
+    np.testing.assert_allclose(o, want, rtol=1e-13, atol=1e-14)
+
+
+@pytest.mark.parametrize("reverse", [False, True])
+def test_constant_per_channel_gate_closed_form(rng, reverse):
+    B, H, L, Dk, Dv = 1, 1, 13, 5, 4
+    q, k, v, _ = _rand(rng, B, H, L, Dk, Dv)
+    gam = -np.abs(rng.standard_normal(Dk)) * 0.3
+    g = np.broadcast_to(gam, (B, H, L, Dk)).copy()
+    i = np.arange(L)
+    dist = (i[None, :] - i[:, None]) if reverse else (i[:, None] - i[None, :])
+    keep = dist >= 0
+    A = np.zeros((L, L))
+    for d in range(Dk):
+        A += np.where(keep, np.outer(q[0, 0, :, d], k[0, 0, :, d]) * np.exp(gam[d] * np.where(keep, dist, 0)), 0.0)
+    want = (Dk ** -0.5) * A @ v[0, 0]
+    o = O.gla_recurrent(q, k, v, g, reverse=reverse)
+    np.testing.assert_allclose(o[0, 0], want, rtol=1e-12, atol=1e-13)
+
+
+@pytest.mark.parametrize("reverse", [False, True])
+def test_bruteforce_tiny(rng, reverse):
+    q, k, v, g = _rand(rng, B=1, H=1, L=7, Dk=3, Dv=2)
+    bf = O.gla_bruteforce(q, k, v, g, reverse=reverse)
+    np.testing.assert_allclose(O.gla_recurrent(q, k, v, g, reverse=reverse), bf, rtol=1e-12, atol=1e-13)
+    np.testing.assert_allclose(O.gla_parallel(q, k, v, g, reverse=reverse), bf, rtol=1e-12, atol=1e-13)
+
+
+@pytest.mark.parametrize("reverse", [False, True])
+def test_parallel_form_matches_recurrence(rng, reverse):
+    q, k, v, g = _rand(rng, B=2, H=2, L=65, Dk=8, Dv=8, gscale=1 / 16)
+    np.testing.assert_allclose(
+        O.gla_recurrent(q, k, v, g, reverse=reverse), O.gla_parallel(q, k, v, g, reverse=reverse), rtol=1e-11, atol=1e-12
+    )
+
+
+def test_flip_symmetry(rng):
+    q, k, v, g = _rand(rng, L=23)
+    f = lambda x: np.flip(x, axis=2)
+    ob = O.gla_recurrent(q, k, v, g, reverse=True)
+    want = f(O.gla_recurrent(f(q), f(k), f(v), f(g)))
+    np.testing.assert_allclose(ob, want, rtol=1e-13, atol=1e-14)
+
+
+def test_state_passing_and_chunk_invariance(rng):
+    q, k, v, g = _rand(rng, B=2, H=1, L=37, Dk=4, Dv=5, gscale=0.3)
+    full, Sfull = O.gla_recurrent(q, k, v, g, return_state=True)
+    a, Sa = O.gla_recurrent(q[:, :, :20], k[:, :, :20], v[:, :, :20], g[:, :, :20], return_state=True)
+    b, Sb = O.gla_recurrent(q[:, :, 20:], k[:, :, 20:], v[:, :, 20:], g[:, :, 20:], initial_state=Sa, return_state=True)
+    np.testing.assert_allclose(np.concatenate([a, b], axis=2), full, rtol=1e-12, atol=1e-13)
+    np.testing.assert_allclose(Sb, Sfull, rtol=1e-12, atol=1e-13)
+    for C in (1, 4, 16, 64):
+        oc, Sc = O.gla_chunked(q, k, v, g, chunk=C, return_state=True)
+        np.testing.assert_allclose(oc, full, rtol=1e-11, atol=1e-12)
+        np.testing.assert_allclose(Sc, Sfull, rtol=1e-11, atol=1e-12)
+
+
+def test_zero_padding_is_a_noop_at_either_end(rng):
+    q, k, v, g = _rand(rng, L=21, Dk=4, Dv=4, gscale=0.2)
+    z = lambda x, n: np.pad(x, ((0, 0), (0, 0), (0, n), (0, 0)))
+    for rev in (False, True):
+        base = O.gla_recurrent(q, k, v, g, reverse=rev)
+        padded = O.gla_recurrent(z(q, 11), z(k, 11), z(v, 11), z(g, 11), reverse=rev)
+        np.testing.assert_allclose(padded[:, :, :21], base, rtol=1e-13, atol=1e-14)
+
+
+def test_linearity_in_v(rng):
+    q, k, v, g = _rand(rng, L=12)
+    v2 = rng.standard_normal(v.shape)
+    lhs = O.bidir_gla_recurrent(q, k, 2.0 * v - 3.0 * v2, g, g * 0.5)
+    rhs = 2.0 * O.bidir_gla_recurrent(q, k, v, g, g * 0.5) - 3.0 * O.bidir_gla_recurrent(q, k, v2, g, g * 0.5)
+    np.testing.assert_allclose(lhs, rhs, rtol=1e-11, atol=1e-12)
+
+
+def test_scale_and_out_scale(rng):
+    q, k, v, g = _rand(rng, L=6)
+    a = O.bidir_gla_recurrent(q, k, v, g, g, scale=1.0, out_scale=1.0)
+    b = O.bidir_gla_recurrent(q, k, v, g, g, scale=0.25, out_scale=0.5)
+    np.testing.assert_allclose(b, a * 0.125, rtol=1e-13)
+
+
+def test_f32_torch_port_matches_fp64():
+    import torch
+    from vig_amd.synthetic import make_gla_inputs
+
+    q, k, v, gf, gb = make_gla_inputs(2, 3, 197, 64, 64, seed=1000)
+    got = O.bidir_naive_recurrent_gla_f32(q, k, v, gf, gb).double().numpy()
+    want = O.bidir_gla_recurrent(q.numpy(), k.numpy(), v.numpy(), gf.numpy(), gb.numpy())
+    assert np.abs(got - want).max() / np.abs(want).max() < 1e-5
+
+
+def test_dirgate_layout_and_values(rng):
+    import torch
+    import torch.nn.functional as F
+
+    B, L, H, Dk = 2, 5, 3, 4
+    x = rng.standard_normal((B, L, 2 * H * Dk)) * 3
+    y = O.dirgate_reference(x, H, 16.0)
+    assert y.shape == (2, B, H, L, Dk)
+    ls = F.logsigmoid(torch.from_numpy(x)).numpy() / 16.0
+    for d in range(2):
+        for b in range(B):
+            for h in range(H):
+                for l in range(L):
+                    for c in range(Dk):
+                        assert abs(y[d, b, h, l, c] - ls[b, l, d * H * Dk + h * Dk + c]) < 1e-14
+    yc = O.dirgate_reference(x, H, 16.0, clamp_min=-0.05)
+    np.testing.assert_allclose(yc, np.maximum(y, -0.05))
+
+
+def test_dwconv_matches_torch_conv2d(rng):
+    import torch
+    import torch.nn.functional as F
+
+    B, h, w, C = 2, 5, 7, 6
+    x = rng.standard_normal((B, h * w, C))
+    wt = rng.standard_normal((C, 1, 3, 3))
+    got = O.dwconv3x3_reference(x, wt, (h, w))
+    x2 = torch.from_numpy(x).reshape(B, h, w, C).permute(0, 3, 1, 2)
+    want = F.conv2d(x2, torch.from_numpy(wt), padding=1, groups=C).flatten(2).permute(0, 2, 1).numpy()
+    np.testing.assert_allclose(got, want, rtol=1e-12, atol=1e-12)
+    got_s = O.dwconv3x3_reference(x, wt, (h, w), silu=True)
+    np.testing.assert_allclose(got_s, F.silu(torch.from_numpy(want)).numpy(), rtol=1e-12, atol=1e-12)
+
+
+def test_blend_matches_torch_expression(rng):
+    import torch
+
+    B, H, L, D = 2, 3, 6, 8
+    o = rng.standard_normal((B, H, L, D))
+    loc = rng.standard_normal((B, L, H * D))
+    gl = rng.standard_normal((B, L, H * D))
+    wg = rng.standard_normal(D)
+    wl = rng.standard_normal(D)
+    got = O.locality_blend_reference(o, loc, gl, wg, wl, eps=1e-6)
+    to = torch.from_numpy(o).permute(0, 2, 1, 3)
+    tl_ = torch.from_numpy(loc).reshape(B, L, H, D)
+    rn = lambda x, w: x * torch.rsqrt(x.pow(2).mean(-1, keepdim=True) + 1e-6) * torch.from_numpy(w)
+    g = torch.sigmoid(torch.from_numpy(gl)).reshape(B, L, H, D)
+    want = (rn(to, wg) * g + rn(tl_, wl) * (1 - g)).reshape(B, L, H * D).numpy()
+    np.testing.assert_allclose(got, want, rtol=1e-12, atol=1e-12)

@@ -1,0 +1,124 @@
+// C ABI of the library (declared in include/vig_gla.h): argument validation and
+// dispatch only.  Nothing here allocates, frees or synchronises.
+#include "../../include/vig_gla.h"
+#include "launch.h"
+
+namespace vig {
+int launch_dirgate(const void* in, void* out, int B, int L, int H, int Dk, float inv_norm, float clamp_min,
+                   int in_dtype, int out_dtype, hipStream_t stream);
+int launch_dwconv3x3(const void* x, const float* wt, const float* bias, void* y, int B, int h, int w, int C,
+                     int silu, int io_dtype, hipStream_t stream);
+int launch_locality_gate(const void* o, const float* wt, void* y, int B, int H, int h, int w, int Dv, int io_dtype,
+                         hipStream_t stream);
+int launch_locality_blend(const void* o, const void* loc, const void* glin, const float* wg, const float* wl, void* y,
+                          int B, int H, int L, int Dv, float eps, int silu_out, int io_dtype, hipStream_t stream);
+}  // namespace vig
+
+static bool dtype_ok(int d) { return d == VIG_F32 || d == VIG_BF16; }
+static bool dk_ok(int d) { return d == 16 || d == 32 || d == 64 || d == 128; }
+static bool dv_ok(int d) { return d == 32 || d == 64; }
+
+extern "C" {
+
+const char* vig_gla_version(void) { return "vig_gla 0.1 gfx950"; }
+
+const char* vig_gla_strerror(int code) {
+  switch (code) {
+    case VIG_OK: return "ok";
+    case VIG_EINVAL: return "invalid argument";
+    case VIG_ENOTSUP: return "shape or dtype combination not built";
+    case VIG_ENOSPC: return "workspace too small";
+    case VIG_ELAUNCH: return "HIP launch error";
+    default: return "unknown error";
+  }
+}
+
+static int fill_args(vig::GlaArgs& a, const void* q, const void* k, const void* v, const void* g_fwd,
+                     const void* g_bwd, void* o, void* workspace, size_t workspace_bytes, int B, int H, int L,
+                     int Dk, int Dv, float scale, float out_scale, int io_dtype, int gate_dtype, void* stream) {
+  if (!q || !k || !v || !g_fwd || !o) return VIG_EINVAL;
+  if (B <= 0 || H <= 0 || L <= 0) return VIG_EINVAL;
+  if ((long long)B * H > 2147483647LL) return VIG_EINVAL;
+  if (!dtype_ok(io_dtype) || !dtype_ok(gate_dtype)) return VIG_ENOTSUP;
+  if (!dk_ok(Dk) || !dv_ok(Dv)) return VIG_ENOTSUP;
+  a = vig::GlaArgs{q, k, v, g_fwd, g_bwd, o, workspace, workspace_bytes, B, H, L, Dk, Dv,
+                   scale, out_scale, io_dtype, gate_dtype, (hipStream_t)stream};
+  return VIG_OK;
+}
+
+size_t vig_gla_bidir_fwd_workspace(int B, int H, int L, int Dk, int Dv, int io_dtype) {
+  if (B <= 0 || H <= 0 || L <= 0) return 0;
+  // The largest requirement over the paths the dispatcher may take for this shape.
+  size_t need = vig::gla_recurrent_workspace(B, H, L, Dv, io_dtype);
+  if (io_dtype == VIG_BF16) {
+    const size_t m = vig::gla_mfma_workspace(B, H, L, Dk, Dv);
+    if (m > need) need = m;
+  }
+  return need;
+}
+
+int vig_gla_bidir_fwd(const void* q, const void* k, const void* v, const void* g_fwd, const void* g_bwd, void* o,
+                      void* workspace, size_t workspace_bytes, int B, int H, int L, int Dk, int Dv, float scale,
+                      float out_scale, int io_dtype, int gate_dtype, void* stream) {
+  vig::GlaArgs a;
+  const int rc = fill_args(a, q, k, v, g_fwd, g_bwd, o, workspace, workspace_bytes, B, H, L, Dk, Dv, scale,
+                           out_scale, io_dtype, gate_dtype, stream);
+  if (rc != VIG_OK) return rc;
+  if (vig::gla_mfma_supported(a)) {
+    if (vig::gla_mfma_workspace(B, H, L, Dk, Dv) > workspace_bytes) return VIG_ENOSPC;
+    if (vig::gla_mfma_workspace(B, H, L, Dk, Dv) > 0 && !workspace) return VIG_EINVAL;
+    return vig::launch_gla_mfma(a);
+  }
+  const size_t need = g_bwd ? vig::gla_recurrent_workspace(B, H, L, Dv, io_dtype) : 0;
+  if (need > workspace_bytes) return VIG_ENOSPC;
+  if (need > 0 && !workspace) return VIG_EINVAL;
+  return vig::launch_gla_recurrent(a);
+}
+
+// Same contract as vig_gla_bidir_fwd, but always takes the fp32-arithmetic
+// token-recurrent kernel (the exact path), whatever the dtypes.
+int vig_gla_bidir_fwd_exact(const void* q, const void* k, const void* v, const void* g_fwd, const void* g_bwd,
+                            void* o, void* workspace, size_t workspace_bytes, int B, int H, int L, int Dk, int Dv,
+                            float scale, float out_scale, int io_dtype, int gate_dtype, void* stream) {
+  vig::GlaArgs a;
+  const int rc = fill_args(a, q, k, v, g_fwd, g_bwd, o, workspace, workspace_bytes, B, H, L, Dk, Dv, scale,
+                           out_scale, io_dtype, gate_dtype, stream);
+  if (rc != VIG_OK) return rc;
+  const size_t need = g_bwd ? vig::gla_recurrent_workspace(B, H, L, Dv, io_dtype) : 0;
+  if (need > workspace_bytes) return VIG_ENOSPC;
+  if (need > 0 && !workspace) return VIG_EINVAL;
+  return vig::launch_gla_recurrent(a);
+}
+
+int vig_dirgate_fwd(const void* gk_lin, void* g_out, int B, int L, int H, int Dk, float inv_normalizer,
+                    float clamp_min, int in_dtype, int out_dtype, void* stream) {
+  if (!gk_lin || !g_out || B <= 0 || L <= 0 || H <= 0 || Dk <= 0) return VIG_EINVAL;
+  if (!dtype_ok(in_dtype) || !dtype_ok(out_dtype) || (Dk % 8) != 0) return VIG_ENOTSUP;
+  return vig::launch_dirgate(gk_lin, g_out, B, L, H, Dk, inv_normalizer, clamp_min, in_dtype, out_dtype,
+                             (hipStream_t)stream);
+}
+
+int vig_dwconv3x3_fwd(const void* x, const float* weight, const float* bias, void* y, int B, int h, int w, int C,
+                      int silu, int io_dtype, void* stream) {
+  if (!x || !weight || !y || B <= 0 || h <= 0 || w <= 0 || C <= 0 || x == y) return VIG_EINVAL;
+  if (!dtype_ok(io_dtype) || (C % 8) != 0) return VIG_ENOTSUP;
+  return vig::launch_dwconv3x3(x, weight, bias, y, B, h, w, C, silu, io_dtype, (hipStream_t)stream);
+}
+
+int vig_locality_gate_fwd(const void* o, const float* weight, void* y, int B, int H, int h, int w, int Dv,
+                          int io_dtype, void* stream) {
+  if (!o || !weight || !y || B <= 0 || H <= 0 || h <= 0 || w <= 0 || o == y) return VIG_EINVAL;
+  if (!dtype_ok(io_dtype) || (Dv % 8) != 0 || Dv <= 0) return VIG_ENOTSUP;
+  return vig::launch_locality_gate(o, weight, y, B, H, h, w, Dv, io_dtype, (hipStream_t)stream);
+}
+
+int vig_locality_blend_fwd(const void* o, const void* local, const void* g_lin, const float* w_g, const float* w_l,
+                           void* y, int B, int H, int L, int Dv, float eps, int silu_out, int io_dtype,
+                           void* stream) {
+  if (!o || !local || !g_lin || !w_g || !w_l || !y || B <= 0 || H <= 0 || L <= 0) return VIG_EINVAL;
+  if (!dtype_ok(io_dtype) || !(Dv == 32 || Dv == 64)) return VIG_ENOTSUP;
+  return vig::launch_locality_blend(o, local, g_lin, w_g, w_l, y, B, H, L, Dv, eps, silu_out, io_dtype,
+                                    (hipStream_t)stream);
+}
+
+}  // extern "C"

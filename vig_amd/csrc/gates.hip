@@ -1,0 +1,284 @@
+// Elementwise / stencil neighbours of the GLA op: direction-wise gate preparation,
+// the 3x3 depthwise stencil on the token grid, the sigmoid locality gate and the
+// RMS-norm blend epilogue.  All are HBM-bound: each element is read once with
+// 16-byte (bf16 x8) or 16-byte (f32 x4) accesses along the channel dimension and
+// written once; stencil neighbours come from L1/L2.
+#include "common.h"
+#include "launch.h"
+
+namespace vig {
+
+// ---------------------------------------------------------------------------
+// vector-of-8 channel access (one 16-byte transaction for bf16, two for f32)
+// ---------------------------------------------------------------------------
+template <typename T> struct Vec8;
+template <> struct Vec8<uint16_t> {
+  static __device__ __forceinline__ void load(const uint16_t* p, float (&x)[8]) {
+    const u32x4_t r = *reinterpret_cast<const u32x4_t*>(p);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      x[2 * i] = bf16lo_to_f32(r[i]);
+      x[2 * i + 1] = bf16hi_to_f32(r[i]);
+    }
+  }
+  static __device__ __forceinline__ void store(uint16_t* p, const float (&x)[8]) {
+    u32x4_t r;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) r[i] = pack_bf16x2(x[2 * i], x[2 * i + 1]);
+    *reinterpret_cast<u32x4_t*>(p) = r;
+  }
+};
+template <> struct Vec8<float> {
+  static __device__ __forceinline__ void load(const float* p, float (&x)[8]) {
+    const f32x4_t a = *reinterpret_cast<const f32x4_t*>(p);
+    const f32x4_t b = *reinterpret_cast<const f32x4_t*>(p + 4);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      x[i] = a[i];
+      x[4 + i] = b[i];
+    }
+  }
+  static __device__ __forceinline__ void store(float* p, const float (&x)[8]) {
+    f32x4_t a, b;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      a[i] = x[i];
+      b[i] = x[4 + i];
+    }
+    *reinterpret_cast<f32x4_t*>(p) = a;
+    *reinterpret_cast<f32x4_t*>(p + 4) = b;
+  }
+};
+
+// ---------------------------------------------------------------------------
+// direction-wise gate preparation
+//   in  [B, L, 2*H*Dk]  ->  out [2, B, H, L, Dk],  logsigmoid(x) * inv_norm, clamp
+// ---------------------------------------------------------------------------
+template <typename TI, typename TO>
+__global__ __launch_bounds__(256) void dirgate_kernel(const TI* __restrict__ in, TO* __restrict__ out,
+                                                       int B, int L, int H, int Dk, float inv_norm,
+                                                       float clamp_min, int use_clamp, size_t nvec) {
+  const int dk8 = Dk >> 3;
+  for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < nvec; i += (size_t)gridDim.x * 256) {
+    // i enumerates output vectors in output order: (((dir*B + b)*H + h)*L + l)*dk8 + d8
+    size_t r = i;
+    const int d8 = (int)(r % dk8);
+    r /= dk8;
+    const int l = (int)(r % L);
+    r /= L;
+    const int h = (int)(r % H);
+    r /= H;
+    const int b = (int)(r % B);
+    const int dir = (int)(r / B);
+    const size_t src = ((size_t)b * L + l) * (size_t)(2 * H * Dk) + (size_t)dir * H * Dk + (size_t)h * Dk + d8 * 8;
+    float x[8];
+    Vec8<TI>::load(in + src, x);
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      // logsigmoid(x) = min(x,0) - log1p(exp(-|x|))
+      float y = fminf(x[j], 0.f) - log1pf(__expf(-fabsf(x[j])));
+      y *= inv_norm;
+      if (use_clamp) y = fmaxf(y, clamp_min);
+      x[j] = y;
+    }
+    Vec8<TO>::store(out + i * 8, x);
+  }
+}
+
+template <typename TI, typename TO>
+static int launch_dirgate_t(const void* in, void* out, int B, int L, int H, int Dk, float inv_norm,
+                            float clamp_min, hipStream_t stream) {
+  const size_t nvec = (size_t)2 * B * H * L * (Dk / 8);
+  const int use_clamp = clamp_min == clamp_min;  // NaN disables
+  const int grid = (int)((nvec + 255) / 256 < 65535 * 8 ? (nvec + 255) / 256 : 65535 * 8);
+  hipLaunchKernelGGL((dirgate_kernel<TI, TO>), dim3(grid), dim3(256), 0, stream, (const TI*)in, (TO*)out, B, L, H,
+                     Dk, inv_norm, clamp_min, use_clamp, nvec);
+  return hipGetLastError() == hipSuccess ? 0 : -5;
+}
+
+int launch_dirgate(const void* in, void* out, int B, int L, int H, int Dk, float inv_norm, float clamp_min,
+                   int in_dtype, int out_dtype, hipStream_t stream) {
+  if (in_dtype == 0 && out_dtype == 0) return launch_dirgate_t<float, float>(in, out, B, L, H, Dk, inv_norm, clamp_min, stream);
+  if (in_dtype == 0 && out_dtype == 1) return launch_dirgate_t<float, uint16_t>(in, out, B, L, H, Dk, inv_norm, clamp_min, stream);
+  if (in_dtype == 1 && out_dtype == 0) return launch_dirgate_t<uint16_t, float>(in, out, B, L, H, Dk, inv_norm, clamp_min, stream);
+  return launch_dirgate_t<uint16_t, uint16_t>(in, out, B, L, H, Dk, inv_norm, clamp_min, stream);
+}
+
+// ---------------------------------------------------------------------------
+// 3x3 depthwise stencil, channels-last:  x [B, h*w, C] -> y [B, h*w, C]
+// one thread = one token x 8 channels; weights [C,3,3] f32
+// ---------------------------------------------------------------------------
+template <typename T>
+__global__ __launch_bounds__(256) void dwconv3x3_kernel(const T* __restrict__ x, const float* __restrict__ wt,
+                                                         const float* __restrict__ bias, T* __restrict__ y, int B,
+                                                         int h, int w, int C, int silu, size_t nvec) {
+  const int c8n = C >> 3;
+  const int L = h * w;
+  for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < nvec; i += (size_t)gridDim.x * 256) {
+    const int c8 = (int)(i % c8n);
+    const size_t bl = i / c8n;
+    const int l = (int)(bl % L);
+    const size_t b = bl / L;
+    const int r = l / w, c = l % w;
+    const int ch = c8 * 8;
+    float accv[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) accv[j] = bias ? bias[ch + j] : 0.f;
+#pragma unroll
+    for (int di = -1; di <= 1; ++di) {
+      const int rr = r + di;
+      if (rr < 0 || rr >= h) continue;
+#pragma unroll
+      for (int dj = -1; dj <= 1; ++dj) {
+        const int cc = c + dj;
+        if (cc < 0 || cc >= w) continue;
+        float xv[8];
+        Vec8<T>::load(x + ((b * L + (size_t)(rr * w + cc)) * C + ch), xv);
+#pragma unroll
+        for (int j = 0; j < 8; ++j) accv[j] += xv[j] * wt[(ch + j) * 9 + (di + 1) * 3 + (dj + 1)];
+      }
+    }
+    if (silu) {
+#pragma unroll
+      for (int j = 0; j < 8; ++j) accv[j] = accv[j] * sigmoidf_(accv[j]);
+    }
+    Vec8<T>::store(y + i * 8, accv);
+  }
+}
+
+int launch_dwconv3x3(const void* x, const float* wt, const float* bias, void* y, int B, int h, int w, int C,
+                     int silu, int io_dtype, hipStream_t stream) {
+  const size_t nvec = (size_t)B * h * w * (C / 8);
+  const int grid = (int)((nvec + 255) / 256 < 65535 * 8 ? (nvec + 255) / 256 : 65535 * 8);
+  if (io_dtype == 0)
+    hipLaunchKernelGGL((dwconv3x3_kernel<float>), dim3(grid), dim3(256), 0, stream, (const float*)x, wt, bias,
+                       (float*)y, B, h, w, C, silu, nvec);
+  else
+    hipLaunchKernelGGL((dwconv3x3_kernel<uint16_t>), dim3(grid), dim3(256), 0, stream, (const uint16_t*)x, wt, bias,
+                       (uint16_t*)y, B, h, w, C, silu, nvec);
+  return hipGetLastError() == hipSuccess ? 0 : -5;
+}
+
+// ---------------------------------------------------------------------------
+// sigmoid locality gate on the head-major layout:
+//   o, y [B, H, L=h*w, Dv];  y = o * sigmoid(dwconv3x3(o)), channel = hd*Dv + d
+// ---------------------------------------------------------------------------
+template <typename T>
+__global__ __launch_bounds__(256) void locality_gate_kernel(const T* __restrict__ o, const float* __restrict__ wt,
+                                                             T* __restrict__ y, int H, int h, int w, int Dv,
+                                                             size_t nvec) {
+  const int d8n = Dv >> 3;
+  const int L = h * w;
+  for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < nvec; i += (size_t)gridDim.x * 256) {
+    const int d8 = (int)(i % d8n);
+    const size_t bhl = i / d8n;
+    const int l = (int)(bhl % L);
+    const size_t bh = bhl / L;
+    const int hd = (int)(bh % H);
+    const int r = l / w, c = l % w;
+    const int ch = hd * Dv + d8 * 8;
+    float accv[8], ctr[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) accv[j] = 0.f, ctr[j] = 0.f;
+#pragma unroll
+    for (int di = -1; di <= 1; ++di) {
+      const int rr = r + di;
+      if (rr < 0 || rr >= h) continue;
+#pragma unroll
+      for (int dj = -1; dj <= 1; ++dj) {
+        const int cc = c + dj;
+        if (cc < 0 || cc >= w) continue;
+        float xv[8];
+        Vec8<T>::load(o + ((bh * L + (size_t)(rr * w + cc)) * Dv + d8 * 8), xv);
+#pragma unroll
+        for (int j = 0; j < 8; ++j) accv[j] += xv[j] * wt[(ch + j) * 9 + (di + 1) * 3 + (dj + 1)];
+        if (di == 0 && dj == 0) {
+#pragma unroll
+          for (int j = 0; j < 8; ++j) ctr[j] = xv[j];
+        }
+      }
+    }
+#pragma unroll
+    for (int j = 0; j < 8; ++j) accv[j] = ctr[j] * sigmoidf_(accv[j]);
+    Vec8<T>::store(y + i * 8, accv);
+  }
+}
+
+int launch_locality_gate(const void* o, const float* wt, void* y, int B, int H, int h, int w, int Dv, int io_dtype,
+                         hipStream_t stream) {
+  const size_t nvec = (size_t)B * H * h * w * (Dv / 8);
+  const int grid = (int)((nvec + 255) / 256 < 65535 * 8 ? (nvec + 255) / 256 : 65535 * 8);
+  if (io_dtype == 0)
+    hipLaunchKernelGGL((locality_gate_kernel<float>), dim3(grid), dim3(256), 0, stream, (const float*)o, wt,
+                       (float*)y, H, h, w, Dv, nvec);
+  else
+    hipLaunchKernelGGL((locality_gate_kernel<uint16_t>), dim3(grid), dim3(256), 0, stream, (const uint16_t*)o, wt,
+                       (uint16_t*)y, H, h, w, Dv, nvec);
+  return hipGetLastError() == hipSuccess ? 0 : -5;
+}
+
+// ---------------------------------------------------------------------------
+// RMS-norm blend epilogue.  One group of Dv/8 lanes owns one (b, l, head) row of
+// Dv values; the two mean-squares are reduced with lane shuffles inside the group.
+//   y[b,l,hd*Dv+d] = rms(o[b,hd,l,:])*w_g*s + rms(local[b,l,hd,:])*w_l*(1-s)
+// ---------------------------------------------------------------------------
+template <typename T>
+__global__ __launch_bounds__(256) void locality_blend_kernel(const T* __restrict__ o, const T* __restrict__ loc,
+                                                              const T* __restrict__ glin,
+                                                              const float* __restrict__ wg,
+                                                              const float* __restrict__ wl, T* __restrict__ y,
+                                                              int H, int L, int Dv, float eps, int silu_out,
+                                                              size_t nvec) {
+  const int d8n = Dv >> 3;  // lanes per row: 4 (Dv=32) or 8 (Dv=64); power of two
+  // nvec is padded to a multiple of 256 by construction of the grid-stride loop bound below,
+  // so every lane of a row group takes the same trip count and the shuffles are well defined.
+  const size_t nround = (nvec + 255) / 256 * 256;
+  for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < nround; i += (size_t)gridDim.x * 256) {
+    const bool live = i < nvec;
+    const size_t ii = live ? i : nvec - 1;
+    const int d8 = (int)(ii % d8n);
+    const size_t blh = ii / d8n;  // output order: (b*L + l)*H + hd
+    const int hd = (int)(blh % H);
+    const size_t bl = blh / H;
+    const int l = (int)(bl % L);
+    const size_t b = bl / L;
+    float xo[8], xl[8], xg[8];
+    Vec8<T>::load(o + (((b * H + hd) * L + l) * (size_t)Dv + d8 * 8), xo);
+    Vec8<T>::load(loc + ii * 8, xl);
+    Vec8<T>::load(glin + ii * 8, xg);
+    float so = 0.f, sl = 0.f;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) so += xo[j] * xo[j], sl += xl[j] * xl[j];
+    for (int m = 1; m < d8n; m <<= 1) {
+      so += __shfl_xor(so, m);
+      sl += __shfl_xor(sl, m);
+    }
+    const float ro = rsqrtf(so / (float)Dv + eps);
+    const float rl = rsqrtf(sl / (float)Dv + eps);
+    float out[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const float s = sigmoidf_(xg[j]);
+      float v = xo[j] * ro * wg[d8 * 8 + j] * s + xl[j] * rl * wl[d8 * 8 + j] * (1.f - s);
+      if (silu_out) v = v * sigmoidf_(v);
+      out[j] = v;
+    }
+    if (live) Vec8<T>::store(y + ii * 8, out);
+  }
+}
+
+int launch_locality_blend(const void* o, const void* loc, const void* glin, const float* wg, const float* wl, void* y,
+                          int B, int H, int L, int Dv, float eps, int silu_out, int io_dtype, hipStream_t stream) {
+  const size_t nvec = (size_t)B * L * H * (Dv / 8);
+  const int grid = (int)((nvec + 255) / 256 < 65535 * 8 ? (nvec + 255) / 256 : 65535 * 8);
+  if (io_dtype == 0)
+    hipLaunchKernelGGL((locality_blend_kernel<float>), dim3(grid), dim3(256), 0, stream, (const float*)o,
+                       (const float*)loc, (const float*)glin, wg, wl, (float*)y, H, L, Dv, eps, silu_out, nvec);
+  else
+    hipLaunchKernelGGL((locality_blend_kernel<uint16_t>), dim3(grid), dim3(256), 0, stream, (const uint16_t*)o,
+                       (const uint16_t*)loc, (const uint16_t*)glin, wg, wl, (uint16_t*)y, H, L, Dv, eps, silu_out,
+                       nvec);
+  return hipGetLastError() == hipSuccess ? 0 : -5;
+}
+
+}  // namespace vig

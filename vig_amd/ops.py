@@ -1,0 +1,222 @@
+"""Op-level Python interface: the reference's GLA call signatures over the HIP library.
+
+Mirrors (same names, positional order, defaults and return convention):
+  fused_chunk_gla              flash-linear-attention/fla/ops/gla/chunk_fuse.py:554-572
+  batch_bid_fused_chunk_gla    fla/ops/gla/chunk_fuse.py:574-596
+  bid_fused_recurrent_gla      fla/ops/gla/recurrent_fuse.py:659-676
+  fused_recurrent_gla          fla/ops/gla/recurrent_fuse.py:631-657
+Forward only: the outputs carry no autograd graph (the reference's own
+bidirectional backward is not functional, recurrent_fuse.py:443,456).
+"""
+from __future__ import annotations
+
+import math
+from typing import Optional, Tuple
+
+import torch
+
+from . import _lib
+
+_DT = {torch.float32: _lib.VIG_F32, torch.bfloat16: _lib.VIG_BF16}
+
+
+def _stream_ptr(t: torch.Tensor) -> int:
+    return torch.cuda.current_stream(t.device).cuda_stream
+
+
+def _dt(t: torch.Tensor) -> int:
+    try:
+        return _DT[t.dtype]
+    except KeyError:
+        raise TypeError(f"unsupported dtype {t.dtype}; float32 and bfloat16 are built") from None
+
+
+def _check_cuda(*ts):
+    for t in ts:
+        if t is None:
+            continue
+        if not t.is_cuda:
+            raise _lib.VigGlaError("vig_amd ops run on the GPU only (tensor is on %s); there is no CPU path" % t.device)
+        if t.device != ts[0].device:
+            raise ValueError("all tensors must be on the same device")
+
+
+def gla_bidir_forward(q, k, v, g_fwd, g_bwd=None, scale: float = -1, out_scale: float = 1.0,
+                      exact: bool = False, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """o = out_scale * (fwd(q,k,v,g_fwd) + bwd(q,k,v,g_bwd)), natural token order.
+
+    q, k, g_*: [B,H,L,Dk]; v: [B,H,L,Dv].  g_bwd=None gives the causal op.
+    `exact=True` forces the fp32-arithmetic recurrent kernel.
+    """
+    lib = _lib.load()
+    _check_cuda(q, k, v, g_fwd, g_bwd)
+    q, k, v, g_fwd = (t.contiguous() for t in (q, k, v, g_fwd))
+    if g_bwd is not None:
+        g_bwd = g_bwd.contiguous()
+        if g_bwd.dtype != g_fwd.dtype or g_bwd.shape != g_fwd.shape:
+            raise ValueError("g_bwd must match g_fwd in dtype and shape")
+    B, H, L, Dk = q.shape
+    Dv = v.shape[-1]
+    if k.shape != q.shape or g_fwd.shape != q.shape or v.shape[:3] != q.shape[:3]:
+        raise ValueError("shape mismatch between q, k, v, g")
+    if k.dtype != q.dtype or v.dtype != q.dtype:
+        raise TypeError("q, k, v must share a dtype")
+    if scale == -1 or scale is None:
+        scale = Dk ** -0.5
+    io_dt, g_dt = _dt(q), _dt(g_fwd)
+    if out is None:
+        out = torch.empty(B, H, L, Dv, dtype=q.dtype, device=q.device)
+    elif not (out.is_contiguous() and out.shape == (B, H, L, Dv) and out.dtype == q.dtype):
+        raise ValueError("bad `out` tensor")
+    fn = lib.vig_gla_bidir_fwd_exact if exact else lib.vig_gla_bidir_fwd
+    ws_bytes = lib.vig_gla_bidir_fwd_workspace(B, H, L, Dk, Dv, io_dt)
+    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=q.device) if ws_bytes else None
+    with torch.cuda.device(q.device):
+        rc = fn(q.data_ptr(), k.data_ptr(), v.data_ptr(), g_fwd.data_ptr(),
+                g_bwd.data_ptr() if g_bwd is not None else None, out.data_ptr(),
+                ws.data_ptr() if ws is not None else None, ws_bytes,
+                B, H, L, Dk, Dv, float(scale), float(out_scale), io_dt, g_dt, _stream_ptr(q))
+    _lib.check(rc, "vig_gla_bidir_fwd")
+    if ws is not None:
+        ws.record_stream(torch.cuda.current_stream(q.device))
+    return out
+
+
+def _split_bid_gates(q, g):
+    B = q.shape[0]
+    if g.shape[0] != 2 * B:
+        raise ValueError(f"bidirectional gates must be [2B,H,L,Dk]; got batch {g.shape[0]} for B={B}")
+    return g[:B], g[B:]
+
+
+def fused_chunk_gla(q, k, v, g, scale: int = -1, initial_state=None, output_final_state: bool = False
+                    ) -> Tuple[torch.Tensor, Optional[torch.Tensor]]:
+    """Causal GLA on [B,H,L,D] tensors; returns (o, final_state=None)."""
+    if initial_state is not None or output_final_state:
+        raise NotImplementedError("initial_state / output_final_state are not built in the HIP path")
+    return gla_bidir_forward(q, k, v, g, None, scale, 1.0), None
+
+
+def fused_recurrent_gla(q, k, v, gk=None, gv=None, scale: int = -1, initial_state=None,
+                        output_final_state: bool = False, causal: bool = True):
+    """Causal recurrent GLA (fp32 state arithmetic); causal=False returns [o, o_reversed] with shared gates."""
+    if gv is not None:
+        raise NotImplementedError("value gates (gv) are not used by ViG and not built")
+    if initial_state is not None or output_final_state:
+        raise NotImplementedError("initial_state / output_final_state are not built in the HIP path")
+    if gk is None:
+        gk = torch.zeros_like(q)
+    o = gla_bidir_forward(q, k, v, gk, None, scale, 1.0, exact=True)
+    if causal:
+        return o, None
+    f = lambda x: x.flip(dims=[2])
+    o_rev = f(gla_bidir_forward(f(q), f(k), f(v), f(gk), None, scale, 1.0, exact=True))
+    return [o, o_rev]
+
+
+def batch_bid_fused_chunk_gla(q, k, v, g, scale: int = -1, initial_state=None, output_final_state: bool = False
+                              ) -> Tuple[torch.Tensor, Optional[torch.Tensor]]:
+    """q,k,v [B,H,L,D]; g [2B,H,L,Dk] = cat(fwd gates, bwd gates), both in natural order; o=(o_f+o_b)/2."""
+    if initial_state is not None or output_final_state:
+        raise NotImplementedError("bidirectional GLA takes no initial/final state")
+    gf, gb = _split_bid_gates(q, g)
+    return gla_bidir_forward(q, k, v, gf, gb, scale, 0.5), None
+
+
+def bid_fused_recurrent_gla(q, k, v, gk=None, gv=None, scale: int = -1, initial_state=None,
+                            output_final_state: bool = False, causal: bool = True
+                            ) -> Tuple[torch.Tensor, Optional[torch.Tensor]]:
+    """Merged bidirectional inference op: gk [2B,H,L,Dk] natural order; o=(o_f+o_b)/2."""
+    if gv is not None:
+        raise NotImplementedError("value gates (gv) are not used by ViG and not built")
+    if initial_state is not None or output_final_state:
+        raise NotImplementedError("bidirectional GLA takes no initial/final state")
+    if not causal:
+        raise NotImplementedError("causal=False on the merged op is unused by ViG and not built")
+    if gk is None:
+        gk = torch.zeros((2 * q.shape[0],) + tuple(q.shape[1:]), dtype=q.dtype, device=q.device)
+    gf, gb = _split_bid_gates(q, gk)
+    return gla_bidir_forward(q, k, v, gf, gb, scale, 0.5), None
+
+
+# ---------------------------------------------------------------------------
+# neighbours
+# ---------------------------------------------------------------------------
+
+def dirgate(gk_lin: torch.Tensor, num_heads: int, gate_logit_normalizer: float = 16.0,
+            clamp_min: Optional[float] = None, out_dtype: Optional[torch.dtype] = None) -> torch.Tensor:
+    """gk_lin [B,L,2*H*Dk] -> [2,B,H,L,Dk] = logsigmoid/normalizer (vig.py:432-441)."""
+    lib = _lib.load()
+    _check_cuda(gk_lin)
+    gk_lin = gk_lin.contiguous()
+    B, L, C2 = gk_lin.shape
+    Dk = C2 // (2 * num_heads)
+    out_dtype = out_dtype or gk_lin.dtype
+    out = torch.empty(2, B, num_heads, L, Dk, dtype=out_dtype, device=gk_lin.device)
+    with torch.cuda.device(gk_lin.device):
+        rc = lib.vig_dirgate_fwd(gk_lin.data_ptr(), out.data_ptr(), B, L, num_heads, Dk,
+                                 1.0 / float(gate_logit_normalizer),
+                                 float("nan") if clamp_min is None else float(clamp_min),
+                                 _dt(gk_lin), _DT[out_dtype], _stream_ptr(gk_lin))
+    _lib.check(rc, "vig_dirgate_fwd")
+    return out
+
+
+def dwconv3x3(x: torch.Tensor, weight: torch.Tensor, hw, bias: Optional[torch.Tensor] = None,
+              silu: bool = False) -> torch.Tensor:
+    """x [B,L,C] on the (h,w) token grid; weight [C,1,3,3] or [C,3,3]; returns [B,L,C]."""
+    lib = _lib.load()
+    _check_cuda(x, weight, bias)
+    x = x.contiguous()
+    B, L, C = x.shape
+    h, w = hw
+    if L != h * w:
+        raise ValueError("L must equal h*w")
+    wt = weight.detach().reshape(C, 9).float().contiguous()
+    bs = bias.detach().float().contiguous() if bias is not None else None
+    y = torch.empty_like(x)
+    with torch.cuda.device(x.device):
+        rc = lib.vig_dwconv3x3_fwd(x.data_ptr(), wt.data_ptr(), bs.data_ptr() if bs is not None else None,
+                                   y.data_ptr(), B, h, w, C, int(silu), _dt(x), _stream_ptr(x))
+    _lib.check(rc, "vig_dwconv3x3_fwd")
+    return y
+
+
+def locality_gate(o: torch.Tensor, weight: torch.Tensor, hw) -> torch.Tensor:
+    """y = o * sigmoid(dwconv3x3(o)) on [B,H,L,Dv] with channel = head*Dv + d."""
+    lib = _lib.load()
+    _check_cuda(o, weight)
+    o = o.contiguous()
+    B, H, L, Dv = o.shape
+    h, w = hw
+    if L != h * w:
+        raise ValueError("L must equal h*w")
+    wt = weight.detach().reshape(H * Dv, 9).float().contiguous()
+    y = torch.empty_like(o)
+    with torch.cuda.device(o.device):
+        rc = lib.vig_locality_gate_fwd(o.data_ptr(), wt.data_ptr(), y.data_ptr(), B, H, h, w, Dv, _dt(o),
+                                       _stream_ptr(o))
+    _lib.check(rc, "vig_locality_gate_fwd")
+    return y
+
+
+def locality_blend(o: torch.Tensor, local: torch.Tensor, g_lin: torch.Tensor, w_g: torch.Tensor,
+                   w_l: torch.Tensor, eps: float = 1e-6, silu_out: bool = False) -> torch.Tensor:
+    """Block epilogue (vig.py:444-457): o [B,H,L,Dv]; local, g_lin [B,L,H*Dv] -> y [B,L,H*Dv]."""
+    lib = _lib.load()
+    _check_cuda(o, local, g_lin, w_g, w_l)
+    o, local, g_lin = o.contiguous(), local.contiguous(), g_lin.contiguous()
+    B, H, L, Dv = o.shape
+    if local.shape != (B, L, H * Dv) or g_lin.shape != (B, L, H * Dv):
+        raise ValueError("local and g_lin must be [B, L, H*Dv]")
+    if local.dtype != o.dtype or g_lin.dtype != o.dtype:
+        raise TypeError("o, local, g_lin must share a dtype")
+    y = torch.empty_like(local)
+    wg = w_g.detach().float().contiguous()
+    wl = w_l.detach().float().contiguous()
+    with torch.cuda.device(o.device):
+        rc = lib.vig_locality_blend_fwd(o.data_ptr(), local.data_ptr(), g_lin.data_ptr(), wg.data_ptr(),
+                                        wl.data_ptr(), y.data_ptr(), B, H, L, Dv, float(eps), int(silu_out),
+                                        _dt(o), _stream_ptr(o))
+    _lib.check(rc, "vig_locality_blend_fwd")
+    return y
