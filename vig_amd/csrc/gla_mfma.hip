@@ -1,23 +1,27 @@
 // Bidirectional chunked GLA forward on bf16 MFMA tiles (gfx950), Dk = Dv = 64.
 //
-// One workgroup (4 waves) per (batch, head) slab of up to 256 tokens; wave w owns a
-// contiguous chunk of ceil(L/4) <= 64 tokens.  Per direction a wave
+// One persistent workgroup of 8 waves per CU walks (batch, head) slabs of up to 256
+// tokens.  A slab is cut into 4 chunks of ceil(L/4) <= 64 tokens; wave (chunk c,
+// direction d) handles one chunk in one direction, so the two directions of a chunk run
+// side by side on the same SIMD and read the same q/k/v lines.  A wave
 //   1. forms the chunk-local cumulative log-gates G with a triangular-ones MFMA
 //      (bf16 gates are exact MFMA inputs, the sums accumulate in fp32),
-//   2. builds end-anchored operands q~ = s*q*exp(G - G_end) (>= |sq|) and
-//      k~ = k*exp(G_end - G) (<= |k|), split into bf16 hi + lo,
+//   2. builds end-anchored operands q~ = q*exp(G - G_end) (>= |q|) and
+//      k~ = k*exp(G_end - G) (<= |k|), each split into bf16 hi + lo,
 //   3. computes the masked intra-chunk scores P^T = k~ q~^T with three MFMA terms
 //      (hi*hi + lo*hi + hi*lo) and P V with P split hi + lo  (V is exact bf16),
-//   4. accumulates the chunk's state contribution U = k~^T V  [Dk x Dv] fp32.
-// The four U's meet once per direction in LDS; each wave folds the ones before it
-// (after it, for the reverse direction) into its incoming state S_in and adds
-// q~ (exp(G_end) * S_in) to its outputs.  Outputs of both directions are summed in
-// the MFMA accumulators and stored once.
+//   4. accumulates the chunk's state contribution U = k~^T V  [Dk x Dv] in fp32.
+// The U's of a direction meet once in LDS, where the four waves of the direction run the
+// chunk-to-chunk state recurrence S <- exp(G_end) * S + U in parallel over disjoint state
+// slices and leave, for every chunk, the decayed incoming state as ready bf16 MFMA
+// fragments; each wave adds q~ (exp(G_end) * S_in) to its outputs.  The two waves of a
+// chunk then swap half of their fp32 output tiles through LDS, add, scale and store
+// bf16 once.  Loads for the next slab are issued before the swap.
 //
 // Chunk algebra follows flash-linear-attention/fla/ops/gla/chunk_util.py:9-78 and
 // chunk_fuse.py:76-97,245-254 (here with 64-token chunks, an end anchor so that the
 // state update needs no second set of factors, and matrix-core intra-chunk scores);
-// the two directions share q/k/v registers as in recurrent_fuse.py:19-148.
+// both directions are served by one launch as in recurrent_fuse.py:19-148.
 //
 // Register layouts (lane l: r = l & 31, h = l >> 5), v_mfma_f32_32x32x16_bf16:
 //   A/B operand: lane supplies index r and contraction slots e = 0..7 (4 VGPRs);
@@ -26,21 +30,44 @@
 // two adjacent channels per token and de-interleaved with v_perm_b32; lane-row rho
 // reads channel pair cpair(rho), chosen so that every accumulator ends up holding
 // 32 contiguous channels (32*h + 8*g + 2*m + p) of one token.
+//
+// Supported gate range: sum of |g| over any 64-token chunk and channel below ~80
+// (exp2 arguments stay finite); ViG's logsigmoid(.)/16 gates are far inside it.
 #include "common.h"
 #include "launch.h"
+#ifdef VIG_TIMING
+#include <stdlib.h>
+#endif
 
 namespace vig {
 
 namespace {
 
+// Scheduling fence: keeps the machine scheduler from hoisting the next phase's loads over this one's math.
+#define VIG_PHASE() __builtin_amdgcn_sched_barrier(0)
+
+// Optional phase timing (development builds only: -DVIG_TIMING): lane 0 of every wave of workgroup 0 records the
+// shader clock at phase boundaries of each slab it walks.
+#ifdef VIG_TIMING
+__device__ unsigned long long g_stamp[4][8][16];
+#define VIG_STAMP(id)                                                                                           \
+  do {                                                                                                          \
+    VIG_PHASE();                                                                                                \
+    if ((lane & 63) == 0 && blockIdx.x == 0 && iter < 4) g_stamp[iter][wi][id] = __builtin_readcyclecounter(); \
+    VIG_PHASE();                                                                                                \
+  } while (0)
+#else
+#define VIG_STAMP(id) \
+  do {                \
+  } while (0)
+#endif
+
 constexpr float kLog2e = 1.4426950408889634f;
-constexpr int kKtStride = 72;                      // bf16 elements per k~ row in LDS (144 B: conflict-free b128 writes)
-constexpr int kKtBytes = 64 * kKtStride * 2;       // per wave
-constexpr int kSlotBytes = 16 * 1024;              // one published U (64x64 fp32)
-constexpr int kLdsKt = 0;
-constexpr int kLdsSlots = 4 * kKtBytes;            // 36864
-constexpr int kLdsDvec = kLdsSlots + 3 * kSlotBytes;  // 86016
-constexpr int kLdsTotal = kLdsDvec + 4 * 64 * 4;   // + 1 KB decay vectors
+constexpr int kKtStride = 72;                // bf16 elements per k~ row in LDS (144 B: conflict-free b128 writes)
+constexpr int kRegionBytes = 16 * 1024;      // per wave: k~ scratch, then published U / state fragments / output half
+constexpr int kLdsDvec = 8 * kRegionBytes;   // per wave: 64 chunk decays exp(G_end)
+constexpr int kLdsGend = kLdsDvec + 8 * 64 * 4;  // per wave: 64 anchors G_end * log2(e), laid out [h][p][16]
+constexpr int kLdsTotal = kLdsGend + 8 * 64 * 4;
 
 __device__ __forceinline__ f32x16_t mfma(const u32x4_t& a, const u32x4_t& b, const f32x16_t& c) {
   return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, a), __builtin_bit_cast(bf16x8_t, b), c, 0,
@@ -54,36 +81,70 @@ __device__ __forceinline__ int jmap(int t, int h, int e) { return 16 * t + 4 * h
 
 __device__ __forceinline__ float exp2_fast(float x) { return __builtin_amdgcn_exp2f(x); }
 
-// Transposed fragments of a row-major [tokens][64] bf16 tile (global memory): frag[t][p] is the operand
-// whose lane index is channel 2*cpair(r)+p and whose slots are the 8 tokens jmap(t,h,.).
-__device__ __forceinline__ void load_tfrags_global(const uint16_t* rows, int nvalid, int r, int h,
-                                                   u32x4_t (&frag)[4][2]) {
-  const int c2 = 2 * cpair(r);
+// LDS traffic inside one wave (k~ rows written by token lanes, read back by channel lanes): the LDS pipe is in
+// order per wave, so only the compiler has to be kept from reordering.
+__device__ __forceinline__ void wave_lds_sync() {
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+  __builtin_amdgcn_wave_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+}
+
+// Workgroup barrier that orders LDS traffic only: global loads issued before it (the next slab's prefetch)
+// stay in flight across it, which a full __syncthreads() fence would drain.
+__device__ __forceinline__ void lds_barrier() {
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
+  __builtin_amdgcn_s_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
+}
+
+// ---------------------------------------------------------------------------------------------------------
+// Loads.  Every load is unconditional on a clamped row (no divergent branches around memory operations);
+// padding rows are zeroed by a select when the data is consumed.  `rows` points at the chunk's first token.
+// ---------------------------------------------------------------------------------------------------------
+
+// raw dwords of the transposed fragments of k-steps [T0, T0+NT): D[t][e] = channels (2*cpair(r), +1) of token jmap(t,h,e)
+template <int T0, int NT>
+__device__ __forceinline__ void issue_tdwords(const uint16_t* rows, int nvalid, int r, int h, uint32_t (&D)[NT][8]) {
+  const unsigned c2 = 2 * cpair(r);
+  const int nlast = max(nvalid - 1, 0);
 #pragma unroll
-  for (int t = 0; t < 4; ++t) {
-    uint32_t D[8];
+  for (int t = 0; t < NT; ++t)
 #pragma unroll
     for (int e = 0; e < 8; ++e) {
-      const int tok = jmap(t, h, e);
-      D[e] = tok < nvalid ? *reinterpret_cast<const uint32_t*>(rows + (size_t)tok * 64 + c2) : 0u;
+      const unsigned tok = (unsigned)min(jmap(T0 + t, h, e), nlast);
+      D[t][e] = *reinterpret_cast<const uint32_t*>(rows + (tok * 64u + c2));
     }
+}
+
+// fragments from raw dwords: frag[t][p] has lane index = channel 2*cpair(r)+p, slots = tokens jmap(t,h,.)
+template <int T0, int NT, bool ZERO_PAD>
+__device__ __forceinline__ void finish_tfrags(const uint32_t (&D)[NT][8], int nvalid, int h, u32x4_t (&frag)[NT][2]) {
+#pragma unroll
+  for (int t = 0; t < NT; ++t) {
+    uint32_t d[8];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) d[e] = (!ZERO_PAD || jmap(T0 + t, h, e) < nvalid) ? D[t][e] : 0u;
 #pragma unroll
     for (int x = 0; x < 4; ++x) {
-      frag[t][0][x] = __builtin_amdgcn_perm(D[2 * x + 1], D[2 * x], 0x05040100u);
-      frag[t][1][x] = __builtin_amdgcn_perm(D[2 * x + 1], D[2 * x], 0x07060302u);
+      frag[t][0][x] = __builtin_amdgcn_perm(d[2 * x + 1], d[2 * x], 0x05040100u);
+      frag[t][1][x] = __builtin_amdgcn_perm(d[2 * x + 1], d[2 * x], 0x07060302u);
     }
   }
 }
 
-// Same, one k-step, from the wave's k~ scratch in LDS.
+// raw rows of one 32-token tile: lane (r, h) reads token 32*it + r, channels [32h, 32h+32) as four 16-byte pieces
+__device__ __forceinline__ void issue_raw_tile(const uint16_t* rows, int it, int nvalid, int r, int h, u32x4_t (&raw)[4]) {
+  const unsigned rowc = (unsigned)min(32 * it + r, max(nvalid - 1, 0));
+#pragma unroll
+  for (int gq = 0; gq < 4; ++gq) raw[gq] = *reinterpret_cast<const u32x4_t*>(rows + (rowc * 64u + 32u * h + 8u * gq));
+}
+
+// one k-step of transposed fragments from the wave's k~ scratch in LDS
 __device__ __forceinline__ void load_tfrag_lds(const uint16_t* kt, int t, int r, int h, u32x4_t (&frag)[2]) {
   const int c2 = 2 * cpair(r);
   uint32_t D[8];
 #pragma unroll
-  for (int e = 0; e < 8; ++e) {
-    const int tok = jmap(t, h, e);
-    D[e] = *reinterpret_cast<const uint32_t*>(kt + tok * kKtStride + c2);
-  }
+  for (int e = 0; e < 8; ++e) D[e] = *reinterpret_cast<const uint32_t*>(kt + jmap(t, h, e) * kKtStride + c2);
 #pragma unroll
   for (int x = 0; x < 4; ++x) {
     frag[0][x] = __builtin_amdgcn_perm(D[2 * x + 1], D[2 * x], 0x05040100u);
@@ -106,53 +167,52 @@ __device__ __forceinline__ u32x4_t tri_frag(int t, int it, int r, int h) {
   return f;
 }
 
-struct Operands {
-  u32x4_t qh[4], ql[4], kh[4], kl[4];  // one 32-token tile, [k-step]
+struct HalfOps {
+  u32x4_t h[4], l[4];  // bf16 hi / lo fragments of one 32-token tile, per k-step (16 channels)
 };
 
-// q~ / k~ of one 32-token tile, split into bf16 hi (round to nearest) + lo (the fp32 remainder, rounded).
-__device__ __forceinline__ void make_operands(const u32x4_t (&qraw)[4], const u32x4_t (&kraw)[4],
-                                              const f32x16_t (&G)[2], const float (&gend2)[2][16], float l2scale,
-                                              Operands& op) {
+// q~ (ISQ) or k~ of one 32-token tile: raw * exp(+-(G - G_end)), split into bf16 hi (round to nearest) and
+// lo (the fp32 remainder, rounded).  `live` zeroes padding rows (needed for k~ only: q~ of a padding row only
+// feeds outputs that are never stored).
+template <bool ISQ>
+__device__ __forceinline__ void make_half(const u32x4_t (&raw)[4], bool live, const f32x16_t (&G)[2],
+                                          const float* gend2 /* LDS, this lane half: [p][16] */, HalfOps& op) {
 #pragma unroll
   for (int g = 0; g < 4; ++g) {
+    const f32x4_t a0 = *reinterpret_cast<const f32x4_t*>(gend2 + 4 * g);
+    const f32x4_t a1 = *reinterpret_cast<const f32x4_t*>(gend2 + 16 + 4 * g);
 #pragma unroll
     for (int m = 0; m < 4; ++m) {
       const int c = 4 * g + m;
-      float qt[2], kt[2];
+      const uint32_t w = (ISQ || live) ? raw[g][m] : 0u;
+      float t[2];
 #pragma unroll
       for (int p = 0; p < 2; ++p) {
-        const float Gv = G[p][c];
-        const float xq = __builtin_fmaf(Gv, kLog2e, l2scale - gend2[p][c]);
-        const float xk = __builtin_fmaf(Gv, -kLog2e, gend2[p][c]);
-        const float qf = p ? bf16hi_to_f32(qraw[g][m]) : bf16lo_to_f32(qraw[g][m]);
-        const float kf = p ? bf16hi_to_f32(kraw[g][m]) : bf16lo_to_f32(kraw[g][m]);
-        qt[p] = qf * exp2_fast(xq);
-        kt[p] = kf * exp2_fast(xk);
+        const float an = p ? a1[m] : a0[m];
+        const float x = ISQ ? __builtin_fmaf(G[p][c], kLog2e, -an) : __builtin_fmaf(G[p][c], -kLog2e, an);
+        const float f = p ? bf16hi_to_f32(w) : bf16lo_to_f32(w);
+        t[p] = f * exp2_fast(x);
       }
-      const uint32_t qhi = pack_bf16x2(qt[0], qt[1]);
-      const uint32_t khi = pack_bf16x2(kt[0], kt[1]);
-      op.qh[g][m] = qhi;
-      op.kh[g][m] = khi;
-      op.ql[g][m] = pack_bf16x2(qt[0] - bf16lo_to_f32(qhi), qt[1] - bf16hi_to_f32(qhi));
-      op.kl[g][m] = pack_bf16x2(kt[0] - bf16lo_to_f32(khi), kt[1] - bf16hi_to_f32(khi));
+      const uint32_t hi = pack_bf16x2(t[0], t[1]);
+      op.h[g][m] = hi;
+      op.l[g][m] = pack_bf16x2(t[0] - bf16lo_to_f32(hi), t[1] - bf16hi_to_f32(hi));
     }
   }
 }
 
 // P^T tile = k~ (rows j) x q~ (columns i), three-term split product.
-__device__ __forceinline__ f32x16_t score_tile(const Operands& kop, const Operands& qop) {
+__device__ __forceinline__ f32x16_t score_tile(const HalfOps& kop, const HalfOps& qop) {
   f32x16_t acc = {0.f};
 #pragma unroll
   for (int ks = 0; ks < 4; ++ks) {
-    acc = mfma(kop.kh[ks], qop.qh[ks], acc);
-    acc = mfma(kop.kl[ks], qop.qh[ks], acc);
-    acc = mfma(kop.kh[ks], qop.ql[ks], acc);
+    acc = mfma(kop.h[ks], qop.h[ks], acc);
+    acc = mfma(kop.l[ks], qop.h[ks], acc);
+    acc = mfma(kop.h[ks], qop.l[ks], acc);
   }
   return acc;
 }
 
-// O^T[p][it] += V^T (k-steps of token tile jt) x P^T tile, with P split hi + lo.
+// O^T[p] += V^T (k-steps 2*jt, 2*jt+1 of vfrag) x P^T tile, with P split hi + lo.
 // MASK: 0 none, 1 keep j <= i (forward diagonal tile), 2 keep j >= i (reverse diagonal tile).
 template <int MASK>
 __device__ __forceinline__ void apply_scores(f32x16_t P, int jt, int r, int h, const u32x4_t (&vfrag)[4][2],
@@ -188,26 +248,53 @@ __device__ __forceinline__ void store_kt(uint16_t* kt, int row, int h, const u32
   for (int g = 0; g < 4; ++g) *reinterpret_cast<u32x4_t*>(kt + row * kKtStride + 32 * h + 8 * g) = kh[g];
 }
 
-// One direction of one wave's chunk: intra-chunk outputs into O, hi q~ fragments kept for the
-// inter-chunk product, chunk state contribution U, and the chunk's total log-decay gend (natural log)
-// for the lane's 32 channels.
+// LDS "unit" u of a region = 64 lanes x 16 B, register-native: lane l owns bytes [(u*64 + l)*16, +16).
+__device__ __forceinline__ char* unit_ptr(char* region, int u, int lane) { return region + (u * 64 + lane) * 16; }
+
+// What a wave carries from the end of one slab to the start of the next: the loads of its first phase.
+struct Prefetch {
+  uint32_t gD[4][8];         // gate dwords, all four k-steps of the chunk
+  uint32_t vD[2][8];         // V dwords of the tile walked first
+  u32x4_t rawk[4], rawq[4];  // raw rows of the tile walked first
+};
+
 template <bool FWD>
-__device__ __forceinline__ void direction_pass(const uint16_t* grows, int nvalid, int r, int h, float l2scale,
-                                               const u32x4_t (&qraw)[2][4], const u32x4_t (&kraw)[2][4],
-                                               const u32x4_t (&vfrag)[4][2], f32x16_t (&O)[2][2],
-                                               u32x4_t (&qkeep)[2][4], float (&gend)[2][16], f32x16_t (&U)[2][2],
-                                               uint16_t* kt) {
-  // ---- cumulative log-gates G[it][p] via triangular-ones MFMA ----
+__device__ __forceinline__ void issue_first_phase(const uint16_t* q, const uint16_t* k, const uint16_t* v,
+                                                  const uint16_t* g, int nvalid, int r, int h, Prefetch& pf) {
+  constexpr int TA = FWD ? 0 : 1;
+  issue_tdwords<0, 4>(g, nvalid, r, h, pf.gD);
+  issue_raw_tile(k, TA, nvalid, r, h, pf.rawk);
+  issue_raw_tile(q, TA, nvalid, r, h, pf.rawq);
+  issue_tdwords<2 * TA, 2>(v, nvalid, r, h, pf.vD);
+}
+
+// Everything one wave does for one slab: chunk c (nvalid tokens starting at the row the pointers address) in
+// direction FWD / reverse.  Every wave of the workgroup passes the same three barriers here (plus the caller's).
+template <bool FWD>
+__device__ __forceinline__ void direction_wave(const uint16_t* q, const uint16_t* k, const uint16_t* v,
+                                               const uint16_t* g, uint16_t* o, const uint16_t* qn, const uint16_t* kn,
+                                               const uint16_t* vn, const uint16_t* gn, bool has_next, int nvalid, int c,
+                                               int lane, char* lds, float oscale, bool bidir, Prefetch& pf, int iter) {
+  const int r = lane & 31, h = lane >> 5;
+  const int wi = (FWD ? 0 : 4) + c;
+  constexpr int TA = FWD ? 0 : 1;  // tile walked first
+  constexpr int TB = FWD ? 1 : 0;
+  char* region = lds + wi * kRegionBytes;
+  uint16_t* kt = reinterpret_cast<uint16_t*>(region);
+  float* dvec_all = reinterpret_cast<float*>(lds + kLdsDvec);
+  if (!FWD) issue_first_phase<FWD>(q, k, v, g, nvalid, r, h, pf);
+  VIG_STAMP(0);
+
+  // ---- cumulative log-gates G[it][p] via triangular-ones MFMA on transposed gate fragments ----
   f32x16_t G[2][2];
   {
     u32x4_t gfrag[4][2];
-    load_tfrags_global(grows, nvalid, r, h, gfrag);
+    finish_tfrags<0, 4, true>(pf.gD, nvalid, h, gfrag);
     const u32x4_t ones = {0x3F803F80u, 0x3F803F80u, 0x3F803F80u, 0x3F803F80u};
 #pragma unroll
     for (int p = 0; p < 2; ++p) {
       f32x16_t g0 = {0.f}, g1 = {0.f};
       if (FWD) {
-        // tokens i of tile 0 see j in tile 0 (masked); tile 1 sees all of tile 0 and masked tile 1
         g0 = mfma(gfrag[0][p], tri_frag<true>(0, 0, r, h), g0);
         g0 = mfma(gfrag[1][p], tri_frag<true>(1, 0, r, h), g0);
         g1 = mfma(gfrag[0][p], ones, g1);
@@ -226,234 +313,323 @@ __device__ __forceinline__ void direction_pass(const uint16_t* grows, int nvalid
       G[1][p] = g1;
     }
   }
-  // ---- anchor: G at the last token (forward) / first token (reverse) of the chunk, same channels per lane half ----
-  float gend2[2][16];
+  VIG_STAMP(1);
+  // ---- anchor: G at the last token (forward) / first token (reverse) of the chunk, same channels per lane half.
+  // The anchors (x log2 e) and the chunk decays exp(G_end) go to LDS: the operand builders re-read the former per
+  // tile, the state recurrence reads the latter after barrier A, and no register holds them across phases. ----
+  float* gend2 = reinterpret_cast<float*>(lds + kLdsGend) + wi * 64 + 32 * h;
   {
     const int src = ((FWD ? 31 : 0) + 32 * h) << 2;
-#pragma unroll
-    for (int p = 0; p < 2; ++p) {
-#pragma unroll
-      for (int c = 0; c < 16; ++c) {
-        const float a = FWD ? G[1][p][c] : G[0][p][c];
-        const float e = __int_as_float(__builtin_amdgcn_ds_bpermute(src, __float_as_int(a)));
-        gend[p][c] = e;
-        gend2[p][c] = e * kLog2e;
-      }
-    }
-  }
-  // ---- intra-chunk scores, tile by tile ----
-  constexpr int TA = FWD ? 0 : 1;  // first tile walked
-  constexpr int TB = FWD ? 1 : 0;
-  Operands a, b;
-  make_operands(qraw[TA], kraw[TA], G[TA], gend2, l2scale, a);
-  apply_scores<FWD ? 1 : 2>(score_tile(a, a), TA, r, h, vfrag, O[0][TA], O[1][TA]);
-  store_kt(kt, 32 * TA + r, h, a.kh);
-#pragma unroll
-  for (int ks = 0; ks < 4; ++ks) qkeep[TA][ks] = a.qh[ks];
-  make_operands(qraw[TB], kraw[TB], G[TB], gend2, l2scale, b);
-  apply_scores<0>(score_tile(a, b), TA, r, h, vfrag, O[0][TB], O[1][TB]);
-  apply_scores<FWD ? 1 : 2>(score_tile(b, b), TB, r, h, vfrag, O[0][TB], O[1][TB]);
-  store_kt(kt, 32 * TB + r, h, b.kh);
-#pragma unroll
-  for (int ks = 0; ks < 4; ++ks) qkeep[TB][ks] = b.qh[ks];
-  __syncthreads();
-  // ---- chunk state contribution U[p'][pv] = k~^T V ----
-#pragma unroll
-  for (int i = 0; i < 2; ++i)
-#pragma unroll
-    for (int j = 0; j < 2; ++j) U[i][j] = f32x16_t{0.f};
-#pragma unroll
-  for (int t = 0; t < 4; ++t) {
-    u32x4_t ktf[2];
-    load_tfrag_lds(kt, t, r, h, ktf);
-#pragma unroll
-    for (int pk = 0; pk < 2; ++pk)
-#pragma unroll
-      for (int pv = 0; pv < 2; ++pv) U[pk][pv] = mfma(ktf[pk], vfrag[t][pv], U[pk][pv]);
-  }
-}
-
-__device__ __forceinline__ void publish_state(char* lds, int slot, int lane, const f32x16_t (&U)[2][2]) {
-  char* base = lds + kLdsSlots + slot * kSlotBytes;
-#pragma unroll
-  for (int pk = 0; pk < 2; ++pk)
-#pragma unroll
-    for (int pv = 0; pv < 2; ++pv)
-#pragma unroll
-      for (int cq = 0; cq < 4; ++cq) {
-        f32x4_t x = {U[pk][pv][4 * cq], U[pk][pv][4 * cq + 1], U[pk][pv][4 * cq + 2], U[pk][pv][4 * cq + 3]};
-        *reinterpret_cast<f32x4_t*>(base + (((pk * 2 + pv) * 4 + cq) * 64 + lane) * 16) = x;
-      }
-}
-
-__device__ __forceinline__ void publish_decay(char* lds, int w, int r, int h, const float (&gend)[2][16]) {
-  if (r == 0) {
-    float* d = reinterpret_cast<float*>(lds + kLdsDvec) + w * 64 + 32 * h;
+    float e2[2][16];
 #pragma unroll
     for (int p = 0; p < 2; ++p)
 #pragma unroll
-      for (int c = 0; c < 16; ++c) d[8 * (c >> 2) + 2 * (c & 3) + p] = gend[p][c];
-  }
-}
-
-// S = exp(gend_w') * S + U_w'  for one published chunk w'
-__device__ __forceinline__ void fold_state(const char* lds, int slot, int wsrc, int lane, int h, f32x16_t (&S)[2][2]) {
-  const float* d = reinterpret_cast<const float*>(lds + kLdsDvec) + wsrc * 64 + 32 * h;
-  const char* base = lds + kLdsSlots + slot * kSlotBytes;
-#pragma unroll
-  for (int pk = 0; pk < 2; ++pk) {
-    float dec[16];
-#pragma unroll
-    for (int c = 0; c < 16; ++c) dec[c] = exp2_fast(d[8 * (c >> 2) + 2 * (c & 3) + pk] * kLog2e);
-#pragma unroll
-    for (int pv = 0; pv < 2; ++pv)
-#pragma unroll
-      for (int cq = 0; cq < 4; ++cq) {
-        const f32x4_t u = *reinterpret_cast<const f32x4_t*>(base + (((pk * 2 + pv) * 4 + cq) * 64 + lane) * 16);
-#pragma unroll
-        for (int m = 0; m < 4; ++m) S[pk][pv][4 * cq + m] = __builtin_fmaf(S[pk][pv][4 * cq + m], dec[4 * cq + m], u[m]);
+      for (int cc = 0; cc < 16; ++cc) {
+        const float a = FWD ? G[1][p][cc] : G[0][p][cc];
+        e2[p][cc] = __int_as_float(__builtin_amdgcn_ds_bpermute(src, __float_as_int(a))) * kLog2e;
       }
-  }
-}
-
-// O^T += (exp(gend) * S_in)^T-fragments x q~hi
-__device__ __forceinline__ void inter_product(const f32x16_t (&S)[2][2], const float (&gend)[2][16],
-                                              const u32x4_t (&qkeep)[2][4], f32x16_t (&O)[2][2]) {
-  float dec[2][16];
+    if (r == 0) {  // every lane of a half holds the same 32 values; one lane writes them
+      float* d = dvec_all + wi * 64 + 32 * h;
 #pragma unroll
-  for (int p = 0; p < 2; ++p)
-#pragma unroll
-    for (int c = 0; c < 16; ++c) dec[p][c] = exp2_fast(gend[p][c] * kLog2e);
-#pragma unroll
-  for (int pv = 0; pv < 2; ++pv) {
-#pragma unroll
-    for (int ks = 0; ks < 4; ++ks) {
-      u32x4_t sf;
-#pragma unroll
-      for (int m = 0; m < 4; ++m) {
-        const int c = 4 * ks + m;
-        sf[m] = pack_bf16x2(S[0][pv][c] * dec[0][c], S[1][pv][c] * dec[1][c]);
+      for (int gq = 0; gq < 4; ++gq) {
+        const f32x4_t x0 = {e2[0][4 * gq], e2[0][4 * gq + 1], e2[0][4 * gq + 2], e2[0][4 * gq + 3]};
+        const f32x4_t x1 = {e2[1][4 * gq], e2[1][4 * gq + 1], e2[1][4 * gq + 2], e2[1][4 * gq + 3]};
+        *reinterpret_cast<f32x4_t*>(gend2 + 4 * gq) = x0;
+        *reinterpret_cast<f32x4_t*>(gend2 + 16 + 4 * gq) = x1;
+        // decay of channel 8*gq + 2*m + p
+        const f32x4_t d0 = {exp2_fast(x0[0]), exp2_fast(x1[0]), exp2_fast(x0[1]), exp2_fast(x1[1])};
+        const f32x4_t d1 = {exp2_fast(x0[2]), exp2_fast(x1[2]), exp2_fast(x0[3]), exp2_fast(x1[3])};
+        *reinterpret_cast<f32x4_t*>(d + 8 * gq) = d0;
+        *reinterpret_cast<f32x4_t*>(d + 8 * gq + 4) = d1;
       }
-#pragma unroll
-      for (int it = 0; it < 2; ++it) O[pv][it] = mfma(sf, qkeep[it][ks], O[pv][it]);
     }
   }
-}
-
-}  // namespace
-
-__global__ __launch_bounds__(256) void gla_mfma_slab_kernel(const uint16_t* __restrict__ q,
-                                                            const uint16_t* __restrict__ k,
-                                                            const uint16_t* __restrict__ v,
-                                                            const uint16_t* __restrict__ gf,
-                                                            const uint16_t* __restrict__ gb,
-                                                            uint16_t* __restrict__ o, int L, float scale,
-                                                            float out_scale) {
-  extern __shared__ __align__(16) char lds[];
-  const int tid = threadIdx.x;
-  const int w = tid >> 6, lane = tid & 63;
-  const int r = lane & 31, h = lane >> 5;
-  const size_t slab = (size_t)blockIdx.x * L * 64;
-  const int cw = (L + 3) >> 2;  // tokens per wave (<= 64)
-  const int row0 = w * cw;
-  const int nvalid = min(max(L - row0, 0), cw);
-  const size_t base = slab + (size_t)row0 * 64;
-  uint16_t* kt = reinterpret_cast<uint16_t*>(lds + kLdsKt + w * kKtBytes);
-  const float l2scale = __log2f(scale);
-
-  // raw q, k rows (lane = token of each 32-token tile, 32 contiguous channels) and transposed V fragments
-  u32x4_t qraw[2][4], kraw[2][4];
-#pragma unroll
-  for (int it = 0; it < 2; ++it) {
-    const int row = 32 * it + r;
-    const bool ok = row < nvalid;
-#pragma unroll
-    for (int g = 0; g < 4; ++g) {
-      const size_t off = base + (size_t)row * 64 + 32 * h + 8 * g;
-      const u32x4_t z = {0u, 0u, 0u, 0u};
-      qraw[it][g] = ok ? *reinterpret_cast<const u32x4_t*>(q + off) : z;
-      kraw[it][g] = ok ? *reinterpret_cast<const u32x4_t*>(k + off) : z;
-    }
-  }
-  u32x4_t vfrag[4][2];
-  load_tfrags_global(v + base, nvalid, r, h, vfrag);
-
+  wave_lds_sync();
+  VIG_STAMP(2);
+  // ---- intra-chunk scores, tile by tile; each tile's rows and V fragments are fetched one phase ahead ----
   f32x16_t O[2][2];
 #pragma unroll
   for (int i = 0; i < 2; ++i)
 #pragma unroll
     for (int j = 0; j < 2; ++j) O[i][j] = f32x16_t{0.f};
-
   u32x4_t qkeep[2][4];
-  float gend[2][16];
-  f32x16_t U[2][2];
-
-  // ------------------------------ forward direction ------------------------------
-  direction_pass<true>(gf + base, nvalid, r, h, l2scale, qraw, kraw, vfrag, O, qkeep, gend, U, kt);
-  if (w < 3) publish_state(lds, w, lane, U);
-  publish_decay(lds, w, r, h, gend);
-  __syncthreads();
-  if (w > 0) {
+  u32x4_t vfrag[4][2];
+  {
+    HalfOps ka, qb;
+    u32x4_t rawk[4], rawq[4];
+    uint32_t vDb[2][8];
+    {
+      HalfOps qa;
+      make_half<false>(pf.rawk, 32 * TA + r < nvalid, G[TA], gend2, ka);
+      make_half<true>(pf.rawq, true, G[TA], gend2, qa);
+      VIG_PHASE();
+      issue_raw_tile(q, TB, nvalid, r, h, rawq);
+      issue_raw_tile(k, TB, nvalid, r, h, rawk);
+      issue_tdwords<2 * TB, 2>(v, nvalid, r, h, vDb);
+      {
+        u32x4_t vf[2][2];
+        finish_tfrags<2 * TA, 2, false>(pf.vD, nvalid, h, vf);
+#pragma unroll
+        for (int tl = 0; tl < 2; ++tl)
+#pragma unroll
+          for (int p = 0; p < 2; ++p) vfrag[2 * TA + tl][p] = vf[tl][p];
+      }
+      apply_scores<FWD ? 1 : 2>(score_tile(ka, qa), TA, r, h, vfrag, O[0][TA], O[1][TA]);
+      store_kt(kt, 32 * TA + r, h, ka.h);
+#pragma unroll
+      for (int ks = 0; ks < 4; ++ks) qkeep[TA][ks] = qa.h[ks];
+    }
+    VIG_PHASE();
+    make_half<true>(rawq, true, G[TB], gend2, qb);
+    apply_scores<0>(score_tile(ka, qb), TA, r, h, vfrag, O[0][TB], O[1][TB]);
+    VIG_PHASE();
+    {
+      HalfOps kb;
+      make_half<false>(rawk, 32 * TB + r < nvalid, G[TB], gend2, kb);
+      {
+        u32x4_t vf[2][2];
+        finish_tfrags<2 * TB, 2, false>(vDb, nvalid, h, vf);
+#pragma unroll
+        for (int tl = 0; tl < 2; ++tl)
+#pragma unroll
+          for (int p = 0; p < 2; ++p) vfrag[2 * TB + tl][p] = vf[tl][p];
+      }
+      apply_scores<FWD ? 1 : 2>(score_tile(kb, qb), TB, r, h, vfrag, O[0][TB], O[1][TB]);
+      store_kt(kt, 32 * TB + r, h, kb.h);
+    }
+#pragma unroll
+    for (int ks = 0; ks < 4; ++ks) qkeep[TB][ks] = qb.h[ks];
+  }
+  VIG_STAMP(3);
+  wave_lds_sync();  // k~ rows of this wave visible to its other lanes
+  VIG_STAMP(4);
+  // ---- chunk state contribution U[pk][pv] = k~^T V; publish it (register-native fp32) with the chunk decay ----
+  {
+    f32x16_t U[2][2];
 #pragma unroll
     for (int i = 0; i < 2; ++i)
 #pragma unroll
       for (int j = 0; j < 2; ++j) U[i][j] = f32x16_t{0.f};
-    for (int ws = 0; ws < w; ++ws) fold_state(lds, ws, ws, lane, h, U);
-    inter_product(U, gend, qkeep, O);
-  }
-  __syncthreads();
-
-  // ------------------------------ reverse direction ------------------------------
-  if (gb != nullptr) {
-    direction_pass<false>(gb + base, nvalid, r, h, l2scale, qraw, kraw, vfrag, O, qkeep, gend, U, kt);
-    if (w > 0) publish_state(lds, w - 1, lane, U);
-    publish_decay(lds, w, r, h, gend);
-    __syncthreads();
-    if (w < 3) {
 #pragma unroll
-      for (int i = 0; i < 2; ++i)
+    for (int t = 0; t < 4; ++t) {
+      u32x4_t ktf[2];
+      load_tfrag_lds(kt, t, r, h, ktf);
 #pragma unroll
-        for (int j = 0; j < 2; ++j) U[i][j] = f32x16_t{0.f};
-      for (int ws = 3; ws > w; --ws) fold_state(lds, ws - 1, ws, lane, h, U);
-      inter_product(U, gend, qkeep, O);
+      for (int pk = 0; pk < 2; ++pk)
+#pragma unroll
+        for (int pv = 0; pv < 2; ++pv) U[pk][pv] = mfma(ktf[pk], vfrag[t][pv], U[pk][pv]);
+    }
+    if (FWD ? (c < 3) : (c > 0)) {
+#pragma unroll
+      for (int pk = 0; pk < 2; ++pk)
+#pragma unroll
+        for (int pv = 0; pv < 2; ++pv)
+#pragma unroll
+          for (int cq = 0; cq < 4; ++cq) {
+            const f32x4_t x = {U[pk][pv][4 * cq], U[pk][pv][4 * cq + 1], U[pk][pv][4 * cq + 2], U[pk][pv][4 * cq + 3]};
+            *reinterpret_cast<f32x4_t*>(unit_ptr(region, (pk * 2 + pv) * 4 + cq, lane)) = x;
+          }
     }
   }
-
-  // ------------------------------ store ------------------------------
+  // ---- forward waves fetch the first phase of the NEXT slab here, reverse waves fetch theirs at the top of the slab:
+  // a wave stalls while the memory pipe accepts its loads, and this way the other wave of the SIMD has math to do ----
+  // (always issued: after the last slab it re-reads the current one, which keeps the loop free of branches around loads)
+  if (FWD) issue_first_phase<FWD>(qn, kn, vn, gn, nvalid, r, h, pf);
+  VIG_STAMP(5);
+  lds_barrier();  // (A) published U's and decays visible
+  VIG_STAMP(6);
+  // ---- state recurrence over the chunks of this direction, one slice (pv, two register quads) per wave ----
+  {
+    const int pv = c & 1, cqa = 2 * (c >> 1);
+    char* dirbase = lds + (FWD ? 0 : 4) * kRegionBytes;
+    const float* ddir = dvec_all + (FWD ? 0 : 4) * 64;
+    constexpr int W0 = FWD ? 0 : 3, STEP = FWD ? 1 : -1;
+    f32x4_t S[2][2];
+#pragma unroll
+    for (int pk = 0; pk < 2; ++pk)
+#pragma unroll
+      for (int j = 0; j < 2; ++j)
+        S[pk][j] =
+            *reinterpret_cast<const f32x4_t*>(unit_ptr(dirbase + W0 * kRegionBytes, (pk * 2 + pv) * 4 + cqa + j, lane));
+#pragma unroll
+    for (int i = 1; i < 4; ++i) {
+      const int wc = W0 + STEP * i;  // consumer chunk: needs exp(G_end(wc)) * S as fragments
+      char* creg = dirbase + wc * kRegionBytes;
+#pragma unroll
+      for (int j = 0; j < 2; ++j) {
+        const int cq = cqa + j;
+        const f32x4_t d0 = *reinterpret_cast<const f32x4_t*>(ddir + wc * 64 + 32 * h + 8 * cq);
+        const f32x4_t d1 = *reinterpret_cast<const f32x4_t*>(ddir + wc * 64 + 32 * h + 8 * cq + 4);
+        // decay of row (m, pk): element 2*m + pk of the eight
+        const float dk0[4] = {d0[0], d0[2], d1[0], d1[2]};
+        const float dk1[4] = {d0[1], d0[3], d1[1], d1[3]};
+        f32x4_t u0 = {0.f, 0.f, 0.f, 0.f}, u1 = {0.f, 0.f, 0.f, 0.f};
+        if (i < 3) {
+          u0 = *reinterpret_cast<const f32x4_t*>(unit_ptr(creg, (0 * 2 + pv) * 4 + cq, lane));
+          u1 = *reinterpret_cast<const f32x4_t*>(unit_ptr(creg, (1 * 2 + pv) * 4 + cq, lane));
+        }
+        u32x4_t fr;
+#pragma unroll
+        for (int m = 0; m < 4; ++m) {
+          const float t0 = S[0][j][m] * dk0[m];
+          const float t1 = S[1][j][m] * dk1[m];
+          fr[m] = pack_bf16x2(t0, t1);
+          S[0][j][m] = t0 + u0[m];
+          S[1][j][m] = t1 + u1[m];
+        }
+        *reinterpret_cast<u32x4_t*>(unit_ptr(creg, pv * 4 + cq, lane)) = fr;
+      }
+    }
+  }
+  VIG_STAMP(7);
+  lds_barrier();  // (B) incoming-state fragments of every chunk visible
+  VIG_STAMP(8);
+  // ---- O^T += (exp(G_end) * S_in) q~hi  for every chunk but the one walked first ----
+  if (FWD ? (c > 0) : (c < 3)) {
+#pragma unroll
+    for (int pv = 0; pv < 2; ++pv)
+#pragma unroll
+      for (int ks = 0; ks < 4; ++ks) {
+        const u32x4_t sf = *reinterpret_cast<const u32x4_t*>(unit_ptr(region, pv * 4 + ks, lane));
+#pragma unroll
+        for (int it = 0; it < 2; ++it) O[pv][it] = mfma(sf, qkeep[it][ks], O[pv][it]);
+      }
+  }
+  VIG_STAMP(9);
+  // ---- the output swap: each wave of a chunk keeps one 32-token tile ----
+  constexpr int KEEP = FWD ? 0 : 1;
+  constexpr int SEND = 1 - KEEP;
+  if (bidir) {
+#pragma unroll
+    for (int pv = 0; pv < 2; ++pv)
+#pragma unroll
+      for (int cq = 0; cq < 4; ++cq) {
+        const f32x4_t x = {O[pv][SEND][4 * cq], O[pv][SEND][4 * cq + 1], O[pv][SEND][4 * cq + 2],
+                           O[pv][SEND][4 * cq + 3]};
+        *reinterpret_cast<f32x4_t*>(unit_ptr(region, pv * 4 + cq, lane)) = x;
+      }
+  }
+  VIG_STAMP(10);
+  lds_barrier();  // (C) swapped output halves visible
+  VIG_STAMP(11);
+  if (bidir) {
+    char* partner = lds + ((FWD ? 4 : 0) + c) * kRegionBytes;
+#pragma unroll
+    for (int pv = 0; pv < 2; ++pv)
+#pragma unroll
+      for (int cq = 0; cq < 4; ++cq) {
+        const f32x4_t x = *reinterpret_cast<const f32x4_t*>(unit_ptr(partner, pv * 4 + cq, lane));
+#pragma unroll
+        for (int m = 0; m < 4; ++m) O[pv][KEEP][4 * cq + m] += x[m];
+      }
+  }
 #pragma unroll
   for (int it = 0; it < 2; ++it) {
+    if (bidir && it != KEEP) continue;
     const int row = 32 * it + r;
     if (row < nvalid) {
 #pragma unroll
-      for (int g = 0; g < 4; ++g) {
+      for (int gq = 0; gq < 4; ++gq) {
         u32x4_t x;
 #pragma unroll
-        for (int m = 0; m < 4; ++m)
-          x[m] = pack_bf16x2(O[0][it][4 * g + m] * out_scale, O[1][it][4 * g + m] * out_scale);
-        *reinterpret_cast<u32x4_t*>(o + base + (size_t)row * 64 + 32 * h + 8 * g) = x;
+        for (int m = 0; m < 4; ++m) x[m] = pack_bf16x2(O[0][it][4 * gq + m] * oscale, O[1][it][4 * gq + m] * oscale);
+        *reinterpret_cast<u32x4_t*>(o + ((unsigned)row * 64u + 32u * h + 8u * gq)) = x;
       }
+    }
+  }
+  VIG_STAMP(12);
+}
+
+template <bool FWD>
+__device__ __forceinline__ void wave_loop(const uint16_t* q, const uint16_t* k, const uint16_t* v, const uint16_t* g,
+                                          uint16_t* o, int L, int nslab, int row0, int nvalid, int c, int lane,
+                                          char* lds, float oscale, bool bidir) {
+  // an empty chunk (nvalid == 0) reads row 0 of its slab instead of running past it; its values are discarded
+  const size_t chunk_off = (size_t)(nvalid > 0 ? row0 : 0) * 64;
+  const size_t slab_elems = (size_t)L * 64;
+  Prefetch pf;
+  int slab = blockIdx.x;
+  if (FWD && slab < nslab) {
+    const size_t b = (size_t)slab * slab_elems + chunk_off;
+    issue_first_phase<FWD>(q + b, k + b, v + b, g + b, nvalid, lane & 31, lane >> 5, pf);
+  }
+  int iter = 0;
+  for (; slab < nslab; slab += gridDim.x, ++iter) {
+    const size_t b = (size_t)slab * slab_elems + chunk_off;
+    const int next = slab + gridDim.x;
+    const bool has_next = next < nslab;
+    const size_t bn = has_next ? (size_t)next * slab_elems + chunk_off : b;
+    asm volatile("" : "+v"(lane));  // per-lane constants are rebuilt per slab instead of living across the loop
+    direction_wave<FWD>(q + b, k + b, v + b, g + b, o + b, q + bn, k + bn, v + bn, g + bn, has_next, nvalid, c, lane,
+                        lds, oscale, bidir, pf, iter);
+    lds_barrier();  // (D) the next slab reuses the LDS regions
+  }
+}
+
+}  // namespace
+
+__global__ __launch_bounds__(512) void gla_mfma_slab_kernel(const uint16_t* __restrict__ q,
+                                                            const uint16_t* __restrict__ k,
+                                                            const uint16_t* __restrict__ v,
+                                                            const uint16_t* __restrict__ gf,
+                                                            const uint16_t* __restrict__ gb,
+                                                            uint16_t* __restrict__ o, int L, int nslab,
+                                                            float oscale) {
+  extern __shared__ __align__(16) char lds[];
+  const int tid = threadIdx.x;
+  const int wi = tid >> 6;
+  const int lane = tid & 63;
+  const int c = wi & 3;
+  const bool bidir = gb != nullptr;
+  const int cw = (L + 3) >> 2;  // tokens per chunk (<= 64)
+  const int row0 = c * cw;
+  const int nvalid = min(max(L - row0, 0), cw);
+  if (wi < 4) {
+    wave_loop<true>(q, k, v, gf, o, L, nslab, row0, nvalid, c, lane, lds, oscale, bidir);
+  } else if (bidir) {
+    wave_loop<false>(q, k, v, gb, o, L, nslab, row0, nvalid, c, lane, lds, oscale, bidir);
+  } else {
+    for (int slab = blockIdx.x; slab < nslab; slab += gridDim.x) {
+      lds_barrier();
+      lds_barrier();
+      lds_barrier();
+      lds_barrier();
     }
   }
 }
 
 bool gla_mfma_supported(const GlaArgs& a) {
-  return a.io_dtype == 1 && a.gate_dtype == 1 && a.Dk == 64 && a.Dv == 64 && a.L <= 256 && a.scale > 0.f;
+  return a.io_dtype == 1 && a.gate_dtype == 1 && a.Dk == 64 && a.Dv == 64 && a.L <= 256;
 }
 
 size_t gla_mfma_workspace(int, int, int, int, int) { return 0; }
 
 int launch_gla_mfma(const GlaArgs& a) {
-  static bool attr_set = false;
-  if (!attr_set) {
+  static int num_cu = 0;
+  if (num_cu == 0) {
+    int dev = 0;
+    hipDeviceProp_t prop;
+    if (hipGetDevice(&dev) != hipSuccess || hipGetDeviceProperties(&prop, dev) != hipSuccess) return -5;
     if (hipFuncSetAttribute(reinterpret_cast<const void*>(gla_mfma_slab_kernel),
                             hipFuncAttributeMaxDynamicSharedMemorySize, kLdsTotal) != hipSuccess)
       return -5;
-    attr_set = true;
+    num_cu = prop.multiProcessorCount > 0 ? prop.multiProcessorCount : 256;
   }
-  hipLaunchKernelGGL(gla_mfma_slab_kernel, dim3(a.B * a.H), dim3(256), kLdsTotal, a.stream, (const uint16_t*)a.q,
+  const int nslab = a.B * a.H;
+  int grid = nslab < num_cu ? nslab : num_cu;
+#ifdef VIG_TIMING
+  if (const char* e = getenv("VIG_GRID")) grid = atoi(e);
+#endif
+  hipLaunchKernelGGL(gla_mfma_slab_kernel, dim3(grid), dim3(512), kLdsTotal, a.stream, (const uint16_t*)a.q,
                      (const uint16_t*)a.k, (const uint16_t*)a.v, (const uint16_t*)a.g_fwd, (const uint16_t*)a.g_bwd,
-                     (uint16_t*)a.o, a.L, a.scale, a.out_scale);
+                     (uint16_t*)a.o, a.L, nslab, a.scale * a.out_scale);
   return hipGetLastError() == hipSuccess ? 0 : -5;
 }
+
+#ifdef VIG_TIMING
+extern "C" int vig_debug_read_stamps(unsigned long long* host_out) {
+  return hipMemcpyFromSymbol(host_out, HIP_SYMBOL(g_stamp), sizeof(g_stamp)) == hipSuccess ? 0 : -5;
+}
+#endif
 
 }  // namespace vig
