@@ -258,23 +258,35 @@ struct Prefetch {
   u32x4_t rawk[4], rawq[4];  // raw rows of the tile walked first
 };
 
-template <bool FWD>
+template <bool FWD, bool WITH_Q>
 __device__ __forceinline__ void issue_first_phase(const uint16_t* q, const uint16_t* k, const uint16_t* v,
                                                   const uint16_t* g, int nvalid, int r, int h, Prefetch& pf) {
   constexpr int TA = FWD ? 0 : 1;
   issue_tdwords<0, 4>(g, nvalid, r, h, pf.gD);
   issue_raw_tile(k, TA, nvalid, r, h, pf.rawk);
-  issue_raw_tile(q, TA, nvalid, r, h, pf.rawq);
+  if (WITH_Q) issue_raw_tile(q, TA, nvalid, r, h, pf.rawq);
   issue_tdwords<2 * TA, 2>(v, nvalid, r, h, pf.vD);
 }
 
-// Everything one wave does for one slab: chunk c (nvalid tokens starting at the row the pointers address) in
+// Segment modes of the kernel.  A sequence longer than 256 tokens is cut into segments of <= 256 tokens that are
+// processed like slabs, chained through per-segment states in a caller workspace:
+//   kModeSlab   whole sequence in one segment, no state in or out;
+//   kModeState  pass 1 of a long sequence: only k~, V and the gates are touched; the segment's end-anchored state
+//               contribution and total decay are written to the workspace (no outputs);
+//   kModeChain  pass 2 of a long sequence: the state entering the segment (from the left for the forward direction,
+//               from the right for the reverse one) is read from the workspace and outputs are produced.
+constexpr int kModeSlab = 0, kModeState = 1, kModeChain = 2;
+constexpr int kStateFloats = 64 * 64 + 64;  // per (sequence, segment, direction): state in unit order, then 64 decays
+
+// Everything one wave does for one segment: chunk c (nvalid tokens starting at the row the pointers address) in
 // direction FWD / reverse.  Every wave of the workgroup passes the same three barriers here (plus the caller's).
-template <bool FWD>
+template <bool FWD, int MODE>
 __device__ __forceinline__ void direction_wave(const uint16_t* q, const uint16_t* k, const uint16_t* v,
                                                const uint16_t* g, uint16_t* o, const uint16_t* qn, const uint16_t* kn,
-                                               const uint16_t* vn, const uint16_t* gn, bool has_next, int nvalid, int c,
-                                               int lane, char* lds, float oscale, bool bidir, Prefetch& pf, int iter) {
+                                               const uint16_t* vn, const uint16_t* gn, int nvalid, int nvalid_next,
+                                               int c, int lane, char* lds, float oscale, bool bidir, float* state,
+                                               Prefetch& pf, int iter) {
+  constexpr bool OUT = MODE != kModeState;  // produces outputs (needs q)
   const int r = lane & 31, h = lane >> 5;
   const int wi = (FWD ? 0 : 4) + c;
   constexpr int TA = FWD ? 0 : 1;  // tile walked first
@@ -282,7 +294,7 @@ __device__ __forceinline__ void direction_wave(const uint16_t* q, const uint16_t
   char* region = lds + wi * kRegionBytes;
   uint16_t* kt = reinterpret_cast<uint16_t*>(region);
   float* dvec_all = reinterpret_cast<float*>(lds + kLdsDvec);
-  if (!FWD) issue_first_phase<FWD>(q, k, v, g, nvalid, r, h, pf);
+  if (!FWD) issue_first_phase<FWD, OUT>(q, k, v, g, nvalid, r, h, pf);
   VIG_STAMP(0);
 
   // ---- cumulative log-gates G[it][p] via triangular-ones MFMA on transposed gate fragments ----
@@ -361,9 +373,9 @@ __device__ __forceinline__ void direction_wave(const uint16_t* q, const uint16_t
     {
       HalfOps qa;
       make_half<false>(pf.rawk, 32 * TA + r < nvalid, G[TA], gend2, ka);
-      make_half<true>(pf.rawq, true, G[TA], gend2, qa);
+      if (OUT) make_half<true>(pf.rawq, true, G[TA], gend2, qa);
       VIG_PHASE();
-      issue_raw_tile(q, TB, nvalid, r, h, rawq);
+      if (OUT) issue_raw_tile(q, TB, nvalid, r, h, rawq);
       issue_raw_tile(k, TB, nvalid, r, h, rawk);
       issue_tdwords<2 * TB, 2>(v, nvalid, r, h, vDb);
       {
@@ -374,14 +386,18 @@ __device__ __forceinline__ void direction_wave(const uint16_t* q, const uint16_t
 #pragma unroll
           for (int p = 0; p < 2; ++p) vfrag[2 * TA + tl][p] = vf[tl][p];
       }
-      apply_scores<FWD ? 1 : 2>(score_tile(ka, qa), TA, r, h, vfrag, O[0][TA], O[1][TA]);
+      if (OUT) apply_scores<FWD ? 1 : 2>(score_tile(ka, qa), TA, r, h, vfrag, O[0][TA], O[1][TA]);
       store_kt(kt, 32 * TA + r, h, ka.h);
+      if (OUT) {
 #pragma unroll
-      for (int ks = 0; ks < 4; ++ks) qkeep[TA][ks] = qa.h[ks];
+        for (int ks = 0; ks < 4; ++ks) qkeep[TA][ks] = qa.h[ks];
+      }
     }
     VIG_PHASE();
-    make_half<true>(rawq, true, G[TB], gend2, qb);
-    apply_scores<0>(score_tile(ka, qb), TA, r, h, vfrag, O[0][TB], O[1][TB]);
+    if (OUT) {
+      make_half<true>(rawq, true, G[TB], gend2, qb);
+      apply_scores<0>(score_tile(ka, qb), TA, r, h, vfrag, O[0][TB], O[1][TB]);
+    }
     VIG_PHASE();
     {
       HalfOps kb;
@@ -394,16 +410,18 @@ __device__ __forceinline__ void direction_wave(const uint16_t* q, const uint16_t
 #pragma unroll
           for (int p = 0; p < 2; ++p) vfrag[2 * TB + tl][p] = vf[tl][p];
       }
-      apply_scores<FWD ? 1 : 2>(score_tile(kb, qb), TB, r, h, vfrag, O[0][TB], O[1][TB]);
+      if (OUT) apply_scores<FWD ? 1 : 2>(score_tile(kb, qb), TB, r, h, vfrag, O[0][TB], O[1][TB]);
       store_kt(kt, 32 * TB + r, h, kb.h);
     }
+    if (OUT) {
 #pragma unroll
-    for (int ks = 0; ks < 4; ++ks) qkeep[TB][ks] = qb.h[ks];
+      for (int ks = 0; ks < 4; ++ks) qkeep[TB][ks] = qb.h[ks];
+    }
   }
   VIG_STAMP(3);
   wave_lds_sync();  // k~ rows of this wave visible to its other lanes
   VIG_STAMP(4);
-  // ---- chunk state contribution U[pk][pv] = k~^T V; publish it (register-native fp32) with the chunk decay ----
+  // ---- chunk state contribution U[pk][pv] = k~^T V; publish it (register-native fp32) ----
   {
     f32x16_t U[2][2];
 #pragma unroll
@@ -419,7 +437,8 @@ __device__ __forceinline__ void direction_wave(const uint16_t* q, const uint16_t
 #pragma unroll
         for (int pv = 0; pv < 2; ++pv) U[pk][pv] = mfma(ktf[pk], vfrag[t][pv], U[pk][pv]);
     }
-    if (FWD ? (c < 3) : (c > 0)) {
+    // the chunk walked last is consumed by nobody inside the segment, unless the segment's own total is wanted
+    if (MODE == kModeState || (FWD ? (c < 3) : (c > 0))) {
 #pragma unroll
       for (int pk = 0; pk < 2; ++pk)
 #pragma unroll
@@ -431,10 +450,10 @@ __device__ __forceinline__ void direction_wave(const uint16_t* q, const uint16_t
           }
     }
   }
-  // ---- forward waves fetch the first phase of the NEXT slab here, reverse waves fetch theirs at the top of the slab:
-  // a wave stalls while the memory pipe accepts its loads, and this way the other wave of the SIMD has math to do ----
-  // (always issued: after the last slab it re-reads the current one, which keeps the loop free of branches around loads)
-  if (FWD) issue_first_phase<FWD>(qn, kn, vn, gn, nvalid, r, h, pf);
+  // ---- forward waves fetch the first phase of the NEXT segment here, reverse waves fetch theirs at the top of the
+  // segment: a wave stalls while the memory pipe accepts its loads, and this way the other wave of the SIMD has math
+  // to do.  (Always issued: after the last segment it re-reads the current one, which keeps branches off the loads.) ----
+  if (FWD) issue_first_phase<FWD, OUT>(qn, kn, vn, gn, nvalid_next, r, h, pf);
   VIG_STAMP(5);
   lds_barrier();  // (A) published U's and decays visible
   VIG_STAMP(6);
@@ -448,13 +467,18 @@ __device__ __forceinline__ void direction_wave(const uint16_t* q, const uint16_t
 #pragma unroll
     for (int pk = 0; pk < 2; ++pk)
 #pragma unroll
-      for (int j = 0; j < 2; ++j)
-        S[pk][j] =
-            *reinterpret_cast<const f32x4_t*>(unit_ptr(dirbase + W0 * kRegionBytes, (pk * 2 + pv) * 4 + cqa + j, lane));
+      for (int j = 0; j < 2; ++j) {
+        const int u = (pk * 2 + pv) * 4 + cqa + j;
+        if (MODE == kModeChain)  // state entering the segment, written by the segment scan in the same unit order
+          S[pk][j] = *reinterpret_cast<const f32x4_t*>(state + (u * 64 + lane) * 4);
+        else
+          S[pk][j] = *reinterpret_cast<const f32x4_t*>(unit_ptr(dirbase + W0 * kRegionBytes, u, lane));
+      }
 #pragma unroll
-    for (int i = 1; i < 4; ++i) {
+    for (int i = (MODE == kModeChain ? 0 : 1); i < 4; ++i) {
       const int wc = W0 + STEP * i;  // consumer chunk: needs exp(G_end(wc)) * S as fragments
       char* creg = dirbase + wc * kRegionBytes;
+      const bool add_u = MODE == kModeState || i < 3;
 #pragma unroll
       for (int j = 0; j < 2; ++j) {
         const int cq = cqa + j;
@@ -464,7 +488,7 @@ __device__ __forceinline__ void direction_wave(const uint16_t* q, const uint16_t
         const float dk0[4] = {d0[0], d0[2], d1[0], d1[2]};
         const float dk1[4] = {d0[1], d0[3], d1[1], d1[3]};
         f32x4_t u0 = {0.f, 0.f, 0.f, 0.f}, u1 = {0.f, 0.f, 0.f, 0.f};
-        if (i < 3) {
+        if (add_u) {
           u0 = *reinterpret_cast<const f32x4_t*>(unit_ptr(creg, (0 * 2 + pv) * 4 + cq, lane));
           u1 = *reinterpret_cast<const f32x4_t*>(unit_ptr(creg, (1 * 2 + pv) * 4 + cq, lane));
         }
@@ -477,119 +501,143 @@ __device__ __forceinline__ void direction_wave(const uint16_t* q, const uint16_t
           S[0][j][m] = t0 + u0[m];
           S[1][j][m] = t1 + u1[m];
         }
-        *reinterpret_cast<u32x4_t*>(unit_ptr(creg, pv * 4 + cq, lane)) = fr;
+        if (OUT) *reinterpret_cast<u32x4_t*>(unit_ptr(creg, pv * 4 + cq, lane)) = fr;
       }
+    }
+    if (MODE == kModeState) {
+      // the segment's end-anchored contribution (unit order) and its total decay per channel
+#pragma unroll
+      for (int pk = 0; pk < 2; ++pk)
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+          *reinterpret_cast<f32x4_t*>(state + (((pk * 2 + pv) * 4 + cqa + j) * 64 + lane) * 4) = S[pk][j];
+      if (c == 0) state[64 * 64 + lane] = ddir[lane] * ddir[64 + lane] * ddir[128 + lane] * ddir[192 + lane];
     }
   }
   VIG_STAMP(7);
   lds_barrier();  // (B) incoming-state fragments of every chunk visible
   VIG_STAMP(8);
-  // ---- O^T += (exp(G_end) * S_in) q~hi  for every chunk but the one walked first ----
-  if (FWD ? (c > 0) : (c < 3)) {
+  if (OUT) {
+    // ---- O^T += (exp(G_end) * S_in) q~hi  for every chunk that has an incoming state ----
+    if (MODE == kModeChain || (FWD ? (c > 0) : (c < 3))) {
 #pragma unroll
-    for (int pv = 0; pv < 2; ++pv)
+      for (int pv = 0; pv < 2; ++pv)
 #pragma unroll
-      for (int ks = 0; ks < 4; ++ks) {
-        const u32x4_t sf = *reinterpret_cast<const u32x4_t*>(unit_ptr(region, pv * 4 + ks, lane));
+        for (int ks = 0; ks < 4; ++ks) {
+          const u32x4_t sf = *reinterpret_cast<const u32x4_t*>(unit_ptr(region, pv * 4 + ks, lane));
 #pragma unroll
-        for (int it = 0; it < 2; ++it) O[pv][it] = mfma(sf, qkeep[it][ks], O[pv][it]);
-      }
-  }
-  VIG_STAMP(9);
-  // ---- the output swap: each wave of a chunk keeps one 32-token tile ----
-  constexpr int KEEP = FWD ? 0 : 1;
-  constexpr int SEND = 1 - KEEP;
-  if (bidir) {
+          for (int it = 0; it < 2; ++it) O[pv][it] = mfma(sf, qkeep[it][ks], O[pv][it]);
+        }
+    }
+    VIG_STAMP(9);
+    // ---- the output swap: each wave of a chunk keeps one 32-token tile ----
+    constexpr int KEEP = FWD ? 0 : 1;
+    constexpr int SEND = 1 - KEEP;
+    if (bidir) {
 #pragma unroll
-    for (int pv = 0; pv < 2; ++pv)
+      for (int pv = 0; pv < 2; ++pv)
 #pragma unroll
-      for (int cq = 0; cq < 4; ++cq) {
-        const f32x4_t x = {O[pv][SEND][4 * cq], O[pv][SEND][4 * cq + 1], O[pv][SEND][4 * cq + 2],
-                           O[pv][SEND][4 * cq + 3]};
-        *reinterpret_cast<f32x4_t*>(unit_ptr(region, pv * 4 + cq, lane)) = x;
-      }
-  }
-  VIG_STAMP(10);
-  lds_barrier();  // (C) swapped output halves visible
-  VIG_STAMP(11);
-  if (bidir) {
-    char* partner = lds + ((FWD ? 4 : 0) + c) * kRegionBytes;
+        for (int cq = 0; cq < 4; ++cq) {
+          const f32x4_t x = {O[pv][SEND][4 * cq], O[pv][SEND][4 * cq + 1], O[pv][SEND][4 * cq + 2],
+                             O[pv][SEND][4 * cq + 3]};
+          *reinterpret_cast<f32x4_t*>(unit_ptr(region, pv * 4 + cq, lane)) = x;
+        }
+    }
+    VIG_STAMP(10);
+    lds_barrier();  // (C) swapped output halves visible
+    VIG_STAMP(11);
+    if (bidir) {
+      char* partner = lds + ((FWD ? 4 : 0) + c) * kRegionBytes;
 #pragma unroll
-    for (int pv = 0; pv < 2; ++pv)
+      for (int pv = 0; pv < 2; ++pv)
 #pragma unroll
-      for (int cq = 0; cq < 4; ++cq) {
-        const f32x4_t x = *reinterpret_cast<const f32x4_t*>(unit_ptr(partner, pv * 4 + cq, lane));
+        for (int cq = 0; cq < 4; ++cq) {
+          const f32x4_t x = *reinterpret_cast<const f32x4_t*>(unit_ptr(partner, pv * 4 + cq, lane));
 #pragma unroll
-        for (int m = 0; m < 4; ++m) O[pv][KEEP][4 * cq + m] += x[m];
-      }
-  }
+          for (int m = 0; m < 4; ++m) O[pv][KEEP][4 * cq + m] += x[m];
+        }
+    }
 #pragma unroll
-  for (int it = 0; it < 2; ++it) {
-    if (bidir && it != KEEP) continue;
-    const int row = 32 * it + r;
-    if (row < nvalid) {
+    for (int it = 0; it < 2; ++it) {
+      if (bidir && it != KEEP) continue;
+      const int row = 32 * it + r;
+      if (row < nvalid) {
 #pragma unroll
-      for (int gq = 0; gq < 4; ++gq) {
-        u32x4_t x;
+        for (int gq = 0; gq < 4; ++gq) {
+          u32x4_t x;
 #pragma unroll
-        for (int m = 0; m < 4; ++m) x[m] = pack_bf16x2(O[0][it][4 * gq + m] * oscale, O[1][it][4 * gq + m] * oscale);
-        *reinterpret_cast<u32x4_t*>(o + ((unsigned)row * 64u + 32u * h + 8u * gq)) = x;
+          for (int m = 0; m < 4; ++m) x[m] = pack_bf16x2(O[0][it][4 * gq + m] * oscale, O[1][it][4 * gq + m] * oscale);
+          *reinterpret_cast<u32x4_t*>(o + ((unsigned)row * 64u + 32u * h + 8u * gq)) = x;
+        }
       }
     }
+  } else {
+    lds_barrier();  // (C) keeps the barrier count of the output modes
   }
   VIG_STAMP(12);
 }
 
-template <bool FWD>
+// Geometry of the work items: item = sequence * nseg + segment; a segment holds seg_len tokens (the last one of a
+// sequence possibly fewer) cut into 4 chunks of cw tokens.
+struct Geometry {
+  int L, nseg, seg_len, cw, nitems;
+};
+
+template <bool FWD, int MODE>
 __device__ __forceinline__ void wave_loop(const uint16_t* q, const uint16_t* k, const uint16_t* v, const uint16_t* g,
-                                          uint16_t* o, int L, int nslab, int row0, int nvalid, int c, int lane,
-                                          char* lds, float oscale, bool bidir) {
-  // an empty chunk (nvalid == 0) reads row 0 of its slab instead of running past it; its values are discarded
-  const size_t chunk_off = (size_t)(nvalid > 0 ? row0 : 0) * 64;
-  const size_t slab_elems = (size_t)L * 64;
+                                          uint16_t* o, const Geometry& geo, int c, int lane, char* lds, float oscale,
+                                          bool bidir, float* state_ws) {
+  constexpr bool OUT = MODE != kModeState;
+  // an empty chunk (nvalid == 0) reads the first row of its segment instead of running past it; its values are discarded
+  auto locate = [&](int item, size_t& off, int& nvalid) {
+    const int seq = item / geo.nseg, seg = item - seq * geo.nseg;
+    const int seg_tokens = min(geo.seg_len, geo.L - seg * geo.seg_len);
+    nvalid = min(max(seg_tokens - c * geo.cw, 0), geo.cw);
+    off = ((size_t)seq * geo.L + (size_t)seg * geo.seg_len + (size_t)(nvalid > 0 ? c * geo.cw : 0)) * 64;
+  };
   Prefetch pf;
-  int slab = blockIdx.x;
-  if (FWD && slab < nslab) {
-    const size_t b = (size_t)slab * slab_elems + chunk_off;
-    issue_first_phase<FWD>(q + b, k + b, v + b, g + b, nvalid, lane & 31, lane >> 5, pf);
+  int item = blockIdx.x;
+  size_t b = 0;
+  int nvalid = 0;
+  if (item < geo.nitems) {
+    locate(item, b, nvalid);
+    if (FWD) issue_first_phase<FWD, OUT>(q + b, k + b, v + b, g + b, nvalid, lane & 31, lane >> 5, pf);
   }
   int iter = 0;
-  for (; slab < nslab; slab += gridDim.x, ++iter) {
-    const size_t b = (size_t)slab * slab_elems + chunk_off;
-    const int next = slab + gridDim.x;
-    const bool has_next = next < nslab;
-    const size_t bn = has_next ? (size_t)next * slab_elems + chunk_off : b;
-    asm volatile("" : "+v"(lane));  // per-lane constants are rebuilt per slab instead of living across the loop
-    direction_wave<FWD>(q + b, k + b, v + b, g + b, o + b, q + bn, k + bn, v + bn, g + bn, has_next, nvalid, c, lane,
-                        lds, oscale, bidir, pf, iter);
-    lds_barrier();  // (D) the next slab reuses the LDS regions
+  for (; item < geo.nitems; item += gridDim.x, ++iter) {
+    const int next = item + gridDim.x;
+    size_t bn = b;
+    int nvalid_next = nvalid;
+    if (next < geo.nitems) locate(next, bn, nvalid_next);
+    float* state = state_ws ? state_ws + ((size_t)item * 2 + (FWD ? 0 : 1)) * kStateFloats : nullptr;
+    asm volatile("" : "+v"(lane));  // per-lane constants are rebuilt per item instead of living across the loop
+    direction_wave<FWD, MODE>(q + b, k + b, v + b, g + b, o + b, q + bn, k + bn, v + bn, g + bn, nvalid, nvalid_next, c,
+                              lane, lds, oscale, bidir, state, pf, iter);
+    lds_barrier();  // (D) the next item reuses the LDS regions
+    b = bn;
+    nvalid = nvalid_next;
   }
 }
 
 }  // namespace
 
-__global__ __launch_bounds__(512) void gla_mfma_slab_kernel(const uint16_t* __restrict__ q,
-                                                            const uint16_t* __restrict__ k,
-                                                            const uint16_t* __restrict__ v,
-                                                            const uint16_t* __restrict__ gf,
-                                                            const uint16_t* __restrict__ gb,
-                                                            uint16_t* __restrict__ o, int L, int nslab,
-                                                            float oscale) {
+template <int MODE>
+__global__ __launch_bounds__(512) void gla_mfma_kernel(const uint16_t* __restrict__ q, const uint16_t* __restrict__ k,
+                                                       const uint16_t* __restrict__ v, const uint16_t* __restrict__ gf,
+                                                       const uint16_t* __restrict__ gb, uint16_t* __restrict__ o,
+                                                       Geometry geo, float oscale, float* state_ws) {
   extern __shared__ __align__(16) char lds[];
   const int tid = threadIdx.x;
   const int wi = tid >> 6;
   const int lane = tid & 63;
   const int c = wi & 3;
   const bool bidir = gb != nullptr;
-  const int cw = (L + 3) >> 2;  // tokens per chunk (<= 64)
-  const int row0 = c * cw;
-  const int nvalid = min(max(L - row0, 0), cw);
   if (wi < 4) {
-    wave_loop<true>(q, k, v, gf, o, L, nslab, row0, nvalid, c, lane, lds, oscale, bidir);
+    wave_loop<true, MODE>(q, k, v, gf, o, geo, c, lane, lds, oscale, bidir, state_ws);
   } else if (bidir) {
-    wave_loop<false>(q, k, v, gb, o, L, nslab, row0, nvalid, c, lane, lds, oscale, bidir);
+    wave_loop<false, MODE>(q, k, v, gb, o, geo, c, lane, lds, oscale, bidir, state_ws);
   } else {
-    for (int slab = blockIdx.x; slab < nslab; slab += gridDim.x) {
+    for (int item = blockIdx.x; item < geo.nitems; item += gridDim.x) {
       lds_barrier();
       lds_barrier();
       lds_barrier();
@@ -598,11 +646,46 @@ __global__ __launch_bounds__(512) void gla_mfma_slab_kernel(const uint16_t* __re
   }
 }
 
-bool gla_mfma_supported(const GlaArgs& a) {
-  return a.io_dtype == 1 && a.gate_dtype == 1 && a.Dk == 64 && a.Dv == 64 && a.L <= 256;
+// Chains the segments of every sequence: in place, the workspace slot of segment s (its own contribution U_s and
+// decay D_s) is replaced by the state entering it,  S_in(s') = D_s * S_in(s) + U_s  with s' the next segment in the
+// direction's walk order.  One thread per state element; all accesses are coalesced (unit order is kept).
+__global__ __launch_bounds__(256) void gla_segment_scan_kernel(float* state_ws, int nseq, int nseg, int ndir) {
+  const int e = blockIdx.x * 256 + threadIdx.x;  // element in unit order: ((u*64 + lane)*4 + m)
+  const int seq = blockIdx.y / ndir, dir = blockIdx.y % ndir;
+  if (seq >= nseq) return;
+  const int m = e & 3, lane = (e >> 2) & 63, u = e >> 8;
+  const int pk = u >> 3, cq = u & 3, h = lane >> 5;
+  const int ch = 32 * h + 8 * cq + 2 * m + pk;
+  float S = 0.f;
+  for (int i = 0; i < nseg; ++i) {
+    const int seg = dir == 0 ? i : nseg - 1 - i;
+    float* slot = state_ws + (((size_t)seq * nseg + seg) * 2 + dir) * kStateFloats;
+    const float u_s = slot[e];
+    const float d_s = slot[64 * 64 + ch];
+    slot[e] = S;
+    S = __builtin_fmaf(d_s, S, u_s);
+  }
 }
 
-size_t gla_mfma_workspace(int, int, int, int, int) { return 0; }
+static Geometry make_geometry(int nseq, int L) {
+  Geometry g;
+  g.L = L;
+  g.nseg = (L + 255) / 256;
+  g.seg_len = (L + g.nseg - 1) / g.nseg;
+  g.cw = (g.seg_len + 3) / 4;
+  g.nitems = nseq * g.nseg;
+  return g;
+}
+
+bool gla_mfma_supported(const GlaArgs& a) {
+  return a.io_dtype == 1 && a.gate_dtype == 1 && a.Dk == 64 && a.Dv == 64;
+}
+
+size_t gla_mfma_workspace(int B, int H, int L, int Dk, int Dv) {
+  if (Dk != 64 || Dv != 64 || L <= 256) return 0;
+  const Geometry g = make_geometry(B * H, L);
+  return (size_t)g.nitems * 2 * kStateFloats * sizeof(float);
+}
 
 int launch_gla_mfma(const GlaArgs& a) {
   static int num_cu = 0;
@@ -610,19 +693,38 @@ int launch_gla_mfma(const GlaArgs& a) {
     int dev = 0;
     hipDeviceProp_t prop;
     if (hipGetDevice(&dev) != hipSuccess || hipGetDeviceProperties(&prop, dev) != hipSuccess) return -5;
-    if (hipFuncSetAttribute(reinterpret_cast<const void*>(gla_mfma_slab_kernel),
-                            hipFuncAttributeMaxDynamicSharedMemorySize, kLdsTotal) != hipSuccess)
-      return -5;
+    const void* kernels[3] = {reinterpret_cast<const void*>(gla_mfma_kernel<kModeSlab>),
+                              reinterpret_cast<const void*>(gla_mfma_kernel<kModeState>),
+                              reinterpret_cast<const void*>(gla_mfma_kernel<kModeChain>)};
+    for (const void* kf : kernels)
+      if (hipFuncSetAttribute(kf, hipFuncAttributeMaxDynamicSharedMemorySize, kLdsTotal) != hipSuccess) return -5;
     num_cu = prop.multiProcessorCount > 0 ? prop.multiProcessorCount : 256;
   }
-  const int nslab = a.B * a.H;
-  int grid = nslab < num_cu ? nslab : num_cu;
+  const Geometry geo = make_geometry(a.B * a.H, a.L);
+  int grid = geo.nitems < num_cu ? geo.nitems : num_cu;
 #ifdef VIG_TIMING
   if (const char* e = getenv("VIG_GRID")) grid = atoi(e);
 #endif
-  hipLaunchKernelGGL(gla_mfma_slab_kernel, dim3(grid), dim3(512), kLdsTotal, a.stream, (const uint16_t*)a.q,
-                     (const uint16_t*)a.k, (const uint16_t*)a.v, (const uint16_t*)a.g_fwd, (const uint16_t*)a.g_bwd,
-                     (uint16_t*)a.o, a.L, nslab, a.scale * a.out_scale);
+  const uint16_t* q = (const uint16_t*)a.q;
+  const uint16_t* k = (const uint16_t*)a.k;
+  const uint16_t* v = (const uint16_t*)a.v;
+  const uint16_t* gf = (const uint16_t*)a.g_fwd;
+  const uint16_t* gb = (const uint16_t*)a.g_bwd;
+  uint16_t* o = (uint16_t*)a.o;
+  const float oscale = a.scale * a.out_scale;
+  if (geo.nseg == 1) {
+    hipLaunchKernelGGL(gla_mfma_kernel<kModeSlab>, dim3(grid), dim3(512), kLdsTotal, a.stream, q, k, v, gf, gb, o, geo,
+                       oscale, (float*)nullptr);
+  } else {
+    float* ws = (float*)a.workspace;
+    hipLaunchKernelGGL(gla_mfma_kernel<kModeState>, dim3(grid), dim3(512), kLdsTotal, a.stream, q, k, v, gf, gb, o, geo,
+                       oscale, ws);
+    const int ndir = gb ? 2 : 1;
+    hipLaunchKernelGGL(gla_segment_scan_kernel, dim3(64 * 64 / 256, a.B * a.H * ndir), dim3(256), 0, a.stream, ws,
+                       a.B * a.H, geo.nseg, ndir);
+    hipLaunchKernelGGL(gla_mfma_kernel<kModeChain>, dim3(grid), dim3(512), kLdsTotal, a.stream, q, k, v, gf, gb, o, geo,
+                       oscale, ws);
+  }
   return hipGetLastError() == hipSuccess ? 0 : -5;
 }
 
