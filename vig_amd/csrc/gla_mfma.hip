@@ -74,7 +74,13 @@ __device__ __forceinline__ f32x16_t mfma(const u32x4_t& a, const u32x4_t& b, con
                                                  0, 0);
 }
 
-__device__ __forceinline__ int cpair(int rho) { return (((rho >> 2) & 1) << 4) | ((rho >> 3) << 2) | (rho & 3); }
+// Channel pair read by lane-row rho of a transposed fragment whose rows span 16*NG channels (NG = 4: 64 channels,
+// every row used; NG = 2: 32 channels, rows 16..31 carry no channel and are zero).  With it, accumulator register
+// 4*g + m of lane half h holds channel 8*NG*h + 8*g + 2*m + p.
+template <int NG>
+__device__ __forceinline__ int cpair(int rho) { return (((rho >> 2) & 1) * (4 * NG)) | ((rho >> 3) << 2) | (rho & 3); }
+template <int NG>
+__device__ __forceinline__ bool row_has_channel(int rho) { return (rho >> 3) < NG; }
 
 // token held by contraction slot e of k-step t for lane half h
 __device__ __forceinline__ int jmap(int t, int h, int e) { return 16 * t + 4 * h + (e & 3) + 8 * (e >> 2); }
@@ -103,27 +109,30 @@ __device__ __forceinline__ void lds_barrier() {
 // ---------------------------------------------------------------------------------------------------------
 
 // raw dwords of the transposed fragments of k-steps [T0, T0+NT): D[t][e] = channels (2*cpair(r), +1) of token jmap(t,h,e)
-template <int T0, int NT>
+template <int T0, int NT, int NG>
 __device__ __forceinline__ void issue_tdwords(const uint16_t* rows, int nvalid, int r, int h, uint32_t (&D)[NT][8]) {
-  const unsigned c2 = 2 * cpair(r);
+  const unsigned c2 = row_has_channel<NG>(r) ? 2 * cpair<NG>(r) : 0;
   const int nlast = max(nvalid - 1, 0);
 #pragma unroll
   for (int t = 0; t < NT; ++t)
 #pragma unroll
     for (int e = 0; e < 8; ++e) {
       const unsigned tok = (unsigned)min(jmap(T0 + t, h, e), nlast);
-      D[t][e] = *reinterpret_cast<const uint32_t*>(rows + (tok * 64u + c2));
+      D[t][e] = *reinterpret_cast<const uint32_t*>(rows + (tok * (16u * NG) + c2));
     }
 }
 
 // fragments from raw dwords: frag[t][p] has lane index = channel 2*cpair(r)+p, slots = tokens jmap(t,h,.)
-template <int T0, int NT, bool ZERO_PAD>
-__device__ __forceinline__ void finish_tfrags(const uint32_t (&D)[NT][8], int nvalid, int h, u32x4_t (&frag)[NT][2]) {
+template <int T0, int NT, bool ZERO_PAD, int NG>
+__device__ __forceinline__ void finish_tfrags(const uint32_t (&D)[NT][8], int nvalid, int r, int h,
+                                              u32x4_t (&frag)[NT][2]) {
+  const bool row_ok = row_has_channel<NG>(r);
 #pragma unroll
   for (int t = 0; t < NT; ++t) {
     uint32_t d[8];
 #pragma unroll
-    for (int e = 0; e < 8; ++e) d[e] = (!ZERO_PAD || jmap(T0 + t, h, e) < nvalid) ? D[t][e] : 0u;
+    for (int e = 0; e < 8; ++e)
+      d[e] = ((NG == 4 || row_ok) && (!ZERO_PAD || jmap(T0 + t, h, e) < nvalid)) ? D[t][e] : 0u;
 #pragma unroll
     for (int x = 0; x < 4; ++x) {
       frag[t][0][x] = __builtin_amdgcn_perm(d[2 * x + 1], d[2 * x], 0x05040100u);
@@ -132,19 +141,27 @@ __device__ __forceinline__ void finish_tfrags(const uint32_t (&D)[NT][8], int nv
   }
 }
 
-// raw rows of one 32-token tile: lane (r, h) reads token 32*it + r, channels [32h, 32h+32) as four 16-byte pieces
-__device__ __forceinline__ void issue_raw_tile(const uint16_t* rows, int it, int nvalid, int r, int h, u32x4_t (&raw)[4]) {
+// raw rows of one 32-token tile: lane (r, h) reads token 32*it + r, channels [8*NG*h, +8*NG) as NG 16-byte pieces
+template <int NG>
+__device__ __forceinline__ void issue_raw_tile(const uint16_t* rows, int it, int nvalid, int r, int h,
+                                               u32x4_t (&raw)[NG]) {
   const unsigned rowc = (unsigned)min(32 * it + r, max(nvalid - 1, 0));
 #pragma unroll
-  for (int gq = 0; gq < 4; ++gq) raw[gq] = *reinterpret_cast<const u32x4_t*>(rows + (rowc * 64u + 32u * h + 8u * gq));
+  for (int gq = 0; gq < NG; ++gq)
+    raw[gq] = *reinterpret_cast<const u32x4_t*>(rows + (rowc * (16u * NG) + (8u * NG) * h + 8u * gq));
 }
 
 // one k-step of transposed fragments from the wave's k~ scratch in LDS
+template <int NG>
 __device__ __forceinline__ void load_tfrag_lds(const uint16_t* kt, int t, int r, int h, u32x4_t (&frag)[2]) {
-  const int c2 = 2 * cpair(r);
+  const bool row_ok = row_has_channel<NG>(r);
+  const int c2 = row_ok ? 2 * cpair<NG>(r) : 0;
   uint32_t D[8];
 #pragma unroll
-  for (int e = 0; e < 8; ++e) D[e] = *reinterpret_cast<const uint32_t*>(kt + jmap(t, h, e) * kKtStride + c2);
+  for (int e = 0; e < 8; ++e) {
+    const uint32_t d = *reinterpret_cast<const uint32_t*>(kt + jmap(t, h, e) * kKtStride + c2);
+    D[e] = (NG == 4 || row_ok) ? d : 0u;
+  }
 #pragma unroll
   for (int x = 0; x < 4; ++x) {
     frag[0][x] = __builtin_amdgcn_perm(D[2 * x + 1], D[2 * x], 0x05040100u);
@@ -167,18 +184,19 @@ __device__ __forceinline__ u32x4_t tri_frag(int t, int it, int r, int h) {
   return f;
 }
 
+template <int NG>
 struct HalfOps {
-  u32x4_t h[4], l[4];  // bf16 hi / lo fragments of one 32-token tile, per k-step (16 channels)
+  u32x4_t h[NG], l[NG];  // bf16 hi / lo fragments of one 32-token tile, per k-step (16 channels)
 };
 
 // q~ (ISQ) or k~ of one 32-token tile: raw * exp(+-(G - G_end)), split into bf16 hi (round to nearest) and
 // lo (the fp32 remainder, rounded).  `live` zeroes padding rows (needed for k~ only: q~ of a padding row only
 // feeds outputs that are never stored).
-template <bool ISQ>
-__device__ __forceinline__ void make_half(const u32x4_t (&raw)[4], bool live, const f32x16_t (&G)[2],
-                                          const float* gend2 /* LDS, this lane half: [p][16] */, HalfOps& op) {
+template <bool ISQ, int NG>
+__device__ __forceinline__ void make_half(const u32x4_t (&raw)[NG], bool live, const f32x16_t (&G)[2],
+                                          const float* gend2 /* LDS, this lane half: [p][16] */, HalfOps<NG>& op) {
 #pragma unroll
-  for (int g = 0; g < 4; ++g) {
+  for (int g = 0; g < NG; ++g) {
     const f32x4_t a0 = *reinterpret_cast<const f32x4_t*>(gend2 + 4 * g);
     const f32x4_t a1 = *reinterpret_cast<const f32x4_t*>(gend2 + 16 + 4 * g);
 #pragma unroll
@@ -201,10 +219,11 @@ __device__ __forceinline__ void make_half(const u32x4_t (&raw)[4], bool live, co
 }
 
 // P^T tile = k~ (rows j) x q~ (columns i), three-term split product.
-__device__ __forceinline__ f32x16_t score_tile(const HalfOps& kop, const HalfOps& qop) {
+template <int NG>
+__device__ __forceinline__ f32x16_t score_tile(const HalfOps<NG>& kop, const HalfOps<NG>& qop) {
   f32x16_t acc = {0.f};
 #pragma unroll
-  for (int ks = 0; ks < 4; ++ks) {
+  for (int ks = 0; ks < NG; ++ks) {
     acc = mfma(kop.h[ks], qop.h[ks], acc);
     acc = mfma(kop.l[ks], qop.h[ks], acc);
     acc = mfma(kop.h[ks], qop.l[ks], acc);
@@ -243,29 +262,31 @@ __device__ __forceinline__ void apply_scores(f32x16_t P, int jt, int r, int h, c
   }
 }
 
-__device__ __forceinline__ void store_kt(uint16_t* kt, int row, int h, const u32x4_t (&kh)[4]) {
+template <int NG>
+__device__ __forceinline__ void store_kt(uint16_t* kt, int row, int h, const u32x4_t (&kh)[NG]) {
 #pragma unroll
-  for (int g = 0; g < 4; ++g) *reinterpret_cast<u32x4_t*>(kt + row * kKtStride + 32 * h + 8 * g) = kh[g];
+  for (int g = 0; g < NG; ++g) *reinterpret_cast<u32x4_t*>(kt + row * kKtStride + 8 * NG * h + 8 * g) = kh[g];
 }
 
 // LDS "unit" u of a region = 64 lanes x 16 B, register-native: lane l owns bytes [(u*64 + l)*16, +16).
 __device__ __forceinline__ char* unit_ptr(char* region, int u, int lane) { return region + (u * 64 + lane) * 16; }
 
 // What a wave carries from the end of one slab to the start of the next: the loads of its first phase.
+template <int NG>
 struct Prefetch {
-  uint32_t gD[4][8];         // gate dwords, all four k-steps of the chunk
-  uint32_t vD[2][8];         // V dwords of the tile walked first
-  u32x4_t rawk[4], rawq[4];  // raw rows of the tile walked first
+  uint32_t gD[4][8];           // gate dwords, all four k-steps of the chunk
+  uint32_t vD[2][8];           // V dwords of the tile walked first
+  u32x4_t rawk[NG], rawq[NG];  // raw rows of the tile walked first
 };
 
-template <bool FWD, bool WITH_Q>
+template <bool FWD, bool WITH_Q, int NG>
 __device__ __forceinline__ void issue_first_phase(const uint16_t* q, const uint16_t* k, const uint16_t* v,
-                                                  const uint16_t* g, int nvalid, int r, int h, Prefetch& pf) {
+                                                  const uint16_t* g, int nvalid, int r, int h, Prefetch<NG>& pf) {
   constexpr int TA = FWD ? 0 : 1;
-  issue_tdwords<0, 4>(g, nvalid, r, h, pf.gD);
-  issue_raw_tile(k, TA, nvalid, r, h, pf.rawk);
-  if (WITH_Q) issue_raw_tile(q, TA, nvalid, r, h, pf.rawq);
-  issue_tdwords<2 * TA, 2>(v, nvalid, r, h, pf.vD);
+  issue_tdwords<0, 4, NG>(g, nvalid, r, h, pf.gD);
+  issue_raw_tile<NG>(k, TA, nvalid, r, h, pf.rawk);
+  if (WITH_Q) issue_raw_tile<NG>(q, TA, nvalid, r, h, pf.rawq);
+  issue_tdwords<2 * TA, 2, 4>(v, nvalid, r, h, pf.vD);
 }
 
 // Segment modes of the kernel.  A sequence longer than 256 tokens is cut into segments of <= 256 tokens that are
@@ -280,12 +301,12 @@ constexpr int kStateFloats = 64 * 64 + 64;  // per (sequence, segment, direction
 
 // Everything one wave does for one segment: chunk c (nvalid tokens starting at the row the pointers address) in
 // direction FWD / reverse.  Every wave of the workgroup passes the same three barriers here (plus the caller's).
-template <bool FWD, int MODE>
+template <bool FWD, int MODE, int NG>
 __device__ __forceinline__ void direction_wave(const uint16_t* q, const uint16_t* k, const uint16_t* v,
                                                const uint16_t* g, uint16_t* o, const uint16_t* qn, const uint16_t* kn,
                                                const uint16_t* vn, const uint16_t* gn, int nvalid, int nvalid_next,
                                                int c, int lane, char* lds, float oscale, bool bidir, float* state,
-                                               Prefetch& pf, int iter) {
+                                               Prefetch<NG>& pf, int iter) {
   constexpr bool OUT = MODE != kModeState;  // produces outputs (needs q)
   const int r = lane & 31, h = lane >> 5;
   const int wi = (FWD ? 0 : 4) + c;
@@ -294,14 +315,14 @@ __device__ __forceinline__ void direction_wave(const uint16_t* q, const uint16_t
   char* region = lds + wi * kRegionBytes;
   uint16_t* kt = reinterpret_cast<uint16_t*>(region);
   float* dvec_all = reinterpret_cast<float*>(lds + kLdsDvec);
-  if (!FWD) issue_first_phase<FWD, OUT>(q, k, v, g, nvalid, r, h, pf);
+  if (!FWD) issue_first_phase<FWD, OUT, NG>(q, k, v, g, nvalid, r, h, pf);
   VIG_STAMP(0);
 
   // ---- cumulative log-gates G[it][p] via triangular-ones MFMA on transposed gate fragments ----
   f32x16_t G[2][2];
   {
     u32x4_t gfrag[4][2];
-    finish_tfrags<0, 4, true>(pf.gD, nvalid, h, gfrag);
+    finish_tfrags<0, 4, true, NG>(pf.gD, nvalid, r, h, gfrag);
     const u32x4_t ones = {0x3F803F80u, 0x3F803F80u, 0x3F803F80u, 0x3F803F80u};
 #pragma unroll
     for (int p = 0; p < 2; ++p) {
@@ -330,6 +351,7 @@ __device__ __forceinline__ void direction_wave(const uint16_t* q, const uint16_t
   // The anchors (x log2 e) and the chunk decays exp(G_end) go to LDS: the operand builders re-read the former per
   // tile, the state recurrence reads the latter after barrier A, and no register holds them across phases. ----
   float* gend2 = reinterpret_cast<float*>(lds + kLdsGend) + wi * 64 + 32 * h;
+  constexpr int HC = 8 * NG;  // channels per lane half
   {
     const int src = ((FWD ? 31 : 0) + 32 * h) << 2;
     float e2[2][16];
@@ -341,9 +363,9 @@ __device__ __forceinline__ void direction_wave(const uint16_t* q, const uint16_t
         e2[p][cc] = __int_as_float(__builtin_amdgcn_ds_bpermute(src, __float_as_int(a))) * kLog2e;
       }
     if (r == 0) {  // every lane of a half holds the same 32 values; one lane writes them
-      float* d = dvec_all + wi * 64 + 32 * h;
+      float* d = dvec_all + wi * 64 + HC * h;
 #pragma unroll
-      for (int gq = 0; gq < 4; ++gq) {
+      for (int gq = 0; gq < NG; ++gq) {
         const f32x4_t x0 = {e2[0][4 * gq], e2[0][4 * gq + 1], e2[0][4 * gq + 2], e2[0][4 * gq + 3]};
         const f32x4_t x1 = {e2[1][4 * gq], e2[1][4 * gq + 1], e2[1][4 * gq + 2], e2[1][4 * gq + 3]};
         *reinterpret_cast<f32x4_t*>(gend2 + 4 * gq) = x0;
@@ -364,58 +386,58 @@ __device__ __forceinline__ void direction_wave(const uint16_t* q, const uint16_t
   for (int i = 0; i < 2; ++i)
 #pragma unroll
     for (int j = 0; j < 2; ++j) O[i][j] = f32x16_t{0.f};
-  u32x4_t qkeep[2][4];
+  u32x4_t qkeep[2][NG];
   u32x4_t vfrag[4][2];
   {
-    HalfOps ka, qb;
-    u32x4_t rawk[4], rawq[4];
+    HalfOps<NG> ka, qb;
+    u32x4_t rawk[NG], rawq[NG];
     uint32_t vDb[2][8];
     {
-      HalfOps qa;
-      make_half<false>(pf.rawk, 32 * TA + r < nvalid, G[TA], gend2, ka);
-      if (OUT) make_half<true>(pf.rawq, true, G[TA], gend2, qa);
+      HalfOps<NG> qa;
+      make_half<false, NG>(pf.rawk, 32 * TA + r < nvalid, G[TA], gend2, ka);
+      if (OUT) make_half<true, NG>(pf.rawq, true, G[TA], gend2, qa);
       VIG_PHASE();
-      if (OUT) issue_raw_tile(q, TB, nvalid, r, h, rawq);
-      issue_raw_tile(k, TB, nvalid, r, h, rawk);
-      issue_tdwords<2 * TB, 2>(v, nvalid, r, h, vDb);
+      if (OUT) issue_raw_tile<NG>(q, TB, nvalid, r, h, rawq);
+      issue_raw_tile<NG>(k, TB, nvalid, r, h, rawk);
+      issue_tdwords<2 * TB, 2, 4>(v, nvalid, r, h, vDb);
       {
         u32x4_t vf[2][2];
-        finish_tfrags<2 * TA, 2, false>(pf.vD, nvalid, h, vf);
+        finish_tfrags<2 * TA, 2, false, 4>(pf.vD, nvalid, r, h, vf);
 #pragma unroll
         for (int tl = 0; tl < 2; ++tl)
 #pragma unroll
           for (int p = 0; p < 2; ++p) vfrag[2 * TA + tl][p] = vf[tl][p];
       }
       if (OUT) apply_scores<FWD ? 1 : 2>(score_tile(ka, qa), TA, r, h, vfrag, O[0][TA], O[1][TA]);
-      store_kt(kt, 32 * TA + r, h, ka.h);
+      store_kt<NG>(kt, 32 * TA + r, h, ka.h);
       if (OUT) {
 #pragma unroll
-        for (int ks = 0; ks < 4; ++ks) qkeep[TA][ks] = qa.h[ks];
+        for (int ks = 0; ks < NG; ++ks) qkeep[TA][ks] = qa.h[ks];
       }
     }
     VIG_PHASE();
     if (OUT) {
-      make_half<true>(rawq, true, G[TB], gend2, qb);
+      make_half<true, NG>(rawq, true, G[TB], gend2, qb);
       apply_scores<0>(score_tile(ka, qb), TA, r, h, vfrag, O[0][TB], O[1][TB]);
     }
     VIG_PHASE();
     {
-      HalfOps kb;
-      make_half<false>(rawk, 32 * TB + r < nvalid, G[TB], gend2, kb);
+      HalfOps<NG> kb;
+      make_half<false, NG>(rawk, 32 * TB + r < nvalid, G[TB], gend2, kb);
       {
         u32x4_t vf[2][2];
-        finish_tfrags<2 * TB, 2, false>(vDb, nvalid, h, vf);
+        finish_tfrags<2 * TB, 2, false, 4>(vDb, nvalid, r, h, vf);
 #pragma unroll
         for (int tl = 0; tl < 2; ++tl)
 #pragma unroll
           for (int p = 0; p < 2; ++p) vfrag[2 * TB + tl][p] = vf[tl][p];
       }
       if (OUT) apply_scores<FWD ? 1 : 2>(score_tile(kb, qb), TB, r, h, vfrag, O[0][TB], O[1][TB]);
-      store_kt(kt, 32 * TB + r, h, kb.h);
+      store_kt<NG>(kt, 32 * TB + r, h, kb.h);
     }
     if (OUT) {
 #pragma unroll
-      for (int ks = 0; ks < 4; ++ks) qkeep[TB][ks] = qb.h[ks];
+      for (int ks = 0; ks < NG; ++ks) qkeep[TB][ks] = qb.h[ks];
     }
   }
   VIG_STAMP(3);
@@ -431,7 +453,7 @@ __device__ __forceinline__ void direction_wave(const uint16_t* q, const uint16_t
 #pragma unroll
     for (int t = 0; t < 4; ++t) {
       u32x4_t ktf[2];
-      load_tfrag_lds(kt, t, r, h, ktf);
+      load_tfrag_lds<NG>(kt, t, r, h, ktf);
 #pragma unroll
       for (int pk = 0; pk < 2; ++pk)
 #pragma unroll
@@ -444,7 +466,7 @@ __device__ __forceinline__ void direction_wave(const uint16_t* q, const uint16_t
 #pragma unroll
         for (int pv = 0; pv < 2; ++pv)
 #pragma unroll
-          for (int cq = 0; cq < 4; ++cq) {
+          for (int cq = 0; cq < NG; ++cq) {  // rows of register quads >= NG carry no channel
             const f32x4_t x = {U[pk][pv][4 * cq], U[pk][pv][4 * cq + 1], U[pk][pv][4 * cq + 2], U[pk][pv][4 * cq + 3]};
             *reinterpret_cast<f32x4_t*>(unit_ptr(region, (pk * 2 + pv) * 4 + cq, lane)) = x;
           }
@@ -453,21 +475,22 @@ __device__ __forceinline__ void direction_wave(const uint16_t* q, const uint16_t
   // ---- forward waves fetch the first phase of the NEXT segment here, reverse waves fetch theirs at the top of the
   // segment: a wave stalls while the memory pipe accepts its loads, and this way the other wave of the SIMD has math
   // to do.  (Always issued: after the last segment it re-reads the current one, which keeps branches off the loads.) ----
-  if (FWD) issue_first_phase<FWD, OUT>(qn, kn, vn, gn, nvalid_next, r, h, pf);
+  if (FWD) issue_first_phase<FWD, OUT, NG>(qn, kn, vn, gn, nvalid_next, r, h, pf);
   VIG_STAMP(5);
   lds_barrier();  // (A) published U's and decays visible
   VIG_STAMP(6);
-  // ---- state recurrence over the chunks of this direction, one slice (pv, two register quads) per wave ----
+  // ---- state recurrence over the chunks of this direction, one slice (pv, NG/2 register quads) per wave ----
   {
-    const int pv = c & 1, cqa = 2 * (c >> 1);
+    constexpr int NQ = NG / 2;
+    const int pv = c & 1, cqa = NQ * (c >> 1);
     char* dirbase = lds + (FWD ? 0 : 4) * kRegionBytes;
     const float* ddir = dvec_all + (FWD ? 0 : 4) * 64;
     constexpr int W0 = FWD ? 0 : 3, STEP = FWD ? 1 : -1;
-    f32x4_t S[2][2];
+    f32x4_t S[2][NQ];
 #pragma unroll
     for (int pk = 0; pk < 2; ++pk)
 #pragma unroll
-      for (int j = 0; j < 2; ++j) {
+      for (int j = 0; j < NQ; ++j) {
         const int u = (pk * 2 + pv) * 4 + cqa + j;
         if (MODE == kModeChain)  // state entering the segment, written by the segment scan in the same unit order
           S[pk][j] = *reinterpret_cast<const f32x4_t*>(state + (u * 64 + lane) * 4);
@@ -480,10 +503,10 @@ __device__ __forceinline__ void direction_wave(const uint16_t* q, const uint16_t
       char* creg = dirbase + wc * kRegionBytes;
       const bool add_u = MODE == kModeState || i < 3;
 #pragma unroll
-      for (int j = 0; j < 2; ++j) {
+      for (int j = 0; j < NQ; ++j) {
         const int cq = cqa + j;
-        const f32x4_t d0 = *reinterpret_cast<const f32x4_t*>(ddir + wc * 64 + 32 * h + 8 * cq);
-        const f32x4_t d1 = *reinterpret_cast<const f32x4_t*>(ddir + wc * 64 + 32 * h + 8 * cq + 4);
+        const f32x4_t d0 = *reinterpret_cast<const f32x4_t*>(ddir + wc * 64 + HC * h + 8 * cq);
+        const f32x4_t d1 = *reinterpret_cast<const f32x4_t*>(ddir + wc * 64 + HC * h + 8 * cq + 4);
         // decay of row (m, pk): element 2*m + pk of the eight
         const float dk0[4] = {d0[0], d0[2], d1[0], d1[2]};
         const float dk1[4] = {d0[1], d0[3], d1[1], d1[3]};
@@ -509,9 +532,10 @@ __device__ __forceinline__ void direction_wave(const uint16_t* q, const uint16_t
 #pragma unroll
       for (int pk = 0; pk < 2; ++pk)
 #pragma unroll
-        for (int j = 0; j < 2; ++j)
+        for (int j = 0; j < NQ; ++j)
           *reinterpret_cast<f32x4_t*>(state + (((pk * 2 + pv) * 4 + cqa + j) * 64 + lane) * 4) = S[pk][j];
-      if (c == 0) state[64 * 64 + lane] = ddir[lane] * ddir[64 + lane] * ddir[128 + lane] * ddir[192 + lane];
+      if (c == 0 && lane < 16 * NG)
+        state[64 * 64 + lane] = ddir[lane] * ddir[64 + lane] * ddir[128 + lane] * ddir[192 + lane];
     }
   }
   VIG_STAMP(7);
@@ -523,7 +547,7 @@ __device__ __forceinline__ void direction_wave(const uint16_t* q, const uint16_t
 #pragma unroll
       for (int pv = 0; pv < 2; ++pv)
 #pragma unroll
-        for (int ks = 0; ks < 4; ++ks) {
+        for (int ks = 0; ks < NG; ++ks) {
           const u32x4_t sf = *reinterpret_cast<const u32x4_t*>(unit_ptr(region, pv * 4 + ks, lane));
 #pragma unroll
           for (int it = 0; it < 2; ++it) O[pv][it] = mfma(sf, qkeep[it][ks], O[pv][it]);
@@ -583,7 +607,7 @@ struct Geometry {
   int L, nseg, seg_len, cw, nitems;
 };
 
-template <bool FWD, int MODE>
+template <bool FWD, int MODE, int NG>
 __device__ __forceinline__ void wave_loop(const uint16_t* q, const uint16_t* k, const uint16_t* v, const uint16_t* g,
                                           uint16_t* o, const Geometry& geo, int c, int lane, char* lds, float oscale,
                                           bool bidir, float* state_ws) {
@@ -593,15 +617,17 @@ __device__ __forceinline__ void wave_loop(const uint16_t* q, const uint16_t* k, 
     const int seq = item / geo.nseg, seg = item - seq * geo.nseg;
     const int seg_tokens = min(geo.seg_len, geo.L - seg * geo.seg_len);
     nvalid = min(max(seg_tokens - c * geo.cw, 0), geo.cw);
-    off = ((size_t)seq * geo.L + (size_t)seg * geo.seg_len + (size_t)(nvalid > 0 ? c * geo.cw : 0)) * 64;
+    off = (size_t)seq * geo.L + (size_t)seg * geo.seg_len + (size_t)(nvalid > 0 ? c * geo.cw : 0);  // in tokens
   };
-  Prefetch pf;
+  constexpr int DK = 16 * NG;
+  Prefetch<NG> pf;
   int item = blockIdx.x;
   size_t b = 0;
   int nvalid = 0;
   if (item < geo.nitems) {
     locate(item, b, nvalid);
-    if (FWD) issue_first_phase<FWD, OUT>(q + b, k + b, v + b, g + b, nvalid, lane & 31, lane >> 5, pf);
+    if (FWD)
+      issue_first_phase<FWD, OUT, NG>(q + b * DK, k + b * DK, v + b * 64, g + b * DK, nvalid, lane & 31, lane >> 5, pf);
   }
   int iter = 0;
   for (; item < geo.nitems; item += gridDim.x, ++iter) {
@@ -611,8 +637,9 @@ __device__ __forceinline__ void wave_loop(const uint16_t* q, const uint16_t* k, 
     if (next < geo.nitems) locate(next, bn, nvalid_next);
     float* state = state_ws ? state_ws + ((size_t)item * 2 + (FWD ? 0 : 1)) * kStateFloats : nullptr;
     asm volatile("" : "+v"(lane));  // per-lane constants are rebuilt per item instead of living across the loop
-    direction_wave<FWD, MODE>(q + b, k + b, v + b, g + b, o + b, q + bn, k + bn, v + bn, g + bn, nvalid, nvalid_next, c,
-                              lane, lds, oscale, bidir, state, pf, iter);
+    direction_wave<FWD, MODE, NG>(q + b * DK, k + b * DK, v + b * 64, g + b * DK, o + b * 64, q + bn * DK, k + bn * DK,
+                                  v + bn * 64, g + bn * DK, nvalid, nvalid_next, c, lane, lds, oscale, bidir, state, pf,
+                                  iter);
     lds_barrier();  // (D) the next item reuses the LDS regions
     b = bn;
     nvalid = nvalid_next;
@@ -621,7 +648,7 @@ __device__ __forceinline__ void wave_loop(const uint16_t* q, const uint16_t* k, 
 
 }  // namespace
 
-template <int MODE>
+template <int MODE, int NG>
 __global__ __launch_bounds__(512) void gla_mfma_kernel(const uint16_t* __restrict__ q, const uint16_t* __restrict__ k,
                                                        const uint16_t* __restrict__ v, const uint16_t* __restrict__ gf,
                                                        const uint16_t* __restrict__ gb, uint16_t* __restrict__ o,
@@ -633,9 +660,9 @@ __global__ __launch_bounds__(512) void gla_mfma_kernel(const uint16_t* __restric
   const int c = wi & 3;
   const bool bidir = gb != nullptr;
   if (wi < 4) {
-    wave_loop<true, MODE>(q, k, v, gf, o, geo, c, lane, lds, oscale, bidir, state_ws);
+    wave_loop<true, MODE, NG>(q, k, v, gf, o, geo, c, lane, lds, oscale, bidir, state_ws);
   } else if (bidir) {
-    wave_loop<false, MODE>(q, k, v, gb, o, geo, c, lane, lds, oscale, bidir, state_ws);
+    wave_loop<false, MODE, NG>(q, k, v, gb, o, geo, c, lane, lds, oscale, bidir, state_ws);
   } else {
     for (int item = blockIdx.x; item < geo.nitems; item += gridDim.x) {
       lds_barrier();
@@ -649,13 +676,14 @@ __global__ __launch_bounds__(512) void gla_mfma_kernel(const uint16_t* __restric
 // Chains the segments of every sequence: in place, the workspace slot of segment s (its own contribution U_s and
 // decay D_s) is replaced by the state entering it,  S_in(s') = D_s * S_in(s) + U_s  with s' the next segment in the
 // direction's walk order.  One thread per state element; all accesses are coalesced (unit order is kept).
-__global__ __launch_bounds__(256) void gla_segment_scan_kernel(float* state_ws, int nseq, int nseg, int ndir) {
+__global__ __launch_bounds__(256) void gla_segment_scan_kernel(float* state_ws, int nseq, int nseg, int ndir, int ng) {
   const int e = blockIdx.x * 256 + threadIdx.x;  // element in unit order: ((u*64 + lane)*4 + m)
   const int seq = blockIdx.y / ndir, dir = blockIdx.y % ndir;
   if (seq >= nseq) return;
   const int m = e & 3, lane = (e >> 2) & 63, u = e >> 8;
   const int pk = u >> 3, cq = u & 3, h = lane >> 5;
-  const int ch = 32 * h + 8 * cq + 2 * m + pk;
+  if (cq >= ng) return;  // register quads beyond Dk/16 carry no channel
+  const int ch = 8 * ng * h + 8 * cq + 2 * m + pk;
   float S = 0.f;
   for (int i = 0; i < nseg; ++i) {
     const int seg = dir == 0 ? i : nseg - 1 - i;
@@ -678,27 +706,25 @@ static Geometry make_geometry(int nseq, int L) {
 }
 
 bool gla_mfma_supported(const GlaArgs& a) {
-  return a.io_dtype == 1 && a.gate_dtype == 1 && a.Dk == 64 && a.Dv == 64;
+  return a.io_dtype == 1 && a.gate_dtype == 1 && (a.Dk == 64 || a.Dk == 32) && a.Dv == 64;
 }
 
 size_t gla_mfma_workspace(int B, int H, int L, int Dk, int Dv) {
-  if (Dk != 64 || Dv != 64 || L <= 256) return 0;
+  if ((Dk != 64 && Dk != 32) || Dv != 64 || L <= 256) return 0;
   const Geometry g = make_geometry(B * H, L);
   return (size_t)g.nitems * 2 * kStateFloats * sizeof(float);
 }
 
-int launch_gla_mfma(const GlaArgs& a) {
-  static int num_cu = 0;
-  if (num_cu == 0) {
-    int dev = 0;
-    hipDeviceProp_t prop;
-    if (hipGetDevice(&dev) != hipSuccess || hipGetDeviceProperties(&prop, dev) != hipSuccess) return -5;
-    const void* kernels[3] = {reinterpret_cast<const void*>(gla_mfma_kernel<kModeSlab>),
-                              reinterpret_cast<const void*>(gla_mfma_kernel<kModeState>),
-                              reinterpret_cast<const void*>(gla_mfma_kernel<kModeChain>)};
+template <int NG>
+static int launch_gla_mfma_t(const GlaArgs& a, int num_cu) {
+  static bool attr_done = false;
+  if (!attr_done) {
+    const void* kernels[3] = {reinterpret_cast<const void*>(gla_mfma_kernel<kModeSlab, NG>),
+                              reinterpret_cast<const void*>(gla_mfma_kernel<kModeState, NG>),
+                              reinterpret_cast<const void*>(gla_mfma_kernel<kModeChain, NG>)};
     for (const void* kf : kernels)
       if (hipFuncSetAttribute(kf, hipFuncAttributeMaxDynamicSharedMemorySize, kLdsTotal) != hipSuccess) return -5;
-    num_cu = prop.multiProcessorCount > 0 ? prop.multiProcessorCount : 256;
+    attr_done = true;
   }
   const Geometry geo = make_geometry(a.B * a.H, a.L);
   int grid = geo.nitems < num_cu ? geo.nitems : num_cu;
@@ -713,19 +739,30 @@ int launch_gla_mfma(const GlaArgs& a) {
   uint16_t* o = (uint16_t*)a.o;
   const float oscale = a.scale * a.out_scale;
   if (geo.nseg == 1) {
-    hipLaunchKernelGGL(gla_mfma_kernel<kModeSlab>, dim3(grid), dim3(512), kLdsTotal, a.stream, q, k, v, gf, gb, o, geo,
-                       oscale, (float*)nullptr);
+    hipLaunchKernelGGL((gla_mfma_kernel<kModeSlab, NG>), dim3(grid), dim3(512), kLdsTotal, a.stream, q, k, v, gf, gb, o,
+                       geo, oscale, (float*)nullptr);
   } else {
     float* ws = (float*)a.workspace;
-    hipLaunchKernelGGL(gla_mfma_kernel<kModeState>, dim3(grid), dim3(512), kLdsTotal, a.stream, q, k, v, gf, gb, o, geo,
-                       oscale, ws);
+    hipLaunchKernelGGL((gla_mfma_kernel<kModeState, NG>), dim3(grid), dim3(512), kLdsTotal, a.stream, q, k, v, gf, gb, o,
+                       geo, oscale, ws);
     const int ndir = gb ? 2 : 1;
     hipLaunchKernelGGL(gla_segment_scan_kernel, dim3(64 * 64 / 256, a.B * a.H * ndir), dim3(256), 0, a.stream, ws,
-                       a.B * a.H, geo.nseg, ndir);
-    hipLaunchKernelGGL(gla_mfma_kernel<kModeChain>, dim3(grid), dim3(512), kLdsTotal, a.stream, q, k, v, gf, gb, o, geo,
-                       oscale, ws);
+                       a.B * a.H, geo.nseg, ndir, NG);
+    hipLaunchKernelGGL((gla_mfma_kernel<kModeChain, NG>), dim3(grid), dim3(512), kLdsTotal, a.stream, q, k, v, gf, gb, o,
+                       geo, oscale, ws);
   }
   return hipGetLastError() == hipSuccess ? 0 : -5;
+}
+
+int launch_gla_mfma(const GlaArgs& a) {
+  static int num_cu = 0;
+  if (num_cu == 0) {
+    int dev = 0;
+    hipDeviceProp_t prop;
+    if (hipGetDevice(&dev) != hipSuccess || hipGetDeviceProperties(&prop, dev) != hipSuccess) return -5;
+    num_cu = prop.multiProcessorCount > 0 ? prop.multiProcessorCount : 256;
+  }
+  return a.Dk == 64 ? launch_gla_mfma_t<4>(a, num_cu) : launch_gla_mfma_t<2>(a, num_cu);
 }
 
 #ifdef VIG_TIMING
