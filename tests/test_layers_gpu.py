@@ -1,0 +1,77 @@
+"""Block- and model-level checks of the host-side mirror against the CPU restatement of the eval path."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import vig_model_ref as R
+from vig_amd import layers
+
+from .util import announce
+
+pytestmark = pytest.mark.gpu
+
+
+def test_reference_parameter_names():
+    """state_dict keys of the GLA block are the reference's (classification/models/vig.py:291-311)."""
+    m = layers.GatedLinearAttention(d_model=384, expand_k=0.5, expand_v=1.0, num_heads=6, use_act_in_conv=False)
+    keys = set(m.state_dict().keys())
+    assert keys == {"in_proj.0.weight", "qkv_proj.weight", "gk_proj.0.weight", "gk_proj.1.weight", "gk_proj.1.bias",
+                    "o_proj.weight", "g_norm.weight", "l_norm.weight", "g_proj.weight", "g_proj.bias"}
+    assert m.qkv_proj.weight.shape == (768, 384) and m.gk_proj[1].weight.shape == (384, 16)
+    assert m.head_qk_dim == 32 and m.head_v_dim == 64
+
+
+@pytest.mark.parametrize("dtype,tol", [(torch.float32, 2e-4), (torch.bfloat16, 6e-2)])
+@pytest.mark.parametrize("variant", ["s", "t"])
+def test_gla_block_matches_restatement(dtype, tol, variant):
+    announce(f"GatedLinearAttention eval forward, vig-{variant}, {dtype}")
+    torch.manual_seed(0)
+    if variant == "s":
+        dim, H, kw = 384, 6, dict(use_act_in_conv=False, use_out_act=False)
+    else:
+        dim, H, kw = 192, 3, dict(use_act_in_conv=True, use_out_act=True)
+    m = layers.GatedLinearAttention(d_model=dim, expand_k=0.5, expand_v=1.0, num_heads=H, layernorm_eps=1e-6, **kw).eval()
+    # non-trivial norm weights and biases
+    with torch.no_grad():
+        m.g_norm.weight.uniform_(0.5, 1.5)
+        m.l_norm.weight.uniform_(0.5, 1.5)
+        m.g_proj.bias.normal_(0, 0.5)
+        m.gk_proj[1].bias.normal_(0, 1.0)
+        for lin in (m.qkv_proj, m.g_proj, m.o_proj, m.gk_proj[0], m.gk_proj[1]):
+            lin.weight.mul_(8.0)  # the 2^-2.5 init makes everything tiny; scale up so errors are visible
+    x = torch.randn(2, 196, dim)
+    sd = {k: v.double() for k, v in m.state_dict().items()}
+    want = R.gla_block_attn(sd, "", x.double(), (14, 14), H, 1e-6, kw["use_act_in_conv"], kw["use_out_act"]).numpy()
+    md = m.to("cuda", dtype)
+    got = md(x.to("cuda", dtype), patch_resolution=(14, 14), token_position=None).double().cpu().numpy()
+    err = np.abs(got - want).max() / np.abs(want).max()
+    print(f"  max-rel err {err:.3e}", flush=True)
+    assert err <= tol
+
+
+def test_gla_block_train_mode_scale():
+    """Training-mode glue averages the directions once (out_scale 1/2), eval halves twice (1/4); the RMS norm that
+    follows hides the factor only up to eps, so compare the pre-norm op directly."""
+    announce("GLA block train/eval scale convention")
+    import vig_amd
+    from vig_amd.synthetic import make_gla_inputs
+
+    q, k, v, gf, gb = [t.cuda() for t in make_gla_inputs(1, 2, 50, 32, 64, seed=3)]
+    a = vig_amd.gla_bidir_forward(q, k, v, gf, gb, out_scale=0.5)
+    b = vig_amd.gla_bidir_forward(q, k, v, gf, gb, out_scale=0.25)
+    assert torch.allclose(a, 2 * b, rtol=1e-6, atol=1e-7)
+
+
+@pytest.mark.parametrize("dtype,tol", [(torch.float32, 5e-4), (torch.bfloat16, 8e-2)])
+def test_vig_small_logits(dtype, tol):
+    """Full ViG-S eval forward (random init, synthetic images) against the float64 restatement on the same state_dict."""
+    announce(f"ViG-S logits {dtype}")
+    torch.manual_seed(0)
+    model = layers.vig_small().eval()
+    images = torch.randn(2, 3, 224, 224)
+    want = R.vig_forward(model.state_dict(), images, num_heads=6, depth=12).numpy()
+    got = model.to("cuda", dtype)(images.to("cuda", dtype)).double().cpu().numpy()
+    err = np.abs(got - want).max() / np.abs(want).max()
+    print(f"  logits max-rel err {err:.3e}  (max |logit| {np.abs(want).max():.3f})", flush=True)
+    assert got.shape == (2, 1000)
+    assert err <= tol

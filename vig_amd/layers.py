@@ -1,0 +1,260 @@
+"""Block- and model-level host side: the reference's module interfaces over the HIP ops.
+
+`GatedLinearAttention` keeps the constructor arguments, forward signature and parameter names of
+classification/models/vig.py:241-464, so a reference state_dict loads unchanged.  The three GEMMs
+(qkv_proj, gk_proj, g_proj, o_proj) stay in torch (hipBLASLt); everything between them runs in this
+package's kernels:
+    3x3 depthwise conv on the token grid   -> vig_dwconv3x3_fwd      (vig.py:291-294,428-430)
+    direction-wise gate preparation        -> vig_dirgate_fwd        (vig.py:432-441)
+    bidirectional GLA                      -> vig_gla_bidir_fwd      (vig.py:442-443)
+    RMS-norm x2 + sigmoid blend (+SiLU)    -> vig_locality_blend_fwd (vig.py:444-457)
+The surrounding ViG shell (patch embedding, residual RMSNorm wiring, SwiGLU MLP, head) is plain torch
+and follows vig.py:469-497,530-618,625-672,705-912 for the options the shipped configs use.
+
+Forward (inference) only: the HIP ops carry no autograd graph.
+"""
+from __future__ import annotations
+
+import math
+from typing import Optional
+
+import torch
+import torch.nn as nn
+import torch.nn.functional as F
+
+from . import ops
+
+
+class RMSNorm(nn.Module):
+    """x * rsqrt(mean(x^2) + eps) * weight, arithmetic in fp32 (fla/modules/rmsnorm.py:38-52,491-512).
+
+    forward(x, residual=None, prenorm=False): with a residual the sum is normalised and, with
+    prenorm=True, also returned (rmsnorm.py:94-106) -- the wiring GLABlock relies on.
+    """
+
+    def __init__(self, hidden_size: int, eps: float = 1e-5):
+        super().__init__()
+        self.eps = eps
+        self.weight = nn.Parameter(torch.ones(hidden_size))
+
+    def forward(self, x, residual=None, prenorm: bool = False):
+        if residual is not None:
+            x = (x + residual).to(x.dtype)
+        xf = x.float()
+        y = xf * torch.rsqrt(xf.pow(2).mean(-1, keepdim=True) + self.eps) * self.weight.float()
+        y = y.to(x.dtype)
+        return (y, x) if prenorm else y
+
+
+class GatedLinearAttention(nn.Module):
+    """ViG's bidirectional GLA token mixer (classification/models/vig.py:241-464)."""
+
+    def __init__(self, d_model: int = 1024, expand_v: float = 2.0, expand_k: float = 1.0, num_heads: int = 4,
+                 gate_fn: str = "swish", layernorm_eps: float = 1e-5, gate_logit_normalizer: int = 16,
+                 gate_low_rank_dim: int = 16, mode: str = "fused_chunk", clamp_min: Optional[float] = None,
+                 fuse_norm: bool = True, use_dirpe: bool = False, use_out_act: bool = False,
+                 use_out_gate: bool = True, rope_mode: str = "none", use_act_in_conv: bool = True,
+                 use_bias_in_dwconv: bool = False, *args, **kwargs):
+        super().__init__()
+        if mode not in ("chunk", "fused_recurrent", "fused_chunk", "bid_fused_chunk", "bidv2_fused_chunk"):
+            raise AssertionError(f"Not suppoerted mode `{mode}`.")
+        if rope_mode != "none":
+            raise NotImplementedError("rope modes other than 'none' are not used by the shipped ViG configs")
+        if use_dirpe:
+            raise NotImplementedError("use_dirpe is not used by the shipped ViG configs")
+        if gate_fn not in ("swish", "silu"):
+            raise NotImplementedError("only the swish/SiLU gate function is built")
+        self.d_model = d_model
+        self.mode = mode
+        self.value_dim = int(d_model * expand_v)
+        self.key_dim = int(d_model * expand_k)
+        self.clamp_min = clamp_min
+        assert self.key_dim % num_heads == 0, f"key dim must be divisible by num_heads of {num_heads}"
+        assert self.value_dim % num_heads == 0, f"value dim must be divisible by num_heads of {num_heads}"
+        self.num_heads = num_heads
+        self.head_qk_dim = self.key_dim // num_heads
+        self.head_v_dim = self.value_dim // num_heads
+        self.use_out_gate = use_out_gate  # stored, never read (as in the reference, vig.py:285)
+        self.use_out_act = use_out_act
+        self.use_act_in_conv = use_act_in_conv
+        self.layernorm_eps = layernorm_eps
+        self.gate_logit_normalizer = gate_logit_normalizer
+
+        self.in_proj = nn.Sequential(
+            nn.Conv2d(d_model, d_model, kernel_size=3, padding=1, groups=d_model, bias=use_bias_in_dwconv),
+            nn.SiLU() if use_act_in_conv else nn.Identity(),
+        )
+        self.qkv_proj = nn.Linear(d_model, 2 * self.key_dim + self.value_dim, bias=False)
+        self.gk_proj = nn.Sequential(nn.Linear(d_model, gate_low_rank_dim, bias=False),
+                                     nn.Linear(gate_low_rank_dim, self.key_dim * 2, bias=True))
+        self.o_proj = nn.Linear(self.value_dim, d_model, bias=False)
+        self.g_norm = RMSNorm(self.head_v_dim, eps=layernorm_eps)
+        self.l_norm = RMSNorm(self.head_v_dim, eps=layernorm_eps)
+        self.g_proj = nn.Linear(d_model, self.value_dim, bias=True)
+        self.reset_parameters()
+
+    def reset_parameters(self):
+        gain = 2 ** -2.5
+        nn.init.xavier_uniform_(self.qkv_proj.weight, gain=gain)
+        nn.init.xavier_uniform_(self.in_proj[0].weight, gain=gain)
+        nn.init.xavier_uniform_(self.g_proj.weight, gain=gain)
+        nn.init.xavier_uniform_(self.o_proj.weight, gain=gain)
+        nn.init.xavier_uniform_(self.gk_proj[0].weight, gain=gain)
+        nn.init.xavier_uniform_(self.gk_proj[1].weight, gain=gain)
+
+    @torch.no_grad()
+    def forward(self, x, lower_bound=0, **kwargs):
+        B, L, C = x.shape
+        if kwargs.get("token_position", None) is not None:
+            raise NotImplementedError("class-token splicing is not built (the shipped configs use IF_CLS_TOKEN False)")
+        hw = tuple(kwargs["patch_resolution"])
+        H = self.num_heads
+        conv = self.in_proj[0]
+        # local_out, already in the [B, L, C] layout the projections consume
+        xs = ops.dwconv3x3(x, conv.weight, hw, bias=conv.bias, silu=self.use_act_in_conv)
+        q, k, v = torch.split(self.qkv_proj(xs), [self.key_dim, self.key_dim, self.value_dim], dim=2)
+        gates = ops.dirgate(self.gk_proj(xs), H, self.gate_logit_normalizer, self.clamp_min)
+        heads = lambda t, d: t.reshape(B, L, H, d).permute(0, 2, 1, 3).contiguous()
+        q, k, v = heads(q, self.head_qk_dim), heads(k, self.head_qk_dim), heads(v, self.head_v_dim)
+        # training glue averages the directions (vig.py:425-426); the eval path halves twice
+        # (recurrent_fuse.py:442, then vig.py:443)
+        out_scale = 0.5 if self.training else 0.25
+        o = ops.gla_bidir_forward(q, k, v, gates[0], gates[1], scale=-1, out_scale=out_scale)
+        y = ops.locality_blend(o, xs, self.g_proj(xs), self.g_norm.weight, self.l_norm.weight,
+                               eps=self.layernorm_eps, silu_out=self.use_out_act)
+        return self.o_proj(y)
+
+
+class GLAMLP(nn.Module):
+    """SwiGLU MLP (vig.py:469-497; swiglu = x*sigmoid(x)*y, fla/modules/activations.py:109-113)."""
+
+    def __init__(self, hidden_size: int, hidden_ratio: Optional[int] = None, intermediate_size: Optional[int] = None,
+                 hidden_act: str = "swish"):
+        super().__init__()
+        if hidden_ratio is None:
+            hidden_ratio = 4
+        if intermediate_size is None:
+            intermediate_size = int(hidden_size * hidden_ratio * 2 / 3)
+            intermediate_size = 256 * ((intermediate_size + 256 - 1) // 256)
+        self.hidden_size, self.hidden_ratio, self.intermediate_size = hidden_size, hidden_ratio, intermediate_size
+        self.gate_proj = nn.Linear(hidden_size, intermediate_size * 2, bias=False)
+        self.down_proj = nn.Linear(intermediate_size, hidden_size, bias=False)
+
+    def forward(self, x):
+        gate, y = self.gate_proj(x).chunk(2, -1)
+        return self.down_proj(F.silu(gate) * y)
+
+
+class GLABlock(nn.Module):
+    """attn_norm -> GLA -> (residual add + mlp_norm, prenorm) -> MLP -> residual (vig.py:530-618), no layer scale."""
+
+    def __init__(self, hidden_size: int, num_heads: int, expand_k: float, expand_v: float, eps: float = 1e-6,
+                 use_out_act: bool = False, use_act_in_conv: bool = True, use_bias_in_dwconv: bool = False,
+                 intermediate_size: Optional[int] = None, mode: str = "fused_chunk"):
+        super().__init__()
+        self.attn_norm = RMSNorm(hidden_size, eps=eps)
+        self.attn = GatedLinearAttention(d_model=hidden_size, expand_k=expand_k, expand_v=expand_v,
+                                         num_heads=num_heads, layernorm_eps=eps, mode=mode, use_out_act=use_out_act,
+                                         use_act_in_conv=use_act_in_conv, use_bias_in_dwconv=use_bias_in_dwconv)
+        self.mlp_norm = RMSNorm(hidden_size, eps=eps)
+        self.mlp = GLAMLP(hidden_size, intermediate_size=intermediate_size)
+
+    def forward(self, hidden_states, **kwargs):
+        residual = hidden_states
+        h = self.attn(self.attn_norm(hidden_states), **kwargs)
+        h, residual = self.mlp_norm(h, residual, True)
+        return (residual + self.mlp(h),)
+
+
+class LayerNorm2d(nn.LayerNorm):
+    def forward(self, x):
+        return F.layer_norm(x.permute(0, 2, 3, 1), self.normalized_shape, self.weight, self.bias, self.eps).permute(0, 3, 1, 2)
+
+
+class V2PatchEmbed(nn.Module):
+    """Two strided convs with LayerNorm2d (vig.py:625-672), use_act_in_patch False."""
+
+    def __init__(self, patch_size=16, in_chans=3, embed_dim=768, use_bias_in_patch=True):
+        super().__init__()
+        stride = patch_size // 2
+        self.proj = nn.Sequential(
+            nn.Conv2d(in_chans, embed_dim // 2, kernel_size=stride + 1, stride=stride, padding=1, bias=use_bias_in_patch),
+            LayerNorm2d(embed_dim // 2),
+            nn.SiLU(),
+            nn.Conv2d(embed_dim // 2, embed_dim, kernel_size=3, stride=2, padding=1, bias=use_bias_in_patch),
+            LayerNorm2d(embed_dim),
+        )
+
+    def forward(self, x):
+        x = self.proj(x)
+        hw = tuple(x.shape[-2:])
+        return x.flatten(2).transpose(1, 2), hw
+
+
+def resize_pos_embed(pos_embed, src_shape, dst_shape):
+    """Bicubic resize of a [1, h*w, C] table (vig.py:915-958), no extra tokens."""
+    if tuple(src_shape) == tuple(dst_shape):
+        return pos_embed
+    _, L, C = pos_embed.shape
+    w = pos_embed.reshape(1, src_shape[0], src_shape[1], C).permute(0, 3, 1, 2)
+    w = F.interpolate(w.float(), size=dst_shape, align_corners=False, mode="bicubic")
+    return torch.flatten(w, 2).transpose(1, 2).to(pos_embed.dtype)
+
+
+class ViG(nn.Module):
+    """Non-hierarchical ViG with the options of the shipped vig-{t,s,b}.yaml (vig.py:705-912): v2 patch embedding,
+    absolute position table, no class token, SwiGLU MLP, average-pool head."""
+
+    def __init__(self, img_size=224, patch_size=16, depth=12, num_heads=6, embed_dim=384, channels=3,
+                 num_classes=1000, expand_k=0.5, expand_v=1.0, use_out_act=False, use_act_in_conv=False,
+                 use_bias_in_dwconv=False, rms_norm_eps=1e-6, initializer_range=0.02):
+        super().__init__()
+        self.embed_dim = embed_dim
+        self.patch_embed = V2PatchEmbed(patch_size=patch_size, in_chans=channels, embed_dim=embed_dim)
+        self.patch_resolution = (img_size // patch_size, img_size // patch_size)
+        self.pos_embed = nn.Parameter(torch.zeros(1, self.patch_resolution[0] * self.patch_resolution[1], embed_dim))
+        self.head = nn.Linear(embed_dim, num_classes)
+        self.blocks = nn.ModuleList([
+            GLABlock(embed_dim, num_heads, expand_k, expand_v, eps=rms_norm_eps, use_out_act=use_out_act,
+                     use_act_in_conv=use_act_in_conv, use_bias_in_dwconv=use_bias_in_dwconv)
+            for _ in range(depth)])
+        self.norm = RMSNorm(embed_dim, eps=rms_norm_eps)
+        # init order of the reference (vig.py:825-837,332-349): every Linear N(0, 0.02) with zero bias, then the
+        # GLA projections xavier-uniform with gain 2^-2.5; convs of the patch embedding keep torch's default
+        for m in self.modules():
+            if isinstance(m, nn.Linear):
+                nn.init.normal_(m.weight, mean=0.0, std=initializer_range)
+                if m.bias is not None:
+                    nn.init.zeros_(m.bias)
+        for m in self.modules():
+            if isinstance(m, GatedLinearAttention):
+                m.reset_parameters()
+        nn.init.trunc_normal_(self.pos_embed, std=0.02)
+
+    def forward_features(self, x):
+        B = x.shape[0]
+        x, hw = self.patch_embed(x)
+        x = x + resize_pos_embed(self.pos_embed, self.patch_resolution, hw)
+        for blk in self.blocks:
+            x = blk(x, patch_resolution=hw, token_position=None)[0]
+        x = self.norm(x)
+        return x.reshape(B, hw[0] * hw[1], -1).mean(dim=1)
+
+    @torch.no_grad()
+    def forward(self, x):
+        return self.head(self.forward_features(x))
+
+
+def vig_small(**kw):
+    """vig-s.yaml: dim 384, 6 heads (Dk 32, Dv 64), depth 12."""
+    return ViG(depth=12, num_heads=6, embed_dim=384, use_out_act=False, use_act_in_conv=False, **kw)
+
+
+def vig_tiny(**kw):
+    """vig-t.yaml: dim 192, 3 heads, depth 12, SiLU after the dwconv and on the blend output."""
+    return ViG(depth=12, num_heads=3, embed_dim=192, use_out_act=True, use_act_in_conv=True, **kw)
+
+
+def vig_base(**kw):
+    """vig-b.yaml: dim 768, 12 heads, depth 12."""
+    return ViG(depth=12, num_heads=12, embed_dim=768, use_out_act=False, use_act_in_conv=False, **kw)
