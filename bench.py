@@ -68,6 +68,28 @@ def cpu_baseline(shape, seed, budget_s=20.0):
     }
 
 
+def model_throughput(dev, batch=256, warmup=10, iters=30):
+    """Full ViG-S eval forward (random init, synthetic images, bf16): images/s the way the reference's
+    throughput() measures it (classification/main.py:389-406: timed forwards of one resident batch)."""
+    import torch
+
+    from vig_amd import layers
+
+    torch.manual_seed(0)
+    model = layers.vig_small().eval().to(dev, torch.bfloat16)
+    images = torch.randn(batch, 3, 224, 224, device=dev, dtype=torch.bfloat16)
+    for _ in range(warmup):
+        model(images)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(iters):
+        model(images)
+    torch.cuda.synchronize()
+    dt = time.perf_counter() - t0
+    return {"images_per_s": iters * batch / dt, "batch": batch, "dtype": "bf16", "iters": iters,
+            "ms_per_forward": dt / iters * 1e3}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -77,6 +99,10 @@ def main():
     ap.add_argument("--sets", type=int, default=0, help="input sets to rotate (0 = enough to exceed 256 MB, >= 3)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--exact", action="store_true", help="time the fp32-arithmetic recurrent kernel instead")
+    ap.add_argument("--model", action="store_true", help="also time the full ViG-S eval forward (images/s)")
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="also run plain device copies of known size (q -> o), so that FETCH_SIZE / WRITE_SIZE "
+                         "counters of a profiled run can be scaled to bytes")
     args = ap.parse_args()
 
     if args.gpus != 1:
@@ -126,6 +152,13 @@ def main():
                 ws.data_ptr(), ws_bytes, s.B, s.H, s.L, s.Dk, s.Dv, scale, 1.0, io_dt, io_dt, sp)
         if rc != 0:
             raise RuntimeError(f"vig_gla_bidir_fwd rc={rc}")
+
+    if args.copy_calibration:
+        # a copy kernel whose traffic is known exactly: numel*2 bytes read, numel*2 bytes written per call
+        for i in range(4):
+            sets[i % nsets][5].copy_(sets[i % nsets][2])
+        torch.cuda.synchronize()
+        log(f"copy calibration: {sets[0][2].numel() * sets[0][2].element_size()} bytes read and written per copy kernel")
 
     for i in range(args.warmup):
         step(i)
@@ -178,6 +211,8 @@ def main():
         "roofline": {"bound": "hbm", "achieved": achieved_gbps, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                      "frac": achieved_gbps / HBM_PEAK_GBPS, "traffic": None},
     }
+    if args.model:
+        out["vig_s_forward"] = model_throughput(dev)
     if not args.no_cpu:
         out["cpu_baseline"] = cpu_baseline(s, 1000 + args.config)
     else:

@@ -308,7 +308,7 @@ __device__ __forceinline__ void direction_wave(const uint16_t* q, const uint16_t
                                                int c, int lane, char* lds, float oscale, bool bidir, float* state,
                                                Prefetch<NG>& pf, int iter) {
   constexpr bool OUT = MODE != kModeState;  // produces outputs (needs q)
-  const int r = lane & 31, h = lane >> 5;
+  int r = lane & 31, h = lane >> 5;
   const int wi = (FWD ? 0 : 4) + c;
   constexpr int TA = FWD ? 0 : 1;  // tile walked first
   constexpr int TB = FWD ? 1 : 0;
@@ -477,6 +477,11 @@ __device__ __forceinline__ void direction_wave(const uint16_t* q, const uint16_t
   // to do.  (Always issued: after the last segment it re-reads the current one, which keeps branches off the loads.) ----
   if (FWD) issue_first_phase<FWD, OUT, NG>(qn, kn, vn, gn, nvalid_next, r, h, pf);
   VIG_STAMP(5);
+  // lane-derived addresses of the exchange phases are rebuilt here instead of being carried (and spilled) across
+  // the register-heavy tile phase
+  asm volatile("" : "+v"(lane));
+  r = lane & 31;
+  h = lane >> 5;
   lds_barrier();  // (A) published U's and decays visible
   VIG_STAMP(6);
   // ---- state recurrence over the chunks of this direction, one slice (pv, NG/2 register quads) per wave ----
@@ -634,7 +639,11 @@ __device__ __forceinline__ void wave_loop(const uint16_t* q, const uint16_t* k, 
     const int next = item + gridDim.x;
     size_t bn = b;
     int nvalid_next = nvalid;
-    if (next < geo.nitems) locate(next, bn, nvalid_next);
+    if (next < geo.nitems) {
+      locate(next, bn, nvalid_next);
+    } else {
+      nvalid_next = min(nvalid, 1);  // nothing follows: the (branch-free) prefetch degenerates to one row per tensor
+    }
     float* state = state_ws ? state_ws + ((size_t)item * 2 + (FWD ? 0 : 1)) * kStateFloats : nullptr;
     asm volatile("" : "+v"(lane));  // per-lane constants are rebuilt per item instead of living across the loop
     direction_wave<FWD, MODE, NG>(q + b * DK, k + b * DK, v + b * 64, g + b * DK, o + b * 64, q + bn * DK, k + bn * DK,
@@ -655,7 +664,7 @@ __global__ __launch_bounds__(512) void gla_mfma_kernel(const uint16_t* __restric
                                                        Geometry geo, float oscale, float* state_ws) {
   extern __shared__ __align__(16) char lds[];
   const int tid = threadIdx.x;
-  const int wi = tid >> 6;
+  const int wi = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform: region / chunk addressing stays scalar
   const int lane = tid & 63;
   const int c = wi & 3;
   const bool bidir = gb != nullptr;
