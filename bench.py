@@ -146,12 +146,24 @@ def main():
     fn = lib.vig_gla_bidir_fwd_exact if args.exact else lib.vig_gla_bidir_fwd
     scale = s.Dk ** -0.5
 
+    # workload 2 adds the sigmoid locality gate on the 14x14 grid of the GLA output (a second, stencil kernel)
+    with_gate = args.config == 2
+    if with_gate:
+        from vig_amd.synthetic import make_locality_weight
+        gate_w = make_locality_weight(s.H * s.Dv, 2002).reshape(s.H * s.Dv, 9).float().contiguous().to(dev)
+        gate_out = [torch.empty_like(t[5]) for t in sets]
+
     def step(i):
         q, k, v, gf, gb, o = sets[i % nsets]
         rc = fn(q.data_ptr(), k.data_ptr(), v.data_ptr(), gf.data_ptr(), gb.data_ptr(), o.data_ptr(),
                 ws.data_ptr(), ws_bytes, s.B, s.H, s.L, s.Dk, s.Dv, scale, 1.0, io_dt, io_dt, sp)
         if rc != 0:
             raise RuntimeError(f"vig_gla_bidir_fwd rc={rc}")
+        if with_gate:
+            rc = lib.vig_locality_gate_fwd(o.data_ptr(), gate_w.data_ptr(), gate_out[i % nsets].data_ptr(), s.B, s.H,
+                                           s.grid[0], s.grid[1], s.Dv, io_dt, sp)
+            if rc != 0:
+                raise RuntimeError(f"vig_locality_gate_fwd rc={rc}")
 
     if args.copy_calibration:
         # a copy kernel whose traffic is known exactly: numel*2 bytes read, numel*2 bytes written per call
@@ -185,6 +197,15 @@ def main():
     k_min = durs[0]
     log(f"wall {ms_per_step*1e3:.1f} us/step; event-bracketed launch avg {k_avg*1e3:.1f} us, median {k_med*1e3:.1f}, min {k_min*1e3:.1f}")
 
+    # HBM bytes per launch measured with rocprofv3 --pmc (FETCH_SIZE / WRITE_SIZE, scaled by a copy kernel of known
+    # size); the figures live with the profile summaries and are keyed by workload
+    traffic = None
+    try:
+        with open(os.path.join(ROOT, "profiles", "hbm_traffic.json")) as f:
+            traffic = json.load(f).get(s.name, {}).get("bytes_per_launch")
+    except (OSError, ValueError):
+        pass
+
     tflops = alg_flops / (ms_per_step * 1e-3) / 1e12
     achieved_gbps = alg_bytes / (k_avg * 1e-3) / 1e9
     exec_flops_tok = 2 * (2 * 64 * (s.Dk + s.Dv) + 4 * s.Dk * s.Dv)  # executed MFMA FLOPs/token at chunk 64
@@ -203,13 +224,14 @@ def main():
         "dtype": s.dtype,
         "data": "synthetic",
         "config": {"workload": s.name, "B": s.B, "H": s.H, "L": s.L, "Dk": s.Dk, "Dv": s.Dv,
-                   "input_sets_rotated": nsets, "kernel_path": "recurrent_fp32" if args.exact else "default"},
+                   "input_sets_rotated": nsets, "kernel_path": "recurrent_fp32" if args.exact else "default",
+                   "locality_gate": "separate stencil kernel after the GLA" if with_gate else None},
         "tokens_per_s": s.tokens / (ms_per_step * 1e-3),
         "mfma_frac_algorithmic": tflops / MFMA_BF16_PEAK_TFLOPS,
         "executed_tflops_chunk64": s.tokens * exec_flops_tok / (ms_per_step * 1e-3) / 1e12,
         "kernel_us": {"avg": k_avg * 1e3, "median": k_med * 1e3, "min": k_min * 1e3},
         "roofline": {"bound": "hbm", "achieved": achieved_gbps, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-                     "frac": achieved_gbps / HBM_PEAK_GBPS, "traffic": None},
+                     "frac": achieved_gbps / HBM_PEAK_GBPS, "traffic": traffic},
     }
     if args.model:
         out["vig_s_forward"] = model_throughput(dev)

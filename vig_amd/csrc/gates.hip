@@ -105,115 +105,89 @@ int launch_dirgate(const void* in, void* out, int B, int L, int H, int Dk, float
 }
 
 // ---------------------------------------------------------------------------
-// 3x3 depthwise stencil, channels-last:  x [B, h*w, C] -> y [B, h*w, C]
-// one thread = one token x 8 channels; weights [C,3,3] f32
+// 3x3 depthwise stencil on the token grid, channels-last.  One workgroup owns one image (or one head slab) and a
+// group of 64 channels: thread = (channel octet, token lane); it keeps the 8x9 weights of its channels in registers
+// and walks tokens lane, lane+32, ...; the nine neighbours of a token are 16-byte reads that hit L1/L2 (the 64-channel
+// slab of one image is a few tens of KB).
+//   GATE = false:  y = conv(x) (+bias) (SiLU optional)          x, y [N, h*w, C] with row stride `stride` elements
+//   GATE = true :  y = x * sigmoid(conv(x))                      (bias / SiLU unused)
+// weights [Ctot, 9] f32; the workgroup's first channel inside the weight table is wch0 = (blockIdx.y * 64 + woff).
 // ---------------------------------------------------------------------------
-template <typename T>
-__global__ __launch_bounds__(256) void dwconv3x3_kernel(const T* __restrict__ x, const float* __restrict__ wt,
-                                                         const float* __restrict__ bias, T* __restrict__ y, int B,
-                                                         int h, int w, int C, int silu, size_t nvec) {
-  const int c8n = C >> 3;
+template <typename T, bool GATE>
+__global__ __launch_bounds__(256) void stencil3x3_kernel(const T* __restrict__ x, const float* __restrict__ wt,
+                                                          const float* __restrict__ bias, T* __restrict__ y, int h, int w,
+                                                          int stride, int groups_per_image, int wmod, int cgroup,
+                                                          int silu) {
+  const int oct = threadIdx.x & 7, tl = threadIdx.x >> 3;  // 8 octets x 32 token lanes
+  const int img = blockIdx.x / groups_per_image, grp = blockIdx.x % groups_per_image;
+  if (grp * 64 + oct * 8 >= cgroup) return;  // channel tail of the last group (no barriers in this kernel)
   const int L = h * w;
-  for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < nvec; i += (size_t)gridDim.x * 256) {
-    const int c8 = (int)(i % c8n);
-    const size_t bl = i / c8n;
-    const int l = (int)(bl % L);
-    const size_t b = bl / L;
-    const int r = l / w, c = l % w;
-    const int ch = c8 * 8;
-    float accv[8];
+  const size_t base = (size_t)img * L * stride + (size_t)grp * 64 + oct * 8;
+  const int wch = (blockIdx.x % wmod) * (GATE ? cgroup : 64) + oct * 8;  // first weight channel of this thread
+  float wreg[8][9];
 #pragma unroll
-    for (int j = 0; j < 8; ++j) accv[j] = bias ? bias[ch + j] : 0.f;
+  for (int j = 0; j < 8; ++j)
+#pragma unroll
+    for (int t = 0; t < 9; ++t) wreg[j][t] = wt[(wch + j) * 9 + t];
+  float breg[8];
+#pragma unroll
+  for (int j = 0; j < 8; ++j) breg[j] = (!GATE && bias) ? bias[wch + j] : 0.f;
+  for (int l = tl; l < L; l += 32) {
+    const int r = l / w, c = l - r * w;
+    float acc[8], ctr[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) acc[j] = breg[j], ctr[j] = 0.f;
 #pragma unroll
     for (int di = -1; di <= 1; ++di) {
-      const int rr = r + di;
-      if (rr < 0 || rr >= h) continue;
 #pragma unroll
       for (int dj = -1; dj <= 1; ++dj) {
-        const int cc = c + dj;
-        if (cc < 0 || cc >= w) continue;
+        // unconditional load from a clamped neighbour; taps outside the grid are zeroed by select (zero padding)
+        const int rr = r + di, cc = c + dj;
+        const bool in = rr >= 0 && rr < h && cc >= 0 && cc < w;
+        const int rc = min(max(rr, 0), h - 1), ccl = min(max(cc, 0), w - 1);
         float xv[8];
-        Vec8<T>::load(x + ((b * L + (size_t)(rr * w + cc)) * C + ch), xv);
+        Vec8<T>::load(x + base + (size_t)(rc * w + ccl) * stride, xv);
 #pragma unroll
-        for (int j = 0; j < 8; ++j) accv[j] += xv[j] * wt[(ch + j) * 9 + (di + 1) * 3 + (dj + 1)];
-      }
-    }
-    if (silu) {
-#pragma unroll
-      for (int j = 0; j < 8; ++j) accv[j] = accv[j] * sigmoidf_(accv[j]);
-    }
-    Vec8<T>::store(y + i * 8, accv);
-  }
-}
-
-int launch_dwconv3x3(const void* x, const float* wt, const float* bias, void* y, int B, int h, int w, int C,
-                     int silu, int io_dtype, hipStream_t stream) {
-  const size_t nvec = (size_t)B * h * w * (C / 8);
-  const int grid = (int)((nvec + 255) / 256 < 65535 * 8 ? (nvec + 255) / 256 : 65535 * 8);
-  if (io_dtype == 0)
-    hipLaunchKernelGGL((dwconv3x3_kernel<float>), dim3(grid), dim3(256), 0, stream, (const float*)x, wt, bias,
-                       (float*)y, B, h, w, C, silu, nvec);
-  else
-    hipLaunchKernelGGL((dwconv3x3_kernel<uint16_t>), dim3(grid), dim3(256), 0, stream, (const uint16_t*)x, wt, bias,
-                       (uint16_t*)y, B, h, w, C, silu, nvec);
-  return hipGetLastError() == hipSuccess ? 0 : -5;
-}
-
-// ---------------------------------------------------------------------------
-// sigmoid locality gate on the head-major layout:
-//   o, y [B, H, L=h*w, Dv];  y = o * sigmoid(dwconv3x3(o)), channel = hd*Dv + d
-// ---------------------------------------------------------------------------
-template <typename T>
-__global__ __launch_bounds__(256) void locality_gate_kernel(const T* __restrict__ o, const float* __restrict__ wt,
-                                                             T* __restrict__ y, int H, int h, int w, int Dv,
-                                                             size_t nvec) {
-  const int d8n = Dv >> 3;
-  const int L = h * w;
-  for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < nvec; i += (size_t)gridDim.x * 256) {
-    const int d8 = (int)(i % d8n);
-    const size_t bhl = i / d8n;
-    const int l = (int)(bhl % L);
-    const size_t bh = bhl / L;
-    const int hd = (int)(bh % H);
-    const int r = l / w, c = l % w;
-    const int ch = hd * Dv + d8 * 8;
-    float accv[8], ctr[8];
-#pragma unroll
-    for (int j = 0; j < 8; ++j) accv[j] = 0.f, ctr[j] = 0.f;
-#pragma unroll
-    for (int di = -1; di <= 1; ++di) {
-      const int rr = r + di;
-      if (rr < 0 || rr >= h) continue;
-#pragma unroll
-      for (int dj = -1; dj <= 1; ++dj) {
-        const int cc = c + dj;
-        if (cc < 0 || cc >= w) continue;
-        float xv[8];
-        Vec8<T>::load(o + ((bh * L + (size_t)(rr * w + cc)) * Dv + d8 * 8), xv);
-#pragma unroll
-        for (int j = 0; j < 8; ++j) accv[j] += xv[j] * wt[(ch + j) * 9 + (di + 1) * 3 + (dj + 1)];
-        if (di == 0 && dj == 0) {
+        for (int j = 0; j < 8; ++j) acc[j] += (in ? xv[j] : 0.f) * wreg[j][(di + 1) * 3 + (dj + 1)];
+        if (GATE && di == 0 && dj == 0) {
 #pragma unroll
           for (int j = 0; j < 8; ++j) ctr[j] = xv[j];
         }
       }
     }
+    if (GATE) {
 #pragma unroll
-    for (int j = 0; j < 8; ++j) accv[j] = ctr[j] * sigmoidf_(accv[j]);
-    Vec8<T>::store(y + i * 8, accv);
+      for (int j = 0; j < 8; ++j) acc[j] = ctr[j] * sigmoidf_(acc[j]);
+    } else if (silu) {
+#pragma unroll
+      for (int j = 0; j < 8; ++j) acc[j] = acc[j] * sigmoidf_(acc[j]);
+    }
+    Vec8<T>::store(y + base + (size_t)l * stride, acc);
   }
+}
+
+int launch_dwconv3x3(const void* x, const float* wt, const float* bias, void* y, int B, int h, int w, int C,
+                     int silu, int io_dtype, hipStream_t stream) {
+  const int groups = (C + 63) / 64;
+  if (io_dtype == 0)
+    hipLaunchKernelGGL((stencil3x3_kernel<float, false>), dim3(B * groups), dim3(256), 0, stream, (const float*)x, wt,
+                       bias, (float*)y, h, w, C, groups, groups, C, silu);
+  else
+    hipLaunchKernelGGL((stencil3x3_kernel<uint16_t, false>), dim3(B * groups), dim3(256), 0, stream, (const uint16_t*)x,
+                       wt, bias, (uint16_t*)y, h, w, C, groups, groups, C, silu);
+  return hipGetLastError() == hipSuccess ? 0 : -5;
 }
 
 int launch_locality_gate(const void* o, const float* wt, void* y, int B, int H, int h, int w, int Dv, int io_dtype,
                          hipStream_t stream) {
-  const size_t nvec = (size_t)B * H * h * w * (Dv / 8);
-  const int grid = (int)((nvec + 255) / 256 < 65535 * 8 ? (nvec + 255) / 256 : 65535 * 8);
+  if (Dv > 64) return -95;
+  // every (batch, head) slab is an "image" of Dv channels; head hd uses weight channels [hd*Dv, hd*Dv + Dv)
   if (io_dtype == 0)
-    hipLaunchKernelGGL((locality_gate_kernel<float>), dim3(grid), dim3(256), 0, stream, (const float*)o, wt,
-                       (float*)y, H, h, w, Dv, nvec);
+    hipLaunchKernelGGL((stencil3x3_kernel<float, true>), dim3(B * H), dim3(256), 0, stream, (const float*)o, wt,
+                       (const float*)nullptr, (float*)y, h, w, Dv, 1, H, Dv, 0);
   else
-    hipLaunchKernelGGL((locality_gate_kernel<uint16_t>), dim3(grid), dim3(256), 0, stream, (const uint16_t*)o, wt,
-                       (uint16_t*)y, H, h, w, Dv, nvec);
+    hipLaunchKernelGGL((stencil3x3_kernel<uint16_t, true>), dim3(B * H), dim3(256), 0, stream, (const uint16_t*)o, wt,
+                       (const float*)nullptr, (uint16_t*)y, h, w, Dv, 1, H, Dv, 0);
   return hipGetLastError() == hipSuccess ? 0 : -5;
 }
 
