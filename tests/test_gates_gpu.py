@@ -69,6 +69,17 @@ def test_dwconv3x3_nonsquare_grid():
     assert max_abs(got, want) <= 1e-5
 
 
+def test_dwconv3x3_large_grid_row_bands():
+    """64x64 token grid (the 1024^2-image shape): the kernel walks it in row bands with halo rows."""
+    announce("dwconv3x3 64x64 grid, bf16, C=192")
+    B, h, w, C = 1, 64, 64, 192
+    x = _randn((B, h * w, C), 21, torch.bfloat16)
+    wt = make_locality_weight(C, 22)
+    want = O.dwconv3x3_reference(f64(x), f64(wt), (h, w), silu=True)
+    got = f64(vig_amd.dwconv3x3(x.cuda(), wt.cuda(), (h, w), silu=True))
+    assert max_abs(got, want) <= 2e-2
+
+
 @pytest.mark.parametrize("dtype,tol", [(torch.float32, 1e-5), (torch.bfloat16, 2e-2)])
 def test_locality_gate(dtype, tol):
     announce(f"locality sigmoid gate {dtype}")

@@ -105,24 +105,41 @@ int launch_dirgate(const void* in, void* out, int B, int L, int H, int Dk, float
 }
 
 // ---------------------------------------------------------------------------
-// 3x3 depthwise stencil on the token grid, channels-last.  One workgroup owns one image (or one head slab) and a
-// group of 64 channels: thread = (channel octet, token lane); it keeps the 8x9 weights of its channels in registers
-// and walks tokens lane, lane+32, ...; the nine neighbours of a token are 16-byte reads that hit L1/L2 (the 64-channel
-// slab of one image is a few tens of KB).
+// 3x3 depthwise stencil on the token grid, channels-last.  One workgroup owns one image (or one head slab), a
+// group of 64 channels and a band of grid rows: it stages the band plus one halo row on each side in LDS with
+// coalesced 16-byte loads (every input byte leaves L2 once), then thread = (channel octet, token lane) keeps the 8x9
+// weights of its channels in registers and walks the band's tokens lane, lane+32, ...; the nine taps are 16-byte LDS
+// reads (a wave reads 8 consecutive tokens x 128 B: conflict-free).
 //   GATE = false:  y = conv(x) (+bias) (SiLU optional)          x, y [N, h*w, C] with row stride `stride` elements
 //   GATE = true :  y = x * sigmoid(conv(x))                      (bias / SiLU unused)
-// weights [Ctot, 9] f32; the workgroup's first channel inside the weight table is wch0 = (blockIdx.y * 64 + woff).
+// weights [Ctot, 9] f32.
 // ---------------------------------------------------------------------------
 template <typename T, bool GATE>
 __global__ __launch_bounds__(256) void stencil3x3_kernel(const T* __restrict__ x, const float* __restrict__ wt,
                                                           const float* __restrict__ bias, T* __restrict__ y, int h, int w,
                                                           int stride, int groups_per_image, int wmod, int cgroup,
-                                                          int silu) {
+                                                          int band_rows, int silu) {
+  extern __shared__ __align__(16) char smem[];
+  T* tile = reinterpret_cast<T*>(smem);  // [(band_rows + 2) * w][64]
   const int oct = threadIdx.x & 7, tl = threadIdx.x >> 3;  // 8 octets x 32 token lanes
   const int img = blockIdx.x / groups_per_image, grp = blockIdx.x % groups_per_image;
-  if (grp * 64 + oct * 8 >= cgroup) return;  // channel tail of the last group (no barriers in this kernel)
+  const int r0 = blockIdx.y * band_rows;                   // first output row of the band
+  const int r1 = min(r0 + band_rows, h);
+  const int s0 = max(r0 - 1, 0), s1 = min(r1 + 1, h);      // staged rows [s0, s1)
   const int L = h * w;
+  const bool ch_ok = grp * 64 + oct * 8 < cgroup;          // channel tail of the last group
   const size_t base = (size_t)img * L * stride + (size_t)grp * 64 + oct * 8;
+  // ---- stage ----
+  const int ntok = (s1 - s0) * w;
+  for (int t = tl; t < ntok; t += 32) {
+    float xv[8];
+    if (ch_ok) {
+      Vec8<T>::load(x + base + (size_t)(s0 * w + t) * stride, xv);
+      Vec8<T>::store(tile + t * 64 + oct * 8, xv);
+    }
+  }
+  __syncthreads();
+  if (!ch_ok) return;
   const int wch = (blockIdx.x % wmod) * (GATE ? cgroup : 64) + oct * 8;  // first weight channel of this thread
   float wreg[8][9];
 #pragma unroll
@@ -132,8 +149,9 @@ __global__ __launch_bounds__(256) void stencil3x3_kernel(const T* __restrict__ x
   float breg[8];
 #pragma unroll
   for (int j = 0; j < 8; ++j) breg[j] = (!GATE && bias) ? bias[wch + j] : 0.f;
-  for (int l = tl; l < L; l += 32) {
-    const int r = l / w, c = l - r * w;
+  const int nout = (r1 - r0) * w;
+  for (int t = tl; t < nout; t += 32) {
+    const int r = r0 + t / w, c = t % w;
     float acc[8], ctr[8];
 #pragma unroll
     for (int j = 0; j < 8; ++j) acc[j] = breg[j], ctr[j] = 0.f;
@@ -141,12 +159,12 @@ __global__ __launch_bounds__(256) void stencil3x3_kernel(const T* __restrict__ x
     for (int di = -1; di <= 1; ++di) {
 #pragma unroll
       for (int dj = -1; dj <= 1; ++dj) {
-        // unconditional load from a clamped neighbour; taps outside the grid are zeroed by select (zero padding)
+        // unconditional read of a clamped neighbour; taps outside the grid are zeroed by select (zero padding)
         const int rr = r + di, cc = c + dj;
         const bool in = rr >= 0 && rr < h && cc >= 0 && cc < w;
-        const int rc = min(max(rr, 0), h - 1), ccl = min(max(cc, 0), w - 1);
+        const int rc = min(max(rr, s0), s1 - 1), ccl = min(max(cc, 0), w - 1);
         float xv[8];
-        Vec8<T>::load(x + base + (size_t)(rc * w + ccl) * stride, xv);
+        Vec8<T>::load(tile + ((rc - s0) * w + ccl) * 64 + oct * 8, xv);
 #pragma unroll
         for (int j = 0; j < 8; ++j) acc[j] += (in ? xv[j] : 0.f) * wreg[j][(di + 1) * 3 + (dj + 1)];
         if (GATE && di == 0 && dj == 0) {
@@ -162,33 +180,38 @@ __global__ __launch_bounds__(256) void stencil3x3_kernel(const T* __restrict__ x
 #pragma unroll
       for (int j = 0; j < 8; ++j) acc[j] = acc[j] * sigmoidf_(acc[j]);
     }
-    Vec8<T>::store(y + base + (size_t)l * stride, acc);
+    Vec8<T>::store(y + base + (size_t)(r * w + c) * stride, acc);
   }
+}
+
+template <typename T, bool GATE>
+static int launch_stencil(const void* x, const float* wt, const float* bias, void* y, int images, int h, int w,
+                          int stride, int groups, int wmod, int cgroup, int silu, hipStream_t stream) {
+  // rows per band so that (band + 2 halo rows) x w tokens x 64 channels fit 48 KB of LDS
+  const int row_bytes = w * 64 * (int)sizeof(T);
+  int band = 48 * 1024 / row_bytes - 2;
+  if (band < 1) return -95;
+  if (band > h) band = h;
+  const int nband = (h + band - 1) / band;
+  const size_t lds = (size_t)(band + 2) * row_bytes;
+  hipLaunchKernelGGL((stencil3x3_kernel<T, GATE>), dim3(images * groups, nband), dim3(256), lds, stream, (const T*)x, wt,
+                     bias, (T*)y, h, w, stride, groups, wmod, cgroup, band, silu);
+  return hipGetLastError() == hipSuccess ? 0 : -5;
 }
 
 int launch_dwconv3x3(const void* x, const float* wt, const float* bias, void* y, int B, int h, int w, int C,
                      int silu, int io_dtype, hipStream_t stream) {
   const int groups = (C + 63) / 64;
-  if (io_dtype == 0)
-    hipLaunchKernelGGL((stencil3x3_kernel<float, false>), dim3(B * groups), dim3(256), 0, stream, (const float*)x, wt,
-                       bias, (float*)y, h, w, C, groups, groups, C, silu);
-  else
-    hipLaunchKernelGGL((stencil3x3_kernel<uint16_t, false>), dim3(B * groups), dim3(256), 0, stream, (const uint16_t*)x,
-                       wt, bias, (uint16_t*)y, h, w, C, groups, groups, C, silu);
-  return hipGetLastError() == hipSuccess ? 0 : -5;
+  if (io_dtype == 0) return launch_stencil<float, false>(x, wt, bias, y, B, h, w, C, groups, groups, C, silu, stream);
+  return launch_stencil<uint16_t, false>(x, wt, bias, y, B, h, w, C, groups, groups, C, silu, stream);
 }
 
 int launch_locality_gate(const void* o, const float* wt, void* y, int B, int H, int h, int w, int Dv, int io_dtype,
                          hipStream_t stream) {
   if (Dv > 64) return -95;
   // every (batch, head) slab is an "image" of Dv channels; head hd uses weight channels [hd*Dv, hd*Dv + Dv)
-  if (io_dtype == 0)
-    hipLaunchKernelGGL((stencil3x3_kernel<float, true>), dim3(B * H), dim3(256), 0, stream, (const float*)o, wt,
-                       (const float*)nullptr, (float*)y, h, w, Dv, 1, H, Dv, 0);
-  else
-    hipLaunchKernelGGL((stencil3x3_kernel<uint16_t, true>), dim3(B * H), dim3(256), 0, stream, (const uint16_t*)o, wt,
-                       (const float*)nullptr, (uint16_t*)y, h, w, Dv, 1, H, Dv, 0);
-  return hipGetLastError() == hipSuccess ? 0 : -5;
+  if (io_dtype == 0) return launch_stencil<float, true>(o, wt, nullptr, y, B * H, h, w, Dv, 1, H, Dv, 0, stream);
+  return launch_stencil<uint16_t, true>(o, wt, nullptr, y, B * H, h, w, Dv, 1, H, Dv, 0, stream);
 }
 
 // ---------------------------------------------------------------------------

@@ -320,6 +320,7 @@ __device__ __forceinline__ void direction_wave(const uint16_t* q, const uint16_t
 
   // ---- cumulative log-gates G[it][p] via triangular-ones MFMA on transposed gate fragments ----
   f32x16_t G[2][2];
+  f32x16_t Gend[2];
   {
     u32x4_t gfrag[4][2];
     finish_tfrags<0, 4, true, NG>(pf.gD, nvalid, r, h, gfrag);
@@ -327,6 +328,11 @@ __device__ __forceinline__ void direction_wave(const uint16_t* q, const uint16_t
 #pragma unroll
     for (int p = 0; p < 2; ++p) {
       f32x16_t g0 = {0.f}, g1 = {0.f};
+      // the chunk total (= G at the anchor token) for every column at once: no cross-lane broadcast needed
+      f32x16_t ge = {0.f};
+#pragma unroll
+      for (int t = 0; t < 4; ++t) ge = mfma(gfrag[t][p], ones, ge);
+      Gend[p] = ge;
       if (FWD) {
         g0 = mfma(gfrag[0][p], tri_frag<true>(0, 0, r, h), g0);
         g0 = mfma(gfrag[1][p], tri_frag<true>(1, 0, r, h), g0);
@@ -353,15 +359,11 @@ __device__ __forceinline__ void direction_wave(const uint16_t* q, const uint16_t
   float* gend2 = reinterpret_cast<float*>(lds + kLdsGend) + wi * 64 + 32 * h;
   constexpr int HC = 8 * NG;  // channels per lane half
   {
-    const int src = ((FWD ? 31 : 0) + 32 * h) << 2;
     float e2[2][16];
 #pragma unroll
     for (int p = 0; p < 2; ++p)
 #pragma unroll
-      for (int cc = 0; cc < 16; ++cc) {
-        const float a = FWD ? G[1][p][cc] : G[0][p][cc];
-        e2[p][cc] = __int_as_float(__builtin_amdgcn_ds_bpermute(src, __float_as_int(a))) * kLog2e;
-      }
+      for (int cc = 0; cc < 16; ++cc) e2[p][cc] = Gend[p][cc] * kLog2e;
     if (r == 0) {  // every lane of a half holds the same 32 values; one lane writes them
       float* d = dvec_all + wi * 64 + HC * h;
 #pragma unroll
