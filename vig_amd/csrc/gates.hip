@@ -53,46 +53,47 @@ template <> struct Vec8<float> {
 // ---------------------------------------------------------------------------
 // direction-wise gate preparation
 //   in  [B, L, 2*H*Dk]  ->  out [2, B, H, L, Dk],  logsigmoid(x) * inv_norm, clamp
+// One workgroup owns 32 consecutive tokens of one batch element: it reads their rows (contiguous, 2*H*Dk channels
+// each) with 16-byte accesses and writes, per (direction, head), a contiguous run of 32 tokens x Dk.  A thread keeps
+// one channel octet for all its tokens, so the layout arithmetic is done once per thread.
 // ---------------------------------------------------------------------------
 template <typename TI, typename TO>
-__global__ __launch_bounds__(256) void dirgate_kernel(const TI* __restrict__ in, TO* __restrict__ out,
-                                                       int B, int L, int H, int Dk, float inv_norm,
-                                                       float clamp_min, int use_clamp, size_t nvec) {
+__global__ __launch_bounds__(256) void dirgate_kernel(const TI* __restrict__ in, TO* __restrict__ out, int B, int L,
+                                                       int H, int Dk, float inv_norm, float clamp_min, int use_clamp) {
+  const int nv = 2 * H * Dk / 8;         // channel octets per token row
   const int dk8 = Dk >> 3;
-  for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < nvec; i += (size_t)gridDim.x * 256) {
-    // i enumerates output vectors in output order: (((dir*B + b)*H + h)*L + l)*dk8 + d8
-    size_t r = i;
-    const int d8 = (int)(r % dk8);
-    r /= dk8;
-    const int l = (int)(r % L);
-    r /= L;
-    const int h = (int)(r % H);
-    r /= H;
-    const int b = (int)(r % B);
-    const int dir = (int)(r / B);
-    const size_t src = ((size_t)b * L + l) * (size_t)(2 * H * Dk) + (size_t)dir * H * Dk + (size_t)h * Dk + d8 * 8;
-    float x[8];
-    Vec8<TI>::load(in + src, x);
+  const int b = blockIdx.y;
+  const int l0 = blockIdx.x * 32;
+  const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;  // 64 octet lanes x 4 token lanes
+  for (int cv = tx; cv < nv; cv += 64) {
+    const int d8 = cv % dk8, hh = (cv / dk8) % H, dir = cv / (dk8 * H);
+    const TI* src = in + ((size_t)b * L) * (size_t)(nv * 8) + (size_t)cv * 8;
+    TO* dst = out + ((((size_t)dir * B + b) * H + hh) * L) * (size_t)Dk + (size_t)d8 * 8;
+    for (int t = ty; t < 32; t += 4) {
+      const int l = l0 + t;
+      if (l >= L) break;
+      float x[8];
+      Vec8<TI>::load(src + (size_t)l * (nv * 8), x);
 #pragma unroll
-    for (int j = 0; j < 8; ++j) {
-      // logsigmoid(x) = min(x,0) - log1p(exp(-|x|))
-      float y = fminf(x[j], 0.f) - log1pf(__expf(-fabsf(x[j])));
-      y *= inv_norm;
-      if (use_clamp) y = fmaxf(y, clamp_min);
-      x[j] = y;
+      for (int j = 0; j < 8; ++j) {
+        // logsigmoid(x) = min(x,0) - log(1 + exp(-|x|)); hardware exp/log are accurate to ~1e-7 absolute here
+        float yv = fminf(x[j], 0.f) - __logf(1.f + __expf(-fabsf(x[j])));
+        yv *= inv_norm;
+        if (use_clamp) yv = fmaxf(yv, clamp_min);
+        x[j] = yv;
+      }
+      Vec8<TO>::store(dst + (size_t)l * Dk, x);
     }
-    Vec8<TO>::store(out + i * 8, x);
   }
 }
 
 template <typename TI, typename TO>
 static int launch_dirgate_t(const void* in, void* out, int B, int L, int H, int Dk, float inv_norm,
                             float clamp_min, hipStream_t stream) {
-  const size_t nvec = (size_t)2 * B * H * L * (Dk / 8);
   const int use_clamp = clamp_min == clamp_min;  // NaN disables
-  const int grid = (int)((nvec + 255) / 256 < 65535 * 8 ? (nvec + 255) / 256 : 65535 * 8);
-  hipLaunchKernelGGL((dirgate_kernel<TI, TO>), dim3(grid), dim3(256), 0, stream, (const TI*)in, (TO*)out, B, L, H,
-                     Dk, inv_norm, clamp_min, use_clamp, nvec);
+  if (B > 65535) return -22;
+  hipLaunchKernelGGL((dirgate_kernel<TI, TO>), dim3((L + 31) / 32, B), dim3(256), 0, stream, (const TI*)in, (TO*)out, B,
+                     L, H, Dk, inv_norm, clamp_min, use_clamp);
   return hipGetLastError() == hipSuccess ? 0 : -5;
 }
 
