@@ -104,51 +104,52 @@ __device__ __forceinline__ void lds_barrier() {
 }
 
 // ---------------------------------------------------------------------------------------------------------
-// Loads.  Every load is unconditional on a clamped row (no divergent branches around memory operations);
-// padding rows are zeroed by a select when the data is consumed.  `rows` points at the chunk's first token.
+// Loads.  Every tensor chunk is addressed through a raw buffer descriptor whose extent is the chunk's valid rows:
+// the hardware returns zero for anything beyond it, so padding rows need neither clamped addresses nor selects
+// (zero gates, keys and values are exactly what padding tokens have to contribute), and token offsets travel as
+// instruction immediates.
 // ---------------------------------------------------------------------------------------------------------
+typedef __amdgpu_buffer_rsrc_t rsrc_t;
 
-// raw dwords of the transposed fragments of k-steps [T0, T0+NT): D[t][e] = channels (2*cpair(r), +1) of token jmap(t,h,e)
+// descriptor of `rows` rows of `row_bytes` starting at p (p and rows are wave-uniform)
+__device__ __forceinline__ rsrc_t chunk_rsrc(const void* p, int rows, int row_bytes) {
+  return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(p), 0, rows * row_bytes, 0x00020000);
+}
+constexpr unsigned kOutOfRange = 0x40000000u;  // byte offset no descriptor of this kernel covers
+
+// raw dwords of the transposed fragments of k-steps [T0, T0+NT): D[t][e] = channels (2*cpair(r), +1) of token
+// jmap(t,h,e); lane rows that carry no channel (NG = 2, rows 16..31) read zeros
 template <int T0, int NT, int NG>
-__device__ __forceinline__ void issue_tdwords(const uint16_t* rows, int nvalid, int r, int h, uint32_t (&D)[NT][8]) {
-  const unsigned c2 = row_has_channel<NG>(r) ? 2 * cpair<NG>(r) : 0;
-  const int nlast = max(nvalid - 1, 0);
+__device__ __forceinline__ void issue_tdwords(rsrc_t rows, int r, int h, uint32_t (&D)[NT][8]) {
+  constexpr unsigned RB = 32u * NG;  // bytes per row
+  const unsigned base = row_has_channel<NG>(r) ? (4u * h) * RB + 4u * cpair<NG>(r) : kOutOfRange;
 #pragma unroll
   for (int t = 0; t < NT; ++t)
 #pragma unroll
-    for (int e = 0; e < 8; ++e) {
-      const unsigned tok = (unsigned)min(jmap(T0 + t, h, e), nlast);
-      D[t][e] = *reinterpret_cast<const uint32_t*>(rows + (tok * (16u * NG) + c2));
-    }
+    for (int e = 0; e < 8; ++e)
+      D[t][e] = __builtin_amdgcn_raw_buffer_load_b32(rows, base + (unsigned)jmap(T0 + t, 0, e) * RB, 0, 0);
 }
 
 // fragments from raw dwords: frag[t][p] has lane index = channel 2*cpair(r)+p, slots = tokens jmap(t,h,.)
-template <int T0, int NT, bool ZERO_PAD, int NG>
-__device__ __forceinline__ void finish_tfrags(const uint32_t (&D)[NT][8], int nvalid, int r, int h,
-                                              u32x4_t (&frag)[NT][2]) {
-  const bool row_ok = row_has_channel<NG>(r);
+template <int NT>
+__device__ __forceinline__ void finish_tfrags(const uint32_t (&D)[NT][8], u32x4_t (&frag)[NT][2]) {
 #pragma unroll
-  for (int t = 0; t < NT; ++t) {
-    uint32_t d[8];
-#pragma unroll
-    for (int e = 0; e < 8; ++e)
-      d[e] = ((NG == 4 || row_ok) && (!ZERO_PAD || jmap(T0 + t, h, e) < nvalid)) ? D[t][e] : 0u;
+  for (int t = 0; t < NT; ++t)
 #pragma unroll
     for (int x = 0; x < 4; ++x) {
-      frag[t][0][x] = __builtin_amdgcn_perm(d[2 * x + 1], d[2 * x], 0x05040100u);
-      frag[t][1][x] = __builtin_amdgcn_perm(d[2 * x + 1], d[2 * x], 0x07060302u);
+      frag[t][0][x] = __builtin_amdgcn_perm(D[t][2 * x + 1], D[t][2 * x], 0x05040100u);
+      frag[t][1][x] = __builtin_amdgcn_perm(D[t][2 * x + 1], D[t][2 * x], 0x07060302u);
     }
-  }
 }
 
 // raw rows of one 32-token tile: lane (r, h) reads token 32*it + r, channels [8*NG*h, +8*NG) as NG 16-byte pieces
 template <int NG>
-__device__ __forceinline__ void issue_raw_tile(const uint16_t* rows, int it, int nvalid, int r, int h,
-                                               u32x4_t (&raw)[NG]) {
-  const unsigned rowc = (unsigned)min(32 * it + r, max(nvalid - 1, 0));
+__device__ __forceinline__ void issue_raw_tile(rsrc_t rows, int it, int r, int h, u32x4_t (&raw)[NG]) {
+  constexpr unsigned RB = 32u * NG;
+  const unsigned base = (unsigned)r * RB + (16u * NG) * h;
 #pragma unroll
   for (int gq = 0; gq < NG; ++gq)
-    raw[gq] = *reinterpret_cast<const u32x4_t*>(rows + (rowc * (16u * NG) + (8u * NG) * h + 8u * gq));
+    raw[gq] = __builtin_amdgcn_raw_buffer_load_b128(rows, base + (unsigned)it * 32u * RB + 16u * gq, 0, 0);
 }
 
 // one k-step of transposed fragments from the wave's k~ scratch in LDS
@@ -190,10 +191,9 @@ struct HalfOps {
 };
 
 // q~ (ISQ) or k~ of one 32-token tile: raw * exp(+-(G - G_end)), split into bf16 hi (round to nearest) and
-// lo (the fp32 remainder, rounded).  `live` zeroes padding rows (needed for k~ only: q~ of a padding row only
-// feeds outputs that are never stored).
+// lo (the fp32 remainder, rounded).  Padding rows arrive as zeros and stay zero (their exponents are finite).
 template <bool ISQ, int NG>
-__device__ __forceinline__ void make_half(const u32x4_t (&raw)[NG], bool live, const f32x16_t (&G)[2],
+__device__ __forceinline__ void make_half(const u32x4_t (&raw)[NG], const f32x16_t (&G)[2],
                                           const float* gend2 /* LDS, this lane half: [p][16] */, HalfOps<NG>& op) {
 #pragma unroll
   for (int g = 0; g < NG; ++g) {
@@ -202,7 +202,7 @@ __device__ __forceinline__ void make_half(const u32x4_t (&raw)[NG], bool live, c
 #pragma unroll
     for (int m = 0; m < 4; ++m) {
       const int c = 4 * g + m;
-      const uint32_t w = (ISQ || live) ? raw[g][m] : 0u;
+      const uint32_t w = raw[g][m];
       float t[2];
 #pragma unroll
       for (int p = 0; p < 2; ++p) {
@@ -279,14 +279,18 @@ struct Prefetch {
   u32x4_t rawk[NG], rawq[NG];  // raw rows of the tile walked first
 };
 
+// The four tensors of one chunk (q, k, g: 32*NG bytes per row; v: 128).
+struct ChunkSrc {
+  rsrc_t q, k, v, g;
+};
+
 template <bool FWD, bool WITH_Q, int NG>
-__device__ __forceinline__ void issue_first_phase(const uint16_t* q, const uint16_t* k, const uint16_t* v,
-                                                  const uint16_t* g, int nvalid, int r, int h, Prefetch<NG>& pf) {
+__device__ __forceinline__ void issue_first_phase(const ChunkSrc& src, int r, int h, Prefetch<NG>& pf) {
   constexpr int TA = FWD ? 0 : 1;
-  issue_tdwords<0, 4, NG>(g, nvalid, r, h, pf.gD);
-  issue_raw_tile<NG>(k, TA, nvalid, r, h, pf.rawk);
-  if (WITH_Q) issue_raw_tile<NG>(q, TA, nvalid, r, h, pf.rawq);
-  issue_tdwords<2 * TA, 2, 4>(v, nvalid, r, h, pf.vD);
+  issue_tdwords<0, 4, NG>(src.g, r, h, pf.gD);
+  issue_raw_tile<NG>(src.k, TA, r, h, pf.rawk);
+  if (WITH_Q) issue_raw_tile<NG>(src.q, TA, r, h, pf.rawq);
+  issue_tdwords<2 * TA, 2, 4>(src.v, r, h, pf.vD);
 }
 
 // Segment modes of the kernel.  A sequence longer than 256 tokens is cut into segments of <= 256 tokens that are
@@ -299,14 +303,12 @@ __device__ __forceinline__ void issue_first_phase(const uint16_t* q, const uint1
 constexpr int kModeSlab = 0, kModeState = 1, kModeChain = 2;
 constexpr int kStateFloats = 64 * 64 + 64;  // per (sequence, segment, direction): state in unit order, then 64 decays
 
-// Everything one wave does for one segment: chunk c (nvalid tokens starting at the row the pointers address) in
+// Everything one wave does for one segment: chunk c (the valid rows its descriptors cover) in
 // direction FWD / reverse.  Every wave of the workgroup passes the same three barriers here (plus the caller's).
 template <bool FWD, int MODE, int NG>
-__device__ __forceinline__ void direction_wave(const uint16_t* q, const uint16_t* k, const uint16_t* v,
-                                               const uint16_t* g, uint16_t* o, const uint16_t* qn, const uint16_t* kn,
-                                               const uint16_t* vn, const uint16_t* gn, int nvalid, int nvalid_next,
-                                               int c, int lane, char* lds, float oscale, bool bidir, float* state,
-                                               Prefetch<NG>& pf, int iter) {
+__device__ __forceinline__ void direction_wave(const ChunkSrc& cur, const ChunkSrc& nxt, rsrc_t o, int c, int lane,
+                                               char* lds, float oscale, bool bidir, float* state, Prefetch<NG>& pf,
+                                               int iter) {
   constexpr bool OUT = MODE != kModeState;  // produces outputs (needs q)
   int r = lane & 31, h = lane >> 5;
   const int wi = (FWD ? 0 : 4) + c;
@@ -315,7 +317,7 @@ __device__ __forceinline__ void direction_wave(const uint16_t* q, const uint16_t
   char* region = lds + wi * kRegionBytes;
   uint16_t* kt = reinterpret_cast<uint16_t*>(region);
   float* dvec_all = reinterpret_cast<float*>(lds + kLdsDvec);
-  if (!FWD) issue_first_phase<FWD, OUT, NG>(q, k, v, g, nvalid, r, h, pf);
+  if (!FWD) issue_first_phase<FWD, OUT, NG>(cur, r, h, pf);
   VIG_STAMP(0);
 
   // ---- cumulative log-gates G[it][p] via triangular-ones MFMA on transposed gate fragments ----
@@ -323,8 +325,9 @@ __device__ __forceinline__ void direction_wave(const uint16_t* q, const uint16_t
   f32x16_t Gend[2];
   {
     u32x4_t gfrag[4][2];
-    finish_tfrags<0, 4, true, NG>(pf.gD, nvalid, r, h, gfrag);
+    finish_tfrags<4>(pf.gD, gfrag);
     const u32x4_t ones = {0x3F803F80u, 0x3F803F80u, 0x3F803F80u, 0x3F803F80u};
+    const u32x4_t tri0 = tri_frag<FWD>(0, 0, r, h), tri1 = tri_frag<FWD>(1, 0, r, h);
 #pragma unroll
     for (int p = 0; p < 2; ++p) {
       f32x16_t g0 = {0.f}, g1 = {0.f};
@@ -333,20 +336,21 @@ __device__ __forceinline__ void direction_wave(const uint16_t* q, const uint16_t
 #pragma unroll
       for (int t = 0; t < 4; ++t) ge = mfma(gfrag[t][p], ones, ge);
       Gend[p] = ge;
+      // the triangular operand depends on (k-step, tile) only through their offset: two distinct fragments
       if (FWD) {
-        g0 = mfma(gfrag[0][p], tri_frag<true>(0, 0, r, h), g0);
-        g0 = mfma(gfrag[1][p], tri_frag<true>(1, 0, r, h), g0);
+        g0 = mfma(gfrag[0][p], tri0, g0);
+        g0 = mfma(gfrag[1][p], tri1, g0);
         g1 = mfma(gfrag[0][p], ones, g1);
         g1 = mfma(gfrag[1][p], ones, g1);
-        g1 = mfma(gfrag[2][p], tri_frag<true>(2, 1, r, h), g1);
-        g1 = mfma(gfrag[3][p], tri_frag<true>(3, 1, r, h), g1);
+        g1 = mfma(gfrag[2][p], tri0, g1);
+        g1 = mfma(gfrag[3][p], tri1, g1);
       } else {
-        g0 = mfma(gfrag[0][p], tri_frag<false>(0, 0, r, h), g0);
-        g0 = mfma(gfrag[1][p], tri_frag<false>(1, 0, r, h), g0);
+        g0 = mfma(gfrag[0][p], tri0, g0);
+        g0 = mfma(gfrag[1][p], tri1, g0);
         g0 = mfma(gfrag[2][p], ones, g0);
         g0 = mfma(gfrag[3][p], ones, g0);
-        g1 = mfma(gfrag[2][p], tri_frag<false>(2, 1, r, h), g1);
-        g1 = mfma(gfrag[3][p], tri_frag<false>(3, 1, r, h), g1);
+        g1 = mfma(gfrag[2][p], tri0, g1);
+        g1 = mfma(gfrag[3][p], tri1, g1);
       }
       G[0][p] = g0;
       G[1][p] = g1;
@@ -396,15 +400,15 @@ __device__ __forceinline__ void direction_wave(const uint16_t* q, const uint16_t
     uint32_t vDb[2][8];
     {
       HalfOps<NG> qa;
-      make_half<false, NG>(pf.rawk, 32 * TA + r < nvalid, G[TA], gend2, ka);
-      if (OUT) make_half<true, NG>(pf.rawq, true, G[TA], gend2, qa);
+      make_half<false, NG>(pf.rawk, G[TA], gend2, ka);
+      if (OUT) make_half<true, NG>(pf.rawq, G[TA], gend2, qa);
       VIG_PHASE();
-      if (OUT) issue_raw_tile<NG>(q, TB, nvalid, r, h, rawq);
-      issue_raw_tile<NG>(k, TB, nvalid, r, h, rawk);
-      issue_tdwords<2 * TB, 2, 4>(v, nvalid, r, h, vDb);
+      if (OUT) issue_raw_tile<NG>(cur.q, TB, r, h, rawq);
+      issue_raw_tile<NG>(cur.k, TB, r, h, rawk);
+      issue_tdwords<2 * TB, 2, 4>(cur.v, r, h, vDb);
       {
         u32x4_t vf[2][2];
-        finish_tfrags<2 * TA, 2, false, 4>(pf.vD, nvalid, r, h, vf);
+        finish_tfrags<2>(pf.vD, vf);
 #pragma unroll
         for (int tl = 0; tl < 2; ++tl)
 #pragma unroll
@@ -419,16 +423,16 @@ __device__ __forceinline__ void direction_wave(const uint16_t* q, const uint16_t
     }
     VIG_PHASE();
     if (OUT) {
-      make_half<true, NG>(rawq, true, G[TB], gend2, qb);
+      make_half<true, NG>(rawq, G[TB], gend2, qb);
       apply_scores<0>(score_tile(ka, qb), TA, r, h, vfrag, O[0][TB], O[1][TB]);
     }
     VIG_PHASE();
     {
       HalfOps<NG> kb;
-      make_half<false, NG>(rawk, 32 * TB + r < nvalid, G[TB], gend2, kb);
+      make_half<false, NG>(rawk, G[TB], gend2, kb);
       {
         u32x4_t vf[2][2];
-        finish_tfrags<2 * TB, 2, false, 4>(vDb, nvalid, r, h, vf);
+        finish_tfrags<2>(vDb, vf);
 #pragma unroll
         for (int tl = 0; tl < 2; ++tl)
 #pragma unroll
@@ -476,8 +480,8 @@ __device__ __forceinline__ void direction_wave(const uint16_t* q, const uint16_t
   }
   // ---- forward waves fetch the first phase of the NEXT segment here, reverse waves fetch theirs at the top of the
   // segment: a wave stalls while the memory pipe accepts its loads, and this way the other wave of the SIMD has math
-  // to do.  (Always issued: after the last segment it re-reads the current one, which keeps branches off the loads.) ----
-  if (FWD) issue_first_phase<FWD, OUT, NG>(qn, kn, vn, gn, nvalid_next, r, h, pf);
+  // to do.  (Always issued: after the last segment its descriptors are empty, which keeps branches off the loads.) ----
+  if (FWD) issue_first_phase<FWD, OUT, NG>(nxt, r, h, pf);
   VIG_STAMP(5);
   // lane-derived addresses of the exchange phases are rebuilt here instead of being carried (and spilled) across
   // the register-heavy tile phase
@@ -591,15 +595,13 @@ __device__ __forceinline__ void direction_wave(const uint16_t* q, const uint16_t
 #pragma unroll
     for (int it = 0; it < 2; ++it) {
       if (bidir && it != KEEP) continue;
-      const int row = 32 * it + r;
-      if (row < nvalid) {
+      const unsigned row = 32u * it + r;  // rows beyond the chunk fall outside the descriptor and are dropped
 #pragma unroll
-        for (int gq = 0; gq < 4; ++gq) {
-          u32x4_t x;
+      for (int gq = 0; gq < 4; ++gq) {
+        u32x4_t x;
 #pragma unroll
-          for (int m = 0; m < 4; ++m) x[m] = pack_bf16x2(O[0][it][4 * gq + m] * oscale, O[1][it][4 * gq + m] * oscale);
-          *reinterpret_cast<u32x4_t*>(o + ((unsigned)row * 64u + 32u * h + 8u * gq)) = x;
-        }
+        for (int m = 0; m < 4; ++m) x[m] = pack_bf16x2(O[0][it][4 * gq + m] * oscale, O[1][it][4 * gq + m] * oscale);
+        __builtin_amdgcn_raw_buffer_store_b128(x, o, row * 128u + 64u * h + 16u * gq, 0, 0);
       }
     }
   } else {
@@ -619,41 +621,40 @@ __device__ __forceinline__ void wave_loop(const uint16_t* q, const uint16_t* k, 
                                           uint16_t* o, const Geometry& geo, int c, int lane, char* lds, float oscale,
                                           bool bidir, float* state_ws) {
   constexpr bool OUT = MODE != kModeState;
-  // an empty chunk (nvalid == 0) reads the first row of its segment instead of running past it; its values are discarded
-  auto locate = [&](int item, size_t& off, int& nvalid) {
-    const int seq = item / geo.nseg, seg = item - seq * geo.nseg;
-    const int seg_tokens = min(geo.seg_len, geo.L - seg * geo.seg_len);
-    nvalid = min(max(seg_tokens - c * geo.cw, 0), geo.cw);
-    off = (size_t)seq * geo.L + (size_t)seg * geo.seg_len + (size_t)(nvalid > 0 ? c * geo.cw : 0);  // in tokens
-  };
   constexpr int DK = 16 * NG;
+  // descriptors of this wave's chunk of an item; past the last item (or for a chunk with no tokens) they are empty
+  auto locate = [&](int item, ChunkSrc& src, rsrc_t& dst) {
+    int nvalid = 0;
+    size_t off = 0;
+    if (item < geo.nitems) {
+      const int seq = item / geo.nseg, seg = item - seq * geo.nseg;
+      const int seg_tokens = min(geo.seg_len, geo.L - seg * geo.seg_len);
+      nvalid = min(max(seg_tokens - c * geo.cw, 0), geo.cw);
+      off = (size_t)seq * geo.L + (size_t)seg * geo.seg_len + (size_t)(nvalid > 0 ? c * geo.cw : 0);  // in tokens
+    }
+    src.q = chunk_rsrc(q + off * DK, nvalid, 2 * DK);
+    src.k = chunk_rsrc(k + off * DK, nvalid, 2 * DK);
+    src.g = chunk_rsrc(g + off * DK, nvalid, 2 * DK);
+    src.v = chunk_rsrc(v + off * 64, nvalid, 128);
+    dst = chunk_rsrc(o + off * 64, nvalid, 128);
+  };
   Prefetch<NG> pf;
   int item = blockIdx.x;
-  size_t b = 0;
-  int nvalid = 0;
-  if (item < geo.nitems) {
-    locate(item, b, nvalid);
-    if (FWD)
-      issue_first_phase<FWD, OUT, NG>(q + b * DK, k + b * DK, v + b * 64, g + b * DK, nvalid, lane & 31, lane >> 5, pf);
-  }
+  ChunkSrc cur;
+  rsrc_t dst;
+  locate(item, cur, dst);
+  if (FWD && item < geo.nitems) issue_first_phase<FWD, OUT, NG>(cur, lane & 31, lane >> 5, pf);
   int iter = 0;
   for (; item < geo.nitems; item += gridDim.x, ++iter) {
-    const int next = item + gridDim.x;
-    size_t bn = b;
-    int nvalid_next = nvalid;
-    if (next < geo.nitems) {
-      locate(next, bn, nvalid_next);
-    } else {
-      nvalid_next = min(nvalid, 1);  // nothing follows: the (branch-free) prefetch degenerates to one row per tensor
-    }
+    ChunkSrc nxt;
+    rsrc_t dst_next;
+    locate(item + gridDim.x, nxt, dst_next);
     float* state = state_ws ? state_ws + ((size_t)item * 2 + (FWD ? 0 : 1)) * kStateFloats : nullptr;
     asm volatile("" : "+v"(lane));  // per-lane constants are rebuilt per item instead of living across the loop
-    direction_wave<FWD, MODE, NG>(q + b * DK, k + b * DK, v + b * 64, g + b * DK, o + b * 64, q + bn * DK, k + bn * DK,
-                                  v + bn * 64, g + bn * DK, nvalid, nvalid_next, c, lane, lds, oscale, bidir, state, pf,
-                                  iter);
+    direction_wave<FWD, MODE, NG>(cur, nxt, dst, c, lane, lds, oscale, bidir, state, pf, iter);
     lds_barrier();  // (D) the next item reuses the LDS regions
-    b = bn;
-    nvalid = nvalid_next;
+    cur = nxt;
+    dst = dst_next;
   }
 }
 
