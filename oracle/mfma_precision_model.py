@@ -1,13 +1,16 @@
-"""CPU emulation of the bf16 MFMA kernel's arithmetic (which operands are rounded where).
+"""CPU emulation of the MFMA kernel's arithmetic (which operands are rounded where).
 
-TEST INFRASTRUCTURE ONLY.  It rebuilds the end-anchored chunk algebra of vig_amd/csrc/gla_mfma.hip in numpy with
-explicit bf16 roundings, so the precision design (which operands carry a bf16 hi + lo pair) can be checked on the
+TEST INFRASTRUCTURE ONLY.  It rebuilds the chunk algebra of vig_amd/csrc/gla_mfma.hip in numpy with explicit
+roundings, so the precision design (which operands are fp16, which carry a bf16 hi + lo pair) can be checked on the
 CPU against the fp64 oracle.  Chunk algebra as in flash-linear-attention/fla/ops/gla/chunk_util.py:9-78 and
-chunk_fuse.py:76-97 with the anchor moved to the chunk end.
+chunk_fuse.py:76-97, here with the anchor at half the chunk total: q~ = q*exp(G - G_end/2), k~ = k*exp(G_end/2 - G),
+so state update and inter-chunk product carry exp(G_end/2) each.
 
-splits:  qk = number of score terms (1: hi*hi, 3: + lo*hi + hi*lo),  p = P terms in P V (1 or 2),
-         iq = q~ terms in the inter-chunk product, st = state terms, u = k~ terms in the state update.
-The shipped kernel is qk=3, p=2, iq=1, st=1, u=1.
+splits:  qk = score operands: "f16" (one fp16 rounding each), 1 (bf16 hi*hi) or 3 (+ lo*hi + hi*lo),
+         p = P terms in P V (1 or 2),  iq = q~ terms in the inter-chunk product, st = state terms,
+         u = k~ terms in the state update.
+The shipped kernel is qk="f16", p=2, iq=1, st=1, u=1 and falls back to qk=3 for chunks whose gate total leaves
+the fp16 range (FALLBACK).
 """
 from __future__ import annotations
 
@@ -31,7 +34,13 @@ def _mm(a, b):
     return np.matmul(a.astype(np.float32), b.astype(np.float32))
 
 
-SHIPPED = dict(qk=3, p=2, iq=1, st=1, u=1)
+def f16_round(x):
+    """fp32 array rounded to fp16 (round to nearest even), returned as fp32."""
+    return np.asarray(x, dtype=np.float32).astype(np.float16).astype(np.float32)
+
+
+SHIPPED = dict(qk="f16", p=2, iq=1, st=1, u=1)
+FALLBACK = dict(qk=3, p=2, iq=1, st=1, u=1)
 PLAIN = dict(qk=1, p=1, iq=1, st=1, u=1)
 
 
@@ -57,22 +66,27 @@ def emulate(q, k, v, gf, gb, chunk, splits=SHIPPED):
             else:
                 G = np.flip(np.cumsum(np.flip(gc, 1), axis=1, dtype=np.float32), 1)
                 Gend = G[:, :1, :]
-            qt = q[:, sl] * np.exp(G - Gend).astype(np.float32)
-            kt = k[:, sl] * np.exp(Gend - G).astype(np.float32)
+            half = np.float32(0.5) * Gend
+            qt = q[:, sl] * np.exp(G - half).astype(np.float32)
+            kt = k[:, sl] * np.exp(half - G).astype(np.float32)
             vc = v[:, sl]
             n = qt.shape[1]
             tri = np.tril(np.ones((n, n), np.float32)) if direction == 0 else np.triu(np.ones((n, n), np.float32))
             qh, ql = _split(qt)
             kh, kl = _split(kt)
-            P = _mm(qh, T(kh))
-            if splits["qk"] >= 3:
-                P += _mm(ql, T(kh)) + _mm(qh, T(kl))
+            if splits["qk"] == "f16":
+                P = _mm(f16_round(qt), T(f16_round(kt)))
+            else:
+                P = _mm(qh, T(kh))
+                if splits["qk"] >= 3:
+                    P += _mm(ql, T(kh)) + _mm(qh, T(kl))
             P *= tri
             Ph, Pl = _split(P)
             oc = _mm(Ph, vc)
             if splits["p"] >= 2:
                 oc += _mm(Pl, vc)
-            Sd = S * T(np.exp(Gend).astype(np.float32))
+            sd = T(np.exp(half).astype(np.float32))  # half decay per key channel
+            Sd = S * sd
             Sh, Sl = _split(Sd)
             oc += _mm(qh, Sh)
             if splits["iq"] >= 2:
@@ -80,7 +94,8 @@ def emulate(q, k, v, gf, gb, chunk, splits=SHIPPED):
             if splits["st"] >= 2:
                 oc += _mm(qh, Sl)
             o[:, sl] += s * oc
-            S = Sd + _mm(T(kh), vc)
+            U = _mm(T(kh), vc)
             if splits["u"] >= 2:
-                S += _mm(T(kl), vc)
+                U += _mm(T(kl), vc)
+            S = (Sd + U) * sd
     return o

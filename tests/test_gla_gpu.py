@@ -130,6 +130,44 @@ def test_bf16_zero_gate_closed_form():
     assert np.all(np.abs(got - want) <= BF16_TOL + 2.0 ** -8 * np.abs(want))
 
 
+@pytest.mark.parametrize("gate_scale,L", [(0.25, 196), (1.0, 196), (1.0, 700)])
+def test_bf16_strong_gates_default_path(gate_scale, L):
+    """Gates far stronger than ViG's /16: chunk totals beyond what the fp16 score operands take, so the kernel has
+    to fall back to its split-bf16 scores (per workgroup, from the first such segment on)."""
+    announce(f"bf16 default path, strong gates x{gate_scale} L={L}")
+    q, k, v, gf, gb = make_gla_inputs(3, 2, L, 64, 64, seed=41, dtype=torch.bfloat16, gate_scale=gate_scale)
+    gf, gb = gf.clamp_min(-3), gb.clamp_min(-3)
+    want = oracle_bidir(q, k, v, gf, gb)
+    got = f64(vig_amd.gla_bidir_forward(*dev(q, k, v, gf, gb)))
+    assert np.isfinite(got).all()
+    assert max_abs(got, want) <= BF16_TOL
+
+
+def test_bf16_mixed_gate_strength_many_items():
+    """More (batch, head) slabs than workgroups, a few of them with strong gates: workgroups switch score variants
+    at different items, and every slab still has to match."""
+    announce("bf16 default path, 600 slabs, every 7th with strong gates")
+    q, k, v, gf, gb = make_gla_inputs(100, 6, 196, 64, 64, seed=43, dtype=torch.bfloat16)
+    _, _, _, sf, sb = make_gla_inputs(100, 6, 196, 64, 64, seed=44, dtype=torch.bfloat16, gate_scale=1.0)
+    strong = (torch.arange(600).reshape(100, 6) % 7 == 3)[:, :, None, None]
+    gf = torch.where(strong, sf.clamp_min(-3), gf)
+    gb = torch.where(strong, sb.clamp_min(-3), gb)
+    want = oracle_bidir(q, k, v, gf, gb)
+    got = f64(vig_amd.gla_bidir_forward(*dev(q, k, v, gf, gb)))
+    assert np.isfinite(got).all()
+    assert max_abs(got, want) <= BF16_TOL
+
+
+def test_bf16_strong_gates_one_direction():
+    announce("bf16 default path, forward direction only, strong gates")
+    q, k, v, gf, _ = make_gla_inputs(2, 3, 300, 64, 64, seed=45, dtype=torch.bfloat16, gate_scale=1.0)
+    gf = gf.clamp_min(-3)
+    want = oracle_bidir(q, k, v, gf, None)
+    got = f64(vig_amd.gla_bidir_forward(*dev(q, k, v, gf, None)))
+    assert np.isfinite(got).all()
+    assert max_abs(got, want) <= BF16_TOL
+
+
 @pytest.mark.parametrize("idx,batch", [(1, None), (2, None), (3, None), (4, 64)])
 def test_bf16_named_configs_full_size(idx, batch):
     """Full-size named workloads against the oracle (the oracle finishes these in seconds)."""

@@ -191,8 +191,9 @@ def test_blend_matches_torch_expression(rng):
 
 
 def test_precision_model_supports_the_shipped_splits():
-    """The kernel's hi/lo splits (scores: 3 terms, P: 2 terms) cut the internal error of a plain bf16 chunk kernel
-    by more than 2x on ViG-S-shaped inputs; the emulation with every operand split reproduces the oracle."""
+    """The kernel's operand precisions (scores: fp16 operands, or three bf16 terms in the fallback; P: 2 terms) cut
+    the internal error of a plain bf16 chunk kernel by more than 2x on ViG-S-shaped inputs; the emulation with every
+    operand split reproduces the oracle."""
     import torch
     from oracle import mfma_precision_model as M
     from vig_amd.synthetic import make_gla_inputs
@@ -205,6 +206,8 @@ def test_precision_model_supports_the_shipped_splits():
     e_plain = rms(M.emulate(*arrs, 49, M.PLAIN))
     e_ship = rms(M.emulate(*arrs, 49, M.SHIPPED))
     e_all = rms(M.emulate(*arrs, 49, dict(qk=3, p=2, iq=2, st=2, u=2)))
+    e_fall = rms(M.emulate(*arrs, 49, M.FALLBACK))
     assert e_all < 2e-5
     assert e_plain > 1.2e-3
     assert e_ship < 0.5 * e_plain
+    assert e_fall < 0.5 * e_plain

@@ -1,4 +1,4 @@
-// Bidirectional chunked GLA forward on bf16 MFMA tiles (gfx950), Dk = Dv = 64.
+// Bidirectional chunked GLA forward on MFMA tiles (gfx950), Dk in {32, 64}, Dv = 64, bf16 in and out.
 //
 // One persistent workgroup of 8 waves per CU walks (batch, head) slabs of up to 256
 // tokens.  A slab is cut into 4 chunks of ceil(L/4) <= 64 tokens; wave (chunk c,
@@ -6,33 +6,36 @@
 // side by side on the same SIMD and read the same q/k/v lines.  A wave
 //   1. forms the chunk-local cumulative log-gates G with a triangular-ones MFMA
 //      (bf16 gates are exact MFMA inputs, the sums accumulate in fp32),
-//   2. builds end-anchored operands q~ = q*exp(G - G_end) (>= |q|) and
-//      k~ = k*exp(G_end - G) (<= |k|), each split into bf16 hi + lo,
-//   3. computes the masked intra-chunk scores P^T = k~ q~^T with three MFMA terms
-//      (hi*hi + lo*hi + hi*lo) and P V with P split hi + lo  (V is exact bf16),
-//   4. accumulates the chunk's state contribution U = k~^T V  [Dk x Dv] in fp32.
+//   2. builds operands anchored at half the chunk total, q~ = q*exp(G - G_end/2) and
+//      k~ = k*exp(G_end/2 - G): both stay within exp(|G_end|/2) of the inputs,
+//   3. computes the masked intra-chunk scores P^T = k~ q~^T on fp16 operands (11-bit
+//      significands, one MFMA term) and P V on bf16 with P split hi + lo (V is exact bf16),
+//   4. accumulates the chunk's state contribution U = k~^T V  [Dk x Dv] in fp32 (k~ as bf16).
 // The U's of a direction meet once in LDS, where the four waves of the direction run the
-// chunk-to-chunk state recurrence S <- exp(G_end) * S + U in parallel over disjoint state
-// slices and leave, for every chunk, the decayed incoming state as ready bf16 MFMA
-// fragments; each wave adds q~ (exp(G_end) * S_in) to its outputs.  The two waves of a
+// chunk-to-chunk state recurrence S <- sqrt(D) (sqrt(D) S + U), D = exp(G_end), in parallel over
+// disjoint state slices and leave, for every chunk, sqrt(D) S_in as ready bf16 MFMA
+// fragments; each wave adds q~ (sqrt(D) S_in) to its outputs.  The two waves of a
 // chunk then swap half of their fp32 output tiles through LDS, add, scale and store
 // bf16 once.  Loads for the next slab are issued before the swap.
 //
-// Chunk algebra follows flash-linear-attention/fla/ops/gla/chunk_util.py:9-78 and
-// chunk_fuse.py:76-97,245-254 (here with 64-token chunks, an end anchor so that the
-// state update needs no second set of factors, and matrix-core intra-chunk scores);
-// both directions are served by one launch as in recurrent_fuse.py:19-148.
+// fp16 score operands need |G_end|/2 * log2(e) <= 6 in every channel of every chunk (ViG's
+// logsigmoid(.)/16 gates reach about 2.5) and inputs below 65504 / 64 in magnitude.  A
+// workgroup that meets a segment with stronger gates redoes it, and does all its later
+// segments, with bf16 hi + lo operands and three score terms per k-step (same algebra,
+// any gate total up to ~80 per chunk and channel).
 //
-// Register layouts (lane l: r = l & 31, h = l >> 5), v_mfma_f32_32x32x16_bf16:
+// Chunk algebra follows flash-linear-attention/fla/ops/gla/chunk_util.py:9-78 and
+// chunk_fuse.py:76-97,245-254 (here with 64-token chunks, a mid-range anchor so that both
+// operands stay small, and matrix-core intra-chunk scores); both directions are served by
+// one launch as in recurrent_fuse.py:19-148.
+//
+// Register layouts (lane l: r = l & 31, h = l >> 5), v_mfma_f32_32x32x16_{bf16,f16}:
 //   A/B operand: lane supplies index r and contraction slots e = 0..7 (4 VGPRs);
 //   C/D: lane holds column r, register c = 4*g + m holds row 8*g + 4*h + m.
 // "Transposed" fragments (tokens in the contraction slots) are read as one dword =
 // two adjacent channels per token and de-interleaved with v_perm_b32; lane-row rho
 // reads channel pair cpair(rho), chosen so that every accumulator ends up holding
 // 32 contiguous channels (32*h + 8*g + 2*m + p) of one token.
-//
-// Supported gate range: sum of |g| over any 64-token chunk and channel below ~80
-// (exp2 arguments stay finite); ViG's logsigmoid(.)/16 gates are far inside it.
 #include "common.h"
 #include "launch.h"
 #ifdef VIG_TIMING
@@ -63,15 +66,31 @@ __device__ unsigned long long g_stamp[4][8][16];
 #endif
 
 constexpr float kLog2e = 1.4426950408889634f;
+// fp16 score operands are used while |G_end|/2 * log2(e) <= this for every channel of the chunk: the scaled
+// operands then stay within 2^6 of the inputs' magnitudes (fp16 holds |x| < 65504 and full precision above 6e-5).
+constexpr float kFastHalfRange = 6.0f;
 constexpr int kKtStride = 72;                // bf16 elements per k~ row in LDS (144 B: conflict-free b128 writes)
 constexpr int kRegionBytes = 16 * 1024;      // per wave: k~ scratch, then published U / state fragments / output half
 constexpr int kLdsDvec = 8 * kRegionBytes;   // per wave: 64 chunk decays exp(G_end)
 constexpr int kLdsGend = kLdsDvec + 8 * 64 * 4;  // per wave: 64 anchors G_end * log2(e), laid out [h][p][16]
-constexpr int kLdsTotal = kLdsGend + 8 * 64 * 4;
+constexpr int kLdsVeto = kLdsGend + 8 * 64 * 4;  // one word: some chunk refused the fp16 variant
+constexpr int kLdsTotal = kLdsVeto + 16;
 
 __device__ __forceinline__ f32x16_t mfma(const u32x4_t& a, const u32x4_t& b, const f32x16_t& c) {
   return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, a), __builtin_bit_cast(bf16x8_t, b), c, 0,
                                                  0, 0);
+}
+
+typedef _Float16 f16x2_t __attribute__((ext_vector_type(2)));
+typedef _Float16 f16x8_t __attribute__((ext_vector_type(8)));
+__device__ __forceinline__ f32x16_t mfma_f16(const u32x4_t& a, const u32x4_t& b, const f32x16_t& c) {
+  return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8_t, a), __builtin_bit_cast(f16x8_t, b), c, 0,
+                                                0, 0);
+}
+__device__ __forceinline__ uint32_t pack_f16x2(float lo, float hi) {
+  f32x2_t x = {lo, hi};
+  f16x2_t y = __builtin_convertvector(x, f16x2_t);  // round to nearest even
+  return __builtin_bit_cast(uint32_t, y);
 }
 
 // Channel pair read by lane-row rho of a transposed fragment whose rows span 16*NG channels (NG = 4: 64 channels,
@@ -218,6 +237,47 @@ __device__ __forceinline__ void make_half(const u32x4_t (&raw)[NG], const f32x16
   }
 }
 
+// q~ and k~ of one 32-token tile for the fp16 score path: one exponent per element serves both (the factors are
+// reciprocal), each product is rounded once to fp16 (11-bit significand) for the scores and once to bf16 for the
+// state path (k~: state update through LDS; q~: inter-chunk product).
+template <bool WITH_Q, int NG>
+__device__ __forceinline__ void make_pair16(const u32x4_t (&rawq)[NG], const u32x4_t (&rawk)[NG],
+                                            const f32x16_t (&G)[2], const float* gend2, u32x4_t (&q16)[NG],
+                                            u32x4_t (&k16)[NG], u32x4_t (&qb)[NG], u32x4_t (&kb)[NG]) {
+#pragma unroll
+  for (int g = 0; g < NG; ++g) {
+    const f32x4_t a0 = *reinterpret_cast<const f32x4_t*>(gend2 + 4 * g);
+    const f32x4_t a1 = *reinterpret_cast<const f32x4_t*>(gend2 + 16 + 4 * g);
+#pragma unroll
+    for (int m = 0; m < 4; ++m) {
+      const int c = 4 * g + m;
+      const float x0 = __builtin_fmaf(G[0][c], kLog2e, -a0[m]);
+      const float x1 = __builtin_fmaf(G[1][c], kLog2e, -a1[m]);
+      const uint32_t wk = rawk[g][m];
+      const float k0 = bf16lo_to_f32(wk) * exp2_fast(-x0);
+      const float k1 = bf16hi_to_f32(wk) * exp2_fast(-x1);
+      k16[g][m] = pack_f16x2(k0, k1);
+      kb[g][m] = pack_bf16x2(k0, k1);
+      if (WITH_Q) {
+        const uint32_t wq = rawq[g][m];
+        const float q0 = bf16lo_to_f32(wq) * exp2_fast(x0);
+        const float q1 = bf16hi_to_f32(wq) * exp2_fast(x1);
+        q16[g][m] = pack_f16x2(q0, q1);
+        qb[g][m] = pack_bf16x2(q0, q1);
+      }
+    }
+  }
+}
+
+// P^T tile = k~ (rows j) x q~ (columns i) on fp16 operands.
+template <int NG>
+__device__ __forceinline__ f32x16_t score_tile16(const u32x4_t (&k16)[NG], const u32x4_t (&q16)[NG]) {
+  f32x16_t acc = {0.f};
+#pragma unroll
+  for (int ks = 0; ks < NG; ++ks) acc = mfma_f16(k16[ks], q16[ks], acc);
+  return acc;
+}
+
 // P^T tile = k~ (rows j) x q~ (columns i), three-term split product.
 template <int NG>
 __device__ __forceinline__ f32x16_t score_tile(const HalfOps<NG>& kop, const HalfOps<NG>& qop) {
@@ -303,10 +363,103 @@ __device__ __forceinline__ void issue_first_phase(const ChunkSrc& src, int r, in
 constexpr int kModeSlab = 0, kModeState = 1, kModeChain = 2;
 constexpr int kStateFloats = 64 * 64 + 64;  // per (sequence, segment, direction): state in unit order, then 64 decays
 
+// Intra-chunk part of one wave: scores of the three tile pairs of its chunk, applied to V; k~ (bf16) goes to the
+// wave's LDS scratch for the state update, q~ (bf16) is kept for the inter-chunk product.  The second tile's rows
+// and V fragments are fetched while the first is worked on.
+//   F16: score operands are single fp16 roundings (valid while the chunk's gate totals keep them inside fp16 range);
+//   otherwise bf16 hi + lo pairs and three MFMA terms per k-step.
+template <bool FWD, int MODE, int NG, bool F16>
+__device__ __forceinline__ void tile_phase(const ChunkSrc& cur, const Prefetch<NG>& pf, const f32x16_t (&G)[2][2],
+                                           const float* gend2, uint16_t* kt, int r, int h, f32x16_t (&O)[2][2],
+                                           u32x4_t (&qkeep)[2][NG], u32x4_t (&vfrag)[4][2]) {
+  constexpr bool OUT = MODE != kModeState;
+  constexpr int TA = FWD ? 0 : 1;  // tile walked first
+  constexpr int TB = FWD ? 1 : 0;
+  constexpr int MASK = FWD ? 1 : 2;
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int j = 0; j < 2; ++j) O[i][j] = f32x16_t{0.f};
+  u32x4_t rawk[NG], rawq[NG];
+  uint32_t vDb[2][8];
+  auto set_vfrag = [&](const uint32_t (&D)[2][8], int t0) {
+    u32x4_t vf[2][2];
+    finish_tfrags<2>(D, vf);
+#pragma unroll
+    for (int tl = 0; tl < 2; ++tl)
+#pragma unroll
+      for (int p = 0; p < 2; ++p) vfrag[t0 + tl][p] = vf[tl][p];
+  };
+  auto fetch_second = [&]() {
+    if (OUT) issue_raw_tile<NG>(cur.q, TB, r, h, rawq);
+    issue_raw_tile<NG>(cur.k, TB, r, h, rawk);
+    issue_tdwords<2 * TB, 2, 4>(cur.v, r, h, vDb);
+  };
+  if (F16) {
+    u32x4_t ka[NG], qb[NG];
+    {
+      u32x4_t qa[NG], kab[NG];
+      make_pair16<OUT, NG>(pf.rawq, pf.rawk, G[TA], gend2, qa, ka, qkeep[TA], kab);
+      store_kt<NG>(kt, 32 * TA + r, h, kab);
+      VIG_PHASE();
+      fetch_second();
+      set_vfrag(pf.vD, 2 * TA);
+      if (OUT) apply_scores<MASK>(score_tile16<NG>(ka, qa), TA, r, h, vfrag, O[0][TA], O[1][TA]);
+    }
+    VIG_PHASE();
+    u32x4_t kb[NG];
+    {
+      u32x4_t kbb[NG];
+      make_pair16<OUT, NG>(rawq, rawk, G[TB], gend2, qb, kb, qkeep[TB], kbb);
+      store_kt<NG>(kt, 32 * TB + r, h, kbb);
+    }
+    if (OUT) apply_scores<0>(score_tile16<NG>(ka, qb), TA, r, h, vfrag, O[0][TB], O[1][TB]);
+    VIG_PHASE();
+    set_vfrag(vDb, 2 * TB);
+    if (OUT) apply_scores<MASK>(score_tile16<NG>(kb, qb), TB, r, h, vfrag, O[0][TB], O[1][TB]);
+  } else {
+    HalfOps<NG> ka, qb;
+    {
+      HalfOps<NG> qa;
+      make_half<false, NG>(pf.rawk, G[TA], gend2, ka);
+      if (OUT) make_half<true, NG>(pf.rawq, G[TA], gend2, qa);
+      VIG_PHASE();
+      fetch_second();
+      set_vfrag(pf.vD, 2 * TA);
+      if (OUT) apply_scores<MASK>(score_tile(ka, qa), TA, r, h, vfrag, O[0][TA], O[1][TA]);
+      store_kt<NG>(kt, 32 * TA + r, h, ka.h);
+      if (OUT) {
+#pragma unroll
+        for (int ks = 0; ks < NG; ++ks) qkeep[TA][ks] = qa.h[ks];
+      }
+    }
+    VIG_PHASE();
+    if (OUT) {
+      make_half<true, NG>(rawq, G[TB], gend2, qb);
+      apply_scores<0>(score_tile(ka, qb), TA, r, h, vfrag, O[0][TB], O[1][TB]);
+    }
+    VIG_PHASE();
+    {
+      HalfOps<NG> kb;
+      make_half<false, NG>(rawk, G[TB], gend2, kb);
+      set_vfrag(vDb, 2 * TB);
+      if (OUT) apply_scores<MASK>(score_tile(kb, qb), TB, r, h, vfrag, O[0][TB], O[1][TB]);
+      store_kt<NG>(kt, 32 * TB + r, h, kb.h);
+    }
+    if (OUT) {
+#pragma unroll
+      for (int ks = 0; ks < NG; ++ks) qkeep[TB][ks] = qb.h[ks];
+    }
+  }
+}
+
+
 // Everything one wave does for one segment: chunk c (the valid rows its descriptors cover) in
 // direction FWD / reverse.  Every wave of the workgroup passes the same three barriers here (plus the caller's).
-template <bool FWD, int MODE, int NG>
-__device__ __forceinline__ void direction_wave(const ChunkSrc& cur, const ChunkSrc& nxt, rsrc_t o, int c, int lane,
+// F16 selects fp16 score operands; that variant returns false (for every wave of the workgroup alike, and without
+// having stored anything) when some chunk of the segment has gates too strong for it.
+template <bool FWD, int MODE, int NG, bool F16>
+__device__ __forceinline__ bool direction_wave(const ChunkSrc& cur, const ChunkSrc& nxt, rsrc_t o, int c, int lane,
                                                char* lds, float oscale, bool bidir, float* state, Prefetch<NG>& pf,
                                                int iter) {
   constexpr bool OUT = MODE != kModeState;  // produces outputs (needs q)
@@ -328,46 +481,48 @@ __device__ __forceinline__ void direction_wave(const ChunkSrc& cur, const ChunkS
     finish_tfrags<4>(pf.gD, gfrag);
     const u32x4_t ones = {0x3F803F80u, 0x3F803F80u, 0x3F803F80u, 0x3F803F80u};
     const u32x4_t tri0 = tri_frag<FWD>(0, 0, r, h), tri1 = tri_frag<FWD>(1, 0, r, h);
+    // k-steps of the tile walked first / second (the triangular operand depends on (k-step, tile) only through
+    // their offset, so two fragments serve both tiles)
+    constexpr int A0 = FWD ? 0 : 2, B0 = FWD ? 2 : 0;
 #pragma unroll
     for (int p = 0; p < 2; ++p) {
-      f32x16_t g0 = {0.f}, g1 = {0.f};
+      // total of the tile walked first, in every column: the second tile's sums start from it
+      f32x16_t carry = {0.f};
+      carry = mfma(gfrag[A0][p], ones, carry);
+      carry = mfma(gfrag[A0 + 1][p], ones, carry);
+      f32x16_t ga = {0.f};
+      ga = mfma(gfrag[A0][p], tri0, ga);
+      ga = mfma(gfrag[A0 + 1][p], tri1, ga);
+      f32x16_t gb = mfma(gfrag[B0][p], tri0, carry);
+      gb = mfma(gfrag[B0 + 1][p], tri1, gb);
       // the chunk total (= G at the anchor token) for every column at once: no cross-lane broadcast needed
-      f32x16_t ge = {0.f};
-#pragma unroll
-      for (int t = 0; t < 4; ++t) ge = mfma(gfrag[t][p], ones, ge);
+      f32x16_t ge = mfma(gfrag[B0][p], ones, carry);
+      ge = mfma(gfrag[B0 + 1][p], ones, ge);
       Gend[p] = ge;
-      // the triangular operand depends on (k-step, tile) only through their offset: two distinct fragments
-      if (FWD) {
-        g0 = mfma(gfrag[0][p], tri0, g0);
-        g0 = mfma(gfrag[1][p], tri1, g0);
-        g1 = mfma(gfrag[0][p], ones, g1);
-        g1 = mfma(gfrag[1][p], ones, g1);
-        g1 = mfma(gfrag[2][p], tri0, g1);
-        g1 = mfma(gfrag[3][p], tri1, g1);
-      } else {
-        g0 = mfma(gfrag[0][p], tri0, g0);
-        g0 = mfma(gfrag[1][p], tri1, g0);
-        g0 = mfma(gfrag[2][p], ones, g0);
-        g0 = mfma(gfrag[3][p], ones, g0);
-        g1 = mfma(gfrag[2][p], tri0, g1);
-        g1 = mfma(gfrag[3][p], tri1, g1);
-      }
-      G[0][p] = g0;
-      G[1][p] = g1;
+      G[FWD ? 0 : 1][p] = ga;
+      G[FWD ? 1 : 0][p] = gb;
     }
   }
   VIG_STAMP(1);
-  // ---- anchor: G at the last token (forward) / first token (reverse) of the chunk, same channels per lane half.
-  // The anchors (x log2 e) and the chunk decays exp(G_end) go to LDS: the operand builders re-read the former per
+  // ---- anchor: half of the chunk total G_end (G at the last token forward / first token reverse), per channel, so
+  // that q~ = q*exp(G - G_end/2) and k~ = k*exp(G_end/2 - G) share the exponent range [-|G_end|/2, |G_end|/2].
+  // The anchors (x log2 e) and the half decays exp(G_end/2) go to LDS: the operand builders re-read the former per
   // tile, the state recurrence reads the latter after barrier A, and no register holds them across phases. ----
   float* gend2 = reinterpret_cast<float*>(lds + kLdsGend) + wi * 64 + 32 * h;
   constexpr int HC = 8 * NG;  // channels per lane half
+  bool fast = true;
   {
     float e2[2][16];
+    float amax = 0.f;
 #pragma unroll
     for (int p = 0; p < 2; ++p)
 #pragma unroll
-      for (int cc = 0; cc < 16; ++cc) e2[p][cc] = Gend[p][cc] * kLog2e;
+      for (int cc = 0; cc < 16; ++cc) {
+        e2[p][cc] = Gend[p][cc] * (0.5f * kLog2e);
+        if (F16) amax = fmaxf(amax, fabsf(e2[p][cc]));
+      }
+    // wave-uniform: fp16 score operands while every channel's exponent range stays within +-kFastHalfRange
+    if (F16) fast = __builtin_amdgcn_ballot_w64(amax > kFastHalfRange) == 0;
     if (r == 0) {  // every lane of a half holds the same 32 values; one lane writes them
       float* d = dvec_all + wi * 64 + HC * h;
 #pragma unroll
@@ -376,7 +531,7 @@ __device__ __forceinline__ void direction_wave(const ChunkSrc& cur, const ChunkS
         const f32x4_t x1 = {e2[1][4 * gq], e2[1][4 * gq + 1], e2[1][4 * gq + 2], e2[1][4 * gq + 3]};
         *reinterpret_cast<f32x4_t*>(gend2 + 4 * gq) = x0;
         *reinterpret_cast<f32x4_t*>(gend2 + 16 + 4 * gq) = x1;
-        // decay of channel 8*gq + 2*m + p
+        // half decay of channel 8*gq + 2*m + p
         const f32x4_t d0 = {exp2_fast(x0[0]), exp2_fast(x1[0]), exp2_fast(x0[1]), exp2_fast(x1[1])};
         const f32x4_t d1 = {exp2_fast(x0[2]), exp2_fast(x1[2]), exp2_fast(x0[3]), exp2_fast(x1[3])};
         *reinterpret_cast<f32x4_t*>(d + 8 * gq) = d0;
@@ -386,66 +541,11 @@ __device__ __forceinline__ void direction_wave(const ChunkSrc& cur, const ChunkS
   }
   wave_lds_sync();
   VIG_STAMP(2);
-  // ---- intra-chunk scores, tile by tile; each tile's rows and V fragments are fetched one phase ahead ----
+  // ---- intra-chunk scores, tile by tile ----
   f32x16_t O[2][2];
-#pragma unroll
-  for (int i = 0; i < 2; ++i)
-#pragma unroll
-    for (int j = 0; j < 2; ++j) O[i][j] = f32x16_t{0.f};
   u32x4_t qkeep[2][NG];
   u32x4_t vfrag[4][2];
-  {
-    HalfOps<NG> ka, qb;
-    u32x4_t rawk[NG], rawq[NG];
-    uint32_t vDb[2][8];
-    {
-      HalfOps<NG> qa;
-      make_half<false, NG>(pf.rawk, G[TA], gend2, ka);
-      if (OUT) make_half<true, NG>(pf.rawq, G[TA], gend2, qa);
-      VIG_PHASE();
-      if (OUT) issue_raw_tile<NG>(cur.q, TB, r, h, rawq);
-      issue_raw_tile<NG>(cur.k, TB, r, h, rawk);
-      issue_tdwords<2 * TB, 2, 4>(cur.v, r, h, vDb);
-      {
-        u32x4_t vf[2][2];
-        finish_tfrags<2>(pf.vD, vf);
-#pragma unroll
-        for (int tl = 0; tl < 2; ++tl)
-#pragma unroll
-          for (int p = 0; p < 2; ++p) vfrag[2 * TA + tl][p] = vf[tl][p];
-      }
-      if (OUT) apply_scores<FWD ? 1 : 2>(score_tile(ka, qa), TA, r, h, vfrag, O[0][TA], O[1][TA]);
-      store_kt<NG>(kt, 32 * TA + r, h, ka.h);
-      if (OUT) {
-#pragma unroll
-        for (int ks = 0; ks < NG; ++ks) qkeep[TA][ks] = qa.h[ks];
-      }
-    }
-    VIG_PHASE();
-    if (OUT) {
-      make_half<true, NG>(rawq, G[TB], gend2, qb);
-      apply_scores<0>(score_tile(ka, qb), TA, r, h, vfrag, O[0][TB], O[1][TB]);
-    }
-    VIG_PHASE();
-    {
-      HalfOps<NG> kb;
-      make_half<false, NG>(rawk, G[TB], gend2, kb);
-      {
-        u32x4_t vf[2][2];
-        finish_tfrags<2>(vDb, vf);
-#pragma unroll
-        for (int tl = 0; tl < 2; ++tl)
-#pragma unroll
-          for (int p = 0; p < 2; ++p) vfrag[2 * TB + tl][p] = vf[tl][p];
-      }
-      if (OUT) apply_scores<FWD ? 1 : 2>(score_tile(kb, qb), TB, r, h, vfrag, O[0][TB], O[1][TB]);
-      store_kt<NG>(kt, 32 * TB + r, h, kb.h);
-    }
-    if (OUT) {
-#pragma unroll
-      for (int ks = 0; ks < NG; ++ks) qkeep[TB][ks] = qb.h[ks];
-    }
-  }
+  tile_phase<FWD, MODE, NG, F16>(cur, pf, G, gend2, kt, r, h, O, qkeep, vfrag);
   VIG_STAMP(3);
   wave_lds_sync();  // k~ rows of this wave visible to its other lanes
   VIG_STAMP(4);
@@ -488,8 +588,13 @@ __device__ __forceinline__ void direction_wave(const ChunkSrc& cur, const ChunkS
   asm volatile("" : "+v"(lane));
   r = lane & 31;
   h = lane >> 5;
+  int* veto = reinterpret_cast<int*>(lds + kLdsVeto);
+  if (F16 && !fast && lane == 0) *veto = 1;
   lds_barrier();  // (A) published U's and decays visible
   VIG_STAMP(6);
+  // same answer in every wave: the word is only written before this barrier and the variant is left once it is set
+  const bool ok = !F16 || __builtin_amdgcn_readfirstlane(*veto) == 0;
+  if (F16 && !ok) o = chunk_rsrc(nullptr, 0, 0);  // nothing of this segment is stored
   // ---- state recurrence over the chunks of this direction, one slice (pv, NG/2 register quads) per wave ----
   {
     constexpr int NQ = NG / 2;
@@ -503,14 +608,18 @@ __device__ __forceinline__ void direction_wave(const ChunkSrc& cur, const ChunkS
 #pragma unroll
       for (int j = 0; j < NQ; ++j) {
         const int u = (pk * 2 + pv) * 4 + cqa + j;
-        if (MODE == kModeChain)  // state entering the segment, written by the segment scan in the same unit order
+        if (MODE == kModeChain) {  // state entering the segment, written by the segment scan in the same unit order
           S[pk][j] = *reinterpret_cast<const f32x4_t*>(state + (u * 64 + lane) * 4);
-        else
+        } else {  // state after the first chunk: its half-anchored contribution times its half decay
           S[pk][j] = *reinterpret_cast<const f32x4_t*>(unit_ptr(dirbase + W0 * kRegionBytes, u, lane));
+          const float* dw = ddir + W0 * 64 + HC * h + 8 * (cqa + j);
+#pragma unroll
+          for (int m = 0; m < 4; ++m) S[pk][j][m] *= dw[2 * m + pk];
+        }
       }
 #pragma unroll
     for (int i = (MODE == kModeChain ? 0 : 1); i < 4; ++i) {
-      const int wc = W0 + STEP * i;  // consumer chunk: needs exp(G_end(wc)) * S as fragments
+      const int wc = W0 + STEP * i;  // consumer chunk: needs exp(G_end(wc)/2) * S as fragments
       char* creg = dirbase + wc * kRegionBytes;
       const bool add_u = MODE == kModeState || i < 3;
 #pragma unroll
@@ -518,7 +627,7 @@ __device__ __forceinline__ void direction_wave(const ChunkSrc& cur, const ChunkS
         const int cq = cqa + j;
         const f32x4_t d0 = *reinterpret_cast<const f32x4_t*>(ddir + wc * 64 + HC * h + 8 * cq);
         const f32x4_t d1 = *reinterpret_cast<const f32x4_t*>(ddir + wc * 64 + HC * h + 8 * cq + 4);
-        // decay of row (m, pk): element 2*m + pk of the eight
+        // half decay of row (m, pk): element 2*m + pk of the eight
         const float dk0[4] = {d0[0], d0[2], d1[0], d1[2]};
         const float dk1[4] = {d0[1], d0[3], d1[1], d1[3]};
         f32x4_t u0 = {0.f, 0.f, 0.f, 0.f}, u1 = {0.f, 0.f, 0.f, 0.f};
@@ -529,24 +638,27 @@ __device__ __forceinline__ void direction_wave(const ChunkSrc& cur, const ChunkS
         u32x4_t fr;
 #pragma unroll
         for (int m = 0; m < 4; ++m) {
+          // with the half anchor: fragment = sqrt(D) * S_in,  S_out = sqrt(D) * (sqrt(D) * S_in + U)
           const float t0 = S[0][j][m] * dk0[m];
           const float t1 = S[1][j][m] * dk1[m];
           fr[m] = pack_bf16x2(t0, t1);
-          S[0][j][m] = t0 + u0[m];
-          S[1][j][m] = t1 + u1[m];
+          S[0][j][m] = (t0 + u0[m]) * dk0[m];
+          S[1][j][m] = (t1 + u1[m]) * dk1[m];
         }
         if (OUT) *reinterpret_cast<u32x4_t*>(unit_ptr(creg, pv * 4 + cq, lane)) = fr;
       }
     }
-    if (MODE == kModeState) {
+    if (MODE == kModeState && ok) {
       // the segment's end-anchored contribution (unit order) and its total decay per channel
 #pragma unroll
       for (int pk = 0; pk < 2; ++pk)
 #pragma unroll
         for (int j = 0; j < NQ; ++j)
           *reinterpret_cast<f32x4_t*>(state + (((pk * 2 + pv) * 4 + cqa + j) * 64 + lane) * 4) = S[pk][j];
-      if (c == 0 && lane < 16 * NG)
-        state[64 * 64 + lane] = ddir[lane] * ddir[64 + lane] * ddir[128 + lane] * ddir[192 + lane];
+      if (c == 0 && lane < 16 * NG) {
+        const float hd = ddir[lane] * ddir[64 + lane] * ddir[128 + lane] * ddir[192 + lane];
+        state[64 * 64 + lane] = hd * hd;
+      }
     }
   }
   VIG_STAMP(7);
@@ -608,6 +720,7 @@ __device__ __forceinline__ void direction_wave(const ChunkSrc& cur, const ChunkS
     lds_barrier();  // (C) keeps the barrier count of the output modes
   }
   VIG_STAMP(12);
+  return ok;
 }
 
 // Geometry of the work items: item = sequence * nseg + segment; a segment holds seg_len tokens (the last one of a
@@ -616,18 +729,18 @@ struct Geometry {
   int L, nseg, seg_len, cw, nitems;
 };
 
-template <bool FWD, int MODE, int NG>
-__device__ __forceinline__ void wave_loop(const uint16_t* q, const uint16_t* k, const uint16_t* v, const uint16_t* g,
-                                          uint16_t* o, const Geometry& geo, int c, int lane, char* lds, float oscale,
-                                          bool bidir, float* state_ws) {
+template <bool FWD, int MODE, int NG, bool F16>
+__device__ __forceinline__ int wave_loop(const uint16_t* q, const uint16_t* k, const uint16_t* v, const uint16_t* g,
+                                         uint16_t* o, const Geometry& geo, int item, int c, int lane, char* lds,
+                                         float oscale, bool bidir, float* state_ws) {
   constexpr bool OUT = MODE != kModeState;
   constexpr int DK = 16 * NG;
   // descriptors of this wave's chunk of an item; past the last item (or for a chunk with no tokens) they are empty
-  auto locate = [&](int item, ChunkSrc& src, rsrc_t& dst) {
+  auto locate = [&](int it, ChunkSrc& src, rsrc_t& dst) {
     int nvalid = 0;
     size_t off = 0;
-    if (item < geo.nitems) {
-      const int seq = item / geo.nseg, seg = item - seq * geo.nseg;
+    if (it < geo.nitems) {
+      const int seq = it / geo.nseg, seg = it - seq * geo.nseg;
       const int seg_tokens = min(geo.seg_len, geo.L - seg * geo.seg_len);
       nvalid = min(max(seg_tokens - c * geo.cw, 0), geo.cw);
       off = (size_t)seq * geo.L + (size_t)seg * geo.seg_len + (size_t)(nvalid > 0 ? c * geo.cw : 0);  // in tokens
@@ -639,7 +752,6 @@ __device__ __forceinline__ void wave_loop(const uint16_t* q, const uint16_t* k, 
     dst = chunk_rsrc(o + off * 64, nvalid, 128);
   };
   Prefetch<NG> pf;
-  int item = blockIdx.x;
   ChunkSrc cur;
   rsrc_t dst;
   locate(item, cur, dst);
@@ -651,11 +763,23 @@ __device__ __forceinline__ void wave_loop(const uint16_t* q, const uint16_t* k, 
     locate(item + gridDim.x, nxt, dst_next);
     float* state = state_ws ? state_ws + ((size_t)item * 2 + (FWD ? 0 : 1)) * kStateFloats : nullptr;
     asm volatile("" : "+v"(lane));  // per-lane constants are rebuilt per item instead of living across the loop
-    direction_wave<FWD, MODE, NG>(cur, nxt, dst, c, lane, lds, oscale, bidir, state, pf, iter);
+    const bool ok = direction_wave<FWD, MODE, NG, F16>(cur, nxt, dst, c, lane, lds, oscale, bidir, state, pf, iter);
     lds_barrier();  // (D) the next item reuses the LDS regions
+    if (F16 && !ok) break;  // this item again, and all that follow, with split-bf16 scores
     cur = nxt;
     dst = dst_next;
   }
+  return item;
+}
+
+// The items of one wave: fp16 score operands until a segment refuses them, split bf16 from there on.
+template <bool FWD, int MODE, int NG>
+__device__ __forceinline__ void wave_items(const uint16_t* q, const uint16_t* k, const uint16_t* v, const uint16_t* g,
+                                           uint16_t* o, const Geometry& geo, int c, int lane, char* lds, float oscale,
+                                           bool bidir, float* state_ws) {
+  const int item = wave_loop<FWD, MODE, NG, true>(q, k, v, g, o, geo, (int)blockIdx.x, c, lane, lds, oscale, bidir,
+                                                  state_ws);
+  wave_loop<FWD, MODE, NG, false>(q, k, v, g, o, geo, item, c, lane, lds, oscale, bidir, state_ws);
 }
 
 }  // namespace
@@ -671,12 +795,26 @@ __global__ __launch_bounds__(512) void gla_mfma_kernel(const uint16_t* __restric
   const int lane = tid & 63;
   const int c = wi & 3;
   const bool bidir = gb != nullptr;
+  if (tid == 0) *reinterpret_cast<int*>(lds + kLdsVeto) = 0;
+  lds_barrier();
   if (wi < 4) {
-    wave_loop<true, MODE, NG>(q, k, v, gf, o, geo, c, lane, lds, oscale, bidir, state_ws);
+    wave_items<true, MODE, NG>(q, k, v, gf, o, geo, c, lane, lds, oscale, bidir, state_ws);
   } else if (bidir) {
-    wave_loop<false, MODE, NG>(q, k, v, gb, o, geo, c, lane, lds, oscale, bidir, state_ws);
+    wave_items<false, MODE, NG>(q, k, v, gb, o, geo, c, lane, lds, oscale, bidir, state_ws);
   } else {
-    for (int item = blockIdx.x; item < geo.nitems; item += gridDim.x) {
+    // idle half of a one-direction launch: keeps the barrier count of the working waves, including the segment
+    // that is walked twice when the fp16 variant is refused
+    const int* veto = reinterpret_cast<const int*>(lds + kLdsVeto);
+    int item = blockIdx.x;
+    for (; item < geo.nitems; item += gridDim.x) {
+      lds_barrier();
+      const bool refused = __builtin_amdgcn_readfirstlane(*veto) != 0;
+      lds_barrier();
+      lds_barrier();
+      lds_barrier();
+      if (refused) break;
+    }
+    for (; item < geo.nitems; item += gridDim.x) {
       lds_barrier();
       lds_barrier();
       lds_barrier();
