@@ -512,32 +512,27 @@ __device__ __forceinline__ bool direction_wave(const ChunkSrc& cur, const ChunkS
   constexpr int HC = 8 * NG;  // channels per lane half
   bool fast = true;
   {
-    float e2[2][16];
-    float amax = 0.f;
+    // every lane of a half holds the same 32 chunk totals, one per register: one lane writes them out, then each
+    // lane of the wave turns one of the 64 values into its anchor and half decay (one exponential per wave
+    // instead of one per value)
+    if (r == 0) {
 #pragma unroll
-    for (int p = 0; p < 2; ++p)
-#pragma unroll
-      for (int cc = 0; cc < 16; ++cc) {
-        e2[p][cc] = Gend[p][cc] * (0.5f * kLog2e);
-        if (F16) amax = fmaxf(amax, fabsf(e2[p][cc]));
-      }
-    // wave-uniform: fp16 score operands while every channel's exponent range stays within +-kFastHalfRange
-    if (F16) fast = __builtin_amdgcn_ballot_w64(amax > kFastHalfRange) == 0;
-    if (r == 0) {  // every lane of a half holds the same 32 values; one lane writes them
-      float* d = dvec_all + wi * 64 + HC * h;
-#pragma unroll
-      for (int gq = 0; gq < NG; ++gq) {
-        const f32x4_t x0 = {e2[0][4 * gq], e2[0][4 * gq + 1], e2[0][4 * gq + 2], e2[0][4 * gq + 3]};
-        const f32x4_t x1 = {e2[1][4 * gq], e2[1][4 * gq + 1], e2[1][4 * gq + 2], e2[1][4 * gq + 3]};
+      for (int gq = 0; gq < 4; ++gq) {
+        const f32x4_t x0 = {Gend[0][4 * gq], Gend[0][4 * gq + 1], Gend[0][4 * gq + 2], Gend[0][4 * gq + 3]};
+        const f32x4_t x1 = {Gend[1][4 * gq], Gend[1][4 * gq + 1], Gend[1][4 * gq + 2], Gend[1][4 * gq + 3]};
         *reinterpret_cast<f32x4_t*>(gend2 + 4 * gq) = x0;
         *reinterpret_cast<f32x4_t*>(gend2 + 16 + 4 * gq) = x1;
-        // half decay of channel 8*gq + 2*m + p
-        const f32x4_t d0 = {exp2_fast(x0[0]), exp2_fast(x1[0]), exp2_fast(x0[1]), exp2_fast(x1[1])};
-        const f32x4_t d1 = {exp2_fast(x0[2]), exp2_fast(x1[2]), exp2_fast(x0[3]), exp2_fast(x1[3])};
-        *reinterpret_cast<f32x4_t*>(d + 8 * gq) = d0;
-        *reinterpret_cast<f32x4_t*>(d + 8 * gq + 4) = d1;
       }
     }
+    wave_lds_sync();
+    float* mine = reinterpret_cast<float*>(lds + kLdsGend) + wi * 64 + lane;  // value (h, p, 4*g + m), lane = 32h+16p+4g+m
+    const float an = *mine * (0.5f * kLog2e);
+    // wave-uniform: fp16 score operands while every channel's exponent range stays within +-kFastHalfRange
+    if (F16) fast = __builtin_amdgcn_ballot_w64(fabsf(an) > kFastHalfRange) == 0;
+    *mine = an;
+    const int p = (lane >> 4) & 1, g = (lane >> 2) & 3, m = lane & 3;
+    // half decay of channel 8*g + 2*m + p of this lane half (register quads >= NG carry no channel)
+    if (g < NG) dvec_all[wi * 64 + HC * h + 8 * g + 2 * m + p] = exp2_fast(an);
   }
   wave_lds_sync();
   VIG_STAMP(2);
