@@ -820,7 +820,8 @@ __global__ __launch_bounds__(512) void gla_mfma_kernel(const uint16_t* __restric
 
 // Chains the segments of every sequence: in place, the workspace slot of segment s (its own contribution U_s and
 // decay D_s) is replaced by the state entering it,  S_in(s') = D_s * S_in(s) + U_s  with s' the next segment in the
-// direction's walk order.  One thread per state element; all accesses are coalesced (unit order is kept).
+// direction's walk order.  One thread per state element; all accesses are coalesced (unit order is kept).  The
+// contributions and decays of eight segments are fetched together, so that the serial part is arithmetic only.
 __global__ __launch_bounds__(256) void gla_segment_scan_kernel(float* state_ws, int nseq, int nseg, int ndir, int ng) {
   const int e = blockIdx.x * 256 + threadIdx.x;  // element in unit order: ((u*64 + lane)*4 + m)
   const int seq = blockIdx.y / ndir, dir = blockIdx.y % ndir;
@@ -829,14 +830,27 @@ __global__ __launch_bounds__(256) void gla_segment_scan_kernel(float* state_ws, 
   const int pk = u >> 3, cq = u & 3, h = lane >> 5;
   if (cq >= ng) return;  // register quads beyond Dk/16 carry no channel
   const int ch = 8 * ng * h + 8 * cq + 2 * m + pk;
+  constexpr int kBatch = 8;
   float S = 0.f;
-  for (int i = 0; i < nseg; ++i) {
-    const int seg = dir == 0 ? i : nseg - 1 - i;
-    float* slot = state_ws + (((size_t)seq * nseg + seg) * 2 + dir) * kStateFloats;
-    const float u_s = slot[e];
-    const float d_s = slot[64 * 64 + ch];
-    slot[e] = S;
-    S = __builtin_fmaf(d_s, S, u_s);
+  for (int i0 = 0; i0 < nseg; i0 += kBatch) {
+    float us[kBatch], ds[kBatch];
+#pragma unroll
+    for (int j = 0; j < kBatch; ++j) {
+      const int i = min(i0 + j, nseg - 1);
+      const int seg = dir == 0 ? i : nseg - 1 - i;
+      const float* slot = state_ws + (((size_t)seq * nseg + seg) * 2 + dir) * kStateFloats;
+      us[j] = slot[e];
+      ds[j] = slot[64 * 64 + ch];
+    }
+#pragma unroll
+    for (int j = 0; j < kBatch; ++j) {
+      const int i = i0 + j;
+      if (i < nseg) {
+        const int seg = dir == 0 ? i : nseg - 1 - i;
+        state_ws[(((size_t)seq * nseg + seg) * 2 + dir) * kStateFloats + e] = S;
+        S = __builtin_fmaf(ds[j], S, us[j]);
+      }
+    }
   }
 }
 
