@@ -55,6 +55,12 @@ const char* vig_gla_strerror(int code);
  * g_bwd == NULL, fused_chunk_gla (chunk_fuse.py:554-572).
  *
  * Built shapes: Dk in {16, 32, 64, 128}, Dv in {32, 64}, any L >= 1.
+ *
+ * Numeric range of the matrix-core path (bf16 tensors and gates, Dk in {32, 64},
+ * Dv = 64): the sum of |g| over any 64 consecutive tokens of one channel must
+ * stay below about 80, and |q|, |k| below about 1000 (beyond either, results
+ * may be inf / NaN, never silently wrong finite numbers).  Other combinations
+ * run on the fp32-arithmetic kernel, which has no such limit.
  */
 int vig_gla_bidir_fwd(const void* q, const void* k, const void* v,
                       const void* g_fwd, const void* g_bwd, void* o,
