@@ -133,6 +133,37 @@ int vig_locality_blend_fwd(const void* o, const void* local, const void* g_lin,
                            int B, int H, int L, int Dv, float eps, int silu_out,
                            int io_dtype, void* stream);
 
+/*
+ * Residual-add + RMS norm over the last dimension (rows x C, C % 8 == 0, C <= 4096):
+ *   s = x (+ residual) in fp32;  residual_out = s (if not NULL);  y = s * rsqrt(mean(s^2) + eps) * weight
+ * residual and residual_out may be NULL; weight [C] f32.  round_sum != 0 first rounds s to the storage
+ * type and normalises the rounded value (what `norm(a + b)` on stored tensors computes); round_sum == 0
+ * is the fused kernel's arithmetic (the unrounded sum is normalised).
+ *
+ * Replaces: flash-linear-attention/fla/modules/rmsnorm.py:69-125 (_layer_norm_fwd_1pass_kernel with
+ * IS_RMS_NORM, HAS_RESIDUAL, STORE_RESIDUAL_OUT) as used at classification/models/vig.py:598,602-606,896.
+ */
+int vig_rmsnorm_fwd(const void* x, const void* residual, const float* weight, void* y, void* residual_out,
+                    long long rows, int C, float eps, int round_sum, int io_dtype, void* stream);
+
+/*
+ * Head-major split of the fused q/k/v projection:
+ *   qkv [B, L, H*Dk | H*Dk | H*Dv]  ->  q, k [B, H, L, Dk],  v [B, H, L, Dv]   (Dk, Dv multiples of 8)
+ *
+ * Replaces: classification/models/vig.py:401-409 (torch.split and the three 'b l (h d) -> b h l d'
+ * rearranges in front of the GLA op).
+ */
+int vig_split_heads_fwd(const void* qkv, void* q, void* k, void* v, int B, int L, int H, int Dk, int Dv,
+                        int io_dtype, void* stream);
+
+/*
+ * SwiGLU product of the MLP:  gate_up [rows, 2*I] = (gate | up)  ->  out [rows, I] = gate * up / (1 + exp(-gate))
+ *
+ * Replaces: swiglu_fwd (flash-linear-attention/fla/modules/activations.py:109-113) on the two halves of
+ * gate_proj's output (classification/models/vig.py:492-495).
+ */
+int vig_swiglu_fwd(const void* gate_up, void* out, long long rows, int I, int io_dtype, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -276,6 +276,40 @@ def rmsnorm_reference(x, weight, eps=1e-6):
     return x * r * np.asarray(weight, dtype=np.float64)
 
 
+def rmsnorm_residual_reference(x, weight, eps=1e-6, residual=None, round_to=None):
+    """Residual-add + RMS norm, float64: s = x + residual; y = s*rsqrt(mean(s^2)+eps)*weight; returns (y, s)
+    (fla/modules/rmsnorm.py:98-125 with IS_RMS_NORM, HAS_RESIDUAL, STORE_RESIDUAL_OUT).  round_to, a function
+    float64 array -> float64 array, rounds s to a storage type before it is normalised (what norm(x + residual) on
+    stored tensors computes, classification/models/vig.py:598,606)."""
+    s = np.asarray(x, dtype=np.float64)
+    if residual is not None:
+        s = s + np.asarray(residual, dtype=np.float64)
+    if round_to is not None:
+        s = round_to(s)
+    return rmsnorm_reference(s, weight, eps), s
+
+
+def split_heads_reference(qkv_blw, num_heads, dk, dv):
+    """qkv [B, L, H*dk | H*dk | H*dv] -> q, k [B,H,L,dk], v [B,H,L,dv] (classification/models/vig.py:401-409)."""
+    x = np.asarray(qkv_blw)
+    B, L, _ = x.shape
+    H = num_heads
+    K = H * dk
+    q = x[..., :K].reshape(B, L, H, dk).transpose(0, 2, 1, 3)
+    k = x[..., K:2 * K].reshape(B, L, H, dk).transpose(0, 2, 1, 3)
+    v = x[..., 2 * K:].reshape(B, L, H, dv).transpose(0, 2, 1, 3)
+    return q, k, v
+
+
+def swiglu_reference(gate_up):
+    """(gate | up) halves of the last dimension -> gate * up / (1 + exp(-gate)), float64
+    (flash-linear-attention/fla/modules/activations.py:109-113)."""
+    x = np.asarray(gate_up, dtype=np.float64)
+    I = x.shape[-1] // 2
+    g, u = x[..., :I], x[..., I:]
+    return g * u / (1.0 + np.exp(-g))
+
+
 def locality_blend_reference(o_bhld, local_blc, glin_blc, w_g, w_l, eps=1e-6, silu_out=False):
     """Block epilogue before o_proj, float64.
 

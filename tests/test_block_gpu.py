@@ -1,0 +1,70 @@
+"""GPU parity of the row-wise block kernels: residual RMS norm, head split, SwiGLU product."""
+import numpy as np
+import pytest
+import torch
+
+import vig_amd
+from oracle import gla_oracle as O
+
+from .util import announce, f64
+
+pytestmark = pytest.mark.gpu
+
+
+def _randn(shape, seed, dtype=torch.float32, scale=1.0):
+    g = torch.Generator(device="cpu").manual_seed(seed)
+    return (torch.randn(*shape, generator=g) * scale).to(dtype)
+
+
+def _close(got, want, tol):
+    """Elementwise |got - want| <= tol * max(1, |want|): bf16 outputs carry half an output ulp (2^-9 relative)."""
+    return bool(np.all(np.abs(got - want) <= tol * np.maximum(1.0, np.abs(want))))
+
+
+def _bf16_round(a):
+    return torch.from_numpy(a).to(torch.bfloat16).double().numpy()
+
+
+@pytest.mark.parametrize("dtype,tol", [(torch.float32, 2e-6), (torch.bfloat16, 2.0 ** -8)])
+@pytest.mark.parametrize("rows,C", [((2, 196), 384), ((3, 5), 192), ((1, 7), 768), ((9,), 8), ((2, 3), 2048)])
+def test_rmsnorm_residual_prenorm(dtype, tol, rows, C):
+    announce(f"rmsnorm {dtype} rows{rows} C{C}")
+    x, r = _randn((*rows, C), 1, dtype), _randn((*rows, C), 2, dtype, 2.0)
+    w = _randn((C,), 3) + 1.0
+    # no residual
+    want, _ = O.rmsnorm_residual_reference(f64(x), f64(w), 1e-6)
+    got = vig_amd.ops.rmsnorm(x.cuda(), w.cuda(), 1e-6)
+    assert _close(f64(got), want, tol)
+    # residual, prenorm: the fused arithmetic normalises the unrounded sum
+    want, s = O.rmsnorm_residual_reference(f64(x), f64(w), 1e-6, residual=f64(r))
+    got, res = vig_amd.ops.rmsnorm(x.cuda(), w.cuda(), 1e-6, residual=r.cuda(), prenorm=True)
+    assert _close(f64(got), want, tol)
+    assert _close(f64(res), s, tol)
+    if dtype == torch.bfloat16:
+        # round_sum: the stored (rounded) sum is what gets normalised, and it is returned bit-exactly
+        want, s = O.rmsnorm_residual_reference(f64(x), f64(w), 1e-6, residual=f64(r), round_to=_bf16_round)
+        got, res = vig_amd.ops.rmsnorm(x.cuda(), w.cuda(), 1e-6, residual=r.cuda(), prenorm=True, round_sum=True)
+        assert np.array_equal(f64(res), s)
+        assert np.array_equal(f64(res), f64(x + r))
+        assert _close(f64(got), want, tol)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("B,L,H,Dk,Dv", [(2, 196, 6, 32, 64), (1, 197, 3, 64, 64), (3, 7, 2, 16, 32)])
+def test_split_heads_is_exact(dtype, B, L, H, Dk, Dv):
+    announce(f"split_heads {dtype} B{B} L{L} H{H} {Dk}/{Dv}")
+    qkv = _randn((B, L, H * (2 * Dk + Dv)), 4, dtype)
+    q, k, v = vig_amd.ops.split_heads(qkv.cuda(), H, Dk, Dv)
+    wq, wk, wv = O.split_heads_reference(f64(qkv), H, Dk, Dv)
+    assert np.array_equal(f64(q), wq) and np.array_equal(f64(k), wk) and np.array_equal(f64(v), wv)
+
+
+@pytest.mark.parametrize("dtype,tol", [(torch.float32, 2e-6), (torch.bfloat16, 2.0 ** -8)])
+@pytest.mark.parametrize("rows,I", [((2, 196), 1024), ((5,), 8), ((3, 4), 512)])
+def test_swiglu(dtype, tol, rows, I):
+    announce(f"swiglu {dtype} rows{rows} I{I}")
+    gu = _randn((*rows, 2 * I), 5, dtype, 2.0)
+    want = O.swiglu_reference(f64(gu))
+    got = vig_amd.ops.swiglu(gu.cuda())
+    assert got.shape == (*rows, I)
+    assert _close(f64(got), want, tol)

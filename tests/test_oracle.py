@@ -211,3 +211,28 @@ def test_precision_model_supports_the_shipped_splits():
     assert e_plain > 1.2e-3
     assert e_ship < 0.5 * e_plain
     assert e_fall < 0.5 * e_plain
+
+
+def test_block_row_ops_against_library_routines():
+    """Residual RMS norm, SwiGLU and the head split against torch's own routines (float64)."""
+    import torch
+    import torch.nn.functional as F
+
+    rng = np.random.default_rng(5)
+    x, r, w = rng.standard_normal((3, 7, 24)), rng.standard_normal((3, 7, 24)), rng.standard_normal(24)
+    y, s = O.rmsnorm_residual_reference(x, w, 1e-6, residual=r)
+    ts = torch.from_numpy(x + r)
+    np.testing.assert_allclose(s, ts.numpy(), rtol=0, atol=0)
+    np.testing.assert_allclose(y, F.rms_norm(ts, (24,), torch.from_numpy(w), 1e-6).numpy(), rtol=1e-12, atol=1e-12)
+    # unit weight, eps -> 0: every row of the output has mean square 1
+    y1, _ = O.rmsnorm_residual_reference(x, np.ones(24), 0.0)
+    np.testing.assert_allclose((y1 ** 2).mean(-1), 1.0, rtol=1e-12)
+    gu = rng.standard_normal((5, 32))
+    tg, tu = torch.from_numpy(gu).chunk(2, -1)
+    np.testing.assert_allclose(O.swiglu_reference(gu), (F.silu(tg) * tu).numpy(), rtol=1e-12, atol=1e-12)
+    qkv = rng.standard_normal((2, 5, 3 * (2 * 4 + 8)))
+    q, k, v = O.split_heads_reference(qkv, 3, 4, 8)
+    tq, tk, tv = torch.split(torch.from_numpy(qkv), [12, 12, 24], dim=2)
+    np.testing.assert_array_equal(q, tq.reshape(2, 5, 3, 4).permute(0, 2, 1, 3).numpy())
+    np.testing.assert_array_equal(k, tk.reshape(2, 5, 3, 4).permute(0, 2, 1, 3).numpy())
+    np.testing.assert_array_equal(v, tv.reshape(2, 5, 3, 8).permute(0, 2, 1, 3).numpy())

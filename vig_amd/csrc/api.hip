@@ -12,6 +12,11 @@ int launch_locality_gate(const void* o, const float* wt, void* y, int B, int H, 
                          hipStream_t stream);
 int launch_locality_blend(const void* o, const void* loc, const void* glin, const float* wg, const float* wl, void* y,
                           int B, int H, int L, int Dv, float eps, int silu_out, int io_dtype, hipStream_t stream);
+int launch_rmsnorm(const void* x, const void* residual, const float* weight, void* y, void* residual_out, int rows,
+                   int C, float eps, int round_sum, int io_dtype, hipStream_t stream);
+int launch_split_heads(const void* qkv, void* q, void* k, void* v, int B, int L, int H, int Dk, int Dv, int io_dtype,
+                       hipStream_t stream);
+int launch_swiglu(const void* in, void* out, long long rows, int I, int io_dtype, hipStream_t stream);
 }  // namespace vig
 
 static bool dtype_ok(int d) { return d == VIG_F32 || d == VIG_BF16; }
@@ -119,6 +124,27 @@ int vig_locality_blend_fwd(const void* o, const void* local, const void* g_lin, 
   if (!dtype_ok(io_dtype) || !(Dv == 32 || Dv == 64)) return VIG_ENOTSUP;
   return vig::launch_locality_blend(o, local, g_lin, w_g, w_l, y, B, H, L, Dv, eps, silu_out, io_dtype,
                                     (hipStream_t)stream);
+}
+
+int vig_rmsnorm_fwd(const void* x, const void* residual, const float* weight, void* y, void* residual_out,
+                    long long rows, int C, float eps, int round_sum, int io_dtype, void* stream) {
+  if (!x || !weight || !y || rows <= 0 || C <= 0 || rows > 0x7fffffffLL) return VIG_EINVAL;
+  if (!dtype_ok(io_dtype) || (C % 8) != 0 || C > 4096) return VIG_ENOTSUP;
+  return vig::launch_rmsnorm(x, residual, weight, y, residual_out, (int)rows, C, eps, round_sum, io_dtype,
+                             (hipStream_t)stream);
+}
+
+int vig_split_heads_fwd(const void* qkv, void* q, void* k, void* v, int B, int L, int H, int Dk, int Dv,
+                        int io_dtype, void* stream) {
+  if (!qkv || !q || !k || !v || B <= 0 || L <= 0 || H <= 0 || Dk <= 0 || Dv <= 0) return VIG_EINVAL;
+  if (!dtype_ok(io_dtype) || (Dk % 8) != 0 || (Dv % 8) != 0 || B > 65535) return VIG_ENOTSUP;
+  return vig::launch_split_heads(qkv, q, k, v, B, L, H, Dk, Dv, io_dtype, (hipStream_t)stream);
+}
+
+int vig_swiglu_fwd(const void* gate_up, void* out, long long rows, int I, int io_dtype, void* stream) {
+  if (!gate_up || !out || rows <= 0 || I <= 0) return VIG_EINVAL;
+  if (!dtype_ok(io_dtype) || (I % 8) != 0) return VIG_ENOTSUP;
+  return vig::launch_swiglu(gate_up, out, rows, I, io_dtype, (hipStream_t)stream);
 }
 
 }  // extern "C"

@@ -1,0 +1,216 @@
+// Row-wise kernels of the ViG block around the GLA op: residual-add + RMS norm, the head-major split of the
+// fused q/k/v projection and the SwiGLU product.  All are HBM-bound: every element is read once and written once
+// with 16-byte accesses, arithmetic in fp32.
+#include "common.h"
+#include "launch.h"
+
+namespace vig {
+
+namespace {
+
+// eight consecutive channels, one 16-byte transaction for bf16 and two for f32
+template <typename T> struct Oct;
+template <> struct Oct<uint16_t> {
+  static __device__ __forceinline__ void load(const uint16_t* p, float (&x)[8]) {
+    const u32x4_t r = *reinterpret_cast<const u32x4_t*>(p);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      x[2 * i] = bf16lo_to_f32(r[i]);
+      x[2 * i + 1] = bf16hi_to_f32(r[i]);
+    }
+  }
+  static __device__ __forceinline__ void store(uint16_t* p, const float (&x)[8]) {
+    u32x4_t r;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) r[i] = pack_bf16x2(x[2 * i], x[2 * i + 1]);
+    *reinterpret_cast<u32x4_t*>(p) = r;
+  }
+  static __device__ __forceinline__ float round(float v) { return bf16_to_f32(f32_to_bf16(v)); }
+};
+template <> struct Oct<float> {
+  static __device__ __forceinline__ void load(const float* p, float (&x)[8]) {
+    const f32x4_t a = *reinterpret_cast<const f32x4_t*>(p);
+    const f32x4_t b = *reinterpret_cast<const f32x4_t*>(p + 4);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      x[i] = a[i];
+      x[4 + i] = b[i];
+    }
+  }
+  static __device__ __forceinline__ void store(float* p, const float (&x)[8]) {
+    f32x4_t a, b;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      a[i] = x[i];
+      b[i] = x[4 + i];
+    }
+    *reinterpret_cast<f32x4_t*>(p) = a;
+    *reinterpret_cast<f32x4_t*>(p + 4) = b;
+  }
+  static __device__ __forceinline__ float round(float v) { return v; }
+};
+
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, 64);
+  return v;
+}
+
+}  // namespace
+
+// ---------------------------------------------------------------------------
+// residual-add + RMS norm, one wave per row of C channels (C % 8 == 0, C <= 64 * 8 * NV):
+//   s = x (+ residual), in fp32;  residual_out = s;  y = s * rsqrt(mean(s^2) + eps) * weight
+// round_sum: s is first rounded to the storage type (the value an explicit add would have stored) and the
+// rounded value is normalised.
+// ---------------------------------------------------------------------------
+template <typename T, int NV>
+__global__ __launch_bounds__(256) void rmsnorm_kernel(const T* __restrict__ x, const T* __restrict__ residual,
+                                                      const float* __restrict__ weight, T* __restrict__ y,
+                                                      T* __restrict__ residual_out, int rows, int C, float eps,
+                                                      int round_sum) {
+  const int lane = threadIdx.x & 63;
+  const int row = blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (row >= rows) return;
+  const int nvec = C >> 3;
+  const size_t base = (size_t)row * C;
+  float s[NV][8];
+  float ss = 0.f;
+#pragma unroll
+  for (int i = 0; i < NV; ++i) {
+    const int v = lane + 64 * i;
+    if (v < nvec) {
+      Oct<T>::load(x + base + 8 * v, s[i]);
+      if (residual) {
+        float rr[8];
+        Oct<T>::load(residual + base + 8 * v, rr);
+#pragma unroll
+        for (int j = 0; j < 8; ++j) s[i][j] += rr[j];
+      }
+      if (round_sum) {
+#pragma unroll
+        for (int j = 0; j < 8; ++j) s[i][j] = Oct<T>::round(s[i][j]);
+      }
+      if (residual_out) Oct<T>::store(residual_out + base + 8 * v, s[i]);
+#pragma unroll
+      for (int j = 0; j < 8; ++j) ss = __builtin_fmaf(s[i][j], s[i][j], ss);
+    }
+  }
+  ss = wave_sum(ss);
+  const float rstd = 1.0f / sqrtf(ss / (float)C + eps);
+#pragma unroll
+  for (int i = 0; i < NV; ++i) {
+    const int v = lane + 64 * i;
+    if (v < nvec) {
+      float w[8];
+      Oct<float>::load(weight + 8 * v, w);
+#pragma unroll
+      for (int j = 0; j < 8; ++j) s[i][j] = s[i][j] * rstd * w[j];
+      Oct<T>::store(y + base + 8 * v, s[i]);
+    }
+  }
+}
+
+template <typename T>
+static int launch_rmsnorm_t(const void* x, const void* residual, const float* weight, void* y, void* residual_out,
+                            int rows, int C, float eps, int round_sum, hipStream_t stream) {
+  const dim3 grid((rows + 3) / 4), block(256);
+  const int nvec = C / 8;
+#define VIG_RMS_CASE(NV)                                                                                          \
+  hipLaunchKernelGGL((rmsnorm_kernel<T, NV>), grid, block, 0, stream, (const T*)x, (const T*)residual, weight, \
+                     (T*)y, (T*)residual_out, rows, C, eps, round_sum)
+  if (nvec <= 64) VIG_RMS_CASE(1);
+  else if (nvec <= 128) VIG_RMS_CASE(2);
+  else if (nvec <= 256) VIG_RMS_CASE(4);
+  else VIG_RMS_CASE(8);
+#undef VIG_RMS_CASE
+  return hipGetLastError() == hipSuccess ? 0 : -5;
+}
+
+int launch_rmsnorm(const void* x, const void* residual, const float* weight, void* y, void* residual_out, int rows,
+                   int C, float eps, int round_sum, int io_dtype, hipStream_t stream) {
+  if (C % 8 != 0 || C > 4096) return -95;
+  return io_dtype == 1 ? launch_rmsnorm_t<uint16_t>(x, residual, weight, y, residual_out, rows, C, eps, round_sum, stream)
+                       : launch_rmsnorm_t<float>(x, residual, weight, y, residual_out, rows, C, eps, round_sum, stream);
+}
+
+// ---------------------------------------------------------------------------
+// head-major split of the fused projection:
+//   qkv [B, L, H*Dk | H*Dk | H*Dv]  ->  q, k [B, H, L, Dk],  v [B, H, L, Dv]
+// One workgroup owns 32 consecutive tokens of one batch element: whole rows are read, and every (tensor, head)
+// receives a contiguous run of 32 tokens.
+// ---------------------------------------------------------------------------
+template <typename T>
+__global__ __launch_bounds__(256) void split_heads_kernel(const T* __restrict__ qkv, T* __restrict__ q,
+                                                          T* __restrict__ k, T* __restrict__ v, int B, int L, int H,
+                                                          int Dk, int Dv) {
+  const int K = H * Dk, V = H * Dv;
+  const int row = 2 * K + V;
+  const int nv = row >> 3;
+  const int b = blockIdx.y;
+  const int l0 = blockIdx.x * 32;
+  const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;
+  for (int cv = tx; cv < nv; cv += 64) {
+    const int ch = cv * 8;
+    T* dst;
+    int D, c;
+    if (ch < K) { dst = q; D = Dk; c = ch; }
+    else if (ch < 2 * K) { dst = k; D = Dk; c = ch - K; }
+    else { dst = v; D = Dv; c = ch - 2 * K; }
+    const int hh = c / D, d = c - hh * D;
+    const T* src = qkv + ((size_t)b * L) * (size_t)row + ch;
+    T* out = dst + (((size_t)b * H + hh) * L) * (size_t)D + d;
+    for (int t = ty; t < 32; t += 4) {
+      const int l = l0 + t;
+      if (l >= L) break;
+      float x[8];
+      Oct<T>::load(src + (size_t)l * row, x);
+      Oct<T>::store(out + (size_t)l * D, x);
+    }
+  }
+}
+
+int launch_split_heads(const void* qkv, void* q, void* k, void* v, int B, int L, int H, int Dk, int Dv, int io_dtype,
+                       hipStream_t stream) {
+  if (Dk % 8 != 0 || Dv % 8 != 0 || B > 65535) return -95;
+  const dim3 grid((L + 31) / 32, B), block(256);
+  if (io_dtype == 1)
+    hipLaunchKernelGGL(split_heads_kernel<uint16_t>, grid, block, 0, stream, (const uint16_t*)qkv, (uint16_t*)q,
+                       (uint16_t*)k, (uint16_t*)v, B, L, H, Dk, Dv);
+  else
+    hipLaunchKernelGGL(split_heads_kernel<float>, grid, block, 0, stream, (const float*)qkv, (float*)q, (float*)k,
+                       (float*)v, B, L, H, Dk, Dv);
+  return hipGetLastError() == hipSuccess ? 0 : -5;
+}
+
+// ---------------------------------------------------------------------------
+// SwiGLU product:  in [rows, 2*I] = (gate | up)  ->  out [rows, I] = gate * up / (1 + exp(-gate))
+// ---------------------------------------------------------------------------
+template <typename T>
+__global__ __launch_bounds__(256) void swiglu_kernel(const T* __restrict__ in, T* __restrict__ out, long long nvec,
+                                                     int I8) {
+  const long long i = (long long)blockIdx.x * 256 + threadIdx.x;
+  if (i >= nvec) return;
+  const long long row = i / I8;
+  const int c = (int)(i - row * I8) * 8;
+  const size_t I = (size_t)I8 * 8;
+  float g[8], u[8];
+  Oct<T>::load(in + (size_t)row * 2 * I + c, g);
+  Oct<T>::load(in + (size_t)row * 2 * I + I + c, u);
+#pragma unroll
+  for (int j = 0; j < 8; ++j) g[j] = g[j] * u[j] / (1.0f + __expf(-g[j]));
+  Oct<T>::store(out + (size_t)row * I + c, g);
+}
+
+int launch_swiglu(const void* in, void* out, long long rows, int I, int io_dtype, hipStream_t stream) {
+  if (I % 8 != 0) return -95;
+  const long long nvec = rows * (I / 8);
+  const dim3 grid((unsigned)((nvec + 255) / 256)), block(256);
+  if (io_dtype == 1)
+    hipLaunchKernelGGL(swiglu_kernel<uint16_t>, grid, block, 0, stream, (const uint16_t*)in, (uint16_t*)out, nvec, I / 8);
+  else
+    hipLaunchKernelGGL(swiglu_kernel<float>, grid, block, 0, stream, (const float*)in, (float*)out, nvec, I / 8);
+  return hipGetLastError() == hipSuccess ? 0 : -5;
+}
+
+}  // namespace vig

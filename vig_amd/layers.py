@@ -8,8 +8,13 @@ package's kernels:
     direction-wise gate preparation        -> vig_dirgate_fwd        (vig.py:432-441)
     bidirectional GLA                      -> vig_gla_bidir_fwd      (vig.py:442-443)
     RMS-norm x2 + sigmoid blend (+SiLU)    -> vig_locality_blend_fwd (vig.py:444-457)
-The surrounding ViG shell (patch embedding, residual RMSNorm wiring, SwiGLU MLP, head) is plain torch
-and follows vig.py:469-497,530-618,625-672,705-912 for the options the shipped configs use.
+    split + three head rearranges          -> vig_split_heads_fwd    (vig.py:401-409)
+    residual add + RMSNorm (prenorm)       -> vig_rmsnorm_fwd        (rmsnorm.py:69-125; vig.py:598,602-606,896)
+    SwiGLU product                         -> vig_swiglu_fwd         (activations.py:109-113; vig.py:492-495)
+The surrounding ViG shell (patch embedding, MLP GEMMs, head) is plain torch and follows
+vig.py:469-497,530-618,625-672,705-912 for the options the shipped configs use.  On CPU tensors the row-wise pieces
+fall back to the same arithmetic in torch (module construction and shape checks only; the GLA op itself has no CPU
+path).
 
 Forward (inference) only: the HIP ops carry no autograd graph.
 """
@@ -37,13 +42,25 @@ class RMSNorm(nn.Module):
         self.eps = eps
         self.weight = nn.Parameter(torch.ones(hidden_size))
 
-    def forward(self, x, residual=None, prenorm: bool = False):
-        if residual is not None:
-            x = (x + residual).to(x.dtype)
+    def _w32(self):
+        """fp32 copy of the weight, refreshed when the parameter changes (the kernels take fp32 weights)."""
+        w = self.weight
+        key = (w.data_ptr(), w._version, w.dtype, w.device)
+        if getattr(self, "_w32_key", None) != key:
+            self._w32_cache = w.detach().float().contiguous()
+            self._w32_key = key
+        return self._w32_cache
+
+    def forward(self, x, residual=None, prenorm: bool = False, round_sum: bool = False):
+        if x.is_cuda:
+            return ops.rmsnorm(x, self._w32(), self.eps, residual=residual, prenorm=prenorm, round_sum=round_sum)
         xf = x.float()
-        y = xf * torch.rsqrt(xf.pow(2).mean(-1, keepdim=True) + self.eps) * self.weight.float()
-        y = y.to(x.dtype)
-        return (y, x) if prenorm else y
+        if residual is not None:
+            xf = xf + residual.float()
+            if round_sum:
+                xf = xf.to(x.dtype).float()
+        y = (xf * torch.rsqrt(xf.pow(2).mean(-1, keepdim=True) + self.eps) * self.weight.float()).to(x.dtype)
+        return (y, xf.to(x.dtype)) if prenorm else y
 
 
 class GatedLinearAttention(nn.Module):
@@ -112,15 +129,13 @@ class GatedLinearAttention(nn.Module):
         conv = self.in_proj[0]
         # local_out, already in the [B, L, C] layout the projections consume
         xs = ops.dwconv3x3(x, conv.weight, hw, bias=conv.bias, silu=self.use_act_in_conv)
-        q, k, v = torch.split(self.qkv_proj(xs), [self.key_dim, self.key_dim, self.value_dim], dim=2)
+        q, k, v = ops.split_heads(self.qkv_proj(xs), H, self.head_qk_dim, self.head_v_dim)
         gates = ops.dirgate(self.gk_proj(xs), H, self.gate_logit_normalizer, self.clamp_min)
-        heads = lambda t, d: t.reshape(B, L, H, d).permute(0, 2, 1, 3).contiguous()
-        q, k, v = heads(q, self.head_qk_dim), heads(k, self.head_qk_dim), heads(v, self.head_v_dim)
         # training glue averages the directions (vig.py:425-426); the eval path halves twice
         # (recurrent_fuse.py:442, then vig.py:443)
         out_scale = 0.5 if self.training else 0.25
         o = ops.gla_bidir_forward(q, k, v, gates[0], gates[1], scale=-1, out_scale=out_scale)
-        y = ops.locality_blend(o, xs, self.g_proj(xs), self.g_norm.weight, self.l_norm.weight,
+        y = ops.locality_blend(o, xs, self.g_proj(xs), self.g_norm._w32(), self.l_norm._w32(),
                                eps=self.layernorm_eps, silu_out=self.use_out_act)
         return self.o_proj(y)
 
@@ -141,7 +156,10 @@ class GLAMLP(nn.Module):
         self.down_proj = nn.Linear(intermediate_size, hidden_size, bias=False)
 
     def forward(self, x):
-        gate, y = self.gate_proj(x).chunk(2, -1)
+        gu = self.gate_proj(x)
+        if gu.is_cuda:
+            return self.down_proj(ops.swiglu(gu))
+        gate, y = gu.chunk(2, -1)
         return self.down_proj(F.silu(gate) * y)
 
 
@@ -164,6 +182,17 @@ class GLABlock(nn.Module):
         h = self.attn(self.attn_norm(hidden_states), **kwargs)
         h, residual = self.mlp_norm(h, residual, True)
         return (residual + self.mlp(h),)
+
+    def forward_carry(self, branch, residual, **kwargs):
+        """Same block, with the closing `residual + mlp(h)` of the previous block folded into this block's first norm:
+        takes (branch, residual) with hidden_states = residual + branch and returns the next such pair."""
+        if residual is None:
+            h, hidden = self.attn_norm(branch), branch
+        else:  # the explicit add stores a rounded sum and attn_norm normalises that (vig.py:598,606)
+            h, hidden = self.attn_norm(branch, residual, True, round_sum=True)
+        h = self.attn(h, **kwargs)
+        h, residual = self.mlp_norm(h, hidden, True)
+        return self.mlp(h), residual
 
 
 class LayerNorm2d(nn.LayerNorm):
@@ -235,9 +264,10 @@ class ViG(nn.Module):
         B = x.shape[0]
         x, hw = self.patch_embed(x)
         x = x + resize_pos_embed(self.pos_embed, self.patch_resolution, hw)
+        branch, residual = x, None
         for blk in self.blocks:
-            x = blk(x, patch_resolution=hw, token_position=None)[0]
-        x = self.norm(x)
+            branch, residual = blk.forward_carry(branch, residual, patch_resolution=hw, token_position=None)
+        x = self.norm(branch, residual, round_sum=True) if residual is not None else self.norm(branch)
         return x.reshape(B, hw[0] * hw[1], -1).mean(dim=1)
 
     @torch.no_grad()

@@ -220,3 +220,68 @@ def locality_blend(o: torch.Tensor, local: torch.Tensor, g_lin: torch.Tensor, w_
                                         _dt(o), _stream_ptr(o))
     _lib.check(rc, "vig_locality_blend_fwd")
     return y
+
+
+def rmsnorm(x: torch.Tensor, weight: torch.Tensor, eps: float = 1e-6, residual: Optional[torch.Tensor] = None,
+            prenorm: bool = False, round_sum: bool = False):
+    """Residual-add + RMS norm over the last dimension (fla/modules/rmsnorm.py:69-125 semantics).
+
+    Returns y, or (y, x + residual) with prenorm=True.  round_sum=True normalises the sum after rounding it to the
+    storage dtype, i.e. what `norm(x + residual)` on stored tensors computes.
+    """
+    lib = _lib.load()
+    _check_cuda(x, weight)
+    x = x.contiguous()
+    C = x.shape[-1]
+    rows = x.numel() // C
+    if residual is not None:
+        _check_cuda(residual)
+        residual = residual.contiguous()
+        if residual.shape != x.shape or residual.dtype != x.dtype:
+            raise ValueError("residual must match x in shape and dtype")
+    w = weight.detach()
+    if w.dtype != torch.float32 or not w.is_contiguous():
+        w = w.float().contiguous()
+    y = torch.empty_like(x)
+    res_out = torch.empty_like(x) if (prenorm and residual is not None) else None
+    with torch.cuda.device(x.device):
+        rc = lib.vig_rmsnorm_fwd(x.data_ptr(), residual.data_ptr() if residual is not None else None, w.data_ptr(),
+                                 y.data_ptr(), res_out.data_ptr() if res_out is not None else None, rows, C,
+                                 float(eps), int(round_sum), _dt(x), _stream_ptr(x))
+    _lib.check(rc, "vig_rmsnorm_fwd")
+    if prenorm:
+        return y, (res_out if res_out is not None else x)
+    return y
+
+
+def split_heads(qkv: torch.Tensor, num_heads: int, head_qk_dim: int, head_v_dim: int):
+    """qkv [B, L, H*Dk | H*Dk | H*Dv] -> q, k [B,H,L,Dk], v [B,H,L,Dv] (vig.py:401-409)."""
+    lib = _lib.load()
+    _check_cuda(qkv)
+    qkv = qkv.contiguous()
+    B, L, W = qkv.shape
+    H = num_heads
+    if W != H * (2 * head_qk_dim + head_v_dim):
+        raise ValueError("last dimension must be H*(2*Dk+Dv)")
+    q = torch.empty(B, H, L, head_qk_dim, dtype=qkv.dtype, device=qkv.device)
+    k = torch.empty_like(q)
+    v = torch.empty(B, H, L, head_v_dim, dtype=qkv.dtype, device=qkv.device)
+    with torch.cuda.device(qkv.device):
+        rc = lib.vig_split_heads_fwd(qkv.data_ptr(), q.data_ptr(), k.data_ptr(), v.data_ptr(), B, L, H, head_qk_dim,
+                                     head_v_dim, _dt(qkv), _stream_ptr(qkv))
+    _lib.check(rc, "vig_split_heads_fwd")
+    return q, k, v
+
+
+def swiglu(gate_up: torch.Tensor) -> torch.Tensor:
+    """gate_up [..., 2*I] = (gate | up) -> gate * up / (1 + exp(-gate))  (fla/modules/activations.py:109-113)."""
+    lib = _lib.load()
+    _check_cuda(gate_up)
+    gate_up = gate_up.contiguous()
+    I = gate_up.shape[-1] // 2
+    rows = gate_up.numel() // (2 * I)
+    out = torch.empty(*gate_up.shape[:-1], I, dtype=gate_up.dtype, device=gate_up.device)
+    with torch.cuda.device(gate_up.device):
+        rc = lib.vig_swiglu_fwd(gate_up.data_ptr(), out.data_ptr(), rows, I, _dt(gate_up), _stream_ptr(gate_up))
+    _lib.check(rc, "vig_swiglu_fwd")
+    return out
