@@ -12,9 +12,8 @@ package's kernels:
     residual add + RMSNorm (prenorm)       -> vig_rmsnorm_fwd        (rmsnorm.py:69-125; vig.py:598,602-606,896)
     SwiGLU product                         -> vig_swiglu_fwd         (activations.py:109-113; vig.py:492-495)
 The surrounding ViG shell (patch embedding, MLP GEMMs, head) is plain torch and follows
-vig.py:469-497,530-618,625-672,705-912 for the options the shipped configs use.  On CPU tensors the row-wise pieces
-fall back to the same arithmetic in torch (module construction and shape checks only; the GLA op itself has no CPU
-path).
+vig.py:469-497,530-618,625-672,705-912 for the options the shipped configs use.  There is no CPU path: every
+library op raises on tensors that are not on the GPU.
 
 Forward (inference) only: the HIP ops carry no autograd graph.
 """
@@ -52,15 +51,7 @@ class RMSNorm(nn.Module):
         return self._w32_cache
 
     def forward(self, x, residual=None, prenorm: bool = False, round_sum: bool = False):
-        if x.is_cuda:
-            return ops.rmsnorm(x, self._w32(), self.eps, residual=residual, prenorm=prenorm, round_sum=round_sum)
-        xf = x.float()
-        if residual is not None:
-            xf = xf + residual.float()
-            if round_sum:
-                xf = xf.to(x.dtype).float()
-        y = (xf * torch.rsqrt(xf.pow(2).mean(-1, keepdim=True) + self.eps) * self.weight.float()).to(x.dtype)
-        return (y, xf.to(x.dtype)) if prenorm else y
+        return ops.rmsnorm(x, self._w32(), self.eps, residual=residual, prenorm=prenorm, round_sum=round_sum)
 
 
 class GatedLinearAttention(nn.Module):
@@ -156,11 +147,7 @@ class GLAMLP(nn.Module):
         self.down_proj = nn.Linear(intermediate_size, hidden_size, bias=False)
 
     def forward(self, x):
-        gu = self.gate_proj(x)
-        if gu.is_cuda:
-            return self.down_proj(ops.swiglu(gu))
-        gate, y = gu.chunk(2, -1)
-        return self.down_proj(F.silu(gate) * y)
+        return self.down_proj(ops.swiglu(self.gate_proj(x)))
 
 
 class GLABlock(nn.Module):
