@@ -75,6 +75,18 @@ def model_throughput(dev, batch=256, warmup=10, iters=30):
 
     from vig_amd import layers
 
+    # the block's GEMMs are hipBLASLt calls made by torch; let torch pick the fastest solution per shape
+    tuned = False
+    try:
+        import torch.cuda.tunable as tunable
+        import tempfile
+        tunable.enable(True)
+        tunable.tuning_enable(True)
+        tunable.set_max_tuning_duration(200)
+        tunable.set_filename(os.path.join(tempfile.gettempdir(), "vig_bench_gemm_solutions.csv"))
+        tuned = True
+    except Exception as e:  # noqa: BLE001 - tuning is optional plumbing
+        log(f"GEMM tuning unavailable: {e}")
     torch.manual_seed(0)
     model = layers.vig_small().eval().to(dev, torch.bfloat16)
     images = torch.randn(batch, 3, 224, 224, device=dev, dtype=torch.bfloat16)
@@ -87,7 +99,7 @@ def model_throughput(dev, batch=256, warmup=10, iters=30):
     torch.cuda.synchronize()
     dt = time.perf_counter() - t0
     return {"images_per_s": iters * batch / dt, "batch": batch, "dtype": "bf16", "iters": iters,
-            "ms_per_forward": dt / iters * 1e3}
+            "ms_per_forward": dt / iters * 1e3, "gemm_solution_tuning": "torch.cuda.tunable" if tuned else None}
 
 
 def main():
