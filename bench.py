@@ -68,7 +68,7 @@ def cpu_baseline(shape, seed, budget_s=20.0):
     }
 
 
-def model_throughput(dev, batch=256, warmup=10, iters=30):
+def model_throughput(dev, batch=256, warmup=10, iters=30, tune_gemm=True):
     """Full ViG-S eval forward (random init, synthetic images, bf16): images/s the way the reference's
     throughput() measures it (classification/main.py:389-406: timed forwards of one resident batch)."""
     import torch
@@ -78,6 +78,8 @@ def model_throughput(dev, batch=256, warmup=10, iters=30):
     # the block's GEMMs are hipBLASLt calls made by torch; let torch pick the fastest solution per shape
     tuned = False
     try:
+        if not tune_gemm:
+            raise RuntimeError("switched off")
         import torch.cuda.tunable as tunable
         import tempfile
         tunable.enable(True)
@@ -112,6 +114,8 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--exact", action="store_true", help="time the fp32-arithmetic recurrent kernel instead")
     ap.add_argument("--model", action="store_true", help="also time the full ViG-S eval forward (images/s)")
+    ap.add_argument("--no-gemm-tuning", action="store_true",
+                    help="with --model: leave torch's GEMM solution tuning off (clean kernel traces)")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run plain device copies of known size (q -> o), so that FETCH_SIZE / WRITE_SIZE "
                          "counters of a profiled run can be scaled to bytes")
@@ -246,7 +250,7 @@ def main():
                      "frac": achieved_gbps / HBM_PEAK_GBPS, "traffic": traffic},
     }
     if args.model:
-        out["vig_s_forward"] = model_throughput(dev)
+        out["vig_s_forward"] = model_throughput(dev, tune_gemm=not args.no_gemm_tuning)
     if not args.no_cpu:
         out["cpu_baseline"] = cpu_baseline(s, 1000 + args.config)
     else:
