@@ -874,9 +874,13 @@ size_t gla_mfma_workspace(int B, int H, int L, int Dk, int Dv) {
   return (size_t)g.nitems * 2 * kStateFloats * sizeof(float);
 }
 
+constexpr int kMaxDevices = 64;
+
 template <int NG>
-static int launch_gla_mfma_t(const GlaArgs& a, int num_cu) {
-  static bool attr_done = false;
+static int launch_gla_mfma_t(const GlaArgs& a, int num_cu, int dev) {
+  // the attribute is per device; concurrent first calls only repeat an idempotent setting
+  static bool attr_done_dev[kMaxDevices] = {};
+  bool& attr_done = attr_done_dev[dev];
   if (!attr_done) {
     const void* kernels[3] = {reinterpret_cast<const void*>(gla_mfma_kernel<kModeSlab, NG>),
                               reinterpret_cast<const void*>(gla_mfma_kernel<kModeState, NG>),
@@ -914,14 +918,16 @@ static int launch_gla_mfma_t(const GlaArgs& a, int num_cu) {
 }
 
 int launch_gla_mfma(const GlaArgs& a) {
-  static int num_cu = 0;
+  static int num_cu_dev[kMaxDevices] = {};
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return -5;
+  int& num_cu = num_cu_dev[dev];
   if (num_cu == 0) {
-    int dev = 0;
-    hipDeviceProp_t prop;
-    if (hipGetDevice(&dev) != hipSuccess || hipGetDeviceProperties(&prop, dev) != hipSuccess) return -5;
-    num_cu = prop.multiProcessorCount > 0 ? prop.multiProcessorCount : 256;
+    int n = 0;
+    if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess) return -5;
+    num_cu = n > 0 ? n : 256;
   }
-  return a.Dk == 64 ? launch_gla_mfma_t<4>(a, num_cu) : launch_gla_mfma_t<2>(a, num_cu);
+  return a.Dk == 64 ? launch_gla_mfma_t<4>(a, num_cu, dev) : launch_gla_mfma_t<2>(a, num_cu, dev);
 }
 
 #ifdef VIG_TIMING
