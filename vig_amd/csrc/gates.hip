@@ -219,63 +219,71 @@ int launch_locality_gate(const void* o, const float* wt, void* y, int B, int H, 
 // RMS-norm blend epilogue.  One group of Dv/8 lanes owns one (b, l, head) row of
 // Dv values; the two mean-squares are reduced with lane shuffles inside the group.
 //   y[b,l,hd*Dv+d] = rms(o[b,hd,l,:])*w_g*s + rms(local[b,l,hd,:])*w_l*(1-s)
+// One workgroup owns 32 consecutive tokens of one batch element; a thread keeps one channel octet (head, d8) for
+// all its tokens, so the layout arithmetic and the norm weights are set up once per thread.
 // ---------------------------------------------------------------------------
 template <typename T>
 __global__ __launch_bounds__(256) void locality_blend_kernel(const T* __restrict__ o, const T* __restrict__ loc,
                                                               const T* __restrict__ glin,
                                                               const float* __restrict__ wg,
                                                               const float* __restrict__ wl, T* __restrict__ y,
-                                                              int H, int L, int Dv, float eps, int silu_out,
-                                                              size_t nvec) {
-  const int d8n = Dv >> 3;  // lanes per row: 4 (Dv=32) or 8 (Dv=64); power of two
-  // nvec is padded to a multiple of 256 by construction of the grid-stride loop bound below,
-  // so every lane of a row group takes the same trip count and the shuffles are well defined.
-  const size_t nround = (nvec + 255) / 256 * 256;
-  for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < nround; i += (size_t)gridDim.x * 256) {
-    const bool live = i < nvec;
-    const size_t ii = live ? i : nvec - 1;
-    const int d8 = (int)(ii % d8n);
-    const size_t blh = ii / d8n;  // output order: (b*L + l)*H + hd
-    const int hd = (int)(blh % H);
-    const size_t bl = blh / H;
-    const int l = (int)(bl % L);
-    const size_t b = bl / L;
-    float xo[8], xl[8], xg[8];
-    Vec8<T>::load(o + (((b * H + hd) * L + l) * (size_t)Dv + d8 * 8), xo);
-    Vec8<T>::load(loc + ii * 8, xl);
-    Vec8<T>::load(glin + ii * 8, xg);
-    float so = 0.f, sl = 0.f;
+                                                              int H, int L, int Dv, float eps, int silu_out) {
+  const int d8n = Dv >> 3;  // lanes per row: 4 (Dv=32) or 8 (Dv=64); divides 64, so groups never straddle a wave
+  const int nv = H * d8n;   // channel octets per token row
+  const int b = blockIdx.y;
+  const int l0 = blockIdx.x * 32;
+  const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;
+  const float inv_dv = 1.0f / (float)Dv;
+  for (int cv0 = 0; cv0 < nv; cv0 += 64) {
+    const int cv = cv0 + tx;
+    const bool has = cv < nv;  // lanes past the row still take part in the shuffles of their (inactive) group
+    const int cvc = has ? cv : 0;
+    const int hd = cvc / d8n, d8 = cvc - hd * d8n;
+    float w_g[8], w_l[8];
 #pragma unroll
-    for (int j = 0; j < 8; ++j) so += xo[j] * xo[j], sl += xl[j] * xl[j];
-    for (int m = 1; m < d8n; m <<= 1) {
-      so += __shfl_xor(so, m);
-      sl += __shfl_xor(sl, m);
-    }
-    const float ro = rsqrtf(so / (float)Dv + eps);
-    const float rl = rsqrtf(sl / (float)Dv + eps);
-    float out[8];
+    for (int j = 0; j < 8; ++j) w_g[j] = wg[d8 * 8 + j], w_l[j] = wl[d8 * 8 + j];
+    const T* po = o + (((size_t)b * H + hd) * L) * (size_t)Dv + d8 * 8;
+    const size_t row0 = ((size_t)b * L) * (size_t)(nv * 8) + (size_t)cvc * 8;
+    for (int t = ty; t < 32; t += 4) {
+      const int l = l0 + t;
+      if (l >= L) break;  // uniform over the wave: a wave shares its token
+      float xo[8], xl[8], xg[8];
+      const size_t tok = row0 + (size_t)l * (nv * 8);
+      Vec8<T>::load(po + (size_t)l * Dv, xo);
+      Vec8<T>::load(loc + tok, xl);
+      Vec8<T>::load(glin + tok, xg);
+      float so = 0.f, sl = 0.f;
 #pragma unroll
-    for (int j = 0; j < 8; ++j) {
-      const float s = sigmoidf_(xg[j]);
-      float v = xo[j] * ro * wg[d8 * 8 + j] * s + xl[j] * rl * wl[d8 * 8 + j] * (1.f - s);
-      if (silu_out) v = v * sigmoidf_(v);
-      out[j] = v;
+      for (int j = 0; j < 8; ++j) so += xo[j] * xo[j], sl += xl[j] * xl[j];
+      for (int m = 1; m < d8n; m <<= 1) {
+        so += __shfl_xor(so, m);
+        sl += __shfl_xor(sl, m);
+      }
+      const float ro = rsqrtf(so * inv_dv + eps);
+      const float rl = rsqrtf(sl * inv_dv + eps);
+      float out[8];
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        const float s = sigmoidf_(xg[j]);
+        float v = xo[j] * ro * w_g[j] * s + xl[j] * rl * w_l[j] * (1.f - s);
+        if (silu_out) v = v * sigmoidf_(v);
+        out[j] = v;
+      }
+      if (has) Vec8<T>::store(y + tok, out);
     }
-    if (live) Vec8<T>::store(y + ii * 8, out);
   }
 }
 
 int launch_locality_blend(const void* o, const void* loc, const void* glin, const float* wg, const float* wl, void* y,
                           int B, int H, int L, int Dv, float eps, int silu_out, int io_dtype, hipStream_t stream) {
-  const size_t nvec = (size_t)B * L * H * (Dv / 8);
-  const int grid = (int)((nvec + 255) / 256 < 65535 * 8 ? (nvec + 255) / 256 : 65535 * 8);
+  if (B > 65535) return -22;
+  const dim3 grid((L + 31) / 32, B), block(256);
   if (io_dtype == 0)
-    hipLaunchKernelGGL((locality_blend_kernel<float>), dim3(grid), dim3(256), 0, stream, (const float*)o,
-                       (const float*)loc, (const float*)glin, wg, wl, (float*)y, H, L, Dv, eps, silu_out, nvec);
+    hipLaunchKernelGGL((locality_blend_kernel<float>), grid, block, 0, stream, (const float*)o, (const float*)loc,
+                       (const float*)glin, wg, wl, (float*)y, H, L, Dv, eps, silu_out);
   else
-    hipLaunchKernelGGL((locality_blend_kernel<uint16_t>), dim3(grid), dim3(256), 0, stream, (const uint16_t*)o,
-                       (const uint16_t*)loc, (const uint16_t*)glin, wg, wl, (uint16_t*)y, H, L, Dv, eps, silu_out,
-                       nvec);
+    hipLaunchKernelGGL((locality_blend_kernel<uint16_t>), grid, block, 0, stream, (const uint16_t*)o,
+                       (const uint16_t*)loc, (const uint16_t*)glin, wg, wl, (uint16_t*)y, H, L, Dv, eps, silu_out);
   return hipGetLastError() == hipSuccess ? 0 : -5;
 }
 
