@@ -107,41 +107,42 @@ int launch_dirgate(const void* in, void* out, int B, int L, int H, int Dk, float
 
 // ---------------------------------------------------------------------------
 // 3x3 depthwise stencil on the token grid, channels-last.  One workgroup owns one image (or one head slab), a
-// group of 64 channels and a band of grid rows: it stages the band plus one halo row on each side in LDS with
-// coalesced 16-byte loads (every input byte leaves L2 once), then thread = (channel octet, token lane) keeps the 8x9
-// weights of its channels in registers and walks the band's tokens lane, lane+32, ...; the nine taps are 16-byte LDS
-// reads (a wave reads 8 consecutive tokens x 128 B: conflict-free).
+// group of 64 channels and a band of grid rows: it stages the band plus a one-cell halo all around in LDS, with
+// zeros where the halo leaves the grid (coalesced 16-byte loads, every input byte leaves L2 once, and no tap needs a
+// bounds check or a clamped address).  Thread = (channel octet, token lane) keeps the 8x9 weights of its channels
+// in registers and walks the band's tokens lane, lane+32, ...
 //   GATE = false:  y = conv(x) (+bias) (SiLU optional)          x, y [N, h*w, C] with row stride `stride` elements
 //   GATE = true :  y = x * sigmoid(conv(x))                      (bias / SiLU unused)
 // weights [Ctot, 9] f32.
 // ---------------------------------------------------------------------------
+constexpr int kStencilGroup = 64;  // channels per workgroup
+
 template <typename T, bool GATE>
 __global__ __launch_bounds__(256) void stencil3x3_kernel(const T* __restrict__ x, const float* __restrict__ wt,
                                                           const float* __restrict__ bias, T* __restrict__ y, int h, int w,
                                                           int stride, int groups_per_image, int wmod, int cgroup,
                                                           int band_rows, int silu) {
   extern __shared__ __align__(16) char smem[];
-  T* tile = reinterpret_cast<T*>(smem);  // [(band_rows + 2) * w][64]
+  T* tile = reinterpret_cast<T*>(smem);  // [(band_rows + 2) * (w + 2)][64]
   const int oct = threadIdx.x & 7, tl = threadIdx.x >> 3;  // 8 octets x 32 token lanes
   const int img = blockIdx.x / groups_per_image, grp = blockIdx.x % groups_per_image;
-  const int r0 = blockIdx.y * band_rows;                   // first output row of the band
+  const int r0 = blockIdx.y * band_rows;  // first output row of the band
   const int r1 = min(r0 + band_rows, h);
-  const int s0 = max(r0 - 1, 0), s1 = min(r1 + 1, h);      // staged rows [s0, s1)
-  const int L = h * w;
-  const bool ch_ok = grp * 64 + oct * 8 < cgroup;          // channel tail of the last group
-  const size_t base = (size_t)img * L * stride + (size_t)grp * 64 + oct * 8;
-  // ---- stage ----
-  const int ntok = (s1 - s0) * w;
-  for (int t = tl; t < ntok; t += 32) {
-    float xv[8];
-    if (ch_ok) {
-      Vec8<T>::load(x + base + (size_t)(s0 * w + t) * stride, xv);
-      Vec8<T>::store(tile + t * 64 + oct * 8, xv);
-    }
+  const int L = h * w, pw = w + 2;
+  const bool ch_ok = grp * kStencilGroup + oct * 8 < cgroup;  // channel tail of the last group
+  const size_t base = (size_t)img * L * stride + (size_t)grp * kStencilGroup + oct * 8;
+  // ---- stage padded cells (pr, pc) <-> grid (r0 - 1 + pr, pc - 1) ----
+  const int ncell = (r1 - r0 + 2) * pw;
+  for (int t = tl; t < ncell; t += 32) {
+    const int pr = t / pw, pc = t - pr * pw;
+    const int r = r0 - 1 + pr, c = pc - 1;
+    float xv[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+    if (ch_ok && r >= 0 && r < h && c >= 0 && c < w) Vec8<T>::load(x + base + (size_t)(r * w + c) * stride, xv);
+    Vec8<T>::store(tile + t * kStencilGroup + oct * 8, xv);
   }
   __syncthreads();
   if (!ch_ok) return;
-  const int wch = (blockIdx.x % wmod) * (GATE ? cgroup : 64) + oct * 8;  // first weight channel of this thread
+  const int wch = (blockIdx.x / groups_per_image % wmod) * cgroup + grp * kStencilGroup + oct * 8;  // first weight channel
   float wreg[8][9];
 #pragma unroll
   for (int j = 0; j < 8; ++j)
@@ -152,23 +153,20 @@ __global__ __launch_bounds__(256) void stencil3x3_kernel(const T* __restrict__ x
   for (int j = 0; j < 8; ++j) breg[j] = (!GATE && bias) ? bias[wch + j] : 0.f;
   const int nout = (r1 - r0) * w;
   for (int t = tl; t < nout; t += 32) {
-    const int r = r0 + t / w, c = t % w;
+    const int rl = t / w, c = t - rl * w;
+    const T* p = tile + (rl * pw + c) * kStencilGroup + oct * 8;  // padded cell of tap (-1, -1)
     float acc[8], ctr[8];
 #pragma unroll
     for (int j = 0; j < 8; ++j) acc[j] = breg[j], ctr[j] = 0.f;
 #pragma unroll
-    for (int di = -1; di <= 1; ++di) {
+    for (int di = 0; di < 3; ++di) {
 #pragma unroll
-      for (int dj = -1; dj <= 1; ++dj) {
-        // unconditional read of a clamped neighbour; taps outside the grid are zeroed by select (zero padding)
-        const int rr = r + di, cc = c + dj;
-        const bool in = rr >= 0 && rr < h && cc >= 0 && cc < w;
-        const int rc = min(max(rr, s0), s1 - 1), ccl = min(max(cc, 0), w - 1);
+      for (int dj = 0; dj < 3; ++dj) {
         float xv[8];
-        Vec8<T>::load(tile + ((rc - s0) * w + ccl) * 64 + oct * 8, xv);
+        Vec8<T>::load(p + (di * pw + dj) * kStencilGroup, xv);
 #pragma unroll
-        for (int j = 0; j < 8; ++j) acc[j] += (in ? xv[j] : 0.f) * wreg[j][(di + 1) * 3 + (dj + 1)];
-        if (GATE && di == 0 && dj == 0) {
+        for (int j = 0; j < 8; ++j) acc[j] = __builtin_fmaf(xv[j], wreg[j][di * 3 + dj], acc[j]);
+        if (GATE && di == 1 && dj == 1) {
 #pragma unroll
           for (int j = 0; j < 8; ++j) ctr[j] = xv[j];
         }
@@ -181,19 +179,20 @@ __global__ __launch_bounds__(256) void stencil3x3_kernel(const T* __restrict__ x
 #pragma unroll
       for (int j = 0; j < 8; ++j) acc[j] = acc[j] * sigmoidf_(acc[j]);
     }
-    Vec8<T>::store(y + base + (size_t)(r * w + c) * stride, acc);
+    Vec8<T>::store(y + base + (size_t)((r0 + rl) * w + c) * stride, acc);
   }
 }
 
 template <typename T, bool GATE>
 static int launch_stencil(const void* x, const float* wt, const float* bias, void* y, int images, int h, int w,
-                          int stride, int groups, int wmod, int cgroup, int silu, hipStream_t stream) {
-  // rows per band so that (band + 2 halo rows) x w tokens x 64 channels fit 48 KB of LDS
-  const int row_bytes = w * 64 * (int)sizeof(T);
+                          int stride, int wmod, int cgroup, int silu, hipStream_t stream) {
+  // rows per band so that (band + 2) x (w + 2) padded cells x 64 channels fit 48 KB of LDS
+  const int row_bytes = (w + 2) * kStencilGroup * (int)sizeof(T);
   int band = 48 * 1024 / row_bytes - 2;
   if (band < 1) return -95;
   if (band > h) band = h;
   const int nband = (h + band - 1) / band;
+  const int groups = (cgroup + kStencilGroup - 1) / kStencilGroup;
   const size_t lds = (size_t)(band + 2) * row_bytes;
   hipLaunchKernelGGL((stencil3x3_kernel<T, GATE>), dim3(images * groups, nband), dim3(256), lds, stream, (const T*)x, wt,
                      bias, (T*)y, h, w, stride, groups, wmod, cgroup, band, silu);
@@ -202,17 +201,17 @@ static int launch_stencil(const void* x, const float* wt, const float* bias, voi
 
 int launch_dwconv3x3(const void* x, const float* wt, const float* bias, void* y, int B, int h, int w, int C,
                      int silu, int io_dtype, hipStream_t stream) {
-  const int groups = (C + 63) / 64;
-  if (io_dtype == 0) return launch_stencil<float, false>(x, wt, bias, y, B, h, w, C, groups, groups, C, silu, stream);
-  return launch_stencil<uint16_t, false>(x, wt, bias, y, B, h, w, C, groups, groups, C, silu, stream);
+  // every batch element is an image of C channels; all images share the C weight channels
+  if (io_dtype == 0) return launch_stencil<float, false>(x, wt, bias, y, B, h, w, C, 1, C, silu, stream);
+  return launch_stencil<uint16_t, false>(x, wt, bias, y, B, h, w, C, 1, C, silu, stream);
 }
 
 int launch_locality_gate(const void* o, const float* wt, void* y, int B, int H, int h, int w, int Dv, int io_dtype,
                          hipStream_t stream) {
   if (Dv > 64) return -95;
   // every (batch, head) slab is an "image" of Dv channels; head hd uses weight channels [hd*Dv, hd*Dv + Dv)
-  if (io_dtype == 0) return launch_stencil<float, true>(o, wt, nullptr, y, B * H, h, w, Dv, 1, H, Dv, 0, stream);
-  return launch_stencil<uint16_t, true>(o, wt, nullptr, y, B * H, h, w, Dv, 1, H, Dv, 0, stream);
+  if (io_dtype == 0) return launch_stencil<float, true>(o, wt, nullptr, y, B * H, h, w, Dv, H, Dv, 0, stream);
+  return launch_stencil<uint16_t, true>(o, wt, nullptr, y, B * H, h, w, Dv, H, Dv, 0, stream);
 }
 
 // ---------------------------------------------------------------------------
