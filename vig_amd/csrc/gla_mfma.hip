@@ -344,13 +344,21 @@ struct ChunkSrc {
   rsrc_t q, k, v, g;
 };
 
-template <bool FWD, bool WITH_Q, int NG>
-__device__ __forceinline__ void issue_first_phase(const ChunkSrc& src, int r, int h, Prefetch<NG>& pf) {
-  constexpr int TA = FWD ? 0 : 1;
+template <int NG>
+__device__ __forceinline__ void issue_gates(const ChunkSrc& src, int r, int h, Prefetch<NG>& pf) {
   issue_tdwords<0, 4, NG>(src.g, r, h, pf.gD);
+}
+template <bool FWD, bool WITH_Q, int NG>
+__device__ __forceinline__ void issue_rows(const ChunkSrc& src, int r, int h, Prefetch<NG>& pf) {
+  constexpr int TA = FWD ? 0 : 1;
   issue_raw_tile<NG>(src.k, TA, r, h, pf.rawk);
   if (WITH_Q) issue_raw_tile<NG>(src.q, TA, r, h, pf.rawq);
   issue_tdwords<2 * TA, 2, 4>(src.v, r, h, pf.vD);
+}
+template <bool FWD, bool WITH_Q, int NG>
+__device__ __forceinline__ void issue_first_phase(const ChunkSrc& src, int r, int h, Prefetch<NG>& pf) {
+  issue_gates<NG>(src, r, h, pf);
+  issue_rows<FWD, WITH_Q, NG>(src, r, h, pf);
 }
 
 // Segment modes of the kernel.  A sequence longer than 256 tokens is cut into segments of <= 256 tokens that are
@@ -470,7 +478,7 @@ __device__ __forceinline__ bool direction_wave(const ChunkSrc& cur, const ChunkS
   char* region = lds + wi * kRegionBytes;
   uint16_t* kt = reinterpret_cast<uint16_t*>(region);
   float* dvec_all = reinterpret_cast<float*>(lds + kLdsDvec);
-  if (!FWD) issue_first_phase<FWD, OUT, NG>(cur, r, h, pf);
+  if (!FWD) issue_rows<FWD, OUT, NG>(cur, r, h, pf);
   VIG_STAMP(0);
 
   // ---- cumulative log-gates G[it][p] via triangular-ones MFMA on transposed gate fragments ----
@@ -573,10 +581,12 @@ __device__ __forceinline__ bool direction_wave(const ChunkSrc& cur, const ChunkS
           }
     }
   }
-  // ---- forward waves fetch the first phase of the NEXT segment here, reverse waves fetch theirs at the top of the
-  // segment: a wave stalls while the memory pipe accepts its loads, and this way the other wave of the SIMD has math
-  // to do.  (Always issued: after the last segment its descriptors are empty, which keeps branches off the loads.) ----
+  // ---- forward waves fetch the whole first phase of the NEXT segment here; reverse waves fetch only its gate
+  // dwords (needed first) here and the rows at the top of the segment: a wave stalls while the memory pipe accepts
+  // its loads, and this way the other wave of the SIMD has math to do.  (Always issued: after the last segment the
+  // descriptors are empty, which keeps branches off the loads.) ----
   if (FWD) issue_first_phase<FWD, OUT, NG>(nxt, r, h, pf);
+  else issue_gates<NG>(nxt, r, h, pf);
   VIG_STAMP(5);
   // lane-derived addresses of the exchange phases are rebuilt here instead of being carried (and spilled) across
   // the register-heavy tile phase
@@ -750,7 +760,10 @@ __device__ __forceinline__ int wave_loop(const uint16_t* q, const uint16_t* k, c
   ChunkSrc cur;
   rsrc_t dst;
   locate(item, cur, dst);
-  if (FWD && item < geo.nitems) issue_first_phase<FWD, OUT, NG>(cur, lane & 31, lane >> 5, pf);
+  if (item < geo.nitems) {
+    if (FWD) issue_first_phase<FWD, OUT, NG>(cur, lane & 31, lane >> 5, pf);
+    else issue_gates<NG>(cur, lane & 31, lane >> 5, pf);
+  }
   int iter = 0;
   for (; item < geo.nitems; item += gridDim.x, ++iter) {
     ChunkSrc nxt;
