@@ -92,14 +92,9 @@ def model_throughput(dev, batch=256, warmup=10, iters=30, tune_gemm=True):
     torch.manual_seed(0)
     model = layers.vig_small().eval().to(dev, torch.bfloat16)
     images = torch.randn(batch, 3, 224, 224, device=dev, dtype=torch.bfloat16)
-    for _ in range(warmup):
-        model(images)
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for _ in range(iters):
-        model(images)
-    torch.cuda.synchronize()
-    dt = time.perf_counter() - t0
+    from vig_amd import evaluate
+    ips = evaluate.throughput(model, images, warmup=warmup, iters=iters)
+    dt = iters * batch / ips
     return {"images_per_s": iters * batch / dt, "batch": batch, "dtype": "bf16", "iters": iters,
             "ms_per_forward": dt / iters * 1e3, "gemm_solution_tuning": "torch.cuda.tunable" if tuned else None}
 

@@ -75,3 +75,37 @@ def test_vig_small_logits(dtype, tol):
     print(f"  logits max-rel err {err:.3e}  (max |logit| {np.abs(want).max():.3f})", flush=True)
     assert got.shape == (2, 1000)
     assert err <= tol
+
+
+def test_evaluate_callers(tmp_path):
+    """Checkpoint round trip (reference layout: weights under 'model'), accuracy, validate and throughput loops."""
+    import torch
+    from vig_amd import evaluate, layers
+
+    announce("evaluate: load_checkpoint / accuracy / validate / throughput on a tiny ViG")
+    torch.manual_seed(0)
+    kw = dict(img_size=64, depth=2, num_heads=3, embed_dim=96, num_classes=10)
+    src = layers.ViG(**kw).eval()
+    path = str(tmp_path / "ckpt.pth")
+    torch.save({"model": src.state_dict(), "epoch": 3}, path)
+    dst = layers.ViG(**kw).eval()
+    res = evaluate.load_checkpoint(dst, path)
+    assert not res.missing_keys and not res.unexpected_keys
+    for (ka, a), (kb, b) in zip(src.state_dict().items(), dst.state_dict().items()):
+        assert ka == kb and torch.equal(a, b)
+    # a position table of another grid is resized
+    big = layers.ViG(**{**kw, "img_size": 96}).eval()
+    evaluate.load_checkpoint(big, path)
+    assert big.pos_embed.shape == (1, 36, 96)
+
+    logits = torch.tensor([[0.1, 0.9, 0.0, 0.2, 0.3, 0.05], [0.8, 0.1, 0.0, 0.7, 0.6, 0.5], [0.0, 0.1, 0.2, 0.3, 0.4, 0.9]])
+    a1, a5 = evaluate.accuracy(logits, torch.tensor([1, 3, 0]), topk=(1, 5))
+    assert abs(a1.item() - 100.0 / 3) < 1e-4 and abs(a5.item() - 200.0 / 3) < 1e-4
+
+    dst = dst.cuda().to(torch.bfloat16)
+    g = torch.Generator().manual_seed(1)
+    loader = [(torch.randn(4, 3, 64, 64, generator=g), torch.randint(0, 10, (4,), generator=g)) for _ in range(3)]
+    acc1, acc5, loss = evaluate.validate(dst, loader)
+    assert 0.0 <= acc1 <= acc5 <= 100.0 and loss > 0
+    ips = evaluate.throughput(dst, loader[0][0].cuda().to(torch.bfloat16), warmup=2, iters=3)
+    assert ips > 0

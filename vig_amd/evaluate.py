@@ -1,0 +1,77 @@
+"""Evaluation-side callers of the ViG shell: checkpoint loading, top-k accuracy, validation and throughput loops.
+
+Own code with the behaviour of classification/main.py:341-406 (validate, throughput) and of timm's `accuracy`
+as used there; one process, one GPU (no reduce over ranks).  Forward only.
+"""
+from __future__ import annotations
+
+import time
+from typing import Iterable, Tuple
+
+import torch
+import torch.nn.functional as F
+
+from .layers import resize_pos_embed
+
+
+def load_checkpoint(model: torch.nn.Module, path: str, strict: bool = True):
+    """Loads a reference checkpoint (classification/utils/utils.py:22-24: the weights sit under 'model') or a bare
+    state_dict.  Tensors only (`weights_only=True`).  A position table of another grid is resized bicubically
+    (classification/models/vig.py:915-958) when the model knows its patch grid."""
+    blob = torch.load(path, map_location="cpu", weights_only=True)
+    state = blob["model"] if isinstance(blob, dict) and "model" in blob and isinstance(blob["model"], dict) else blob
+    state = dict(state)
+    own = model.state_dict()
+    if "pos_embed" in state and "pos_embed" in own and state["pos_embed"].shape != own["pos_embed"].shape:
+        n_src = state["pos_embed"].shape[1]
+        side = int(round(n_src ** 0.5))
+        if side * side != n_src or not hasattr(model, "patch_resolution"):
+            raise ValueError("cannot resize pos_embed: source grid is not square or the model has no patch_resolution")
+        state["pos_embed"] = resize_pos_embed(state["pos_embed"], (side, side), tuple(model.patch_resolution))
+    return model.load_state_dict(state, strict=strict)
+
+
+def accuracy(output: torch.Tensor, target: torch.Tensor, topk: Tuple[int, ...] = (1,)):
+    """Top-k accuracies in percent over a batch of logits."""
+    maxk = min(max(topk), output.shape[1])
+    _, pred = output.topk(maxk, dim=1, largest=True, sorted=True)
+    correct = pred.eq(target.reshape(-1, 1))
+    n = target.shape[0]
+    return [correct[:, :min(k, maxk)].any(dim=1).float().sum() * (100.0 / n) for k in topk]
+
+
+@torch.no_grad()
+def validate(model: torch.nn.Module, data_loader: Iterable, dtype: torch.dtype = torch.bfloat16):
+    """Weighted averages of top-1, top-5 and cross-entropy over a loader of (images, target) batches
+    (classification/main.py:341-385).  Images are cast to `dtype`; the loss is taken on fp32 logits."""
+    model.eval()
+    dev = next(model.parameters()).device
+    n_total, acc1_sum, acc5_sum, loss_sum = 0, 0.0, 0.0, 0.0
+    for images, target in data_loader:
+        images = images.to(dev, dtype, non_blocking=True)
+        target = target.to(dev, non_blocking=True)
+        logits = model(images).float()
+        a1, a5 = accuracy(logits, target, topk=(1, 5))
+        n = target.shape[0]
+        n_total += n
+        acc1_sum += a1.item() * n
+        acc5_sum += a5.item() * n
+        loss_sum += F.cross_entropy(logits, target).item() * n
+    if n_total == 0:
+        raise ValueError("empty data loader")
+    return acc1_sum / n_total, acc5_sum / n_total, loss_sum / n_total
+
+
+@torch.no_grad()
+def throughput(model: torch.nn.Module, images: torch.Tensor, warmup: int = 50, iters: int = 30) -> float:
+    """Images per second of repeated forwards of one resident batch: `warmup` untimed and `iters` timed forwards
+    between synchronisations (classification/main.py:388-406)."""
+    model.eval()
+    for _ in range(warmup):
+        model(images)
+    torch.cuda.synchronize(images.device)
+    t0 = time.perf_counter()
+    for _ in range(iters):
+        model(images)
+    torch.cuda.synchronize(images.device)
+    return iters * images.shape[0] / (time.perf_counter() - t0)
