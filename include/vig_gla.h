@@ -87,6 +87,27 @@ int vig_gla_bidir_fwd_exact(const void* q, const void* k, const void* v,
                             int io_dtype, int gate_dtype, void* stream);
 
 /*
+ * Backward of vig_gla_bidir_fwd: given d_o = dL/do [B, H, L, Dv], writes
+ *   dq, dk [B, H, L, Dk], dv [B, H, L, Dv] (summed over the directions) in io_dtype and
+ *   dg_fwd, dg_bwd [B, H, L, Dk] in gate_dtype (dg_bwd only when g_bwd != NULL).
+ * fp32 arithmetic, token-recurrent.  `workspace` must hold vig_gla_bidir_bwd_workspace(...) bytes.
+ * Built shapes: (Dk, Dv) in {(16,32), (32,32), (32,64), (64,32), (64,64)}, any L >= 1.
+ *
+ * Replaces: FusedChunkGLAFunction.backward (flash-linear-attention/fla/ops/gla/chunk_fuse.py:413-518; gate
+ * gradient :505-518) under the flip-concat glue of classification/models/vig.py:407-426, for both directions in
+ * natural token order.
+ */
+int vig_gla_bidir_bwd(const void* q, const void* k, const void* v,
+                      const void* g_fwd, const void* g_bwd, const void* d_o,
+                      void* dq, void* dk, void* dv, void* dg_fwd, void* dg_bwd,
+                      void* workspace, size_t workspace_bytes,
+                      int B, int H, int L, int Dk, int Dv,
+                      float scale, float out_scale,
+                      int io_dtype, int gate_dtype, void* stream);
+
+size_t vig_gla_bidir_bwd_workspace(int B, int H, int L, int Dk, int Dv, int bidirectional);
+
+/*
  * Direction-wise gate preparation.
  *   gk_lin [B, L, 2*H*Dk]  ->  g_out [2, B, H, L, Dk]
  *   g_out[dir,b,h,l,d] = max(logsigmoid(gk_lin[b,l,dir*H*Dk + h*Dk + d]) * inv_normalizer, clamp_min)

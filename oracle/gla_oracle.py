@@ -88,6 +88,60 @@ def bidir_gla_recurrent(q, k, v, g_fwd, g_bwd, scale=None, out_scale=1.0):
     return out_scale * (of + ob)
 
 
+def gla_recurrent_backward(q, k, v, g, do, scale=None, reverse=False):
+    """Gradients of gla_recurrent's output contracted with `do`, float64, by the adjoint recurrences.
+
+    Same derivatives as the reference's chunked backward (fla/ops/gla/chunk_fuse.py:413-518 with the
+    gate gradient of :505-518, `dg = q*dq - k*dk` followed by a reversed cumulative sum), written per token:
+        dS_t = (scale*q_t) do_t^T + diag(exp(g_{t'})) dS_{t'}      (t' = the token walked after t)
+        dq_t = scale * S_t do_t ;  dk_t = dS_t v_t ;  dv_t = dS_t^T k_t
+        dG_t = q_t*dq_t - k_t*dk_t ;  dg_t = sum of dG over t and every token walked after it.
+    Returns dq, dk, dv, dg with the shapes of q, k, v, g.
+    """
+    q = np.asarray(q, dtype=np.float64)
+    k = np.asarray(k, dtype=np.float64)
+    v = np.asarray(v, dtype=np.float64)
+    g = np.asarray(g, dtype=np.float64)
+    do = np.asarray(do, dtype=np.float64)
+    B, H, L, Dk = q.shape
+    Dv = v.shape[-1]
+    if scale is None or scale == -1:
+        scale = Dk ** -0.5
+    a = np.exp(g)
+    order = list(range(L - 1, -1, -1) if reverse else range(L))
+    dq = np.zeros_like(q)
+    S = np.zeros((B, H, Dk, Dv))
+    for t in order:
+        S = S * a[:, :, t, :, None] + k[:, :, t, :, None] * v[:, :, t, None, :]
+        dq[:, :, t] = scale * np.einsum("bhkv,bhv->bhk", S, do[:, :, t])
+    dk = np.zeros_like(k)
+    dv = np.zeros_like(v)
+    dg = np.zeros_like(g)
+    dS = np.zeros((B, H, Dk, Dv))
+    run = np.zeros((B, H, Dk))
+    prev = None
+    for t in reversed(order):
+        if prev is not None:
+            dS = dS * a[:, :, prev, :, None]
+        dS = dS + scale * q[:, :, t, :, None] * do[:, :, t, None, :]
+        dk[:, :, t] = np.einsum("bhkv,bhv->bhk", dS, v[:, :, t])
+        dv[:, :, t] = np.einsum("bhkv,bhk->bhv", dS, k[:, :, t])
+        run = run + q[:, :, t] * dq[:, :, t] - k[:, :, t] * dk[:, :, t]
+        dg[:, :, t] = run
+        prev = t
+    return dq, dk, dv, dg
+
+
+def bidir_gla_backward(q, k, v, g_fwd, g_bwd, do, scale=None, out_scale=1.0):
+    """Gradients of bidir_gla_recurrent: (dq, dk, dv, dg_fwd, dg_bwd); dq, dk, dv are summed over the directions."""
+    do = out_scale * np.asarray(do, dtype=np.float64)
+    fq, fk, fv, fg = gla_recurrent_backward(q, k, v, g_fwd, do, scale=scale, reverse=False)
+    if g_bwd is None:
+        return fq, fk, fv, fg, None
+    bq, bk, bv, bg = gla_recurrent_backward(q, k, v, g_bwd, do, scale=scale, reverse=True)
+    return fq + bq, fk + bk, fv + bv, fg, bg
+
+
 def gla_parallel(q, k, v, g, scale=None, reverse=False):
     """Quadratic ("parallel") form, derived independently of the recurrence.
 

@@ -1,0 +1,92 @@
+"""GPU parity of the backward of the bidirectional GLA op (through the C ABI and through autograd) against the
+fp64 oracle's adjoint recurrences (themselves pinned by finite differences and autograd in tests/test_oracle.py)."""
+import numpy as np
+import pytest
+import torch
+
+import vig_amd
+from oracle import gla_oracle as O
+from vig_amd.synthetic import make_gla_inputs
+
+from .util import announce, f64
+
+pytestmark = pytest.mark.gpu
+
+
+def _do(shape, seed, dtype):
+    g = torch.Generator(device="cpu").manual_seed(seed)
+    return torch.randn(*shape, generator=g).to(dtype)
+
+
+def _rel(got, want, floor=0.0):
+    """max|got - want| over the larger of max|want| and `floor`.  The gate gradient is a difference of two terms
+    (q*dq - k*dk) that can cancel exactly (L = 1), so it is measured against the size of those terms."""
+    return float(np.abs(got - want).max() / max(np.abs(want).max(), floor, 1e-30))
+
+
+def _check_all(got, want, q, tol=1e-4):
+    floor = float(np.abs(f64(q) * want[0]).max())
+    for name, g_, w_ in zip(("dq", "dk", "dv", "dg_fwd", "dg_bwd"), got, want):
+        if w_ is None:
+            assert g_ is None
+            continue
+        assert _rel(f64(g_), w_, floor if name.startswith("dg") else 0.0) <= tol, name
+
+
+@pytest.mark.parametrize("L", [1, 2, 15, 16, 17, 64, 196, 300])
+def test_backward_fp32_ragged_lengths(L):
+    announce(f"backward fp32 L={L}")
+    q, k, v, gf, gb = make_gla_inputs(2, 2, L, 64, 64, seed=300 + L)
+    do = _do(v.shape, 7, torch.float32)
+    want = O.bidir_gla_backward(f64(q), f64(k), f64(v), f64(gf), f64(gb), f64(do), out_scale=0.5)
+    got = vig_amd.gla_bidir_backward(*(t.cuda() for t in (q, k, v, gf, gb, do)), out_scale=0.5)
+    _check_all(got, want, q)
+
+
+@pytest.mark.parametrize("Dk,Dv", [(16, 32), (32, 32), (32, 64), (64, 32)])
+def test_backward_fp32_head_dims_and_causal(Dk, Dv):
+    announce(f"backward fp32 Dk={Dk} Dv={Dv}, causal only")
+    q, k, v, gf, _ = make_gla_inputs(1, 3, 50, Dk, Dv, seed=9, gate_scale=0.5)
+    do = _do(v.shape, 8, torch.float32)
+    want = O.bidir_gla_backward(f64(q), f64(k), f64(v), f64(gf), None, f64(do))
+    got = vig_amd.gla_bidir_backward(q.cuda(), k.cuda(), v.cuda(), gf.cuda(), None, do.cuda())
+    _check_all(got, want, q)
+
+
+def test_backward_bf16_io():
+    """bf16 tensors and gates, fp32 arithmetic inside: every gradient within half an output ulp (2^-8 relative,
+    elementwise, plus a small absolute floor) of the oracle on the same bf16-rounded inputs."""
+    announce("backward bf16 io, ViG-S head shape")
+    q, k, v, gf, gb = make_gla_inputs(2, 3, 196, 32, 64, seed=12, dtype=torch.bfloat16)
+    do = _do(v.shape, 9, torch.bfloat16)
+    want = O.bidir_gla_backward(f64(q), f64(k), f64(v), f64(gf), f64(gb), f64(do), out_scale=0.25)
+    got = vig_amd.gla_bidir_backward(*(t.cuda() for t in (q, k, v, gf, gb, do)), out_scale=0.25)
+    for name, g_, w_ in zip(("dq", "dk", "dv", "dg_fwd", "dg_bwd"), got, want):
+        err = np.abs(f64(g_) - w_)
+        assert np.all(err <= 2.0 ** -8 * np.abs(w_) + 1e-3 * np.abs(w_).max()), name
+
+
+def test_autograd_through_the_wrappers():
+    """loss.backward() through batch_bid_fused_chunk_gla (gates as one [2B,...] tensor) and fused_chunk_gla."""
+    announce("autograd through the op wrappers")
+    q, k, v, gf, gb = make_gla_inputs(2, 2, 70, 32, 64, seed=21)
+    do = _do(v.shape, 10, torch.float32)
+    tq, tk, tv = (t.cuda().requires_grad_(True) for t in (q, k, v))
+    tg = torch.cat([gf, gb], 0).cuda().requires_grad_(True)
+    o, _ = vig_amd.batch_bid_fused_chunk_gla(tq, tk, tv, tg)
+    assert o.requires_grad
+    (o * do.cuda()).sum().backward()
+    want = O.bidir_gla_backward(f64(q), f64(k), f64(v), f64(gf), f64(gb), f64(do), out_scale=0.5)
+    assert _rel(f64(tq.grad), want[0]) <= 1e-4 and _rel(f64(tk.grad), want[1]) <= 1e-4
+    assert _rel(f64(tv.grad), want[2]) <= 1e-4
+    assert _rel(f64(tg.grad[:2]), want[3]) <= 1e-4 and _rel(f64(tg.grad[2:]), want[4]) <= 1e-4
+    # forward value of the recorded call equals the plain call
+    with torch.no_grad():
+        o2, _ = vig_amd.batch_bid_fused_chunk_gla(tq, tk, tv, tg)
+    assert torch.equal(o.detach(), o2)
+    # causal wrapper
+    tq2 = q.cuda().requires_grad_(True)
+    o3, _ = vig_amd.fused_chunk_gla(tq2, k.cuda(), v.cuda(), gf.cuda())
+    (o3 * do.cuda()).sum().backward()
+    want = O.bidir_gla_backward(f64(q), f64(k), f64(v), f64(gf), None, f64(do))
+    assert _rel(f64(tq2.grad), want[0]) <= 1e-4

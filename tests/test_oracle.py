@@ -236,3 +236,50 @@ def test_block_row_ops_against_library_routines():
     np.testing.assert_array_equal(q, tq.reshape(2, 5, 3, 4).permute(0, 2, 1, 3).numpy())
     np.testing.assert_array_equal(k, tk.reshape(2, 5, 3, 4).permute(0, 2, 1, 3).numpy())
     np.testing.assert_array_equal(v, tv.reshape(2, 5, 3, 8).permute(0, 2, 1, 3).numpy())
+
+
+def test_backward_against_finite_differences_and_autograd():
+    """The adjoint recurrences against (i) central differences of the pinned forward oracle and (ii) torch autograd
+    through an independently written float64 quadratic form."""
+    import torch
+
+    rng = np.random.default_rng(11)
+    B, H, L, Dk, Dv = 1, 2, 7, 4, 3
+    q, k = rng.standard_normal((B, H, L, Dk)), rng.standard_normal((B, H, L, Dk))
+    v, do = rng.standard_normal((B, H, L, Dv)), rng.standard_normal((B, H, L, Dv))
+    gf = -np.abs(rng.standard_normal((B, H, L, Dk))) * 0.3
+    gb = -np.abs(rng.standard_normal((B, H, L, Dk))) * 0.3
+    dq, dk, dv, dgf, dgb = O.bidir_gla_backward(q, k, v, gf, gb, do, out_scale=0.5)
+
+    def loss(q_, k_, v_, gf_, gb_):
+        return float((O.bidir_gla_recurrent(q_, k_, v_, gf_, gb_, out_scale=0.5) * do).sum())
+
+    args = [q, k, v, gf, gb]
+    for which, grad in enumerate((dq, dk, dv, dgf, dgb)):
+        num = np.zeros_like(grad)
+        it = np.nditer(args[which], flags=["multi_index"])
+        for _ in it:
+            i = it.multi_index
+            hi = [a.copy() for a in args]
+            lo = [a.copy() for a in args]
+            hi[which][i] += 1e-6
+            lo[which][i] -= 1e-6
+            num[i] = (loss(*hi) - loss(*lo)) / 2e-6
+        np.testing.assert_allclose(grad, num, rtol=1e-6, atol=1e-8)
+
+    # autograd through a quadratic form written with torch primitives
+    tq, tk, tv, tgf, tgb = (torch.tensor(a, requires_grad=True) for a in args)
+
+    def direction(tg, reverse):
+        G = torch.flip(torch.cumsum(torch.flip(tg, [2]), 2), [2]) if reverse else torch.cumsum(tg, 2)
+        E = G[:, :, :, None, :] - G[:, :, None, :, :]
+        idx = torch.arange(L)
+        keep = (idx[None, :] >= idx[:, None]) if reverse else (idx[None, :] <= idx[:, None])
+        W = torch.where(keep[None, None, :, :, None], torch.exp(torch.where(keep[None, None, :, :, None], E, torch.zeros_like(E))), torch.zeros_like(E))
+        A = (Dk ** -0.5) * torch.einsum("bhid,bhjd,bhijd->bhij", tq, tk, W)
+        return torch.einsum("bhij,bhjv->bhiv", A, tv)
+
+    out = 0.5 * (direction(tgf, False) + direction(tgb, True))
+    (out * torch.tensor(do)).sum().backward()
+    for grad, t in zip((dq, dk, dv, dgf, dgb), (tq, tk, tv, tgf, tgb)):
+        np.testing.assert_allclose(grad, t.grad.numpy(), rtol=1e-10, atol=1e-12)

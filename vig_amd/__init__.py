@@ -12,6 +12,7 @@ from .ops import (  # noqa: F401
     dwconv3x3,
     fused_chunk_gla,
     fused_recurrent_gla,
+    gla_bidir_backward,
     gla_bidir_forward,
     locality_blend,
     locality_gate,
@@ -22,5 +23,5 @@ from .ops import (  # noqa: F401
 
 __all__ = [
     "batch_bid_fused_chunk_gla", "bid_fused_recurrent_gla", "dirgate", "dwconv3x3", "fused_chunk_gla",
-    "fused_recurrent_gla", "gla_bidir_forward", "locality_blend", "locality_gate", "rmsnorm", "split_heads", "swiglu",
+    "fused_recurrent_gla", "gla_bidir_backward", "gla_bidir_forward", "locality_blend", "locality_gate", "rmsnorm", "split_heads", "swiglu",
 ]

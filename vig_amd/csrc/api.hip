@@ -17,6 +17,11 @@ int launch_rmsnorm(const void* x, const void* residual, const float* weight, voi
 int launch_split_heads(const void* qkv, void* q, void* k, void* v, int B, int L, int H, int Dk, int Dv, int io_dtype,
                        hipStream_t stream);
 int launch_swiglu(const void* in, void* out, long long rows, int I, int io_dtype, hipStream_t stream);
+int launch_gla_backward(const void* q, const void* k, const void* v, const void* g_fwd, const void* g_bwd,
+                        const void* d_o, void* dq, void* dk, void* dv, void* dg_fwd, void* dg_bwd, void* workspace,
+                        int B, int H, int L, int Dk, int Dv, float scale, float out_scale, int io_dtype,
+                        int gate_dtype, hipStream_t stream);
+size_t gla_backward_workspace(int B, int H, int L, int Dk, int Dv, int bidir);
 }  // namespace vig
 
 static bool dtype_ok(int d) { return d == VIG_F32 || d == VIG_BF16; }
@@ -145,6 +150,29 @@ int vig_swiglu_fwd(const void* gate_up, void* out, long long rows, int I, int io
   if (!gate_up || !out || rows <= 0 || I <= 0) return VIG_EINVAL;
   if (!dtype_ok(io_dtype) || (I % 8) != 0) return VIG_ENOTSUP;
   return vig::launch_swiglu(gate_up, out, rows, I, io_dtype, (hipStream_t)stream);
+}
+
+static bool bwd_shape_ok(int Dk, int Dv) {
+  return (Dk == 16 && Dv == 32) || (Dk == 32 && (Dv == 32 || Dv == 64)) || (Dk == 64 && (Dv == 32 || Dv == 64));
+}
+
+size_t vig_gla_bidir_bwd_workspace(int B, int H, int L, int Dk, int Dv, int bidirectional) {
+  if (B <= 0 || H <= 0 || L <= 0 || !bwd_shape_ok(Dk, Dv)) return 0;
+  return vig::gla_backward_workspace(B, H, L, Dk, Dv, bidirectional);
+}
+
+int vig_gla_bidir_bwd(const void* q, const void* k, const void* v, const void* g_fwd, const void* g_bwd,
+                      const void* d_o, void* dq, void* dk, void* dv, void* dg_fwd, void* dg_bwd, void* workspace,
+                      size_t workspace_bytes, int B, int H, int L, int Dk, int Dv, float scale, float out_scale,
+                      int io_dtype, int gate_dtype, void* stream) {
+  if (!q || !k || !v || !g_fwd || !d_o || !dq || !dk || !dv || !dg_fwd || (g_bwd && !dg_bwd) || B <= 0 || H <= 0 ||
+      L <= 0)
+    return VIG_EINVAL;
+  if (!dtype_ok(io_dtype) || !dtype_ok(gate_dtype) || !bwd_shape_ok(Dk, Dv)) return VIG_ENOTSUP;
+  const size_t need = vig::gla_backward_workspace(B, H, L, Dk, Dv, g_bwd != nullptr);
+  if (!workspace || workspace_bytes < need) return VIG_ENOSPC;
+  return vig::launch_gla_backward(q, k, v, g_fwd, g_bwd, d_o, dq, dk, dv, dg_fwd, dg_bwd, workspace, B, H, L, Dk, Dv,
+                                  scale, out_scale, io_dtype, gate_dtype, (hipStream_t)stream);
 }
 
 }  // extern "C"

@@ -47,7 +47,67 @@ def gla_bidir_forward(q, k, v, g_fwd, g_bwd=None, scale: float = -1, out_scale: 
 
     q, k, g_*: [B,H,L,Dk]; v: [B,H,L,Dv].  g_bwd=None gives the causal op.
     `exact=True` forces the fp32-arithmetic recurrent kernel.
+    Differentiable: when autograd is recording and an input requires grad, the backward runs vig_gla_bidir_bwd.
     """
+    tensors = (q, k, v, g_fwd) + ((g_bwd,) if g_bwd is not None else ())
+    if torch.is_grad_enabled() and any(t.requires_grad for t in tensors):
+        if out is not None:
+            raise ValueError("`out` cannot be given when a gradient is recorded")
+        if scale == -1 or scale is None:
+            scale = q.shape[-1] ** -0.5
+        return _GLABidirFunction.apply(q, k, v, g_fwd, g_bwd, float(scale), float(out_scale), bool(exact))
+    return _gla_bidir_forward_raw(q, k, v, g_fwd, g_bwd, scale, out_scale, exact, out)
+
+
+def gla_bidir_backward(q, k, v, g_fwd, g_bwd, d_o, scale: float = -1, out_scale: float = 1.0):
+    """Gradients of gla_bidir_forward contracted with d_o: (dq, dk, dv, dg_fwd, dg_bwd or None).  fp32 arithmetic."""
+    lib = _lib.load()
+    _check_cuda(q, k, v, g_fwd, g_bwd, d_o)
+    q, k, v, g_fwd, d_o = (t.contiguous() for t in (q, k, v, g_fwd, d_o))
+    if g_bwd is not None:
+        g_bwd = g_bwd.contiguous()
+    B, H, L, Dk = q.shape
+    Dv = v.shape[-1]
+    if d_o.shape != v.shape or d_o.dtype != q.dtype:
+        raise ValueError("d_o must match the output in shape and dtype")
+    if scale == -1 or scale is None:
+        scale = Dk ** -0.5
+    dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
+    dgf = torch.empty_like(g_fwd)
+    dgb = torch.empty_like(g_bwd) if g_bwd is not None else None
+    ws_bytes = lib.vig_gla_bidir_bwd_workspace(B, H, L, Dk, Dv, int(g_bwd is not None))
+    if ws_bytes == 0:
+        raise _lib.VigGlaError(f"vig_gla_bidir_bwd: shape Dk={Dk}, Dv={Dv} is not built")
+    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=q.device)
+    with torch.cuda.device(q.device):
+        rc = lib.vig_gla_bidir_bwd(q.data_ptr(), k.data_ptr(), v.data_ptr(), g_fwd.data_ptr(),
+                                   g_bwd.data_ptr() if g_bwd is not None else None, d_o.data_ptr(),
+                                   dq.data_ptr(), dk.data_ptr(), dv.data_ptr(), dgf.data_ptr(),
+                                   dgb.data_ptr() if dgb is not None else None, ws.data_ptr(), ws_bytes,
+                                   B, H, L, Dk, Dv, float(scale), float(out_scale), _dt(q), _dt(g_fwd), _stream_ptr(q))
+    _lib.check(rc, "vig_gla_bidir_bwd")
+    ws.record_stream(torch.cuda.current_stream(q.device))
+    return dq, dk, dv, dgf, dgb
+
+
+class _GLABidirFunction(torch.autograd.Function):
+    """Autograd node of the bidirectional op (the reference's FusedChunkGLAFunction, chunk_fuse.py:315-518)."""
+
+    @staticmethod
+    def forward(ctx, q, k, v, g_fwd, g_bwd, scale, out_scale, exact):
+        o = _gla_bidir_forward_raw(q, k, v, g_fwd, g_bwd, scale, out_scale, exact, None)
+        ctx.save_for_backward(q, k, v, g_fwd, g_bwd)
+        ctx.scale, ctx.out_scale = scale, out_scale
+        return o
+
+    @staticmethod
+    def backward(ctx, d_o):
+        q, k, v, g_fwd, g_bwd = ctx.saved_tensors
+        dq, dk, dv, dgf, dgb = gla_bidir_backward(q, k, v, g_fwd, g_bwd, d_o, ctx.scale, ctx.out_scale)
+        return dq, dk, dv, dgf, dgb, None, None, None
+
+
+def _gla_bidir_forward_raw(q, k, v, g_fwd, g_bwd, scale, out_scale, exact, out):
     lib = _lib.load()
     _check_cuda(q, k, v, g_fwd, g_bwd)
     q, k, v, g_fwd = (t.contiguous() for t in (q, k, v, g_fwd))
