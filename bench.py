@@ -99,6 +99,40 @@ def model_throughput(dev, batch=256, warmup=10, iters=30, tune_gemm=True):
             "ms_per_forward": dt / iters * 1e3, "gemm_solution_tuning": "torch.cuda.tunable" if tuned else None}
 
 
+def backward_time(lib, tensors, s, io_dt, scale, sp, stream, dev, iters=20):
+    """Event-bracketed time of vig_gla_bidir_bwd (fp32 token-recurrent arithmetic) on one input set."""
+    import torch
+
+    q, k, v, gf, gb, o = tensors
+    d_o = torch.randn_like(v)
+    dq, dk, dv, dgf, dgb = (torch.empty_like(t) for t in (q, k, v, gf, gb))
+    n = lib.vig_gla_bidir_bwd_workspace(s.B, s.H, s.L, s.Dk, s.Dv, 1)
+    if n == 0:
+        return None
+    ws = torch.empty(n, dtype=torch.uint8, device=dev)
+
+    def run():
+        rc = lib.vig_gla_bidir_bwd(q.data_ptr(), k.data_ptr(), v.data_ptr(), gf.data_ptr(), gb.data_ptr(), d_o.data_ptr(),
+                                   dq.data_ptr(), dk.data_ptr(), dv.data_ptr(), dgf.data_ptr(), dgb.data_ptr(),
+                                   ws.data_ptr(), n, s.B, s.H, s.L, s.Dk, s.Dv, scale, 1.0, io_dt, io_dt, sp)
+        if rc != 0:
+            raise RuntimeError(f"vig_gla_bidir_bwd rc={rc}")
+
+    for _ in range(3):
+        run()
+    evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(iters)]
+    for a, b in evs:
+        a.record(stream)
+        run()
+        b.record(stream)
+    torch.cuda.synchronize()
+    us = sum(a.elapsed_time(b) for a, b in evs) / iters * 1e3
+    esz = 4 if s.dtype == "f32" else 2
+    alg = s.tokens * esz * ((2 * s.Dk + 2 * s.Dv) + 2 * s.Dk + (2 * s.Dk + s.Dv) + 2 * s.Dk)
+    return {"us": us, "algorithmic_bytes": alg, "algorithmic_GBps": alg / (us * 1e-6) / 1e9,
+            "frac_of_hbm_peak": alg / (us * 1e-6) / 1e9 / HBM_PEAK_GBPS, "kernel": "fp32 token-recurrent"}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -109,6 +143,7 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--exact", action="store_true", help="time the fp32-arithmetic recurrent kernel instead")
     ap.add_argument("--model", action="store_true", help="also time the full ViG-S eval forward (images/s)")
+    ap.add_argument("--backward", action="store_true", help="also time the backward of the op on the same workload")
     ap.add_argument("--no-gemm-tuning", action="store_true",
                     help="with --model: leave torch's GEMM solution tuning off (clean kernel traces)")
     ap.add_argument("--copy-calibration", action="store_true",
@@ -244,6 +279,8 @@ def main():
         "roofline": {"bound": "hbm", "achieved": achieved_gbps, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                      "frac": achieved_gbps / HBM_PEAK_GBPS, "traffic": traffic},
     }
+    if args.backward:
+        out["backward"] = backward_time(lib, sets[0], s, io_dt, scale, sp, stream, dev)
     if args.model:
         out["vig_s_forward"] = model_throughput(dev, tune_gemm=not args.no_gemm_tuning)
     if not args.no_cpu:
