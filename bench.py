@@ -147,6 +147,8 @@ def main():
     ap.add_argument("--backward", action="store_true", help="also time the backward of the op on the same workload")
     ap.add_argument("--no-gemm-tuning", action="store_true",
                     help="with --model: leave torch's GEMM solution tuning off (clean kernel traces)")
+    ap.add_argument("--unfused-gate", action="store_true",
+                    help="workload 2: run the locality gate as a second kernel instead of inside the GLA kernel")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="also run plain device copies of known size (q -> o), so that FETCH_SIZE / WRITE_SIZE "
                          "counters of a profiled run can be scaled to bytes")
@@ -193,8 +195,10 @@ def main():
     fn = lib.vig_gla_bidir_fwd_exact if args.exact else lib.vig_gla_bidir_fwd
     scale = s.Dk ** -0.5
 
-    # workload 2 adds the sigmoid locality gate on the 14x14 grid of the GLA output (a second, stencil kernel)
+    # workload 2 adds the sigmoid locality gate on the 14x14 grid of the GLA output: inside the GLA kernel, or with
+    # --unfused-gate as a second (stencil) kernel over the stored output
     with_gate = args.config == 2
+    fused_gate = with_gate and not args.unfused_gate and not args.exact
     if with_gate:
         from vig_amd.synthetic import make_locality_weight
         gate_w = make_locality_weight(s.H * s.Dv, 2002).reshape(s.H * s.Dv, 9).float().contiguous().to(dev)
@@ -202,6 +206,13 @@ def main():
 
     def step(i):
         q, k, v, gf, gb, o = sets[i % nsets]
+        if fused_gate:
+            rc = lib.vig_gla_bidir_locgate_fwd(q.data_ptr(), k.data_ptr(), v.data_ptr(), gf.data_ptr(), gb.data_ptr(),
+                                               gate_w.data_ptr(), gate_out[i % nsets].data_ptr(), s.B, s.H, s.L, s.Dk,
+                                               s.Dv, s.grid[0], s.grid[1], scale, 1.0, io_dt, io_dt, sp)
+            if rc != 0:
+                raise RuntimeError(f"vig_gla_bidir_locgate_fwd rc={rc}")
+            return
         rc = fn(q.data_ptr(), k.data_ptr(), v.data_ptr(), gf.data_ptr(), gb.data_ptr(), o.data_ptr(),
                 ws.data_ptr(), ws_bytes, s.B, s.H, s.L, s.Dk, s.Dv, scale, 1.0, io_dt, io_dt, sp)
         if rc != 0:
@@ -272,7 +283,8 @@ def main():
         "data": "synthetic",
         "config": {"workload": s.name, "B": s.B, "H": s.H, "L": s.L, "Dk": s.Dk, "Dv": s.Dv,
                    "input_sets_rotated": nsets, "kernel_path": "recurrent_fp32" if args.exact else "default",
-                   "locality_gate": "separate stencil kernel after the GLA" if with_gate else None},
+                   "locality_gate": ("inside the GLA kernel" if fused_gate else "separate stencil kernel after the GLA")
+                   if with_gate else None},
         "tokens_per_s": s.tokens / (ms_per_step * 1e-3),
         "mfma_frac_algorithmic": tflops / MFMA_BF16_PEAK_TFLOPS,
         "executed_tflops_chunk64": s.tokens * exec_flops_tok / (ms_per_step * 1e-3) / 1e12,

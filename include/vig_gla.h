@@ -141,6 +141,22 @@ int vig_locality_gate_fwd(const void* o, const float* weight, void* y,
                           int B, int H, int h, int w, int Dv, int io_dtype, void* stream);
 
 /*
+ * vig_gla_bidir_fwd and vig_locality_gate_fwd in one kernel: the GLA output o = out_scale * (o_fwd + o_bwd) is
+ * rounded to bf16, staged on chip, and y = o * sigmoid(dwconv3x3(o)) is what reaches memory (bit-identical to the
+ * two calls in a row).  Same tensors as vig_gla_bidir_fwd; weight [H*Dv, 3, 3] f32; L = grid_h * grid_w.
+ * Built for bf16 tensors and gates, Dk in {32, 64}, Dv = 64, L <= 256, both directions, and token grids with
+ * grid_w <= 62 and grid_h + 2 <= 8 * floor(64 / (grid_w + 2)) (14x14 and 16x16 are); VIG_ENOTSUP otherwise
+ * (the caller then makes the two calls).  No workspace.
+ *
+ * Replaces: the GLA call of classification/models/vig.py:442 followed by the benchmark's sigmoid locality gate
+ * (the synthetic restatement of vig.py:291-294,447-454 on the op's own output).
+ */
+int vig_gla_bidir_locgate_fwd(const void* q, const void* k, const void* v, const void* g_fwd, const void* g_bwd,
+                              const float* gate_weight, void* y, int B, int H, int L, int Dk, int Dv,
+                              int grid_h, int grid_w, float scale, float out_scale, int io_dtype, int gate_dtype,
+                              void* stream);
+
+/*
  * Block epilogue before o_proj:
  *   y[b,l,hd*Dv+d] = rms(o[b,hd,l,:])*w_g * s + rms(local[b,l,hd,:])*w_l * (1-s),  s = sigmoid(g_lin[b,l,hd*Dv+d])
  *   rms(x) = x * rsqrt(mean(x^2) + eps); optional SiLU on y.

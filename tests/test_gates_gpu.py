@@ -105,3 +105,66 @@ def test_locality_blend(dtype, tol, H, Dv, L):
         want = O.locality_blend_reference(f64(o), f64(loc), f64(gl), f64(wg), f64(wl), 1e-6, silu)
         got = f64(vig_amd.locality_blend(o.cuda(), loc.cuda(), gl.cuda(), wg.cuda(), wl.cuda(), 1e-6, silu))
         assert max_abs(got, want) <= tol
+
+
+# ---- the locality gate fused into the GLA kernel (vig_gla_bidir_locgate_fwd) ----
+def _gla_inputs(B, H, L, Dk, seed, gate_scale=None):
+    from vig_amd.synthetic import make_gla_inputs
+    kw = {} if gate_scale is None else {"gate_scale": gate_scale}
+    q, k, v, gf, gb = make_gla_inputs(B, H, L, Dk, 64, seed=seed, dtype=torch.bfloat16, **kw)
+    if gate_scale is not None:
+        gf, gb = gf.clamp_min(-3), gb.clamp_min(-3)
+    return q, k, v, gf, gb
+
+
+@pytest.mark.parametrize("B,H,hw,Dk", [(2, 12, (14, 14), 64), (3, 2, (16, 16), 64), (5, 3, (7, 7), 32),
+                                        (2, 2, (3, 5), 64), (1, 3, (1, 9), 64), (2, 1, (12, 1), 32),
+                                        (1, 2, (6, 40), 64), (1, 1, (1, 1), 64)])
+def test_fused_locality_gate_matches_two_calls_and_oracle(B, H, hw, Dk):
+    """One kernel against (a) the GLA call followed by the stencil call, bit for bit, and (b) the fp64 oracle:
+    recurrent GLA, then o * sigmoid(conv(o)), within the bf16 bound."""
+    from .util import oracle_bidir
+    announce(f"fused locality gate B{B} H{H} grid {hw} Dk{Dk}")
+    L = hw[0] * hw[1]
+    q, k, v, gf, gb = _gla_inputs(B, H, L, Dk, seed=300 + L)
+    wt = make_locality_weight(H * 64, 31)
+    dq, dk, dv, dgf, dgb = (t.cuda() for t in (q, k, v, gf, gb))
+    got = vig_amd.gla_bidir_locality_gate(dq, dk, dv, dgf, dgb, wt.cuda(), hw)
+    two = vig_amd.locality_gate(vig_amd.gla_bidir_forward(dq, dk, dv, dgf, dgb), wt.cuda(), hw)
+    assert torch.equal(got, two)
+    o = oracle_bidir(q, k, v, gf, gb)
+    want = O.locality_sigmoid_gate_reference(o, f64(wt), hw)
+    assert max_abs(f64(got), want) <= 2e-2
+
+
+def test_fused_locality_gate_many_slabs_mixed_gate_strength():
+    """More slabs than workgroups, every 5th with gates too strong for the fp16 score operands: the slab that is
+    walked twice must not leave anything of its first walk in the output."""
+    announce("fused locality gate, 420 slabs, every 5th with strong gates")
+    B, H, hw = 70, 6, (14, 14)
+    q, k, v, gf, gb = _gla_inputs(B, H, 196, 64, seed=51)
+    _, _, _, sf, sb = _gla_inputs(B, H, 196, 64, seed=52, gate_scale=1.0)
+    strong = (torch.arange(B * H).reshape(B, H) % 5 == 2)[:, :, None, None]
+    gf, gb = torch.where(strong, sf, gf), torch.where(strong, sb, gb)
+    wt = make_locality_weight(H * 64, 33)
+    dq, dk, dv, dgf, dgb = (t.cuda() for t in (q, k, v, gf, gb))
+    got = vig_amd.gla_bidir_locality_gate(dq, dk, dv, dgf, dgb, wt.cuda(), hw)
+    two = vig_amd.locality_gate(vig_amd.gla_bidir_forward(dq, dk, dv, dgf, dgb), wt.cuda(), hw)
+    assert torch.isfinite(got.float()).all()
+    assert torch.equal(got, two)
+
+
+def test_fused_locality_gate_other_shapes_take_two_calls():
+    """Shapes outside the one-kernel form (long sequence, fp32) go through the two calls and still match the oracle."""
+    from .util import oracle_bidir
+    announce("fused locality gate wrapper on L=18x18 and on fp32")
+    hw = (18, 18)
+    q, k, v, gf, gb = _gla_inputs(1, 2, 324, 64, seed=61)
+    wt = make_locality_weight(2 * 64, 35)
+    got = vig_amd.gla_bidir_locality_gate(*(t.cuda() for t in (q, k, v, gf, gb)), wt.cuda(), hw)
+    want = O.locality_sigmoid_gate_reference(oracle_bidir(q, k, v, gf, gb), f64(wt), hw)
+    assert max_abs(f64(got), want) <= 2e-2
+    q, k, v, gf, gb = (t.float() for t in _gla_inputs(1, 2, 49, 64, seed=62))
+    got = vig_amd.gla_bidir_locality_gate(*(t.cuda() for t in (q, k, v, gf, gb)), wt.cuda(), (7, 7))
+    want = O.locality_sigmoid_gate_reference(oracle_bidir(q, k, v, gf, gb), f64(wt), (7, 7))
+    assert max_abs(f64(got), want) <= 1e-4 * max(1.0, float(np.abs(want).max()))

@@ -30,6 +30,7 @@ SIGNATURES = {
     "vig_gla_bidir_bwd_workspace": (_c_size_t, [_c_int] * 6),
     "vig_dirgate_fwd": (_c_int, [_c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_float, _c_float, _c_int, _c_int, _c_void_p]),
     "vig_dwconv3x3_fwd": (_c_int, [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_void_p]),
+    "vig_gla_bidir_locgate_fwd": (_c_int, [_c_void_p] * 7 + [_c_int] * 7 + [_c_float, _c_float, _c_int, _c_int, _c_void_p]),
     "vig_locality_gate_fwd": (_c_int, [_c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_void_p]),
     "vig_locality_blend_fwd": (_c_int, [_c_void_p] * 6 + [_c_int, _c_int, _c_int, _c_int, _c_float, _c_int, _c_int, _c_void_p]),
     "vig_rmsnorm_fwd": (_c_int, [_c_void_p] * 5 + [ctypes.c_longlong, _c_int, _c_float, _c_int, _c_int, _c_void_p]),

@@ -85,6 +85,25 @@ int vig_gla_bidir_fwd(const void* q, const void* k, const void* v, const void* g
   return vig::launch_gla_recurrent(a);
 }
 
+// vig_gla_bidir_fwd followed by vig_locality_gate_fwd in one kernel: y = o * sigmoid(conv3x3(o)) with o the rounded
+// GLA output, never written to memory.  Only shapes of the bf16 MFMA path with the whole sequence in one slab.
+int vig_gla_bidir_locgate_fwd(const void* q, const void* k, const void* v, const void* g_fwd, const void* g_bwd,
+                              const float* gate_weight, void* y, int B, int H, int L, int Dk, int Dv, int grid_h,
+                              int grid_w, float scale, float out_scale, int io_dtype, int gate_dtype, void* stream) {
+  vig::GlaArgs a;
+  const int rc = fill_args(a, q, k, v, g_fwd, g_bwd, y, nullptr, 0, B, H, L, Dk, Dv, scale, out_scale, io_dtype,
+                           gate_dtype, stream);
+  if (rc != VIG_OK) return rc;
+  if (!gate_weight || !g_bwd || grid_h <= 0 || grid_w <= 0 || (long long)grid_h * grid_w != L) return VIG_EINVAL;
+  if (!vig::gla_mfma_supported(a) || vig::gla_mfma_workspace(B, H, L, Dk, Dv) > 0 ||
+      !vig::gla_mfma_gate_grid_ok(grid_h, grid_w))
+    return VIG_ENOTSUP;
+  a.gate_w = gate_weight;
+  a.gate_rows = grid_h;
+  a.gate_cols = grid_w;
+  return vig::launch_gla_mfma(a);
+}
+
 // Same contract as vig_gla_bidir_fwd, but always takes the fp32-arithmetic
 // token-recurrent kernel (the exact path), whatever the dtypes.
 int vig_gla_bidir_fwd_exact(const void* q, const void* k, const void* v, const void* g_fwd, const void* g_bwd,

@@ -74,7 +74,8 @@ constexpr int kRegionBytes = 16 * 1024;      // per wave: k~ scratch, then publi
 constexpr int kLdsDvec = 8 * kRegionBytes;   // per wave: 64 chunk decays exp(G_end)
 constexpr int kLdsGend = kLdsDvec + 8 * 64 * 4;  // per wave: 64 anchors G_end * log2(e), laid out [h][p][16]
 constexpr int kLdsVeto = kLdsGend + 8 * 64 * 4;  // one word: some chunk refused the fp16 variant
-constexpr int kLdsTotal = kLdsVeto + 16;
+constexpr int kLdsGateW = kLdsVeto + 16;          // fused locality gate: the 64 x 9 stencil weights of the slab's head
+constexpr int kLdsTotal = kLdsGateW + 64 * 9 * 4;
 
 __device__ __forceinline__ f32x16_t mfma(const u32x4_t& a, const u32x4_t& b, const f32x16_t& c) {
   return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, a), __builtin_bit_cast(bf16x8_t, b), c, 0,
@@ -467,14 +468,38 @@ __device__ __forceinline__ void tile_phase(const ChunkSrc& cur, const Prefetch<N
 }
 
 
+// Locality gate fused into the output of a whole-sequence slab:  y = o * sigmoid(conv3x3(o)), the depthwise 3x3
+// stencil taken over the gw x gh token grid of the slab (zero padding), per channel, on the bf16-rounded o.
+struct GateCtx {
+  const float* w;  // [64][9] stencil weights of this slab's head
+  int gw, gh;      // token grid: gw columns, gh rows, gw * gh = L
+  int t0, nvalid;  // first token of this wave's chunk in the slab and its number of rows
+};
+// The rounded outputs of the slab are staged as a zero-padded (gh+2) x (gw+2) grid of 128-byte cells in the upper
+// halves of the LDS regions (free after barrier B).  A padded row never straddles two regions: each upper half takes
+// rph = 64 / (gw+2) whole rows, so the three taps of a stencil row are at constant offsets from the first.
+constexpr int kGateCellsPerRegion = 64;
+struct GateLayout {
+  int pw, rph;
+  float inv_rph;
+  __device__ __forceinline__ GateLayout(int gw) : pw(gw + 2), rph(kGateCellsPerRegion / (gw + 2)) {
+    inv_rph = 1.0f / (float)rph;
+  }
+  // byte offset in LDS of padded cell (py, 0); exact for py < 2^20
+  __device__ __forceinline__ int row(int py) const {
+    const int reg = (int)(((float)py + 0.5f) * inv_rph);
+    return reg * kRegionBytes + kRegionBytes / 2 + __mul24(py - __mul24(reg, rph), pw * 128);  // (24-bit: full rate)
+  }
+};
+
 // Everything one wave does for one segment: chunk c (the valid rows its descriptors cover) in
 // direction FWD / reverse.  Every wave of the workgroup passes the same three barriers here (plus the caller's).
 // F16 selects fp16 score operands; that variant returns false (for every wave of the workgroup alike, and without
 // having stored anything) when some chunk of the segment has gates too strong for it.
-template <bool FWD, int MODE, int NG, bool F16>
+template <bool FWD, int MODE, int NG, bool F16, bool GATE>
 __device__ __forceinline__ bool direction_wave(const ChunkSrc& cur, const ChunkSrc& nxt, rsrc_t o, int c, int lane,
                                                char* lds, float oscale, bool bidir, float* state, Prefetch<NG>& pf,
-                                               int iter) {
+                                               int iter, const GateCtx& gate) {
   constexpr bool OUT = MODE != kModeState;  // produces outputs (needs q)
   int r = lane & 31, h = lane >> 5;
   const int wi = (FWD ? 0 : 4) + c;
@@ -485,6 +510,10 @@ __device__ __forceinline__ bool direction_wave(const ChunkSrc& cur, const ChunkS
   float* dvec_all = reinterpret_cast<float*>(lds + kLdsDvec);
   if (!FWD) issue_rows<FWD, OUT, NG>(cur, r, h, pf);
   VIG_STAMP(0);
+  // fused gate: the first 144 threads fetch the head's stencil weights now and park them in LDS before barrier A
+  f32x4_t gate_w4 = {0.f, 0.f, 0.f, 0.f};
+  const bool gate_w_mine = GATE && wi * 64 + lane < 64 * 9 / 4;
+  if (GATE && gate_w_mine) gate_w4 = reinterpret_cast<const f32x4_t*>(gate.w)[wi * 64 + lane];
 
   // ---- cumulative log-gates G[it][p] via triangular-ones MFMA on transposed gate fragments ----
   f32x16_t G[2][2];
@@ -600,6 +629,7 @@ __device__ __forceinline__ bool direction_wave(const ChunkSrc& cur, const ChunkS
   h = lane >> 5;
   int* veto = reinterpret_cast<int*>(lds + kLdsVeto);
   if (F16 && !fast && lane == 0) *veto = 1;
+  if (GATE && gate_w_mine) reinterpret_cast<f32x4_t*>(lds + kLdsGateW)[wi * 64 + lane] = gate_w4;
   lds_barrier();  // (A) published U's and decays visible
   VIG_STAMP(6);
   // same answer in every wave: the word is only written before this barrier and the variant is left once it is set
@@ -714,6 +744,84 @@ __device__ __forceinline__ bool direction_wave(const ChunkSrc& cur, const ChunkS
           for (int m = 0; m < 4; ++m) O[pv][KEEP][4 * cq + m] += x[m];
         }
     }
+    if (GATE) {
+      // (needs both directions: every wave owns the 32-row tile KEEP of its chunk)
+      const GateLayout lay(gate.gw);
+      const float inv_w = 1.0f / (float)gate.gw;
+      {
+        const int row = 32 * KEEP + r;
+        if (row < gate.nvalid) {
+          const int T = gate.t0 + row;
+          const int y = (int)(((float)T + 0.5f) * inv_w), x = T - __mul24(y, gate.gw);
+          char* cell = lds + lay.row(y + 1) + (x + 1) * 128 + 64 * h;
+#pragma unroll
+          for (int gq = 0; gq < 4; ++gq) {
+            u32x4_t w;
+#pragma unroll
+            for (int m = 0; m < 4; ++m)
+              w[m] = pack_bf16x2(O[0][KEEP][4 * gq + m] * oscale, O[1][KEEP][4 * gq + m] * oscale);
+            *reinterpret_cast<u32x4_t*>(cell + 16 * gq) = w;
+          }
+        }
+      }
+      const int oct = lane & 7, tl = lane >> 3;
+      {  // the border cells, by the whole workgroup: top row, bottom row, then the two ends of every other row
+        const int nborder = 2 * lay.pw + 2 * gate.gh;
+        const u32x4_t zero = {0u, 0u, 0u, 0u};
+        for (int bc = wi * 8 + tl; bc < nborder; bc += 64) {
+          int py, px;
+          if (bc < 2 * lay.pw) {
+            py = bc < lay.pw ? 0 : gate.gh + 1;
+            px = bc < lay.pw ? bc : bc - lay.pw;
+          } else {
+            const int j = bc - 2 * lay.pw;
+            py = 1 + (j >> 1);
+            px = (j & 1) ? lay.pw - 1 : 0;
+          }
+          *reinterpret_cast<u32x4_t*>(lds + lay.row(py) + px * 128 + 16 * oct) = zero;
+        }
+      }
+      float wreg[8][9];
+      {
+        const f32x4_t* wp = reinterpret_cast<const f32x4_t*>(lds + kLdsGateW + oct * 72 * 4);
+#pragma unroll
+        for (int i = 0; i < 18; ++i) {
+          const f32x4_t x = wp[i];
+#pragma unroll
+          for (int m = 0; m < 4; ++m) wreg[(4 * i + m) / 9][(4 * i + m) % 9] = x[m];
+        }
+      }
+      lds_barrier();  // (C') the slab's outputs and the zero border are staged
+#pragma unroll 1
+      for (int i = 0; i < 4; ++i) {
+        const int row = 32 * KEEP + tl + 8 * i;
+        if (row < gate.nvalid) {
+          const int T = gate.t0 + row;
+          const int y = (int)(((float)T + 0.5f) * inv_w), x = T - __mul24(y, gate.gw);
+          float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f}, ctr[8];
+#pragma unroll
+          for (int di = 0; di < 3; ++di) {
+            const char* tap = lds + lay.row(y + di) + x * 128 + 16 * oct;  // padded cell of tap (di - 1, -1)
+#pragma unroll
+            for (int dj = 0; dj < 3; ++dj) {
+              const u32x4_t w = *reinterpret_cast<const u32x4_t*>(tap + dj * 128);
+#pragma unroll
+              for (int m = 0; m < 4; ++m) {
+                const float lo = bf16lo_to_f32(w[m]), hi = bf16hi_to_f32(w[m]);
+                acc[2 * m] = __builtin_fmaf(lo, wreg[2 * m][di * 3 + dj], acc[2 * m]);
+                acc[2 * m + 1] = __builtin_fmaf(hi, wreg[2 * m + 1][di * 3 + dj], acc[2 * m + 1]);
+                if (di == 1 && dj == 1) ctr[2 * m] = lo, ctr[2 * m + 1] = hi;
+              }
+            }
+          }
+          u32x4_t out;
+#pragma unroll
+          for (int m = 0; m < 4; ++m)
+            out[m] = pack_bf16x2(ctr[2 * m] * sigmoidf_(acc[2 * m]), ctr[2 * m + 1] * sigmoidf_(acc[2 * m + 1]));
+          __builtin_amdgcn_raw_buffer_store_b128(out, o, (unsigned)row * 128u + 16u * oct, 0, 0);
+        }
+      }
+    } else
 #pragma unroll
     for (int it = 0; it < 2; ++it) {
       if (bidir && it != KEEP) continue;
@@ -737,12 +845,13 @@ __device__ __forceinline__ bool direction_wave(const ChunkSrc& cur, const ChunkS
 // sequence possibly fewer) cut into 4 chunks of cw tokens.
 struct Geometry {
   int L, nseg, seg_len, cw, nitems;
+  int gw, gh, heads;  // fused locality gate only: token grid and heads per batch element
 };
 
-template <bool FWD, int MODE, int NG, bool F16>
+template <bool FWD, int MODE, int NG, bool F16, bool GATE>
 __device__ __forceinline__ int wave_loop(const uint16_t* q, const uint16_t* k, const uint16_t* v, const uint16_t* g,
                                          uint16_t* o, const Geometry& geo, int item, int c, int lane, char* lds,
-                                         float oscale, bool bidir, float* state_ws) {
+                                         float oscale, bool bidir, float* state_ws, const float* gate_w) {
   constexpr bool OUT = MODE != kModeState;
   constexpr int DK = 16 * NG;
   // descriptors of this wave's chunk of an item; past the last item (or for a chunk with no tokens) they are empty
@@ -776,7 +885,13 @@ __device__ __forceinline__ int wave_loop(const uint16_t* q, const uint16_t* k, c
     locate(item + gridDim.x, nxt, dst_next);
     float* state = state_ws ? state_ws + ((size_t)item * 2 + (FWD ? 0 : 1)) * kStateFloats : nullptr;
     asm volatile("" : "+v"(lane));  // per-lane constants are rebuilt per item instead of living across the loop
-    const bool ok = direction_wave<FWD, MODE, NG, F16>(cur, nxt, dst, c, lane, lds, oscale, bidir, state, pf, iter);
+    GateCtx gate{};
+    if (GATE) {  // slab mode: item = sequence = batch element * heads + head
+      const int nvalid = min(max(geo.L - c * geo.cw, 0), geo.cw);
+      gate = GateCtx{gate_w + (size_t)(item % geo.heads) * (64 * 9), geo.gw, geo.gh, c * geo.cw, nvalid};
+    }
+    const bool ok =
+        direction_wave<FWD, MODE, NG, F16, GATE>(cur, nxt, dst, c, lane, lds, oscale, bidir, state, pf, iter, gate);
     lds_barrier();  // (D) the next item reuses the LDS regions
     if (F16 && !ok) break;  // this item again, and all that follow, with split-bf16 scores
     cur = nxt;
@@ -786,22 +901,23 @@ __device__ __forceinline__ int wave_loop(const uint16_t* q, const uint16_t* k, c
 }
 
 // The items of one wave: fp16 score operands until a segment refuses them, split bf16 from there on.
-template <bool FWD, int MODE, int NG>
+template <bool FWD, int MODE, int NG, bool GATE>
 __device__ __forceinline__ void wave_items(const uint16_t* q, const uint16_t* k, const uint16_t* v, const uint16_t* g,
                                            uint16_t* o, const Geometry& geo, int c, int lane, char* lds, float oscale,
-                                           bool bidir, float* state_ws) {
-  const int item = wave_loop<FWD, MODE, NG, true>(q, k, v, g, o, geo, (int)blockIdx.x, c, lane, lds, oscale, bidir,
-                                                  state_ws);
-  wave_loop<FWD, MODE, NG, false>(q, k, v, g, o, geo, item, c, lane, lds, oscale, bidir, state_ws);
+                                           bool bidir, float* state_ws, const float* gate_w) {
+  const int item = wave_loop<FWD, MODE, NG, true, GATE>(q, k, v, g, o, geo, (int)blockIdx.x, c, lane, lds, oscale,
+                                                        bidir, state_ws, gate_w);
+  wave_loop<FWD, MODE, NG, false, GATE>(q, k, v, g, o, geo, item, c, lane, lds, oscale, bidir, state_ws, gate_w);
 }
 
 }  // namespace
 
-template <int MODE, int NG>
+template <int MODE, int NG, bool GATE = false>
 __global__ __launch_bounds__(512) void gla_mfma_kernel(const uint16_t* __restrict__ q, const uint16_t* __restrict__ k,
                                                        const uint16_t* __restrict__ v, const uint16_t* __restrict__ gf,
                                                        const uint16_t* __restrict__ gb, uint16_t* __restrict__ o,
-                                                       Geometry geo, float oscale, float* state_ws) {
+                                                       Geometry geo, float oscale, float* state_ws,
+                                                       const float* __restrict__ gate_w) {
   extern __shared__ __align__(16) char lds[];
   const int tid = threadIdx.x;
   const int wi = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform: region / chunk addressing stays scalar
@@ -811,9 +927,9 @@ __global__ __launch_bounds__(512) void gla_mfma_kernel(const uint16_t* __restric
   if (tid == 0) *reinterpret_cast<int*>(lds + kLdsVeto) = 0;
   lds_barrier();
   if (wi < 4) {
-    wave_items<true, MODE, NG>(q, k, v, gf, o, geo, c, lane, lds, oscale, bidir, state_ws);
+    wave_items<true, MODE, NG, GATE>(q, k, v, gf, o, geo, c, lane, lds, oscale, bidir, state_ws, gate_w);
   } else if (bidir) {
-    wave_items<false, MODE, NG>(q, k, v, gb, o, geo, c, lane, lds, oscale, bidir, state_ws);
+    wave_items<false, MODE, NG, GATE>(q, k, v, gb, o, geo, c, lane, lds, oscale, bidir, state_ws, gate_w);
   } else {
     // idle half of a one-direction launch: keeps the barrier count of the working waves, including the segment
     // that is walked twice when the fp16 variant is refused
@@ -873,13 +989,19 @@ __global__ __launch_bounds__(256) void gla_segment_scan_kernel(float* state_ws, 
 }
 
 static Geometry make_geometry(int nseq, int L) {
-  Geometry g;
+  Geometry g{};
   g.L = L;
   g.nseg = (L + 255) / 256;
   g.seg_len = (L + g.nseg - 1) / g.nseg;
   g.cw = (g.seg_len + 3) / 4;
   g.nitems = nseq * g.nseg;
   return g;
+}
+
+// the padded grid must fit the staging cells: whole padded rows per region half, eight halves
+bool gla_mfma_gate_grid_ok(int rows, int cols) {
+  if (rows <= 0 || cols <= 0 || cols + 2 > kGateCellsPerRegion) return false;
+  return rows + 2 <= 8 * (kGateCellsPerRegion / (cols + 2));
 }
 
 bool gla_mfma_supported(const GlaArgs& a) {
@@ -900,14 +1022,15 @@ static int launch_gla_mfma_t(const GlaArgs& a, int num_cu, int dev) {
   static bool attr_done_dev[kMaxDevices] = {};
   bool& attr_done = attr_done_dev[dev];
   if (!attr_done) {
-    const void* kernels[3] = {reinterpret_cast<const void*>(gla_mfma_kernel<kModeSlab, NG>),
+    const void* kernels[4] = {reinterpret_cast<const void*>(gla_mfma_kernel<kModeSlab, NG>),
                               reinterpret_cast<const void*>(gla_mfma_kernel<kModeState, NG>),
-                              reinterpret_cast<const void*>(gla_mfma_kernel<kModeChain, NG>)};
+                              reinterpret_cast<const void*>(gla_mfma_kernel<kModeChain, NG>),
+                              reinterpret_cast<const void*>(gla_mfma_kernel<kModeSlab, NG, true>)};
     for (const void* kf : kernels)
       if (hipFuncSetAttribute(kf, hipFuncAttributeMaxDynamicSharedMemorySize, kLdsTotal) != hipSuccess) return -5;
     attr_done = true;
   }
-  const Geometry geo = make_geometry(a.B * a.H, a.L);
+  Geometry geo = make_geometry(a.B * a.H, a.L);
   int grid = geo.nitems < num_cu ? geo.nitems : num_cu;
 #ifdef VIG_TIMING
   if (const char* e = getenv("VIG_GRID")) grid = atoi(e);
@@ -919,18 +1042,29 @@ static int launch_gla_mfma_t(const GlaArgs& a, int num_cu, int dev) {
   const uint16_t* gb = (const uint16_t*)a.g_bwd;
   uint16_t* o = (uint16_t*)a.o;
   const float oscale = a.scale * a.out_scale;
-  if (geo.nseg == 1) {
+  const float* no_gate = nullptr;
+  if (a.gate_w) {
+    // fused locality gate: whole-sequence slabs, both directions, the padded token grid must fit the staging cells
+    if (geo.nseg != 1 || !gb || a.gate_cols <= 0 || a.gate_rows <= 0 || a.gate_cols * a.gate_rows != a.L ||
+        !gla_mfma_gate_grid_ok(a.gate_rows, a.gate_cols))
+      return -95;
+    geo.gw = a.gate_cols;
+    geo.gh = a.gate_rows;
+    geo.heads = a.H;
+    hipLaunchKernelGGL((gla_mfma_kernel<kModeSlab, NG, true>), dim3(grid), dim3(512), kLdsTotal, a.stream, q, k, v, gf,
+                       gb, o, geo, oscale, (float*)nullptr, a.gate_w);
+  } else if (geo.nseg == 1) {
     hipLaunchKernelGGL((gla_mfma_kernel<kModeSlab, NG>), dim3(grid), dim3(512), kLdsTotal, a.stream, q, k, v, gf, gb, o,
-                       geo, oscale, (float*)nullptr);
+                       geo, oscale, (float*)nullptr, no_gate);
   } else {
     float* ws = (float*)a.workspace;
     hipLaunchKernelGGL((gla_mfma_kernel<kModeState, NG>), dim3(grid), dim3(512), kLdsTotal, a.stream, q, k, v, gf, gb, o,
-                       geo, oscale, ws);
+                       geo, oscale, ws, no_gate);
     const int ndir = gb ? 2 : 1;
     hipLaunchKernelGGL(gla_segment_scan_kernel, dim3(64 * 64 / 256, a.B * a.H * ndir), dim3(256), 0, a.stream, ws,
                        a.B * a.H, geo.nseg, ndir, NG);
     hipLaunchKernelGGL((gla_mfma_kernel<kModeChain, NG>), dim3(grid), dim3(512), kLdsTotal, a.stream, q, k, v, gf, gb, o,
-                       geo, oscale, ws);
+                       geo, oscale, ws, no_gate);
   }
   return hipGetLastError() == hipSuccess ? 0 : -5;
 }

@@ -18,6 +18,10 @@ struct GlaArgs {
   float scale, out_scale;
   int io_dtype, gate_dtype;  // 0 = f32, 1 = bf16
   hipStream_t stream;
+  // fused locality gate (bf16 MFMA path only): o * sigmoid(conv3x3(o)) on the gate_rows x gate_cols token grid is
+  // stored instead of o; weights [H*Dv, 9] f32.  Null: plain output.
+  const float* gate_w = nullptr;
+  int gate_rows = 0, gate_cols = 0;
 };
 
 // fp32-arithmetic token-recurrent path (any supported dtype combination).
@@ -27,6 +31,7 @@ size_t gla_recurrent_workspace(int B, int H, int L, int Dv, int io_dtype);
 // bf16 MFMA chunked path (bf16 io and gates).
 bool gla_mfma_supported(const GlaArgs& a);
 int launch_gla_mfma(const GlaArgs& a);
+bool gla_mfma_gate_grid_ok(int rows, int cols);  // token grids the fused locality gate takes
 size_t gla_mfma_workspace(int B, int H, int L, int Dk, int Dv);
 
 }  // namespace vig

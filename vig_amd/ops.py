@@ -260,6 +260,41 @@ def locality_gate(o: torch.Tensor, weight: torch.Tensor, hw) -> torch.Tensor:
     return y
 
 
+def gla_bidir_locality_gate(q, k, v, g_fwd, g_bwd, weight: torch.Tensor, hw, scale: float = -1,
+                            out_scale: float = 1.0) -> torch.Tensor:
+    """locality_gate(gla_bidir_forward(q, k, v, g_fwd, g_bwd), weight, hw), bit for bit.
+
+    Shapes the one-kernel form is built for (bf16, Dk in {32,64}, Dv=64, L=h*w<=256) never write the ungated
+    output to memory; every other shape makes the two calls.  Inference only.
+    """
+    lib = _lib.load()
+    _check_cuda(q, k, v, g_fwd, g_bwd, weight)
+    B, H, L, Dk = q.shape
+    Dv = v.shape[-1]
+    h, w = hw
+    if L != h * w:
+        raise ValueError("L must equal h*w")
+    if scale == -1 or scale is None:
+        scale = Dk ** -0.5
+    fusable = (g_bwd is not None and q.dtype == torch.bfloat16 and g_fwd.dtype == torch.bfloat16 and Dk in (32, 64)
+               and Dv == 64 and L <= 256 and w + 2 <= 64 and h + 2 <= 8 * (64 // (w + 2)))
+    if not fusable:
+        return locality_gate(gla_bidir_forward(q, k, v, g_fwd, g_bwd, scale, out_scale), weight, hw)
+    q, k, v, g_fwd, g_bwd = (t.detach().contiguous() for t in (q, k, v, g_fwd, g_bwd))
+    if k.shape != q.shape or g_fwd.shape != q.shape or g_bwd.shape != q.shape or v.shape[:3] != q.shape[:3]:
+        raise ValueError("shape mismatch between q, k, v, g")
+    if k.dtype != q.dtype or v.dtype != q.dtype or g_bwd.dtype != g_fwd.dtype:
+        raise TypeError("q, k, v must share a dtype, and so must the gates")
+    wt = weight.detach().reshape(H * Dv, 9).float().contiguous()
+    y = torch.empty(B, H, L, Dv, dtype=q.dtype, device=q.device)
+    with torch.cuda.device(q.device):
+        rc = lib.vig_gla_bidir_locgate_fwd(q.data_ptr(), k.data_ptr(), v.data_ptr(), g_fwd.data_ptr(),
+                                           g_bwd.data_ptr(), wt.data_ptr(), y.data_ptr(), B, H, L, Dk, Dv, h, w,
+                                           float(scale), float(out_scale), _dt(q), _dt(g_fwd), _stream_ptr(q))
+    _lib.check(rc, "vig_gla_bidir_locgate_fwd")
+    return y
+
+
 def locality_blend(o: torch.Tensor, local: torch.Tensor, g_lin: torch.Tensor, w_g: torch.Tensor,
                    w_l: torch.Tensor, eps: float = 1e-6, silu_out: bool = False) -> torch.Tensor:
     """Block epilogue (vig.py:444-457): o [B,H,L,Dv]; local, g_lin [B,L,H*Dv] -> y [B,L,H*Dv]."""
