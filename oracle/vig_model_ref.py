@@ -30,8 +30,10 @@ def _ln2d(x, w, b, eps=1e-5):
     return F.layer_norm(x.permute(0, 2, 3, 1), (x.shape[1],), w, b, eps).permute(0, 3, 1, 2)
 
 
-def gla_block_attn(sd, pre, x, hw, num_heads, eps=1e-6, act_in_conv=False, out_act=False, normalizer=16.0):
-    """Eval-mode GatedLinearAttention.forward on x [B, L, C] (float64)."""
+def gla_block_attn(sd, pre, x, hw, num_heads, eps=1e-6, act_in_conv=False, out_act=False, normalizer=16.0,
+                   second_halving=True):
+    """Eval-mode GatedLinearAttention.forward on x [B, L, C] (float64).  second_halving=False gives HierViG's
+    GLA2D (classification/models/vig_h.py:536-606), whose `o /= 2` after the op is commented out (:579)."""
     B, L, C = x.shape
     h, w = hw
     x2 = x.reshape(B, h, w, C).permute(0, 3, 1, 2)
@@ -52,7 +54,9 @@ def gla_block_attn(sd, pre, x, hw, num_heads, eps=1e-6, act_in_conv=False, out_a
     gb = F.logsigmoid(heads(bw)) / normalizer
     o = O.bidir_gla_recurrent(heads(q).numpy(), heads(k).numpy(), heads(v).numpy(), gf.numpy(), gb.numpy(),
                               out_scale=0.5)
-    o = torch.from_numpy(o) / 2  # the second halving of the eval path (vig.py:443)
+    o = torch.from_numpy(o)
+    if second_halving:
+        o = o / 2  # the second halving of the eval path (vig.py:443)
     o = o.permute(0, 2, 1, 3)  # b l h d
     Dv = value_dim // H
     loc = local.reshape(B, H, Dv, L).permute(0, 3, 1, 2)  # 'b (h d) l -> b l h d'

@@ -109,3 +109,44 @@ def test_evaluate_callers(tmp_path):
     assert 0.0 <= acc1 <= acc5 <= 100.0 and loss > 0
     ips = evaluate.throughput(dst, loader[0][0].cuda().to(torch.bfloat16), warmup=2, iters=3)
     assert ips > 0
+
+
+# ---- HierViG's GLA2D (classification/models/vig_h.py:338-606): Dk 16, Dv 32 at every stage ----
+def test_gla2d_parameter_names():
+    m = layers.GLA2D(d_model=96, expand_k=0.5, expand_v=1.0, num_heads=3, use_act_in_conv=False, channel_first=True)
+    assert set(m.state_dict().keys()) == {
+        "in_proj.0.weight", "qkv_proj.weight", "gk_proj.0.weight", "gk_proj.1.weight", "gk_proj.1.bias",
+        "o_proj.weight", "g_norm.weight", "l_norm.weight", "g_proj.weight", "g_proj.bias"}
+    assert m.head_qk_dim == 16 and m.head_v_dim == 32 and m.qkv_proj.weight.shape == (192, 96)
+
+
+@pytest.mark.parametrize("dtype,tol", [(torch.float32, 2e-4), (torch.bfloat16, 6e-2)])
+@pytest.mark.parametrize("dim,H,hw,channel_first", [(96, 3, (28, 28), True), (96, 3, (9, 13), False),
+                                                    (192, 6, (14, 14), True), (768, 24, (7, 7), False)])
+def test_gla2d_matches_restatement(dtype, tol, dim, H, hw, channel_first):
+    announce(f"GLA2D eval forward dim {dim} heads {H} grid {hw} channel_first={channel_first} {dtype}")
+    torch.manual_seed(1)
+    m = layers.GLA2D(d_model=dim, expand_k=0.5, expand_v=1.0, num_heads=H, layernorm_eps=1e-6,
+                     use_act_in_conv=False, use_out_act=False, channel_first=channel_first).eval()
+    with torch.no_grad():
+        m.g_norm.weight.uniform_(0.5, 1.5)
+        m.l_norm.weight.uniform_(0.5, 1.5)
+        m.g_proj.bias.normal_(0, 0.5)
+        m.gk_proj[1].bias.normal_(0, 1.0)
+        for lin in (m.qkv_proj, m.g_proj, m.o_proj, m.gk_proj[0], m.gk_proj[1]):
+            lin.weight.mul_(8.0)
+    B, (h, w) = 2, hw
+    x = torch.randn(B, h, w, dim)  # channels last; the restatement consumes tokens in row-major grid order
+    sd = {k: v.double() for k, v in m.state_dict().items()}
+    want = R.gla_block_attn(sd, "", x.reshape(B, h * w, dim).double(), hw, H, 1e-6, False, False,
+                            second_halving=False).reshape(B, h, w, dim).numpy()
+    md = m.to("cuda", dtype)
+    xin = x.permute(0, 3, 1, 2).contiguous() if channel_first else x
+    got = md(xin.to("cuda", dtype))
+    if channel_first:
+        assert got.shape == (B, dim, h, w)
+        got = got.permute(0, 2, 3, 1)
+    got = got.double().cpu().numpy()
+    err = np.abs(got - want).max() / np.abs(want).max()
+    print(f"  max-rel err {err:.3e}", flush=True)
+    assert err <= tol

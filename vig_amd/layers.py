@@ -110,25 +110,58 @@ class GatedLinearAttention(nn.Module):
         nn.init.xavier_uniform_(self.gk_proj[0].weight, gain=gain)
         nn.init.xavier_uniform_(self.gk_proj[1].weight, gain=gain)
 
-    @torch.no_grad()
-    def forward(self, x, lower_bound=0, **kwargs):
-        B, L, C = x.shape
-        if kwargs.get("token_position", None) is not None:
-            raise NotImplementedError("class-token splicing is not built (the shipped configs use IF_CLS_TOKEN False)")
-        hw = tuple(kwargs["patch_resolution"])
+    def _mix(self, x, hw, out_scale):
+        """The token mixer on x [B, L, C] with L = h*w tokens in row-major grid order."""
         H = self.num_heads
         conv = self.in_proj[0]
         # local_out, already in the [B, L, C] layout the projections consume
         xs = ops.dwconv3x3(x, conv.weight, hw, bias=conv.bias, silu=self.use_act_in_conv)
         q, k, v = ops.split_heads(self.qkv_proj(xs), H, self.head_qk_dim, self.head_v_dim)
         gates = ops.dirgate(self.gk_proj(xs), H, self.gate_logit_normalizer, self.clamp_min)
-        # training glue averages the directions (vig.py:425-426); the eval path halves twice
-        # (recurrent_fuse.py:442, then vig.py:443)
-        out_scale = 0.5 if self.training else 0.25
         o = ops.gla_bidir_forward(q, k, v, gates[0], gates[1], scale=-1, out_scale=out_scale)
         y = ops.locality_blend(o, xs, self.g_proj(xs), self.g_norm._w32(), self.l_norm._w32(),
                                eps=self.layernorm_eps, silu_out=self.use_out_act)
         return self.o_proj(y)
+
+    @torch.no_grad()
+    def forward(self, x, lower_bound=0, **kwargs):
+        if kwargs.get("token_position", None) is not None:
+            raise NotImplementedError("class-token splicing is not built (the shipped configs use IF_CLS_TOKEN False)")
+        # training glue averages the directions (vig.py:425-426); the eval path halves twice
+        # (recurrent_fuse.py:442, then vig.py:443)
+        return self._mix(x, tuple(kwargs["patch_resolution"]), 0.5 if self.training else 0.25)
+
+
+class GLA2D(GatedLinearAttention):
+    """HierViG's token mixer (classification/models/vig_h.py:338-606): the same block on a feature map,
+    x [B, H, W, C] (or [B, C, H, W] with channel_first), same parameter names (its Linear2d keeps nn.Linear's weight
+    shape, vig_h.py:202-209).  Both branches of the reference average the two directions once (training glue
+    vig_h.py:531-532; eval bid_fused_recurrent_gla with the second halving commented out, vig_h.py:578-579)."""
+
+    def __init__(self, d_model: int = 1024, expand_v: float = 2.0, expand_k: float = 1.0, num_heads: int = 4,
+                 gate_fn: str = "swish", layernorm_eps: float = 1e-5, gate_logit_normalizer: int = 16,
+                 gate_low_rank_dim: int = 16, mode: str = "fused_chunk", clamp_min: Optional[float] = None,
+                 fuse_norm: bool = True, use_dirpe: bool = False, use_out_act: bool = False,
+                 use_act_in_conv: bool = True, rope_mode: str = "none", channel_first: bool = False, *args, **kwargs):
+        super().__init__(d_model=d_model, expand_v=expand_v, expand_k=expand_k, num_heads=num_heads, gate_fn=gate_fn,
+                         layernorm_eps=layernorm_eps, gate_logit_normalizer=gate_logit_normalizer,
+                         gate_low_rank_dim=gate_low_rank_dim, mode=mode, clamp_min=clamp_min, fuse_norm=fuse_norm,
+                         use_dirpe=use_dirpe, use_out_act=use_out_act, rope_mode=rope_mode,
+                         use_act_in_conv=use_act_in_conv, use_bias_in_dwconv=False)
+        self.channel_first = channel_first
+        self.d_group = 2
+
+    @torch.no_grad()
+    def forward(self, x, **kwargs):
+        if self.channel_first:
+            B, C, H, W = x.shape
+            x = x.permute(0, 2, 3, 1)
+        else:
+            B, H, W, C = x.shape
+        y = self._mix(x.reshape(B, H * W, C), (H, W), 0.5)
+        if self.channel_first:
+            return y.permute(0, 2, 1).reshape(B, -1, H, W)
+        return y.reshape(B, H, W, -1)
 
 
 class GLAMLP(nn.Module):
