@@ -90,8 +90,11 @@ int vig_gla_bidir_fwd_exact(const void* q, const void* k, const void* v,
  * Backward of vig_gla_bidir_fwd: given d_o = dL/do [B, H, L, Dv], writes
  *   dq, dk [B, H, L, Dk], dv [B, H, L, Dv] (summed over the directions) in io_dtype and
  *   dg_fwd, dg_bwd [B, H, L, Dk] in gate_dtype (dg_bwd only when g_bwd != NULL).
- * fp32 arithmetic, token-recurrent.  `workspace` must hold vig_gla_bidir_bwd_workspace(...) bytes.
+ * `workspace` must hold vig_gla_bidir_bwd_workspace(...) bytes.
  * Built shapes: (Dk, Dv) in {(16,32), (32,32), (32,64), (64,32), (64,64)}, any L >= 1.
+ * Dispatch: bf16 tensors + bf16 gates + Dk = Dv = 64 + L <= 256 + both directions -> matrix-core kernel (bf16
+ * operands, fp32 accumulation; gradients within ~1e-2 of their largest magnitude); a slab whose gate total exceeds
+ * ~83 in some channel, and every other case -> fp32-arithmetic token-recurrent kernel.
  *
  * Replaces: FusedChunkGLAFunction.backward (flash-linear-attention/fla/ops/gla/chunk_fuse.py:413-518; gate
  * gradient :505-518) under the flip-concat glue of classification/models/vig.py:407-426, for both directions in
@@ -106,6 +109,15 @@ int vig_gla_bidir_bwd(const void* q, const void* k, const void* v,
                       int io_dtype, int gate_dtype, void* stream);
 
 size_t vig_gla_bidir_bwd_workspace(int B, int H, int L, int Dk, int Dv, int bidirectional);
+
+/* Same contract as vig_gla_bidir_bwd, always the fp32-arithmetic token-recurrent kernel (the exact path). */
+int vig_gla_bidir_bwd_exact(const void* q, const void* k, const void* v,
+                            const void* g_fwd, const void* g_bwd, const void* d_o,
+                            void* dq, void* dk, void* dv, void* dg_fwd, void* dg_bwd,
+                            void* workspace, size_t workspace_bytes,
+                            int B, int H, int L, int Dk, int Dv,
+                            float scale, float out_scale,
+                            int io_dtype, int gate_dtype, void* stream);
 
 /*
  * Direction-wise gate preparation.

@@ -90,3 +90,61 @@ def test_autograd_through_the_wrappers():
     (o3 * do.cuda()).sum().backward()
     want = O.bidir_gla_backward(f64(q), f64(k), f64(v), f64(gf), None, f64(do))
     assert _rel(f64(tq2.grad), want[0]) <= 1e-4
+
+
+# ---- the matrix-core backward (bf16 tensors and gates, Dk = Dv = 64, L <= 256, both directions) ----
+MFMA_BWD_TOL = 2e-2  # max |error| over the gradient's largest magnitude (bf16 operands, fp32 accumulation)
+
+
+def _check_mfma(got, want, q, tol=MFMA_BWD_TOL):
+    floor = float(np.abs(f64(q) * want[0]).max())
+    worst = {}
+    for name, g_, w_ in zip(("dq", "dk", "dv", "dg_fwd", "dg_bwd"), got, want):
+        assert np.isfinite(f64(g_)).all(), name
+        worst[name] = _rel(f64(g_), w_, floor if name.startswith("dg") else 0.0)
+    print("  " + " ".join(f"{k}:{v:.2e}" for k, v in worst.items()), flush=True)
+    for name, e in worst.items():
+        assert e <= tol, (name, e)
+
+
+@pytest.mark.parametrize("B,H,L", [(2, 2, 1), (1, 3, 17), (2, 1, 32), (1, 2, 33), (2, 2, 64), (2, 3, 196),
+                                   (1, 2, 255), (1, 3, 256)])
+def test_backward_mfma_lengths(B, H, L):
+    announce(f"backward on the matrix cores B{B} H{H} L={L}")
+    q, k, v, gf, gb = make_gla_inputs(B, H, L, 64, 64, seed=500 + L, dtype=torch.bfloat16)
+    do = _do(v.shape, 10, torch.bfloat16)
+    want = O.bidir_gla_backward(f64(q), f64(k), f64(v), f64(gf), f64(gb), f64(do), out_scale=0.5)
+    got = vig_amd.gla_bidir_backward(*(t.cuda() for t in (q, k, v, gf, gb, do)), out_scale=0.5)
+    _check_mfma(got, want, q)
+
+
+def test_backward_mfma_many_slabs_against_exact_path():
+    """More slabs than workgroups (persistent loop), against the fp32-arithmetic kernel on the same inputs."""
+    announce("backward on the matrix cores, 600 slabs, against the recurrent kernel")
+    q, k, v, gf, gb = (t.cuda() for t in make_gla_inputs(100, 6, 196, 64, 64, seed=77, dtype=torch.bfloat16))
+    do = _do(v.shape, 11, torch.bfloat16).cuda()
+    want = [f64(t) for t in vig_amd.gla_bidir_backward(q, k, v, gf, gb, do, out_scale=0.5, exact=True)]
+    got = vig_amd.gla_bidir_backward(q, k, v, gf, gb, do, out_scale=0.5)
+    _check_mfma(got, want, q.cpu())
+
+
+def test_backward_mfma_strong_gates_fall_back_per_slab():
+    """Every third slab has gates beyond the quadratic form's range: those come from the recurrent kernel, bit for
+    bit, the others from the matrix cores."""
+    announce("backward, strong gates in every third slab")
+    B, H, L = 4, 3, 196
+    q, k, v, gf, gb = make_gla_inputs(B, H, L, 64, 64, seed=81, dtype=torch.bfloat16)
+    _, _, _, sf, sb = make_gla_inputs(B, H, L, 64, 64, seed=82, dtype=torch.bfloat16, gate_scale=2.0)
+    strong = (torch.arange(B * H).reshape(B, H) % 3 == 1)[:, :, None, None]
+    gf, gb = torch.where(strong, sf, gf), torch.where(strong, sb, gb)
+    do = _do(v.shape, 12, torch.bfloat16)
+    dev = [t.cuda() for t in (q, k, v, gf, gb, do)]
+    exact = vig_amd.gla_bidir_backward(*dev, out_scale=0.5, exact=True)
+    got = vig_amd.gla_bidir_backward(*dev, out_scale=0.5)
+    sel = strong[:, :, 0, 0].cuda()
+    for name, g_, e_ in zip(("dq", "dk", "dv", "dg_fwd", "dg_bwd"), got, exact):
+        assert torch.isfinite(g_.float()).all(), name
+        assert torch.equal(g_[sel], e_[sel]), name
+    want = O.bidir_gla_backward(f64(q), f64(k), f64(v), f64(gf), f64(gb), f64(do), out_scale=0.5)
+    keep = ~strong[:, :, 0, 0].numpy()
+    _check_mfma([g_.cpu()[keep] for g_ in got], [w_[keep] for w_ in want], q[keep])

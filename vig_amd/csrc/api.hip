@@ -20,7 +20,7 @@ int launch_swiglu(const void* in, void* out, long long rows, int I, int io_dtype
 int launch_gla_backward(const void* q, const void* k, const void* v, const void* g_fwd, const void* g_bwd,
                         const void* d_o, void* dq, void* dk, void* dv, void* dg_fwd, void* dg_bwd, void* workspace,
                         int B, int H, int L, int Dk, int Dv, float scale, float out_scale, int io_dtype,
-                        int gate_dtype, hipStream_t stream);
+                        int gate_dtype, bool exact, hipStream_t stream);
 size_t gla_backward_workspace(int B, int H, int L, int Dk, int Dv, int bidir);
 }  // namespace vig
 
@@ -180,10 +180,10 @@ size_t vig_gla_bidir_bwd_workspace(int B, int H, int L, int Dk, int Dv, int bidi
   return vig::gla_backward_workspace(B, H, L, Dk, Dv, bidirectional);
 }
 
-int vig_gla_bidir_bwd(const void* q, const void* k, const void* v, const void* g_fwd, const void* g_bwd,
-                      const void* d_o, void* dq, void* dk, void* dv, void* dg_fwd, void* dg_bwd, void* workspace,
-                      size_t workspace_bytes, int B, int H, int L, int Dk, int Dv, float scale, float out_scale,
-                      int io_dtype, int gate_dtype, void* stream) {
+static int gla_bidir_bwd(const void* q, const void* k, const void* v, const void* g_fwd, const void* g_bwd,
+                         const void* d_o, void* dq, void* dk, void* dv, void* dg_fwd, void* dg_bwd, void* workspace,
+                         size_t workspace_bytes, int B, int H, int L, int Dk, int Dv, float scale, float out_scale,
+                         int io_dtype, int gate_dtype, bool exact, void* stream) {
   if (!q || !k || !v || !g_fwd || !d_o || !dq || !dk || !dv || !dg_fwd || (g_bwd && !dg_bwd) || B <= 0 || H <= 0 ||
       L <= 0)
     return VIG_EINVAL;
@@ -191,7 +191,24 @@ int vig_gla_bidir_bwd(const void* q, const void* k, const void* v, const void* g
   const size_t need = vig::gla_backward_workspace(B, H, L, Dk, Dv, g_bwd != nullptr);
   if (!workspace || workspace_bytes < need) return VIG_ENOSPC;
   return vig::launch_gla_backward(q, k, v, g_fwd, g_bwd, d_o, dq, dk, dv, dg_fwd, dg_bwd, workspace, B, H, L, Dk, Dv,
-                                  scale, out_scale, io_dtype, gate_dtype, (hipStream_t)stream);
+                                  scale, out_scale, io_dtype, gate_dtype, exact, (hipStream_t)stream);
+}
+
+int vig_gla_bidir_bwd(const void* q, const void* k, const void* v, const void* g_fwd, const void* g_bwd,
+                      const void* d_o, void* dq, void* dk, void* dv, void* dg_fwd, void* dg_bwd, void* workspace,
+                      size_t workspace_bytes, int B, int H, int L, int Dk, int Dv, float scale, float out_scale,
+                      int io_dtype, int gate_dtype, void* stream) {
+  return gla_bidir_bwd(q, k, v, g_fwd, g_bwd, d_o, dq, dk, dv, dg_fwd, dg_bwd, workspace, workspace_bytes, B, H, L, Dk,
+                       Dv, scale, out_scale, io_dtype, gate_dtype, false, stream);
+}
+
+// Same contract, always the fp32-arithmetic token-recurrent kernel.
+int vig_gla_bidir_bwd_exact(const void* q, const void* k, const void* v, const void* g_fwd, const void* g_bwd,
+                            const void* d_o, void* dq, void* dk, void* dv, void* dg_fwd, void* dg_bwd,
+                            void* workspace, size_t workspace_bytes, int B, int H, int L, int Dk, int Dv, float scale,
+                            float out_scale, int io_dtype, int gate_dtype, void* stream) {
+  return gla_bidir_bwd(q, k, v, g_fwd, g_bwd, d_o, dq, dk, dv, dg_fwd, dg_bwd, workspace, workspace_bytes, B, H, L, Dk,
+                       Dv, scale, out_scale, io_dtype, gate_dtype, true, stream);
 }
 
 }  // extern "C"

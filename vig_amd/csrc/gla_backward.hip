@@ -29,13 +29,17 @@ struct GlaBwdArgs {
   float scale, out_scale;
   int io_dtype, gate_dtype;
   hipStream_t stream;
+  const int* only_flagged;  // null: every slab; else one int per (batch, head): slabs with 0 are skipped
 };
 
 template <typename TIO, typename TG, int DK, int DV, int TB>
 __global__ __launch_bounds__(256) void gla_backward_kernel(
     const TIO* __restrict__ q, const TIO* __restrict__ k, const TIO* __restrict__ v, const TG* __restrict__ gf,
     const TG* __restrict__ gb, const TIO* __restrict__ d_o, TIO* dq, TIO* dk, TIO* dv, TG* dgf, TG* dgb,
-    float* ws_dq, float* ws_acc_k, float* ws_acc_v, int L, float scale, float out_scale) {
+    float* ws_dq, float* ws_acc_k, float* ws_acc_v, int L, float scale, float out_scale,
+    const int* __restrict__ only_flagged) {
+  // second pass behind the matrix-core kernel: only the slabs it left out (uniform per workgroup, before any barrier)
+  if (only_flagged && only_flagged[blockIdx.x] == 0) return;
   constexpr int DKG = DK / 4;  // rows per wave, layout A
   constexpr int DVG = DV / 4;  // columns per wave, layout B
   __shared__ __align__(16) float sq[TB][DK];   // scale * q
@@ -237,7 +241,7 @@ static int launch_bwd_t(const GlaBwdArgs& a) {
   hipLaunchKernelGGL((gla_backward_kernel<TIO, TG, DK, DV, TB>), dim3(a.B * a.H), dim3(256), 0, a.stream,
                      (const TIO*)a.q, (const TIO*)a.k, (const TIO*)a.v, (const TG*)a.g_fwd, (const TG*)a.g_bwd,
                      (const TIO*)a.d_o, (TIO*)a.dq, (TIO*)a.dk, (TIO*)a.dv, (TG*)a.dg_fwd, (TG*)a.dg_bwd, ws_dq,
-                     ws_acc_k, ws_acc_v, a.L, a.scale, a.out_scale);
+                     ws_acc_k, ws_acc_v, a.L, a.scale, a.out_scale, a.only_flagged);
   return hipGetLastError() == hipSuccess ? 0 : -5;
 }
 
@@ -254,17 +258,28 @@ static int launch_bwd_d(const GlaBwdArgs& a) {
   return -95;
 }
 
-size_t gla_backward_workspace(int B, int H, int L, int Dk, int Dv, int bidir) {
+// fp32 scratch of the recurrent kernel, then one flag per slab for the matrix-core kernel
+static size_t recurrent_floats(int B, int H, int L, int Dk, int Dv, int bidir) {
   const size_t n_qk = (size_t)B * H * L * Dk, n_v = (size_t)B * H * L * Dv;
-  return (bidir ? 3 * n_qk + n_v : n_qk) * sizeof(float);
+  return bidir ? 3 * n_qk + n_v : n_qk;
+}
+size_t gla_backward_workspace(int B, int H, int L, int Dk, int Dv, int bidir) {
+  return recurrent_floats(B, H, L, Dk, Dv, bidir) * sizeof(float) + (size_t)B * H * sizeof(int);
 }
 
 int launch_gla_backward(const void* q, const void* k, const void* v, const void* g_fwd, const void* g_bwd,
                         const void* d_o, void* dq, void* dk, void* dv, void* dg_fwd, void* dg_bwd, void* workspace,
                         int B, int H, int L, int Dk, int Dv, float scale, float out_scale, int io_dtype,
-                        int gate_dtype, hipStream_t stream) {
+                        int gate_dtype, bool exact, hipStream_t stream) {
   GlaBwdArgs a{q, k, v, g_fwd, g_bwd, d_o, dq, dk, dv, dg_fwd, dg_bwd, workspace, B, H, L, Dk, Dv,
-               scale, out_scale, io_dtype, gate_dtype, stream};
+               scale, out_scale, io_dtype, gate_dtype, stream, nullptr};
+  if (!exact && gla_backward_mfma_supported(L, Dk, Dv, io_dtype, gate_dtype, g_bwd != nullptr)) {
+    int* flags = reinterpret_cast<int*>((float*)workspace + recurrent_floats(B, H, L, Dk, Dv, 1));
+    const int rc = launch_gla_backward_mfma(q, k, v, g_fwd, g_bwd, d_o, dq, dk, dv, dg_fwd, dg_bwd, flags, B, H, L,
+                                            scale * out_scale, stream);
+    if (rc != 0) return rc;
+    a.only_flagged = flags;  // slabs with gates beyond the matrix-core kernel's range
+  }
   if (io_dtype == 0) return gate_dtype == 0 ? launch_bwd_d<float, float>(a) : launch_bwd_d<float, uint16_t>(a);
   return gate_dtype == 0 ? launch_bwd_d<uint16_t, float>(a) : launch_bwd_d<uint16_t, uint16_t>(a);
 }

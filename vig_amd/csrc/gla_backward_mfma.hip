@@ -1,0 +1,376 @@
+// Backward of the bidirectional GLA op on MFMA tiles (gfx950): bf16 tensors and gates, Dk = Dv = 64, L <= 256.
+//
+// Per direction the whole (batch, head) slab is one quadratic form (no chunk states): with G the inclusive
+// cumulative log-gate along the direction and the anchor a = G_total / 2,
+//   q~_i = q_i e^{G_i - a},  k~_j = k_j e^{a - G_j}   (both within e^{|G_total|/2} of the inputs),
+//   P_ij = q~_i . k~_j,  A_ij = do_i . v_j            for the pairs the direction keeps (j <= i forward, j >= i reverse),
+//   dv_j = s sum_i P_ij do_i,   dq_i = s e^{G_i - a} (.) sum_j A_ij k~_j,   dk_j = s e^{a - G_j} (.) sum_i A_ij q~_i,
+//   dg_t = sum over the tokens i the gate of t acts on (i >= t forward, i <= t reverse) of q_i (.) dq_i - k_i (.) dk_i,
+// s = scale * out_scale.  This is the natural-order form of flash-linear-attention/fla/ops/gla/chunk_fuse.py:413-518
+// with one chunk per sequence; the flip-concat glue of classification/models/vig.py:407-426 never materialises.
+//
+// One persistent workgroup of 8 waves per CU walks slabs; wave w owns the 32-token tile w.  Per direction the
+// workgroup stages q~, k~ (and once v, do) as bf16 rows in LDS; then wave w accumulates dq of its tile over the key
+// tiles the direction keeps, and dk, dv of its tile over the query tiles: score tiles P, A come out of the matrix
+// cores in the register layout that feeds the next product directly (mfma_tiles.h), operands with tokens in the
+// contraction slots are read from the LDS rows as dwords.  The two directions take turns in LDS, so the work of a
+// tile pair (w, direction) and (w, other direction) adds up to the same for every wave.  dg needs a running sum over
+// tokens: the tile's q dq - k dk goes through LDS, lane = channel scans its 32 tokens, tile totals are exchanged.
+//
+// Slabs whose gate totals exceed the anchor's range (|G_total| / 2 * log2(e) > 60 in some channel) are not computed
+// here: the workgroup raises the slab's flag and the token-recurrent kernel, launched afterwards with that flag
+// array, computes exactly those.
+#include "common.h"
+#include "launch.h"
+#include "mfma_tiles.h"
+
+namespace vig {
+
+namespace {
+
+constexpr int kBwdTiles = 8;                                // 32-token tiles per slab
+constexpr int kBwdMatBytes = kBwdTiles * 32 * kKtStride * 2;  // one staged 256 x 64 bf16 matrix, 144-byte rows
+constexpr int kBwdLdsQ = 0;
+constexpr int kBwdLdsK = kBwdMatBytes;
+constexpr int kBwdLdsV = 2 * kBwdMatBytes;
+constexpr int kBwdLdsDo = 3 * kBwdMatBytes;
+constexpr int kBwdLdsTot = 4 * kBwdMatBytes;           // [8][64] f32: gate totals of the tiles
+constexpr int kBwdLdsOff = kBwdLdsTot + 8 * 64 * 4;    // [8][64] f32: per wave, (prefix - anchor) of its tile
+constexpr int kBwdLdsDgTot = kBwdLdsOff + 8 * 64 * 4;  // [8][64] f32: totals of q dq - k dk of the tiles
+constexpr int kBwdLdsTotal = kBwdLdsDgTot + 8 * 64 * 4;
+constexpr int kXStride = 68;  // floats per token row of the dg scratch (272 B: conflict-free 16-byte writes)
+static_assert(8 * 32 * kXStride * 4 <= 2 * kBwdMatBytes, "dg scratch overlays the q~ and k~ matrices");
+constexpr float kBwdHalfRange = 60.0f;
+
+// fragment of 8 consecutive channels (k-step ks, lane half h) of a staged row: contraction over channels
+__device__ __forceinline__ u32x4_t row_frag(const uint16_t* mat, int row, int ks, int h) {
+  return *reinterpret_cast<const u32x4_t*>(mat + row * kKtStride + 16 * ks + 8 * h);
+}
+
+// accumulator tile (rows 8g+4h+m in registers, column = lane) -> operand fragments with its rows in the contraction
+// slots, k-steps t = 0, 1
+__device__ __forceinline__ void tile_frags(const f32x16_t& T, u32x4_t (&f)[2]) {
+#pragma unroll
+  for (int t = 0; t < 2; ++t)
+#pragma unroll
+    for (int x = 0; x < 4; ++x) f[t][x] = pack_bf16x2(T[8 * t + 2 * x], T[8 * t + 2 * x + 1]);
+}
+
+// keeps the entries of a diagonal tile the direction uses; ROWS_ARE_QUERIES: rows i, column j (else rows j, column i)
+template <bool FWD, bool ROWS_ARE_QUERIES>
+__device__ __forceinline__ void mask_diag(f32x16_t& T, int r, int h) {
+#pragma unroll
+  for (int c = 0; c < 16; ++c) {
+    const int row = 8 * (c >> 2) + 4 * h + (c & 3);
+    const int i = ROWS_ARE_QUERIES ? row : r, j = ROWS_ARE_QUERIES ? r : row;
+    const bool keep = FWD ? (j <= i) : (j >= i);
+    T[c] = keep ? T[c] : 0.f;
+  }
+}
+
+struct BwdSlab {
+  const uint16_t *q, *k, *v, *gf, *gb, *d_o;
+  uint16_t *dq, *dk, *dv, *dgf, *dgb;
+};
+
+// One direction of one slab, for wave w (tile w).  dv accumulates over both directions (raw, unscaled).  The first
+// direction (LAST = false) leaves its dq and dk as bf16 pairs in keepq / keepk and stages v and do; the second adds its
+// own and stores dq, dk, dv.  Returns false, for every wave alike and before it has stored anything, when the gates
+// are out of range.
+template <bool FWD, bool LAST>
+__device__ __forceinline__ bool bwd_direction(const BwdSlab& sl, int L, int ntiles, int w, int lane, char* lds,
+                                              float s, f32x16_t (&dv)[2], uint32_t (&keepq)[16],
+                                              uint32_t (&keepk)[16]) {
+  constexpr bool stage_vdo = !LAST;
+  const int r = lane & 31, h = lane >> 5;
+  uint16_t* Q = reinterpret_cast<uint16_t*>(lds + kBwdLdsQ);
+  uint16_t* K = reinterpret_cast<uint16_t*>(lds + kBwdLdsK);
+  uint16_t* V = reinterpret_cast<uint16_t*>(lds + kBwdLdsV);
+  uint16_t* DO = reinterpret_cast<uint16_t*>(lds + kBwdLdsDo);
+  float* tot = reinterpret_cast<float*>(lds + kBwdLdsTot);
+  float* offs = reinterpret_cast<float*>(lds + kBwdLdsOff) + w * 64;
+  float* dgtot = reinterpret_cast<float*>(lds + kBwdLdsDgTot);
+  const int rows = min(max(L - 32 * w, 0), 32);  // valid tokens of this wave's tile
+  const size_t toff = (size_t)32 * w * 64;
+  const uint16_t* g = FWD ? sl.gf : sl.gb;
+  const rsrc_t rq = chunk_rsrc(sl.q + toff, rows, 128), rk = chunk_rsrc(sl.k + toff, rows, 128);
+  const rsrc_t rg = chunk_rsrc(g + toff, rows, 128);
+
+  // ---- loads of this tile: gates (tokens in the contraction slots), q and k rows; v and do rows once per slab ----
+  uint32_t gD[2][8];
+  issue_tdwords<0, 2, 4>(rg, r, h, gD);
+  u32x4_t rawq[4], rawk[4];
+  issue_raw_tile<4>(rq, 0, r, h, rawq);
+  issue_raw_tile<4>(rk, 0, r, h, rawk);
+  if (stage_vdo) {
+    u32x4_t rv[4], rd[4];
+    issue_raw_tile<4>(chunk_rsrc(sl.v + toff, rows, 128), 0, r, h, rv);
+    issue_raw_tile<4>(chunk_rsrc(sl.d_o + toff, rows, 128), 0, r, h, rd);
+    store_kt<4>(V, 32 * w + r, h, rv);
+    store_kt<4>(DO, 32 * w + r, h, rd);
+  }
+
+  // ---- tile-local cumulative gates: G^T = g^T T, lane = token, registers = channels 32h + 8g + 2m + p ----
+  f32x16_t G[2];
+  {
+    u32x4_t gfrag[2][2];
+    finish_tfrags<2>(gD, gfrag);
+    const u32x4_t tri0 = tri_frag<FWD>(0, 0, r, h), tri1 = tri_frag<FWD>(1, 0, r, h);
+#pragma unroll
+    for (int p = 0; p < 2; ++p) {
+      f32x16_t z = {0.f};
+      z = mfma(gfrag[0][p], tri0, z);
+      G[p] = mfma(gfrag[1][p], tri1, z);
+    }
+  }
+  // the tile total sits at its last token in walking order
+  if (r == (FWD ? 31 : 0)) {
+#pragma unroll
+    for (int c = 0; c < 16; ++c) {
+      const int ch = 32 * h + 8 * (c >> 2) + 2 * (c & 3);
+      tot[w * 64 + ch] = G[0][c];
+      tot[w * 64 + ch + 1] = G[1][c];
+    }
+  }
+  lds_barrier();  // (1) tile totals (and v, do rows) visible; the previous direction's scratch is dead
+  // lane = channel: gates before this tile in walking order, minus the anchor (half the slab total)
+  bool out_of_range;
+  {
+    float pre = 0.f, all = 0.f;
+#pragma unroll
+    for (int t = 0; t < kBwdTiles; ++t) {
+      const float x = tot[t * 64 + lane];
+      all += x;
+      pre += (FWD ? (t < w) : (t > w)) ? x : 0.f;
+    }
+    offs[lane] = pre - 0.5f * all;
+    out_of_range = __builtin_amdgcn_ballot_w64(fabsf(all) * (0.5f * kLog2e) > kBwdHalfRange) != 0;
+  }
+  if (out_of_range) return false;  // same totals in every wave: the whole workgroup leaves together
+  wave_lds_sync();
+  // x = (G - a) * log2(e) per (token, channel): q~ = q 2^x, k~ = k 2^-x
+  f32x16_t x[2];
+#pragma unroll
+  for (int gq = 0; gq < 4; ++gq) {
+    const f32x4_t o0 = *reinterpret_cast<const f32x4_t*>(offs + 32 * h + 8 * gq);
+    const f32x4_t o1 = *reinterpret_cast<const f32x4_t*>(offs + 32 * h + 8 * gq + 4);
+    const float o8[8] = {o0[0], o0[1], o0[2], o0[3], o1[0], o1[1], o1[2], o1[3]};
+#pragma unroll
+    for (int m = 0; m < 4; ++m)
+#pragma unroll
+      for (int p = 0; p < 2; ++p) x[p][4 * gq + m] = (G[p][4 * gq + m] + o8[2 * m + p]) * kLog2e;
+  }
+  {
+    u32x4_t qt[4], kt[4];
+#pragma unroll
+    for (int gq = 0; gq < 4; ++gq)
+#pragma unroll
+      for (int m = 0; m < 4; ++m) {
+        const int c = 4 * gq + m;
+        const float e0 = exp2_fast(x[0][c]), e1 = exp2_fast(x[1][c]);
+        const uint32_t wq = rawq[gq][m], wk = rawk[gq][m];
+        qt[gq][m] = pack_bf16x2(bf16lo_to_f32(wq) * e0, bf16hi_to_f32(wq) * e1);
+        kt[gq][m] = pack_bf16x2(bf16lo_to_f32(wk) * exp2_fast(-x[0][c]), bf16hi_to_f32(wk) * exp2_fast(-x[1][c]));
+      }
+    store_kt<4>(Q, 32 * w + r, h, qt);
+    store_kt<4>(K, 32 * w + r, h, kt);
+  }
+  lds_barrier();  // (2) q~, k~ of every tile visible
+
+  // ---- dq of tile w: over the key tiles J the direction keeps ----
+  f32x16_t dqh[2] = {{0.f}, {0.f}};
+  if (w < ntiles) {
+    u32x4_t doB[4];
+#pragma unroll
+    for (int ks = 0; ks < 4; ++ks) doB[ks] = row_frag(DO, 32 * w + r, ks, h);
+    const int j0 = FWD ? 0 : w, j1 = FWD ? w : ntiles - 1;
+#pragma unroll 1
+    for (int J = j0; J <= j1; ++J) {
+      f32x16_t T = {0.f};  // A^T tile: rows j in J, columns i in tile w
+#pragma unroll
+      for (int ks = 0; ks < 4; ++ks) T = mfma(row_frag(V, 32 * J + r, ks, h), doB[ks], T);
+      if (J == w) mask_diag<FWD, false>(T, r, h);
+      u32x4_t f[2];
+      tile_frags(T, f);
+#pragma unroll
+      for (int t = 0; t < 2; ++t) {
+        u32x4_t kf[2];
+        load_tfrag_lds<4>(K + 32 * J * kKtStride, t, r, h, kf);
+        dqh[0] = mfma(kf[0], f[t], dqh[0]);
+        dqh[1] = mfma(kf[1], f[t], dqh[1]);
+      }
+    }
+  }
+  // dq^ waits as bf16 pairs while the other accumulators are at work
+  uint32_t dqp[16];
+#pragma unroll
+  for (int c = 0; c < 16; ++c) dqp[c] = pack_bf16x2(dqh[0][c], dqh[1][c]);
+  // ---- dk, dv of tile w: over the query tiles I the direction keeps ----
+  f32x16_t dkh[2] = {{0.f}, {0.f}};
+  if (w < ntiles) {
+    const int i0 = FWD ? w : 0, i1 = FWD ? ntiles - 1 : w;
+#pragma unroll 1
+    for (int I = i0; I <= i1; ++I) {
+      f32x16_t P = {0.f}, A = {0.f};  // rows i in I, columns j in tile w
+#pragma unroll
+      for (int ks = 0; ks < 4; ++ks) {
+        P = mfma(row_frag(Q, 32 * I + r, ks, h), row_frag(K, 32 * w + r, ks, h), P);
+        A = mfma(row_frag(DO, 32 * I + r, ks, h), row_frag(V, 32 * w + r, ks, h), A);
+      }
+      if (I == w) {
+        mask_diag<FWD, true>(P, r, h);
+        mask_diag<FWD, true>(A, r, h);
+      }
+      u32x4_t pf[2], af[2];
+      tile_frags(P, pf);
+      tile_frags(A, af);
+#pragma unroll
+      for (int t = 0; t < 2; ++t) {
+        u32x4_t df[2], qf[2];
+        load_tfrag_lds<4>(DO + 32 * I * kKtStride, t, r, h, df);
+        load_tfrag_lds<4>(Q + 32 * I * kKtStride, t, r, h, qf);
+        dv[0] = mfma(df[0], pf[t], dv[0]);
+        dv[1] = mfma(df[1], pf[t], dv[1]);
+        dkh[0] = mfma(qf[0], af[t], dkh[0]);
+        dkh[1] = mfma(qf[1], af[t], dkh[1]);
+      }
+    }
+  }
+  // ---- scale back; X = q dq - k dk = s (q~ dq^ - k~ dk^): the exponentials cancel, and the staged rows serve ----
+  f32x16_t X[2];
+  {
+    const int rows_out = rows;
+    const rsrc_t oq = chunk_rsrc(sl.dq + toff, rows_out, 128), okk = chunk_rsrc(sl.dk + toff, rows_out, 128);
+    const rsrc_t ov = chunk_rsrc(sl.dv + toff, rows_out, 128);
+#pragma unroll
+    for (int gq = 0; gq < 4; ++gq) {
+      const u32x4_t qrow = *reinterpret_cast<const u32x4_t*>(Q + (32 * w + r) * kKtStride + 32 * h + 8 * gq);
+      const u32x4_t krow = *reinterpret_cast<const u32x4_t*>(K + (32 * w + r) * kKtStride + 32 * h + 8 * gq);
+      u32x4_t xq, xk, xv;
+#pragma unroll
+      for (int m = 0; m < 4; ++m) {
+        const int c = 4 * gq + m;
+        float a[2], b[2];
+#pragma unroll
+        for (int p = 0; p < 2; ++p) {
+          const float dqc = p ? bf16hi_to_f32(dqp[c]) : bf16lo_to_f32(dqp[c]);
+          const float dkc = dkh[p][c];
+          const float qt = p ? bf16hi_to_f32(qrow[m]) : bf16lo_to_f32(qrow[m]);
+          const float kt = p ? bf16hi_to_f32(krow[m]) : bf16lo_to_f32(krow[m]);
+          X[p][c] = s * (qt * dqc - kt * dkc);
+          a[p] = s * exp2_fast(x[p][c]) * dqc;
+          b[p] = s * exp2_fast(-x[p][c]) * dkc;
+          if (LAST) {
+            a[p] += p ? bf16hi_to_f32(keepq[c]) : bf16lo_to_f32(keepq[c]);
+            b[p] += p ? bf16hi_to_f32(keepk[c]) : bf16lo_to_f32(keepk[c]);
+          }
+        }
+        xq[m] = pack_bf16x2(a[0], a[1]);
+        xk[m] = pack_bf16x2(b[0], b[1]);
+        if (LAST) xv[m] = pack_bf16x2(dv[0][c] * s, dv[1][c] * s);
+        if (!LAST) keepq[c] = xq[m], keepk[c] = xk[m];
+      }
+      if (LAST) {
+        const unsigned off = (unsigned)r * 128u + 64u * h + 16u * gq;
+        __builtin_amdgcn_raw_buffer_store_b128(xq, oq, off, 0, 0);
+        __builtin_amdgcn_raw_buffer_store_b128(xk, okk, off, 0, 0);
+        __builtin_amdgcn_raw_buffer_store_b128(xv, ov, off, 0, 0);
+      }
+    }
+  }
+  lds_barrier();  // (3) nobody reads q~, k~ any more: their space becomes the dg scratch
+  {
+    float* xs = reinterpret_cast<float*>(lds + kBwdLdsQ) + w * 32 * kXStride;
+#pragma unroll
+    for (int gq = 0; gq < 4; ++gq) {
+      const f32x4_t a = {X[0][4 * gq], X[1][4 * gq], X[0][4 * gq + 1], X[1][4 * gq + 1]};
+      const f32x4_t b = {X[0][4 * gq + 2], X[1][4 * gq + 2], X[0][4 * gq + 3], X[1][4 * gq + 3]};
+      *reinterpret_cast<f32x4_t*>(xs + r * kXStride + 32 * h + 8 * gq) = a;
+      *reinterpret_cast<f32x4_t*>(xs + r * kXStride + 32 * h + 8 * gq + 4) = b;
+    }
+    wave_lds_sync();
+    // lane = channel: the tile's total, then (with the totals of the tiles behind it) the running sum over its
+    // tokens against the walking order
+    float acc = 0.f;
+#pragma unroll
+    for (int t = 0; t < 32; ++t) acc += xs[t * kXStride + lane];
+    dgtot[w * 64 + lane] = acc;
+    lds_barrier();  // (4) tile totals of X visible
+    float run = 0.f;
+#pragma unroll
+    for (int t = 0; t < kBwdTiles; ++t) {
+      const float y = dgtot[t * 64 + lane];
+      run += (FWD ? (t > w) : (t < w)) ? y : 0.f;
+    }
+    uint16_t* dg = FWD ? sl.dgf : sl.dgb;
+    const rsrc_t rdg = chunk_rsrc(dg + toff, rows, 128);
+#pragma unroll
+    for (int i = 0; i < 32; ++i) {
+      const int t = FWD ? 31 - i : i;
+      run += xs[t * kXStride + lane];
+      __builtin_amdgcn_raw_buffer_store_b16(f32_to_bf16(run), rdg, (unsigned)t * 128u + 2u * lane, 0, 0);
+    }
+  }
+  return true;
+}
+
+}  // namespace
+
+__global__ __launch_bounds__(512) void gla_backward_mfma_kernel(
+    const uint16_t* __restrict__ q, const uint16_t* __restrict__ k, const uint16_t* __restrict__ v,
+    const uint16_t* __restrict__ gf, const uint16_t* __restrict__ gb, const uint16_t* __restrict__ d_o,
+    uint16_t* __restrict__ dq, uint16_t* __restrict__ dk, uint16_t* __restrict__ dv, uint16_t* __restrict__ dgf,
+    uint16_t* __restrict__ dgb, int* __restrict__ flags, int nslabs, int L, float s) {
+  extern __shared__ __align__(16) char lds[];
+  const int tid = threadIdx.x;
+  const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int lane = tid & 63;
+  const int ntiles = (L + 31) / 32;
+  for (int slab = blockIdx.x; slab < nslabs; slab += gridDim.x) {
+    const size_t base = (size_t)slab * L * 64;
+    const BwdSlab sl{q + base, k + base, v + base, gf + base, gb + base, d_o + base,
+                     dq + base, dk + base, dv + base, dgf + base, dgb + base};
+    f32x16_t dvacc[2] = {{0.f}, {0.f}};
+    uint32_t keepq[16], keepk[16];
+    bool ok = bwd_direction<true, false>(sl, L, ntiles, w, lane, lds, s, dvacc, keepq, keepk);
+    if (ok) {
+      lds_barrier();  // (5) the dg scratch of direction 1 is dead before q~, k~ of direction 2 are staged
+      ok = bwd_direction<false, true>(sl, L, ntiles, w, lane, lds, s, dvacc, keepq, keepk);
+    }
+    if (tid == 0) flags[slab] = ok ? 0 : 1;
+    lds_barrier();  // the next slab restages everything
+  }
+}
+
+bool gla_backward_mfma_supported(int L, int Dk, int Dv, int io_dtype, int gate_dtype, bool bidir) {
+  return bidir && io_dtype == 1 && gate_dtype == 1 && Dk == 64 && Dv == 64 && L <= 32 * kBwdTiles;
+}
+
+// flags: one int per (batch, head) slab, written by every launch: 1 = not computed here (gates out of range)
+int launch_gla_backward_mfma(const void* q, const void* k, const void* v, const void* gf, const void* gb,
+                             const void* d_o, void* dq, void* dk, void* dv, void* dgf, void* dgb, int* flags, int B,
+                             int H, int L, float s, hipStream_t stream) {
+  constexpr int kMaxDevices = 64;
+  static bool attr_done_dev[kMaxDevices] = {};
+  static int num_cu_dev[kMaxDevices] = {};
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return -5;
+  if (!attr_done_dev[dev]) {
+    if (hipFuncSetAttribute(reinterpret_cast<const void*>(gla_backward_mfma_kernel),
+                            hipFuncAttributeMaxDynamicSharedMemorySize, kBwdLdsTotal) != hipSuccess)
+      return -5;
+    int n = 0;
+    if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess) return -5;
+    num_cu_dev[dev] = n > 0 ? n : 256;
+    attr_done_dev[dev] = true;
+  }
+  const int nslabs = B * H;
+  const int grid = nslabs < num_cu_dev[dev] ? nslabs : num_cu_dev[dev];
+  hipLaunchKernelGGL(gla_backward_mfma_kernel, dim3(grid), dim3(512), kBwdLdsTotal, stream, (const uint16_t*)q,
+                     (const uint16_t*)k, (const uint16_t*)v, (const uint16_t*)gf, (const uint16_t*)gb,
+                     (const uint16_t*)d_o, (uint16_t*)dq, (uint16_t*)dk, (uint16_t*)dv, (uint16_t*)dgf, (uint16_t*)dgb,
+                     flags, nslabs, L, s);
+  return hipGetLastError() == hipSuccess ? 0 : -5;
+}
+
+}  // namespace vig

@@ -38,6 +38,7 @@
 // 32 contiguous channels (32*h + 8*g + 2*m + p) of one token.
 #include "common.h"
 #include "launch.h"
+#include "mfma_tiles.h"
 #ifdef VIG_TIMING
 #include <stdlib.h>
 #endif
@@ -65,22 +66,15 @@ __device__ unsigned long long g_stamp[4][8][16];
   } while (0)
 #endif
 
-constexpr float kLog2e = 1.4426950408889634f;
 // fp16 score operands are used while |G_end|/2 * log2(e) <= this for every channel of the chunk: the scaled
 // operands then stay within 2^6 of the inputs' magnitudes (fp16 holds |x| < 65504 and full precision above 6e-5).
 constexpr float kFastHalfRange = 6.0f;
-constexpr int kKtStride = 72;                // bf16 elements per k~ row in LDS (144 B: conflict-free b128 writes)
 constexpr int kRegionBytes = 16 * 1024;      // per wave: k~ scratch, then published U / state fragments / output half
 constexpr int kLdsDvec = 8 * kRegionBytes;   // per wave: 64 chunk decays exp(G_end)
 constexpr int kLdsGend = kLdsDvec + 8 * 64 * 4;  // per wave: 64 anchors G_end * log2(e), laid out [h][p][16]
 constexpr int kLdsVeto = kLdsGend + 8 * 64 * 4;  // one word: some chunk refused the fp16 variant
 constexpr int kLdsGateW = kLdsVeto + 16;          // fused locality gate: the 64 x 9 stencil weights of the slab's head
 constexpr int kLdsTotal = kLdsGateW + 64 * 9 * 4;
-
-__device__ __forceinline__ f32x16_t mfma(const u32x4_t& a, const u32x4_t& b, const f32x16_t& c) {
-  return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, a), __builtin_bit_cast(bf16x8_t, b), c, 0,
-                                                 0, 0);
-}
 
 typedef _Float16 f16x2_t __attribute__((ext_vector_type(2)));
 typedef _Float16 f16x8_t __attribute__((ext_vector_type(8)));
@@ -92,117 +86,6 @@ __device__ __forceinline__ uint32_t pack_f16x2(float lo, float hi) {
   f32x2_t x = {lo, hi};
   f16x2_t y = __builtin_convertvector(x, f16x2_t);  // round to nearest even
   return __builtin_bit_cast(uint32_t, y);
-}
-
-// Channel pair read by lane-row rho of a transposed fragment whose rows span 16*NG channels (NG = 4: 64 channels,
-// every row used; NG = 2: 32 channels, rows 16..31 carry no channel and are zero).  With it, accumulator register
-// 4*g + m of lane half h holds channel 8*NG*h + 8*g + 2*m + p.
-template <int NG>
-__device__ __forceinline__ int cpair(int rho) { return (((rho >> 2) & 1) * (4 * NG)) | ((rho >> 3) << 2) | (rho & 3); }
-template <int NG>
-__device__ __forceinline__ bool row_has_channel(int rho) { return (rho >> 3) < NG; }
-
-// token held by contraction slot e of k-step t for lane half h
-__device__ __forceinline__ int jmap(int t, int h, int e) { return 16 * t + 4 * h + (e & 3) + 8 * (e >> 2); }
-
-__device__ __forceinline__ float exp2_fast(float x) { return __builtin_amdgcn_exp2f(x); }
-
-// LDS traffic inside one wave (k~ rows written by token lanes, read back by channel lanes): the LDS pipe is in
-// order per wave, so only the compiler has to be kept from reordering.
-__device__ __forceinline__ void wave_lds_sync() {
-  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-  __builtin_amdgcn_wave_barrier();
-  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-}
-
-// Workgroup barrier that orders LDS traffic only: global loads issued before it (the next slab's prefetch)
-// stay in flight across it, which a full __syncthreads() fence would drain.
-__device__ __forceinline__ void lds_barrier() {
-  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
-  __builtin_amdgcn_s_barrier();
-  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
-}
-
-// ---------------------------------------------------------------------------------------------------------
-// Loads.  Every tensor chunk is addressed through a raw buffer descriptor whose extent is the chunk's valid rows:
-// the hardware returns zero for anything beyond it, so padding rows need neither clamped addresses nor selects
-// (zero gates, keys and values are exactly what padding tokens have to contribute), and token offsets travel as
-// instruction immediates.
-// ---------------------------------------------------------------------------------------------------------
-typedef __amdgpu_buffer_rsrc_t rsrc_t;
-
-// descriptor of `rows` rows of `row_bytes` starting at p (p and rows are wave-uniform)
-__device__ __forceinline__ rsrc_t chunk_rsrc(const void* p, int rows, int row_bytes) {
-  return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(p), 0, rows * row_bytes, 0x00020000);
-}
-constexpr unsigned kOutOfRange = 0x40000000u;  // byte offset no descriptor of this kernel covers
-
-// raw dwords of the transposed fragments of k-steps [T0, T0+NT): D[t][e] = channels (2*cpair(r), +1) of token
-// jmap(t,h,e); lane rows that carry no channel (NG = 2, rows 16..31) read zeros
-template <int T0, int NT, int NG>
-__device__ __forceinline__ void issue_tdwords(rsrc_t rows, int r, int h, uint32_t (&D)[NT][8]) {
-  constexpr unsigned RB = 32u * NG;  // bytes per row
-  const unsigned base = row_has_channel<NG>(r) ? (4u * h) * RB + 4u * cpair<NG>(r) : kOutOfRange;
-#pragma unroll
-  for (int t = 0; t < NT; ++t)
-#pragma unroll
-    for (int e = 0; e < 8; ++e)
-      D[t][e] = __builtin_amdgcn_raw_buffer_load_b32(rows, base + (unsigned)jmap(T0 + t, 0, e) * RB, 0, 0);
-}
-
-// fragments from raw dwords: frag[t][p] has lane index = channel 2*cpair(r)+p, slots = tokens jmap(t,h,.)
-template <int NT>
-__device__ __forceinline__ void finish_tfrags(const uint32_t (&D)[NT][8], u32x4_t (&frag)[NT][2]) {
-#pragma unroll
-  for (int t = 0; t < NT; ++t)
-#pragma unroll
-    for (int x = 0; x < 4; ++x) {
-      frag[t][0][x] = __builtin_amdgcn_perm(D[t][2 * x + 1], D[t][2 * x], 0x05040100u);
-      frag[t][1][x] = __builtin_amdgcn_perm(D[t][2 * x + 1], D[t][2 * x], 0x07060302u);
-    }
-}
-
-// raw rows of one 32-token tile: lane (r, h) reads token 32*it + r, channels [8*NG*h, +8*NG) as NG 16-byte pieces
-template <int NG>
-__device__ __forceinline__ void issue_raw_tile(rsrc_t rows, int it, int r, int h, u32x4_t (&raw)[NG]) {
-  constexpr unsigned RB = 32u * NG;
-  const unsigned base = (unsigned)r * RB + (16u * NG) * h;
-#pragma unroll
-  for (int gq = 0; gq < NG; ++gq)
-    raw[gq] = __builtin_amdgcn_raw_buffer_load_b128(rows, base + (unsigned)it * 32u * RB + 16u * gq, 0, 0);
-}
-
-// one k-step of transposed fragments from the wave's k~ scratch in LDS
-template <int NG>
-__device__ __forceinline__ void load_tfrag_lds(const uint16_t* kt, int t, int r, int h, u32x4_t (&frag)[2]) {
-  const bool row_ok = row_has_channel<NG>(r);
-  const int c2 = row_ok ? 2 * cpair<NG>(r) : 0;
-  uint32_t D[8];
-#pragma unroll
-  for (int e = 0; e < 8; ++e) {
-    const uint32_t d = *reinterpret_cast<const uint32_t*>(kt + jmap(t, h, e) * kKtStride + c2);
-    D[e] = (NG == 4 || row_ok) ? d : 0u;
-  }
-#pragma unroll
-  for (int x = 0; x < 4; ++x) {
-    frag[0][x] = __builtin_amdgcn_perm(D[2 * x + 1], D[2 * x], 0x05040100u);
-    frag[1][x] = __builtin_amdgcn_perm(D[2 * x + 1], D[2 * x], 0x07060302u);
-  }
-}
-
-// B operand of the cumulative-sum MFMA: ones where token slot j is on the kept side of column token i.
-template <bool FWD>
-__device__ __forceinline__ u32x4_t tri_frag(int t, int it, int r, int h) {
-  const int i = 32 * it + r;
-  u32x4_t f;
-#pragma unroll
-  for (int x = 0; x < 4; ++x) {
-    const int j0 = jmap(t, h, 2 * x), j1 = jmap(t, h, 2 * x + 1);
-    const bool b0 = FWD ? (j0 <= i) : (j0 >= i);
-    const bool b1 = FWD ? (j1 <= i) : (j1 >= i);
-    f[x] = (b0 ? 0x00003F80u : 0u) | (b1 ? 0x3F800000u : 0u);
-  }
-  return f;
 }
 
 template <int NG>
@@ -321,12 +204,6 @@ __device__ __forceinline__ void apply_scores(f32x16_t P, int jt, int r, int h, c
     O1 = mfma(vfrag[t][1], ph, O1);
     O1 = mfma(vfrag[t][1], pl, O1);
   }
-}
-
-template <int NG>
-__device__ __forceinline__ void store_kt(uint16_t* kt, int row, int h, const u32x4_t (&kh)[NG]) {
-#pragma unroll
-  for (int g = 0; g < NG; ++g) *reinterpret_cast<u32x4_t*>(kt + row * kKtStride + 8 * NG * h + 8 * g) = kh[g];
 }
 
 // LDS "unit" u of a region = 64 lanes x 16 B, register-native: lane l owns bytes [(u*64 + l)*16, +16).

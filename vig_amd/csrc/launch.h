@@ -34,4 +34,10 @@ int launch_gla_mfma(const GlaArgs& a);
 bool gla_mfma_gate_grid_ok(int rows, int cols);  // token grids the fused locality gate takes
 size_t gla_mfma_workspace(int B, int H, int L, int Dk, int Dv);
 
+// bf16 matrix-core backward (whole-slab quadratic form); flags[b*H + h] = 1 marks slabs it left to the recurrent kernel
+bool gla_backward_mfma_supported(int L, int Dk, int Dv, int io_dtype, int gate_dtype, bool bidir);
+int launch_gla_backward_mfma(const void* q, const void* k, const void* v, const void* gf, const void* gb,
+                             const void* d_o, void* dq, void* dk, void* dv, void* dgf, void* dgb, int* flags, int B,
+                             int H, int L, float s, hipStream_t stream);
+
 }  // namespace vig

@@ -59,8 +59,13 @@ def gla_bidir_forward(q, k, v, g_fwd, g_bwd=None, scale: float = -1, out_scale: 
     return _gla_bidir_forward_raw(q, k, v, g_fwd, g_bwd, scale, out_scale, exact, out)
 
 
-def gla_bidir_backward(q, k, v, g_fwd, g_bwd, d_o, scale: float = -1, out_scale: float = 1.0):
-    """Gradients of gla_bidir_forward contracted with d_o: (dq, dk, dv, dg_fwd, dg_bwd or None).  fp32 arithmetic."""
+def gla_bidir_backward(q, k, v, g_fwd, g_bwd, d_o, scale: float = -1, out_scale: float = 1.0,
+                       exact: bool = False):
+    """Gradients of gla_bidir_forward contracted with d_o: (dq, dk, dv, dg_fwd, dg_bwd or None).
+
+    bf16 tensors and gates with Dk = Dv = 64, L <= 256 and both directions run on the matrix cores (bf16 operands,
+    fp32 accumulation); everything else, and `exact=True`, on the fp32-arithmetic token-recurrent kernel.
+    """
     lib = _lib.load()
     _check_cuda(q, k, v, g_fwd, g_bwd, d_o)
     q, k, v, g_fwd, d_o = (t.contiguous() for t in (q, k, v, g_fwd, d_o))
@@ -80,7 +85,8 @@ def gla_bidir_backward(q, k, v, g_fwd, g_bwd, d_o, scale: float = -1, out_scale:
         raise _lib.VigGlaError(f"vig_gla_bidir_bwd: shape Dk={Dk}, Dv={Dv} is not built")
     ws = torch.empty(ws_bytes, dtype=torch.uint8, device=q.device)
     with torch.cuda.device(q.device):
-        rc = lib.vig_gla_bidir_bwd(q.data_ptr(), k.data_ptr(), v.data_ptr(), g_fwd.data_ptr(),
+        fn = lib.vig_gla_bidir_bwd_exact if exact else lib.vig_gla_bidir_bwd
+        rc = fn(q.data_ptr(), k.data_ptr(), v.data_ptr(), g_fwd.data_ptr(),
                                    g_bwd.data_ptr() if g_bwd is not None else None, d_o.data_ptr(),
                                    dq.data_ptr(), dk.data_ptr(), dv.data_ptr(), dgf.data_ptr(),
                                    dgb.data_ptr() if dgb is not None else None, ws.data_ptr(), ws_bytes,
