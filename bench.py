@@ -100,38 +100,42 @@ def model_throughput(dev, batch=256, warmup=10, iters=30, tune_gemm=True):
             "ms_per_forward": dt / iters * 1e3, "gemm_solution_tuning": "torch.cuda.tunable" if tuned else None}
 
 
-def backward_time(lib, tensors, s, io_dt, scale, sp, stream, dev, iters=20):
-    """Event-bracketed time of vig_gla_bidir_bwd (fp32 token-recurrent arithmetic) on one input set."""
+def backward_time(lib, sets, s, io_dt, scale, sp, stream, dev, iters=60):
+    """Event-bracketed time of vig_gla_bidir_bwd, rotating over the input sets like the forward loop does."""
     import torch
 
-    q, k, v, gf, gb, o = tensors
-    d_o = torch.randn_like(v)
+    q, k, v, gf, gb, o = sets[0]
+    d_os = [torch.randn_like(t[2]) for t in sets]
     dq, dk, dv, dgf, dgb = (torch.empty_like(t) for t in (q, k, v, gf, gb))
     n = lib.vig_gla_bidir_bwd_workspace(s.B, s.H, s.L, s.Dk, s.Dv, 1)
     if n == 0:
         return None
     ws = torch.empty(n, dtype=torch.uint8, device=dev)
 
-    def run():
+    def run(i):
+        q, k, v, gf, gb, _ = sets[i % len(sets)]
+        d_o = d_os[i % len(sets)]
         rc = lib.vig_gla_bidir_bwd(q.data_ptr(), k.data_ptr(), v.data_ptr(), gf.data_ptr(), gb.data_ptr(), d_o.data_ptr(),
                                    dq.data_ptr(), dk.data_ptr(), dv.data_ptr(), dgf.data_ptr(), dgb.data_ptr(),
                                    ws.data_ptr(), n, s.B, s.H, s.L, s.Dk, s.Dv, scale, 1.0, io_dt, io_dt, sp)
         if rc != 0:
             raise RuntimeError(f"vig_gla_bidir_bwd rc={rc}")
 
-    for _ in range(3):
-        run()
+    for i in range(3):
+        run(i)
     evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(iters)]
-    for a, b in evs:
+    for i, (a, b) in enumerate(evs):
         a.record(stream)
-        run()
+        run(i)
         b.record(stream)
     torch.cuda.synchronize()
     us = sum(a.elapsed_time(b) for a, b in evs) / iters * 1e3
     esz = 4 if s.dtype == "f32" else 2
+    mfma = s.dtype != "f32" and s.Dk == 64 and s.Dv == 64 and s.L <= 256
     alg = s.tokens * esz * ((2 * s.Dk + 2 * s.Dv) + 2 * s.Dk + (2 * s.Dk + s.Dv) + 2 * s.Dk)
     return {"us": us, "algorithmic_bytes": alg, "algorithmic_GBps": alg / (us * 1e-6) / 1e9,
-            "frac_of_hbm_peak": alg / (us * 1e-6) / 1e9 / HBM_PEAK_GBPS, "kernel": "fp32 token-recurrent"}
+            "frac_of_hbm_peak": alg / (us * 1e-6) / 1e9 / HBM_PEAK_GBPS,
+            "kernel": "matrix cores (whole-slab quadratic form), bf16 operands" if mfma else "fp32 token-recurrent"}
 
 
 def main():
@@ -293,7 +297,7 @@ def main():
                      "frac": achieved_gbps / HBM_PEAK_GBPS, "traffic": traffic},
     }
     if args.backward:
-        out["backward"] = backward_time(lib, sets[0], s, io_dt, scale, sp, stream, dev)
+        out["backward"] = backward_time(lib, sets, s, io_dt, scale, sp, stream, dev)
     if args.model:
         out["vig_s_forward"] = model_throughput(dev, tune_gemm=not args.no_gemm_tuning)
     if not args.no_cpu:

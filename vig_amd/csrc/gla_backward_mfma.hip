@@ -42,6 +42,22 @@ constexpr int kXStride = 68;  // floats per token row of the dg scratch (272 B: 
 static_assert(8 * 32 * kXStride * 4 <= 2 * kBwdMatBytes, "dg scratch overlays the q~ and k~ matrices");
 constexpr float kBwdHalfRange = 60.0f;
 
+// Optional phase timing (development builds only: -DVIG_TIMING): lane 0 of every wave of workgroup 0 records the
+// shader clock at the phase boundaries of the first slab, per direction.
+#ifdef VIG_TIMING
+__device__ unsigned long long g_bwd_stamp[2][8][16];
+#define VIG_BWD_STAMP(id)                                                                                   \
+  do {                                                                                                      \
+    __builtin_amdgcn_sched_barrier(0);                                                                      \
+    if (lane == 0 && blockIdx.x == 0 && first_slab) g_bwd_stamp[LAST ? 1 : 0][w][id] = __builtin_readcyclecounter(); \
+    __builtin_amdgcn_sched_barrier(0);                                                                      \
+  } while (0)
+#else
+#define VIG_BWD_STAMP(id) \
+  do {                    \
+  } while (0)
+#endif
+
 // fragment of 8 consecutive channels (k-step ks, lane half h) of a staged row: contraction over channels
 __device__ __forceinline__ u32x4_t row_frag(const uint16_t* mat, int row, int ks, int h) {
   return *reinterpret_cast<const u32x4_t*>(mat + row * kKtStride + 16 * ks + 8 * h);
@@ -73,15 +89,40 @@ struct BwdSlab {
   uint16_t *dq, *dk, *dv, *dgf, *dgb;
 };
 
+// What a wave loads for one direction of one slab (its own 32-token tile), issued one phase ahead.
+struct BwdLoads {
+  uint32_t gD[2][8];             // gate dwords (tokens in the contraction slots)
+  u32x4_t rawq[4], rawk[4];      // q and k rows
+  u32x4_t rawv[4], rawd[4];      // v and do rows (first direction of a slab only)
+};
+struct BwdNext {  // the direction whose loads are issued while this one finishes
+  BwdSlab sl;
+  const uint16_t* g;
+  int L;  // 0: nothing follows (empty descriptors, no memory traffic)
+};
+template <bool WITH_VDO>
+__device__ __forceinline__ void issue_bwd_loads(const BwdNext& n, int w, int r, int h, BwdLoads& ld) {
+  const int rows = __builtin_amdgcn_readfirstlane(min(max(n.L - 32 * w, 0), 32));  // (scalar: descriptors stay in SGPRs)
+  const size_t toff = (size_t)32 * w * 64;
+  issue_tdwords<0, 2, 4>(chunk_rsrc(n.g + toff, rows, 128), r, h, ld.gD);
+  issue_raw_tile<4>(chunk_rsrc(n.sl.q + toff, rows, 128), 0, r, h, ld.rawq);
+  issue_raw_tile<4>(chunk_rsrc(n.sl.k + toff, rows, 128), 0, r, h, ld.rawk);
+  if (WITH_VDO) {
+    issue_raw_tile<4>(chunk_rsrc(n.sl.v + toff, rows, 128), 0, r, h, ld.rawv);
+    issue_raw_tile<4>(chunk_rsrc(n.sl.d_o + toff, rows, 128), 0, r, h, ld.rawd);
+  }
+}
+
 // One direction of one slab, for wave w (tile w).  dv accumulates over both directions (raw, unscaled).  The first
-// direction (LAST = false) leaves its dq and dk as bf16 pairs in keepq / keepk and stages v and do; the second adds its
-// own and stores dq, dk, dv.  Returns false, for every wave alike and before it has stored anything, when the gates
+// direction (LAST = false) stages v and do and parks its dq and dk, rounded to bf16, in the output tensors; the second
+// adds its own to them and stores dq, dk, dv.  Returns false, for every wave alike and before it has stored anything, when the gates
 // are out of range.
 template <bool FWD, bool LAST>
 __device__ __forceinline__ bool bwd_direction(const BwdSlab& sl, int L, int ntiles, int w, int lane, char* lds,
-                                              float s, f32x16_t (&dv)[2], uint32_t (&keepq)[16],
-                                              uint32_t (&keepk)[16]) {
+                                              float s, f32x16_t (&dv)[2], BwdLoads& ld, const BwdNext& nxt,
+                                              bool first_slab) {
   constexpr bool stage_vdo = !LAST;
+  asm volatile("" : "+v"(lane));  // per-lane constants are rebuilt per direction instead of living across the slab loop
   const int r = lane & 31, h = lane >> 5;
   uint16_t* Q = reinterpret_cast<uint16_t*>(lds + kBwdLdsQ);
   uint16_t* K = reinterpret_cast<uint16_t*>(lds + kBwdLdsK);
@@ -90,31 +131,24 @@ __device__ __forceinline__ bool bwd_direction(const BwdSlab& sl, int L, int ntil
   float* tot = reinterpret_cast<float*>(lds + kBwdLdsTot);
   float* offs = reinterpret_cast<float*>(lds + kBwdLdsOff) + w * 64;
   float* dgtot = reinterpret_cast<float*>(lds + kBwdLdsDgTot);
-  const int rows = min(max(L - 32 * w, 0), 32);  // valid tokens of this wave's tile
+  const int rows = __builtin_amdgcn_readfirstlane(min(max(L - 32 * w, 0), 32));  // valid tokens of this wave's tile
   const size_t toff = (size_t)32 * w * 64;
-  const uint16_t* g = FWD ? sl.gf : sl.gb;
-  const rsrc_t rq = chunk_rsrc(sl.q + toff, rows, 128), rk = chunk_rsrc(sl.k + toff, rows, 128);
-  const rsrc_t rg = chunk_rsrc(g + toff, rows, 128);
 
-  // ---- loads of this tile: gates (tokens in the contraction slots), q and k rows; v and do rows once per slab ----
-  uint32_t gD[2][8];
-  issue_tdwords<0, 2, 4>(rg, r, h, gD);
-  u32x4_t rawq[4], rawk[4];
-  issue_raw_tile<4>(rq, 0, r, h, rawq);
-  issue_raw_tile<4>(rk, 0, r, h, rawk);
+  VIG_BWD_STAMP(0);
+  // ---- this tile's loads were issued a phase ago; v and do rows go to LDS once per slab ----
   if (stage_vdo) {
-    u32x4_t rv[4], rd[4];
-    issue_raw_tile<4>(chunk_rsrc(sl.v + toff, rows, 128), 0, r, h, rv);
-    issue_raw_tile<4>(chunk_rsrc(sl.d_o + toff, rows, 128), 0, r, h, rd);
-    store_kt<4>(V, 32 * w + r, h, rv);
-    store_kt<4>(DO, 32 * w + r, h, rd);
+    store_kt<4>(V, 32 * w + r, h, ld.rawv);
+    store_kt<4>(DO, 32 * w + r, h, ld.rawd);
   }
+  u32x4_t rawq[4], rawk[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) rawq[i] = ld.rawq[i], rawk[i] = ld.rawk[i];
 
   // ---- tile-local cumulative gates: G^T = g^T T, lane = token, registers = channels 32h + 8g + 2m + p ----
   f32x16_t G[2];
   {
     u32x4_t gfrag[2][2];
-    finish_tfrags<2>(gD, gfrag);
+    finish_tfrags<2>(ld.gD, gfrag);
     const u32x4_t tri0 = tri_frag<FWD>(0, 0, r, h), tri1 = tri_frag<FWD>(1, 0, r, h);
 #pragma unroll
     for (int p = 0; p < 2; ++p) {
@@ -132,6 +166,7 @@ __device__ __forceinline__ bool bwd_direction(const BwdSlab& sl, int L, int ntil
       tot[w * 64 + ch + 1] = G[1][c];
     }
   }
+  VIG_BWD_STAMP(1);
   lds_barrier();  // (1) tile totals (and v, do rows) visible; the previous direction's scratch is dead
   // lane = channel: gates before this tile in walking order, minus the anchor (half the slab total)
   bool out_of_range;
@@ -146,6 +181,7 @@ __device__ __forceinline__ bool bwd_direction(const BwdSlab& sl, int L, int ntil
     offs[lane] = pre - 0.5f * all;
     out_of_range = __builtin_amdgcn_ballot_w64(fabsf(all) * (0.5f * kLog2e) > kBwdHalfRange) != 0;
   }
+  VIG_BWD_STAMP(2);
   if (out_of_range) return false;  // same totals in every wave: the whole workgroup leaves together
   wave_lds_sync();
   // x = (G - a) * log2(e) per (token, channel): q~ = q 2^x, k~ = k 2^-x
@@ -175,7 +211,9 @@ __device__ __forceinline__ bool bwd_direction(const BwdSlab& sl, int L, int ntil
     store_kt<4>(Q, 32 * w + r, h, qt);
     store_kt<4>(K, 32 * w + r, h, kt);
   }
+  VIG_BWD_STAMP(3);
   lds_barrier();  // (2) q~, k~ of every tile visible
+  VIG_BWD_STAMP(4);
 
   // ---- dq of tile w: over the key tiles J the direction keeps ----
   f32x16_t dqh[2] = {{0.f}, {0.f}};
@@ -201,47 +239,64 @@ __device__ __forceinline__ bool bwd_direction(const BwdSlab& sl, int L, int ntil
       }
     }
   }
+  VIG_BWD_STAMP(5);
   // dq^ waits as bf16 pairs while the other accumulators are at work
   uint32_t dqp[16];
 #pragma unroll
   for (int c = 0; c < 16; ++c) dqp[c] = pack_bf16x2(dqh[0][c], dqh[1][c]);
-  // ---- dk, dv of tile w: over the query tiles I the direction keeps ----
+  // the first direction parked its dq and dk (rounded to bf16) in the output tensors; fetch them under the loops
+  const rsrc_t oq = chunk_rsrc(sl.dq + toff, rows, 128), okk = chunk_rsrc(sl.dk + toff, rows, 128);
+  u32x4_t prevq[4], prevk[4];
+  if (LAST) {
+#pragma unroll
+    for (int gq = 0; gq < 4; ++gq) {
+      const unsigned off = (unsigned)r * 128u + 64u * h + 16u * gq;
+      prevq[gq] = __builtin_amdgcn_raw_buffer_load_b128(oq, off, 0, 0);
+      prevk[gq] = __builtin_amdgcn_raw_buffer_load_b128(okk, off, 0, 0);
+    }
+  }
+  // ---- dv, then dk of tile w: over the query tiles I the direction keeps (two loops: fewer live registers) ----
   f32x16_t dkh[2] = {{0.f}, {0.f}};
   if (w < ntiles) {
     const int i0 = FWD ? w : 0, i1 = FWD ? ntiles - 1 : w;
 #pragma unroll 1
     for (int I = i0; I <= i1; ++I) {
-      f32x16_t P = {0.f}, A = {0.f};  // rows i in I, columns j in tile w
+      f32x16_t P = {0.f};  // rows i in I, columns j in tile w
 #pragma unroll
-      for (int ks = 0; ks < 4; ++ks) {
-        P = mfma(row_frag(Q, 32 * I + r, ks, h), row_frag(K, 32 * w + r, ks, h), P);
-        A = mfma(row_frag(DO, 32 * I + r, ks, h), row_frag(V, 32 * w + r, ks, h), A);
-      }
-      if (I == w) {
-        mask_diag<FWD, true>(P, r, h);
-        mask_diag<FWD, true>(A, r, h);
-      }
-      u32x4_t pf[2], af[2];
+      for (int ks = 0; ks < 4; ++ks) P = mfma(row_frag(Q, 32 * I + r, ks, h), row_frag(K, 32 * w + r, ks, h), P);
+      if (I == w) mask_diag<FWD, true>(P, r, h);
+      u32x4_t pf[2];
       tile_frags(P, pf);
+#pragma unroll
+      for (int t = 0; t < 2; ++t) {
+        u32x4_t df[2];
+        load_tfrag_lds<4>(DO + 32 * I * kKtStride, t, r, h, df);
+        dv[0] = mfma(df[0], pf[t], dv[0]);
+        dv[1] = mfma(df[1], pf[t], dv[1]);
+      }
+    }
+#pragma unroll 1
+    for (int I = i0; I <= i1; ++I) {
+      f32x16_t A = {0.f};
+#pragma unroll
+      for (int ks = 0; ks < 4; ++ks) A = mfma(row_frag(DO, 32 * I + r, ks, h), row_frag(V, 32 * w + r, ks, h), A);
+      if (I == w) mask_diag<FWD, true>(A, r, h);
+      u32x4_t af[2];
       tile_frags(A, af);
 #pragma unroll
       for (int t = 0; t < 2; ++t) {
-        u32x4_t df[2], qf[2];
-        load_tfrag_lds<4>(DO + 32 * I * kKtStride, t, r, h, df);
+        u32x4_t qf[2];
         load_tfrag_lds<4>(Q + 32 * I * kKtStride, t, r, h, qf);
-        dv[0] = mfma(df[0], pf[t], dv[0]);
-        dv[1] = mfma(df[1], pf[t], dv[1]);
         dkh[0] = mfma(qf[0], af[t], dkh[0]);
         dkh[1] = mfma(qf[1], af[t], dkh[1]);
       }
     }
   }
+  VIG_BWD_STAMP(6);
   // ---- scale back; X = q dq - k dk = s (q~ dq^ - k~ dk^): the exponentials cancel, and the staged rows serve ----
   f32x16_t X[2];
   {
-    const int rows_out = rows;
-    const rsrc_t oq = chunk_rsrc(sl.dq + toff, rows_out, 128), okk = chunk_rsrc(sl.dk + toff, rows_out, 128);
-    const rsrc_t ov = chunk_rsrc(sl.dv + toff, rows_out, 128);
+    const rsrc_t ov = chunk_rsrc(sl.dv + toff, rows, 128);
 #pragma unroll
     for (int gq = 0; gq < 4; ++gq) {
       const u32x4_t qrow = *reinterpret_cast<const u32x4_t*>(Q + (32 * w + r) * kKtStride + 32 * h + 8 * gq);
@@ -261,23 +316,21 @@ __device__ __forceinline__ bool bwd_direction(const BwdSlab& sl, int L, int ntil
           a[p] = s * exp2_fast(x[p][c]) * dqc;
           b[p] = s * exp2_fast(-x[p][c]) * dkc;
           if (LAST) {
-            a[p] += p ? bf16hi_to_f32(keepq[c]) : bf16lo_to_f32(keepq[c]);
-            b[p] += p ? bf16hi_to_f32(keepk[c]) : bf16lo_to_f32(keepk[c]);
+            a[p] += p ? bf16hi_to_f32(prevq[gq][m]) : bf16lo_to_f32(prevq[gq][m]);
+            b[p] += p ? bf16hi_to_f32(prevk[gq][m]) : bf16lo_to_f32(prevk[gq][m]);
           }
         }
         xq[m] = pack_bf16x2(a[0], a[1]);
         xk[m] = pack_bf16x2(b[0], b[1]);
         if (LAST) xv[m] = pack_bf16x2(dv[0][c] * s, dv[1][c] * s);
-        if (!LAST) keepq[c] = xq[m], keepk[c] = xk[m];
       }
-      if (LAST) {
-        const unsigned off = (unsigned)r * 128u + 64u * h + 16u * gq;
-        __builtin_amdgcn_raw_buffer_store_b128(xq, oq, off, 0, 0);
-        __builtin_amdgcn_raw_buffer_store_b128(xk, okk, off, 0, 0);
-        __builtin_amdgcn_raw_buffer_store_b128(xv, ov, off, 0, 0);
-      }
+      const unsigned off = (unsigned)r * 128u + 64u * h + 16u * gq;
+      __builtin_amdgcn_raw_buffer_store_b128(xq, oq, off, 0, 0);
+      __builtin_amdgcn_raw_buffer_store_b128(xk, okk, off, 0, 0);
+      if (LAST) __builtin_amdgcn_raw_buffer_store_b128(xv, ov, off, 0, 0);
     }
   }
+  VIG_BWD_STAMP(7);
   lds_barrier();  // (3) nobody reads q~, k~ any more: their space becomes the dg scratch
   {
     float* xs = reinterpret_cast<float*>(lds + kBwdLdsQ) + w * 32 * kXStride;
@@ -289,28 +342,43 @@ __device__ __forceinline__ bool bwd_direction(const BwdSlab& sl, int L, int ntil
       *reinterpret_cast<f32x4_t*>(xs + r * kXStride + 32 * h + 8 * gq + 4) = b;
     }
     wave_lds_sync();
+    // the next direction's loads travel while this one scans and stores
+    issue_bwd_loads<LAST>(nxt, w, r, h, ld);
     // lane = channel: the tile's total, then (with the totals of the tiles behind it) the running sum over its
-    // tokens against the walking order
+    // tokens against the walking order, written back in place
     float acc = 0.f;
 #pragma unroll
     for (int t = 0; t < 32; ++t) acc += xs[t * kXStride + lane];
     dgtot[w * 64 + lane] = acc;
+    VIG_BWD_STAMP(8);
     lds_barrier();  // (4) tile totals of X visible
+    VIG_BWD_STAMP(9);
     float run = 0.f;
 #pragma unroll
     for (int t = 0; t < kBwdTiles; ++t) {
       const float y = dgtot[t * 64 + lane];
       run += (FWD ? (t > w) : (t < w)) ? y : 0.f;
     }
-    uint16_t* dg = FWD ? sl.dgf : sl.dgb;
-    const rsrc_t rdg = chunk_rsrc(dg + toff, rows, 128);
 #pragma unroll
     for (int i = 0; i < 32; ++i) {
       const int t = FWD ? 31 - i : i;
       run += xs[t * kXStride + lane];
-      __builtin_amdgcn_raw_buffer_store_b16(f32_to_bf16(run), rdg, (unsigned)t * 128u + 2u * lane, 0, 0);
+      xs[t * kXStride + lane] = run;
+    }
+    wave_lds_sync();
+    // back to lane = token: 16-byte stores of the gate gradient
+    uint16_t* dg = FWD ? sl.dgf : sl.dgb;
+    const rsrc_t rdg = chunk_rsrc(dg + toff, rows, 128);
+#pragma unroll
+    for (int gq = 0; gq < 4; ++gq) {
+      const f32x4_t a = *reinterpret_cast<const f32x4_t*>(xs + r * kXStride + 32 * h + 8 * gq);
+      const f32x4_t b = *reinterpret_cast<const f32x4_t*>(xs + r * kXStride + 32 * h + 8 * gq + 4);
+      const u32x4_t out = {pack_bf16x2(a[0], a[1]), pack_bf16x2(a[2], a[3]), pack_bf16x2(b[0], b[1]),
+                           pack_bf16x2(b[2], b[3])};
+      __builtin_amdgcn_raw_buffer_store_b128(out, rdg, (unsigned)r * 128u + 64u * h + 16u * gq, 0, 0);
     }
   }
+  VIG_BWD_STAMP(10);
   return true;
 }
 
@@ -326,21 +394,48 @@ __global__ __launch_bounds__(512) void gla_backward_mfma_kernel(
   const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int lane = tid & 63;
   const int ntiles = (L + 31) / 32;
+  auto slab_of = [&](int i) {
+    const size_t base = (size_t)i * L * 64;
+    return BwdSlab{q + base, k + base, v + base, gf + base, gb + base, d_o + base,
+                   dq + base, dk + base, dv + base, dgf + base, dgb + base};
+  };
+  const int r = lane & 31, h = lane >> 5;
+#ifdef VIG_BWD_STAGGER
+  // experiment: half of the workgroups start late, so that their memory phases meet the others' compute phases
+  if ((blockIdx.x >> 3) & 1) {
+    const unsigned long long t0 = wall_clock64();
+    while (wall_clock64() - t0 < (unsigned long long)(VIG_BWD_STAGGER) * 100ull) __builtin_amdgcn_s_sleep(16);
+  }
+#endif
+  BwdLoads ld;
+  if ((int)blockIdx.x < nslabs) {
+    const BwdSlab s0 = slab_of(blockIdx.x);
+    issue_bwd_loads<true>(BwdNext{s0, s0.gf, L}, w, r, h, ld);
+  }
   for (int slab = blockIdx.x; slab < nslabs; slab += gridDim.x) {
-    const size_t base = (size_t)slab * L * 64;
-    const BwdSlab sl{q + base, k + base, v + base, gf + base, gb + base, d_o + base,
-                     dq + base, dk + base, dv + base, dgf + base, dgb + base};
+    const BwdSlab sl = slab_of(slab);
+    const int following = slab + (int)gridDim.x;
+    const BwdSlab sn = slab_of(following < nslabs ? following : slab);
+    const BwdNext second{sl, sl.gb, L}, next_first{sn, sn.gf, following < nslabs ? L : 0};
     f32x16_t dvacc[2] = {{0.f}, {0.f}};
-    uint32_t keepq[16], keepk[16];
-    bool ok = bwd_direction<true, false>(sl, L, ntiles, w, lane, lds, s, dvacc, keepq, keepk);
+    const bool first_slab = slab == (int)blockIdx.x;
+    bool ok = bwd_direction<true, false>(sl, L, ntiles, w, lane, lds, s, dvacc, ld, second, first_slab);
     if (ok) {
       lds_barrier();  // (5) the dg scratch of direction 1 is dead before q~, k~ of direction 2 are staged
-      ok = bwd_direction<false, true>(sl, L, ntiles, w, lane, lds, s, dvacc, keepq, keepk);
+      ok = bwd_direction<false, true>(sl, L, ntiles, w, lane, lds, s, dvacc, ld, next_first, first_slab);
     }
+    // a direction that left early has not issued the loads of the slab that follows
+    if (!ok) issue_bwd_loads<true>(next_first, w, r, h, ld);
     if (tid == 0) flags[slab] = ok ? 0 : 1;
     lds_barrier();  // the next slab restages everything
   }
 }
+
+#ifdef VIG_TIMING
+extern "C" int vig_debug_read_bwd_stamps(unsigned long long* host_out) {
+  return hipMemcpyFromSymbol(host_out, HIP_SYMBOL(g_bwd_stamp), sizeof(g_bwd_stamp)) == hipSuccess ? 0 : -5;
+}
+#endif
 
 bool gla_backward_mfma_supported(int L, int Dk, int Dv, int io_dtype, int gate_dtype, bool bidir) {
   return bidir && io_dtype == 1 && gate_dtype == 1 && Dk == 64 && Dv == 64 && L <= 32 * kBwdTiles;
