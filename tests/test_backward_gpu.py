@@ -54,13 +54,13 @@ def test_backward_fp32_head_dims_and_causal(Dk, Dv):
 
 
 def test_backward_bf16_io():
-    """bf16 tensors and gates, fp32 arithmetic inside: every gradient within half an output ulp (2^-8 relative,
+    """bf16 tensors and gates through the exact path, fp32 arithmetic inside: every gradient within half an output ulp (2^-8 relative,
     elementwise, plus a small absolute floor) of the oracle on the same bf16-rounded inputs."""
     announce("backward bf16 io, ViG-S head shape")
     q, k, v, gf, gb = make_gla_inputs(2, 3, 196, 32, 64, seed=12, dtype=torch.bfloat16)
     do = _do(v.shape, 9, torch.bfloat16)
     want = O.bidir_gla_backward(f64(q), f64(k), f64(v), f64(gf), f64(gb), f64(do), out_scale=0.25)
-    got = vig_amd.gla_bidir_backward(*(t.cuda() for t in (q, k, v, gf, gb, do)), out_scale=0.25)
+    got = vig_amd.gla_bidir_backward(*(t.cuda() for t in (q, k, v, gf, gb, do)), out_scale=0.25, exact=True)
     for name, g_, w_ in zip(("dq", "dk", "dv", "dg_fwd", "dg_bwd"), got, want):
         err = np.abs(f64(g_) - w_)
         assert np.all(err <= 2.0 ** -8 * np.abs(w_) + 1e-3 * np.abs(w_).max()), name
@@ -107,21 +107,23 @@ def _check_mfma(got, want, q, tol=MFMA_BWD_TOL):
         assert e <= tol, (name, e)
 
 
-@pytest.mark.parametrize("B,H,L", [(2, 2, 1), (1, 3, 17), (2, 1, 32), (1, 2, 33), (2, 2, 64), (2, 3, 196),
-                                   (1, 2, 255), (1, 3, 256)])
-def test_backward_mfma_lengths(B, H, L):
-    announce(f"backward on the matrix cores B{B} H{H} L={L}")
-    q, k, v, gf, gb = make_gla_inputs(B, H, L, 64, 64, seed=500 + L, dtype=torch.bfloat16)
+@pytest.mark.parametrize("B,H,L,Dk", [(2, 2, 1, 64), (1, 3, 17, 64), (2, 1, 32, 64), (1, 2, 33, 64), (2, 2, 64, 64),
+                                      (2, 3, 196, 64), (1, 2, 255, 64), (1, 3, 256, 64), (2, 2, 1, 32), (1, 3, 33, 32),
+                                      (2, 6, 196, 32), (1, 2, 256, 32)])
+def test_backward_mfma_lengths(B, H, L, Dk):
+    announce(f"backward on the matrix cores B{B} H{H} L={L} Dk={Dk}")
+    q, k, v, gf, gb = make_gla_inputs(B, H, L, Dk, 64, seed=500 + L, dtype=torch.bfloat16)
     do = _do(v.shape, 10, torch.bfloat16)
     want = O.bidir_gla_backward(f64(q), f64(k), f64(v), f64(gf), f64(gb), f64(do), out_scale=0.5)
     got = vig_amd.gla_bidir_backward(*(t.cuda() for t in (q, k, v, gf, gb, do)), out_scale=0.5)
     _check_mfma(got, want, q)
 
 
-def test_backward_mfma_many_slabs_against_exact_path():
+@pytest.mark.parametrize("Dk", [64, 32])
+def test_backward_mfma_many_slabs_against_exact_path(Dk):
     """More slabs than workgroups (persistent loop), against the fp32-arithmetic kernel on the same inputs."""
-    announce("backward on the matrix cores, 600 slabs, against the recurrent kernel")
-    q, k, v, gf, gb = (t.cuda() for t in make_gla_inputs(100, 6, 196, 64, 64, seed=77, dtype=torch.bfloat16))
+    announce(f"backward on the matrix cores, 600 slabs, Dk={Dk}, against the recurrent kernel")
+    q, k, v, gf, gb = (t.cuda() for t in make_gla_inputs(100, 6, 196, Dk, 64, seed=77, dtype=torch.bfloat16))
     do = _do(v.shape, 11, torch.bfloat16).cuda()
     want = [f64(t) for t in vig_amd.gla_bidir_backward(q, k, v, gf, gb, do, out_scale=0.5, exact=True)]
     got = vig_amd.gla_bidir_backward(q, k, v, gf, gb, do, out_scale=0.5)

@@ -276,7 +276,7 @@ int launch_gla_backward(const void* q, const void* k, const void* v, const void*
   if (!exact && gla_backward_mfma_supported(L, Dk, Dv, io_dtype, gate_dtype, g_bwd != nullptr)) {
     int* flags = reinterpret_cast<int*>((float*)workspace + recurrent_floats(B, H, L, Dk, Dv, 1));
     const int rc = launch_gla_backward_mfma(q, k, v, g_fwd, g_bwd, d_o, dq, dk, dv, dg_fwd, dg_bwd, flags, B, H, L,
-                                            scale * out_scale, stream);
+                                            Dk, scale * out_scale, stream);
     if (rc != 0) return rc;
     a.only_flagged = flags;  // slabs with gates beyond the matrix-core kernel's range
   }

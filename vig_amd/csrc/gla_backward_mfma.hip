@@ -1,4 +1,5 @@
-// Backward of the bidirectional GLA op on MFMA tiles (gfx950): bf16 tensors and gates, Dk = Dv = 64, L <= 256.
+// Backward of the bidirectional GLA op on MFMA tiles (gfx950): bf16 tensors and gates, Dk in {32, 64}, Dv = 64,
+// L <= 256.
 //
 // Per direction the whole (batch, head) slab is one quadratic form (no chunk states): with G the inclusive
 // cumulative log-gate along the direction and the anchor a = G_total / 2,
@@ -72,14 +73,16 @@ __device__ __forceinline__ void tile_frags(const f32x16_t& T, u32x4_t (&f)[2]) {
     for (int x = 0; x < 4; ++x) f[t][x] = pack_bf16x2(T[8 * t + 2 * x], T[8 * t + 2 * x + 1]);
 }
 
-// keeps the entries of a diagonal tile the direction uses; ROWS_ARE_QUERIES: rows i, column j (else rows j, column i)
+// keeps the entries of a diagonal tile (diag) the direction uses, and all of any other tile; ROWS_ARE_QUERIES: rows
+// i, column j (else rows j, column i).  Selects, not a branch around them: a branch between the matrix instructions
+// and the first vector read of their result left that read without its wait states in one build of this kernel.
 template <bool FWD, bool ROWS_ARE_QUERIES>
-__device__ __forceinline__ void mask_diag(f32x16_t& T, int r, int h) {
+__device__ __forceinline__ void mask_diag(f32x16_t& T, int r, int h, bool diag) {
 #pragma unroll
   for (int c = 0; c < 16; ++c) {
     const int row = 8 * (c >> 2) + 4 * h + (c & 3);
     const int i = ROWS_ARE_QUERIES ? row : r, j = ROWS_ARE_QUERIES ? r : row;
-    const bool keep = FWD ? (j <= i) : (j >= i);
+    const bool keep = !diag || (FWD ? (j <= i) : (j >= i));
     T[c] = keep ? T[c] : 0.f;
   }
 }
@@ -90,9 +93,10 @@ struct BwdSlab {
 };
 
 // What a wave loads for one direction of one slab (its own 32-token tile), issued one phase ahead.
+template <int NG>
 struct BwdLoads {
   uint32_t gD[2][8];             // gate dwords (tokens in the contraction slots)
-  u32x4_t rawq[4], rawk[4];      // q and k rows
+  u32x4_t rawq[NG], rawk[NG];    // q and k rows
   u32x4_t rawv[4], rawd[4];      // v and do rows (first direction of a slab only)
 };
 struct BwdNext {  // the direction whose loads are issued while this one finishes
@@ -100,16 +104,17 @@ struct BwdNext {  // the direction whose loads are issued while this one finishe
   const uint16_t* g;
   int L;  // 0: nothing follows (empty descriptors, no memory traffic)
 };
-template <bool WITH_VDO>
-__device__ __forceinline__ void issue_bwd_loads(const BwdNext& n, int w, int r, int h, BwdLoads& ld) {
+template <bool WITH_VDO, int NG>
+__device__ __forceinline__ void issue_bwd_loads(const BwdNext& n, int w, int r, int h, BwdLoads<NG>& ld) {
+  constexpr int DK = 16 * NG;
   const int rows = __builtin_amdgcn_readfirstlane(min(max(n.L - 32 * w, 0), 32));  // (scalar: descriptors stay in SGPRs)
-  const size_t toff = (size_t)32 * w * 64;
-  issue_tdwords<0, 2, 4>(chunk_rsrc(n.g + toff, rows, 128), r, h, ld.gD);
-  issue_raw_tile<4>(chunk_rsrc(n.sl.q + toff, rows, 128), 0, r, h, ld.rawq);
-  issue_raw_tile<4>(chunk_rsrc(n.sl.k + toff, rows, 128), 0, r, h, ld.rawk);
+  const size_t tk = (size_t)32 * w * DK, tv = (size_t)32 * w * 64;
+  issue_tdwords<0, 2, NG>(chunk_rsrc(n.g + tk, rows, 2 * DK), r, h, ld.gD);
+  issue_raw_tile<NG>(chunk_rsrc(n.sl.q + tk, rows, 2 * DK), 0, r, h, ld.rawq);
+  issue_raw_tile<NG>(chunk_rsrc(n.sl.k + tk, rows, 2 * DK), 0, r, h, ld.rawk);
   if (WITH_VDO) {
-    issue_raw_tile<4>(chunk_rsrc(n.sl.v + toff, rows, 128), 0, r, h, ld.rawv);
-    issue_raw_tile<4>(chunk_rsrc(n.sl.d_o + toff, rows, 128), 0, r, h, ld.rawd);
+    issue_raw_tile<4>(chunk_rsrc(n.sl.v + tv, rows, 128), 0, r, h, ld.rawv);
+    issue_raw_tile<4>(chunk_rsrc(n.sl.d_o + tv, rows, 128), 0, r, h, ld.rawd);
   }
 }
 
@@ -117,11 +122,13 @@ __device__ __forceinline__ void issue_bwd_loads(const BwdNext& n, int w, int r, 
 // direction (LAST = false) stages v and do and parks its dq and dk, rounded to bf16, in the output tensors; the second
 // adds its own to them and stores dq, dk, dv.  Returns false, for every wave alike and before it has stored anything, when the gates
 // are out of range.
-template <bool FWD, bool LAST>
+template <bool FWD, bool LAST, int NG>
 __device__ __forceinline__ bool bwd_direction(const BwdSlab& sl, int L, int ntiles, int w, int lane, char* lds,
-                                              float s, f32x16_t (&dv)[2], BwdLoads& ld, const BwdNext& nxt,
+                                              float s, f32x16_t (&dv)[2], BwdLoads<NG>& ld, const BwdNext& nxt,
                                               bool first_slab) {
   constexpr bool stage_vdo = !LAST;
+  constexpr int DK = 16 * NG;   // channels of q, k and the gates
+  constexpr int HC = 8 * NG;    // channels per lane half
   asm volatile("" : "+v"(lane));  // per-lane constants are rebuilt per direction instead of living across the slab loop
   const int r = lane & 31, h = lane >> 5;
   uint16_t* Q = reinterpret_cast<uint16_t*>(lds + kBwdLdsQ);
@@ -132,7 +139,7 @@ __device__ __forceinline__ bool bwd_direction(const BwdSlab& sl, int L, int ntil
   float* offs = reinterpret_cast<float*>(lds + kBwdLdsOff) + w * 64;
   float* dgtot = reinterpret_cast<float*>(lds + kBwdLdsDgTot);
   const int rows = __builtin_amdgcn_readfirstlane(min(max(L - 32 * w, 0), 32));  // valid tokens of this wave's tile
-  const size_t toff = (size_t)32 * w * 64;
+  const size_t tk = (size_t)32 * w * DK, tv = (size_t)32 * w * 64;
 
   VIG_BWD_STAMP(0);
   // ---- this tile's loads were issued a phase ago; v and do rows go to LDS once per slab ----
@@ -140,15 +147,15 @@ __device__ __forceinline__ bool bwd_direction(const BwdSlab& sl, int L, int ntil
     store_kt<4>(V, 32 * w + r, h, ld.rawv);
     store_kt<4>(DO, 32 * w + r, h, ld.rawd);
   }
-  u32x4_t rawq[4], rawk[4];
+  u32x4_t rawq[NG], rawk[NG];
 #pragma unroll
-  for (int i = 0; i < 4; ++i) rawq[i] = ld.rawq[i], rawk[i] = ld.rawk[i];
+  for (int i = 0; i < NG; ++i) rawq[i] = ld.rawq[i], rawk[i] = ld.rawk[i];
 
-  // ---- tile-local cumulative gates: G^T = g^T T, lane = token, registers = channels 32h + 8g + 2m + p ----
+  // ---- tile-local cumulative gates: G^T = g^T T, lane = token, registers = channels HC*h + 8g + 2m + p ----
   f32x16_t G[2];
   {
     u32x4_t gfrag[2][2];
-    finish_tfrags<2>(ld.gD, gfrag);
+    finish_tfrags<2>(ld.gD, gfrag);  // (rows that carry no channel, NG = 2, hold zeros)
     const u32x4_t tri0 = tri_frag<FWD>(0, 0, r, h), tri1 = tri_frag<FWD>(1, 0, r, h);
 #pragma unroll
     for (int p = 0; p < 2; ++p) {
@@ -160,8 +167,8 @@ __device__ __forceinline__ bool bwd_direction(const BwdSlab& sl, int L, int ntil
   // the tile total sits at its last token in walking order
   if (r == (FWD ? 31 : 0)) {
 #pragma unroll
-    for (int c = 0; c < 16; ++c) {
-      const int ch = 32 * h + 8 * (c >> 2) + 2 * (c & 3);
+    for (int c = 0; c < 4 * NG; ++c) {
+      const int ch = HC * h + 8 * (c >> 2) + 2 * (c & 3);
       tot[w * 64 + ch] = G[0][c];
       tot[w * 64 + ch + 1] = G[1][c];
     }
@@ -174,7 +181,7 @@ __device__ __forceinline__ bool bwd_direction(const BwdSlab& sl, int L, int ntil
     float pre = 0.f, all = 0.f;
 #pragma unroll
     for (int t = 0; t < kBwdTiles; ++t) {
-      const float x = tot[t * 64 + lane];
+      const float x = lane < DK ? tot[t * 64 + lane] : 0.f;
       all += x;
       pre += (FWD ? (t < w) : (t > w)) ? x : 0.f;
     }
@@ -185,11 +192,11 @@ __device__ __forceinline__ bool bwd_direction(const BwdSlab& sl, int L, int ntil
   if (out_of_range) return false;  // same totals in every wave: the whole workgroup leaves together
   wave_lds_sync();
   // x = (G - a) * log2(e) per (token, channel): q~ = q 2^x, k~ = k 2^-x
-  f32x16_t x[2];
+  f32x16_t x[2] = {{0.f}, {0.f}};
 #pragma unroll
-  for (int gq = 0; gq < 4; ++gq) {
-    const f32x4_t o0 = *reinterpret_cast<const f32x4_t*>(offs + 32 * h + 8 * gq);
-    const f32x4_t o1 = *reinterpret_cast<const f32x4_t*>(offs + 32 * h + 8 * gq + 4);
+  for (int gq = 0; gq < NG; ++gq) {
+    const f32x4_t o0 = *reinterpret_cast<const f32x4_t*>(offs + HC * h + 8 * gq);
+    const f32x4_t o1 = *reinterpret_cast<const f32x4_t*>(offs + HC * h + 8 * gq + 4);
     const float o8[8] = {o0[0], o0[1], o0[2], o0[3], o1[0], o1[1], o1[2], o1[3]};
 #pragma unroll
     for (int m = 0; m < 4; ++m)
@@ -197,9 +204,9 @@ __device__ __forceinline__ bool bwd_direction(const BwdSlab& sl, int L, int ntil
       for (int p = 0; p < 2; ++p) x[p][4 * gq + m] = (G[p][4 * gq + m] + o8[2 * m + p]) * kLog2e;
   }
   {
-    u32x4_t qt[4], kt[4];
+    u32x4_t qt[NG], kt[NG];
 #pragma unroll
-    for (int gq = 0; gq < 4; ++gq)
+    for (int gq = 0; gq < NG; ++gq)
 #pragma unroll
       for (int m = 0; m < 4; ++m) {
         const int c = 4 * gq + m;
@@ -208,8 +215,8 @@ __device__ __forceinline__ bool bwd_direction(const BwdSlab& sl, int L, int ntil
         qt[gq][m] = pack_bf16x2(bf16lo_to_f32(wq) * e0, bf16hi_to_f32(wq) * e1);
         kt[gq][m] = pack_bf16x2(bf16lo_to_f32(wk) * exp2_fast(-x[0][c]), bf16hi_to_f32(wk) * exp2_fast(-x[1][c]));
       }
-    store_kt<4>(Q, 32 * w + r, h, qt);
-    store_kt<4>(K, 32 * w + r, h, kt);
+    store_kt<NG>(Q, 32 * w + r, h, qt);
+    store_kt<NG>(K, 32 * w + r, h, kt);
   }
   VIG_BWD_STAMP(3);
   lds_barrier();  // (2) q~, k~ of every tile visible
@@ -227,13 +234,13 @@ __device__ __forceinline__ bool bwd_direction(const BwdSlab& sl, int L, int ntil
       f32x16_t T = {0.f};  // A^T tile: rows j in J, columns i in tile w
 #pragma unroll
       for (int ks = 0; ks < 4; ++ks) T = mfma(row_frag(V, 32 * J + r, ks, h), doB[ks], T);
-      if (J == w) mask_diag<FWD, false>(T, r, h);
+      mask_diag<FWD, false>(T, r, h, J == w);
       u32x4_t f[2];
       tile_frags(T, f);
 #pragma unroll
       for (int t = 0; t < 2; ++t) {
         u32x4_t kf[2];
-        load_tfrag_lds<4>(K + 32 * J * kKtStride, t, r, h, kf);
+        load_tfrag_lds<NG>(K + 32 * J * kKtStride, t, r, h, kf);
         dqh[0] = mfma(kf[0], f[t], dqh[0]);
         dqh[1] = mfma(kf[1], f[t], dqh[1]);
       }
@@ -245,12 +252,12 @@ __device__ __forceinline__ bool bwd_direction(const BwdSlab& sl, int L, int ntil
 #pragma unroll
   for (int c = 0; c < 16; ++c) dqp[c] = pack_bf16x2(dqh[0][c], dqh[1][c]);
   // the first direction parked its dq and dk (rounded to bf16) in the output tensors; fetch them under the loops
-  const rsrc_t oq = chunk_rsrc(sl.dq + toff, rows, 128), okk = chunk_rsrc(sl.dk + toff, rows, 128);
-  u32x4_t prevq[4], prevk[4];
+  const rsrc_t oq = chunk_rsrc(sl.dq + tk, rows, 2 * DK), okk = chunk_rsrc(sl.dk + tk, rows, 2 * DK);
+  u32x4_t prevq[NG], prevk[NG];
   if (LAST) {
 #pragma unroll
-    for (int gq = 0; gq < 4; ++gq) {
-      const unsigned off = (unsigned)r * 128u + 64u * h + 16u * gq;
+    for (int gq = 0; gq < NG; ++gq) {
+      const unsigned off = (unsigned)r * (2u * DK) + (2u * HC) * h + 16u * gq;
       prevq[gq] = __builtin_amdgcn_raw_buffer_load_b128(oq, off, 0, 0);
       prevk[gq] = __builtin_amdgcn_raw_buffer_load_b128(okk, off, 0, 0);
     }
@@ -263,8 +270,8 @@ __device__ __forceinline__ bool bwd_direction(const BwdSlab& sl, int L, int ntil
     for (int I = i0; I <= i1; ++I) {
       f32x16_t P = {0.f};  // rows i in I, columns j in tile w
 #pragma unroll
-      for (int ks = 0; ks < 4; ++ks) P = mfma(row_frag(Q, 32 * I + r, ks, h), row_frag(K, 32 * w + r, ks, h), P);
-      if (I == w) mask_diag<FWD, true>(P, r, h);
+      for (int ks = 0; ks < NG; ++ks) P = mfma(row_frag(Q, 32 * I + r, ks, h), row_frag(K, 32 * w + r, ks, h), P);
+      mask_diag<FWD, true>(P, r, h, I == w);
       u32x4_t pf[2];
       tile_frags(P, pf);
 #pragma unroll
@@ -280,13 +287,13 @@ __device__ __forceinline__ bool bwd_direction(const BwdSlab& sl, int L, int ntil
       f32x16_t A = {0.f};
 #pragma unroll
       for (int ks = 0; ks < 4; ++ks) A = mfma(row_frag(DO, 32 * I + r, ks, h), row_frag(V, 32 * w + r, ks, h), A);
-      if (I == w) mask_diag<FWD, true>(A, r, h);
+      mask_diag<FWD, true>(A, r, h, I == w);
       u32x4_t af[2];
       tile_frags(A, af);
 #pragma unroll
       for (int t = 0; t < 2; ++t) {
         u32x4_t qf[2];
-        load_tfrag_lds<4>(Q + 32 * I * kKtStride, t, r, h, qf);
+        load_tfrag_lds<NG>(Q + 32 * I * kKtStride, t, r, h, qf);
         dkh[0] = mfma(qf[0], af[t], dkh[0]);
         dkh[1] = mfma(qf[1], af[t], dkh[1]);
       }
@@ -296,12 +303,21 @@ __device__ __forceinline__ bool bwd_direction(const BwdSlab& sl, int L, int ntil
   // ---- scale back; X = q dq - k dk = s (q~ dq^ - k~ dk^): the exponentials cancel, and the staged rows serve ----
   f32x16_t X[2];
   {
-    const rsrc_t ov = chunk_rsrc(sl.dv + toff, rows, 128);
+    const rsrc_t ov = chunk_rsrc(sl.dv + tv, rows, 128);
+    if (LAST) {
 #pragma unroll
-    for (int gq = 0; gq < 4; ++gq) {
-      const u32x4_t qrow = *reinterpret_cast<const u32x4_t*>(Q + (32 * w + r) * kKtStride + 32 * h + 8 * gq);
-      const u32x4_t krow = *reinterpret_cast<const u32x4_t*>(K + (32 * w + r) * kKtStride + 32 * h + 8 * gq);
-      u32x4_t xq, xk, xv;
+      for (int gq = 0; gq < 4; ++gq) {
+        u32x4_t xv;
+#pragma unroll
+        for (int m = 0; m < 4; ++m) xv[m] = pack_bf16x2(dv[0][4 * gq + m] * s, dv[1][4 * gq + m] * s);
+        __builtin_amdgcn_raw_buffer_store_b128(xv, ov, (unsigned)r * 128u + 64u * h + 16u * gq, 0, 0);
+      }
+    }
+#pragma unroll
+    for (int gq = 0; gq < NG; ++gq) {
+      const u32x4_t qrow = *reinterpret_cast<const u32x4_t*>(Q + (32 * w + r) * kKtStride + HC * h + 8 * gq);
+      const u32x4_t krow = *reinterpret_cast<const u32x4_t*>(K + (32 * w + r) * kKtStride + HC * h + 8 * gq);
+      u32x4_t xq, xk;
 #pragma unroll
       for (int m = 0; m < 4; ++m) {
         const int c = 4 * gq + m;
@@ -322,12 +338,10 @@ __device__ __forceinline__ bool bwd_direction(const BwdSlab& sl, int L, int ntil
         }
         xq[m] = pack_bf16x2(a[0], a[1]);
         xk[m] = pack_bf16x2(b[0], b[1]);
-        if (LAST) xv[m] = pack_bf16x2(dv[0][c] * s, dv[1][c] * s);
       }
-      const unsigned off = (unsigned)r * 128u + 64u * h + 16u * gq;
+      const unsigned off = (unsigned)r * (2u * DK) + (2u * HC) * h + 16u * gq;
       __builtin_amdgcn_raw_buffer_store_b128(xq, oq, off, 0, 0);
       __builtin_amdgcn_raw_buffer_store_b128(xk, okk, off, 0, 0);
-      if (LAST) __builtin_amdgcn_raw_buffer_store_b128(xv, ov, off, 0, 0);
     }
   }
   VIG_BWD_STAMP(7);
@@ -335,47 +349,48 @@ __device__ __forceinline__ bool bwd_direction(const BwdSlab& sl, int L, int ntil
   {
     float* xs = reinterpret_cast<float*>(lds + kBwdLdsQ) + w * 32 * kXStride;
 #pragma unroll
-    for (int gq = 0; gq < 4; ++gq) {
+    for (int gq = 0; gq < NG; ++gq) {
       const f32x4_t a = {X[0][4 * gq], X[1][4 * gq], X[0][4 * gq + 1], X[1][4 * gq + 1]};
       const f32x4_t b = {X[0][4 * gq + 2], X[1][4 * gq + 2], X[0][4 * gq + 3], X[1][4 * gq + 3]};
-      *reinterpret_cast<f32x4_t*>(xs + r * kXStride + 32 * h + 8 * gq) = a;
-      *reinterpret_cast<f32x4_t*>(xs + r * kXStride + 32 * h + 8 * gq + 4) = b;
+      *reinterpret_cast<f32x4_t*>(xs + r * kXStride + HC * h + 8 * gq) = a;
+      *reinterpret_cast<f32x4_t*>(xs + r * kXStride + HC * h + 8 * gq + 4) = b;
     }
     wave_lds_sync();
     // the next direction's loads travel while this one scans and stores
-    issue_bwd_loads<LAST>(nxt, w, r, h, ld);
-    // lane = channel: the tile's total, then (with the totals of the tiles behind it) the running sum over its
-    // tokens against the walking order, written back in place
+    issue_bwd_loads<LAST, NG>(nxt, w, r, h, ld);
+    // lane = channel (lanes past Dk idle along): the tile's total, then (with the totals of the tiles behind it) the
+    // running sum over its tokens against the walking order, written back in place
+    const int cl = lane < DK ? lane : 0;
     float acc = 0.f;
 #pragma unroll
-    for (int t = 0; t < 32; ++t) acc += xs[t * kXStride + lane];
-    dgtot[w * 64 + lane] = acc;
+    for (int t = 0; t < 32; ++t) acc += xs[t * kXStride + cl];
+    if (lane < DK) dgtot[w * 64 + lane] = acc;
     VIG_BWD_STAMP(8);
     lds_barrier();  // (4) tile totals of X visible
     VIG_BWD_STAMP(9);
     float run = 0.f;
 #pragma unroll
     for (int t = 0; t < kBwdTiles; ++t) {
-      const float y = dgtot[t * 64 + lane];
+      const float y = dgtot[t * 64 + cl];
       run += (FWD ? (t > w) : (t < w)) ? y : 0.f;
     }
 #pragma unroll
     for (int i = 0; i < 32; ++i) {
       const int t = FWD ? 31 - i : i;
-      run += xs[t * kXStride + lane];
-      xs[t * kXStride + lane] = run;
+      run += xs[t * kXStride + cl];
+      if (lane < DK) xs[t * kXStride + lane] = run;
     }
     wave_lds_sync();
     // back to lane = token: 16-byte stores of the gate gradient
     uint16_t* dg = FWD ? sl.dgf : sl.dgb;
-    const rsrc_t rdg = chunk_rsrc(dg + toff, rows, 128);
+    const rsrc_t rdg = chunk_rsrc(dg + tk, rows, 2 * DK);
 #pragma unroll
-    for (int gq = 0; gq < 4; ++gq) {
-      const f32x4_t a = *reinterpret_cast<const f32x4_t*>(xs + r * kXStride + 32 * h + 8 * gq);
-      const f32x4_t b = *reinterpret_cast<const f32x4_t*>(xs + r * kXStride + 32 * h + 8 * gq + 4);
+    for (int gq = 0; gq < NG; ++gq) {
+      const f32x4_t a = *reinterpret_cast<const f32x4_t*>(xs + r * kXStride + HC * h + 8 * gq);
+      const f32x4_t b = *reinterpret_cast<const f32x4_t*>(xs + r * kXStride + HC * h + 8 * gq + 4);
       const u32x4_t out = {pack_bf16x2(a[0], a[1]), pack_bf16x2(a[2], a[3]), pack_bf16x2(b[0], b[1]),
                            pack_bf16x2(b[2], b[3])};
-      __builtin_amdgcn_raw_buffer_store_b128(out, rdg, (unsigned)r * 128u + 64u * h + 16u * gq, 0, 0);
+      __builtin_amdgcn_raw_buffer_store_b128(out, rdg, (unsigned)r * (2u * DK) + (2u * HC) * h + 16u * gq, 0, 0);
     }
   }
   VIG_BWD_STAMP(10);
@@ -384,6 +399,7 @@ __device__ __forceinline__ bool bwd_direction(const BwdSlab& sl, int L, int ntil
 
 }  // namespace
 
+template <int NG>
 __global__ __launch_bounds__(512) void gla_backward_mfma_kernel(
     const uint16_t* __restrict__ q, const uint16_t* __restrict__ k, const uint16_t* __restrict__ v,
     const uint16_t* __restrict__ gf, const uint16_t* __restrict__ gb, const uint16_t* __restrict__ d_o,
@@ -395,9 +411,8 @@ __global__ __launch_bounds__(512) void gla_backward_mfma_kernel(
   const int lane = tid & 63;
   const int ntiles = (L + 31) / 32;
   auto slab_of = [&](int i) {
-    const size_t base = (size_t)i * L * 64;
-    return BwdSlab{q + base, k + base, v + base, gf + base, gb + base, d_o + base,
-                   dq + base, dk + base, dv + base, dgf + base, dgb + base};
+    const size_t bk = (size_t)i * L * (16 * NG), bv = (size_t)i * L * 64;
+    return BwdSlab{q + bk, k + bk, v + bv, gf + bk, gb + bk, d_o + bv, dq + bk, dk + bk, dv + bv, dgf + bk, dgb + bk};
   };
   const int r = lane & 31, h = lane >> 5;
 #ifdef VIG_BWD_STAGGER
@@ -407,10 +422,10 @@ __global__ __launch_bounds__(512) void gla_backward_mfma_kernel(
     while (wall_clock64() - t0 < (unsigned long long)(VIG_BWD_STAGGER) * 100ull) __builtin_amdgcn_s_sleep(16);
   }
 #endif
-  BwdLoads ld;
+  BwdLoads<NG> ld;
   if ((int)blockIdx.x < nslabs) {
     const BwdSlab s0 = slab_of(blockIdx.x);
-    issue_bwd_loads<true>(BwdNext{s0, s0.gf, L}, w, r, h, ld);
+    issue_bwd_loads<true, NG>(BwdNext{s0, s0.gf, L}, w, r, h, ld);
   }
   for (int slab = blockIdx.x; slab < nslabs; slab += gridDim.x) {
     const BwdSlab sl = slab_of(slab);
@@ -419,17 +434,24 @@ __global__ __launch_bounds__(512) void gla_backward_mfma_kernel(
     const BwdNext second{sl, sl.gb, L}, next_first{sn, sn.gf, following < nslabs ? L : 0};
     f32x16_t dvacc[2] = {{0.f}, {0.f}};
     const bool first_slab = slab == (int)blockIdx.x;
-    bool ok = bwd_direction<true, false>(sl, L, ntiles, w, lane, lds, s, dvacc, ld, second, first_slab);
+    bool ok = bwd_direction<true, false, NG>(sl, L, ntiles, w, lane, lds, s, dvacc, ld, second, first_slab);
     if (ok) {
       lds_barrier();  // (5) the dg scratch of direction 1 is dead before q~, k~ of direction 2 are staged
-      ok = bwd_direction<false, true>(sl, L, ntiles, w, lane, lds, s, dvacc, ld, next_first, first_slab);
+      ok = bwd_direction<false, true, NG>(sl, L, ntiles, w, lane, lds, s, dvacc, ld, next_first, first_slab);
     }
     // a direction that left early has not issued the loads of the slab that follows
-    if (!ok) issue_bwd_loads<true>(next_first, w, r, h, ld);
+    if (!ok) issue_bwd_loads<true, NG>(next_first, w, r, h, ld);
     if (tid == 0) flags[slab] = ok ? 0 : 1;
     lds_barrier();  // the next slab restages everything
   }
 }
+
+template __global__ void gla_backward_mfma_kernel<4>(const uint16_t*, const uint16_t*, const uint16_t*,
+                                                     const uint16_t*, const uint16_t*, const uint16_t*, uint16_t*,
+                                                     uint16_t*, uint16_t*, uint16_t*, uint16_t*, int*, int, int, float);
+template __global__ void gla_backward_mfma_kernel<2>(const uint16_t*, const uint16_t*, const uint16_t*,
+                                                     const uint16_t*, const uint16_t*, const uint16_t*, uint16_t*,
+                                                     uint16_t*, uint16_t*, uint16_t*, uint16_t*, int*, int, int, float);
 
 #ifdef VIG_TIMING
 extern "C" int vig_debug_read_bwd_stamps(unsigned long long* host_out) {
@@ -438,22 +460,23 @@ extern "C" int vig_debug_read_bwd_stamps(unsigned long long* host_out) {
 #endif
 
 bool gla_backward_mfma_supported(int L, int Dk, int Dv, int io_dtype, int gate_dtype, bool bidir) {
-  return bidir && io_dtype == 1 && gate_dtype == 1 && Dk == 64 && Dv == 64 && L <= 32 * kBwdTiles;
+  return bidir && io_dtype == 1 && gate_dtype == 1 && (Dk == 64 || Dk == 32) && Dv == 64 && L <= 32 * kBwdTiles;
 }
 
 // flags: one int per (batch, head) slab, written by every launch: 1 = not computed here (gates out of range)
 int launch_gla_backward_mfma(const void* q, const void* k, const void* v, const void* gf, const void* gb,
                              const void* d_o, void* dq, void* dk, void* dv, void* dgf, void* dgb, int* flags, int B,
-                             int H, int L, float s, hipStream_t stream) {
+                             int H, int L, int Dk, float s, hipStream_t stream) {
   constexpr int kMaxDevices = 64;
   static bool attr_done_dev[kMaxDevices] = {};
   static int num_cu_dev[kMaxDevices] = {};
   int dev = 0;
   if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return -5;
   if (!attr_done_dev[dev]) {
-    if (hipFuncSetAttribute(reinterpret_cast<const void*>(gla_backward_mfma_kernel),
-                            hipFuncAttributeMaxDynamicSharedMemorySize, kBwdLdsTotal) != hipSuccess)
-      return -5;
+    const void* kernels[2] = {reinterpret_cast<const void*>(gla_backward_mfma_kernel<4>),
+                              reinterpret_cast<const void*>(gla_backward_mfma_kernel<2>)};
+    for (const void* kf : kernels)
+      if (hipFuncSetAttribute(kf, hipFuncAttributeMaxDynamicSharedMemorySize, kBwdLdsTotal) != hipSuccess) return -5;
     int n = 0;
     if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess) return -5;
     num_cu_dev[dev] = n > 0 ? n : 256;
@@ -461,10 +484,14 @@ int launch_gla_backward_mfma(const void* q, const void* k, const void* v, const 
   }
   const int nslabs = B * H;
   const int grid = nslabs < num_cu_dev[dev] ? nslabs : num_cu_dev[dev];
-  hipLaunchKernelGGL(gla_backward_mfma_kernel, dim3(grid), dim3(512), kBwdLdsTotal, stream, (const uint16_t*)q,
-                     (const uint16_t*)k, (const uint16_t*)v, (const uint16_t*)gf, (const uint16_t*)gb,
-                     (const uint16_t*)d_o, (uint16_t*)dq, (uint16_t*)dk, (uint16_t*)dv, (uint16_t*)dgf, (uint16_t*)dgb,
-                     flags, nslabs, L, s);
+#define VIG_BWD_LAUNCH(NG)                                                                                          \
+  hipLaunchKernelGGL(gla_backward_mfma_kernel<NG>, dim3(grid), dim3(512), kBwdLdsTotal, stream, (const uint16_t*)q, \
+                     (const uint16_t*)k, (const uint16_t*)v, (const uint16_t*)gf, (const uint16_t*)gb,              \
+                     (const uint16_t*)d_o, (uint16_t*)dq, (uint16_t*)dk, (uint16_t*)dv, (uint16_t*)dgf,             \
+                     (uint16_t*)dgb, flags, nslabs, L, s)
+  if (Dk == 64) VIG_BWD_LAUNCH(4);
+  else VIG_BWD_LAUNCH(2);
+#undef VIG_BWD_LAUNCH
   return hipGetLastError() == hipSuccess ? 0 : -5;
 }
 

@@ -38,6 +38,6 @@ size_t gla_mfma_workspace(int B, int H, int L, int Dk, int Dv);
 bool gla_backward_mfma_supported(int L, int Dk, int Dv, int io_dtype, int gate_dtype, bool bidir);
 int launch_gla_backward_mfma(const void* q, const void* k, const void* v, const void* gf, const void* gb,
                              const void* d_o, void* dq, void* dk, void* dv, void* dgf, void* dgb, int* flags, int B,
-                             int H, int L, float s, hipStream_t stream);
+                             int H, int L, int Dk, float s, hipStream_t stream);
 
 }  // namespace vig
