@@ -59,8 +59,11 @@ const char* vig_gla_strerror(int code);
  * Numeric range of the matrix-core path (bf16 tensors and gates, Dk in {32, 64},
  * Dv = 64): the sum of |g| over any 64 consecutive tokens of one channel must
  * stay below about 80, and |q|, |k| below about 1000 (beyond either, results
- * may be inf / NaN, never silently wrong finite numbers).  Other combinations
- * run on the fp32-arithmetic kernel, which has no such limit.
+ * may be inf / NaN, never silently wrong finite numbers).  HierViG's head shape
+ * (bf16, Dk = 16, Dv = 32, both directions) takes the same path from L = 128 on,
+ * zero-padded to Dk 32 / Dv 64 in the workspace (classification/models/vig_h.py:
+ * 377-385 with EXPAND_K 0.5, EXPAND_V 1.0).  Other combinations run on the
+ * fp32-arithmetic kernel, which has no such limit.
  */
 int vig_gla_bidir_fwd(const void* q, const void* k, const void* v,
                       const void* g_fwd, const void* g_bwd, void* o,

@@ -199,3 +199,20 @@ def test_bf16_flip_symmetry_full_size():
     fl = lambda x: x.flip(dims=[2]).contiguous()
     b = fl(vig_amd.gla_bidir_forward(fl(dq), fl(dk_), fl(dv_), fl(dgb), fl(dgf)))
     assert (a.float() - b.float()).abs().max().item() <= BF16_TOL
+
+
+@pytest.mark.parametrize("B,H,L", [(2, 3, 128), (2, 3, 196), (1, 6, 784), (1, 3, 3136)])
+def test_bf16_hiervig_head_shape_on_the_matrix_cores(B, H, L):
+    """Dk 16 / Dv 32 (HierViG) from L = 128 on: zero-padded to Dk 32 / Dv 64 inside the library; against the oracle,
+    and against the fp32-arithmetic kernel on the same inputs."""
+    announce(f"bf16 Dk=16 Dv=32 B{B} H{H} L={L} (padded onto the matrix-core kernel)")
+    q, k, v, gf, gb = make_gla_inputs(B, H, L, 16, 32, seed=600 + L, dtype=torch.bfloat16)
+    want = oracle_bidir(q, k, v, gf, gb)
+    got = vig_amd.gla_bidir_forward(*dev(q, k, v, gf, gb))
+    assert got.shape == (B, H, L, 32)
+    # |o| reaches ~5 here (k is scaled by 16^-0.5 only), where the bf16 output grid alone is coarser than 2e-2:
+    # allow half an output ulp (2^-8 relative) on top of the absolute tolerance
+    assert np.all(np.abs(f64(got) - want) <= BF16_TOL + 2.0 ** -8 * np.abs(want))
+    exact = vig_amd.gla_bidir_forward(*dev(q, k, v, gf, gb), exact=True)
+    assert np.all(np.abs(f64(got) - f64(exact)) <= BF16_TOL + 2.0 ** -7 * np.abs(want))
+    assert not torch.equal(got, exact)  # (the two kernels round differently: proves the padded path ran)

@@ -213,4 +213,28 @@ int launch_swiglu(const void* in, void* out, long long rows, int I, int io_dtype
   return hipGetLastError() == hipSuccess ? 0 : -5;
 }
 
+// ---------------------------------------------------------------------------
+// Channel padding / cropping of bf16 rows:  dst[row, c] = c < src_c ? src[row, c] : 0  for c < dst_c.
+// Used to run head shapes narrower than the matrix-core kernel's (Dk 16, Dv 32) on it: zero q, k and v channels
+// contribute nothing, zero log-gates mean no decay, and the surplus output channels are cropped.
+// ---------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void pad_channels_kernel(const uint16_t* __restrict__ src, uint16_t* __restrict__ dst,
+                                                           long long nvec, int src_c8, int dst_c8) {
+  const long long i = (long long)blockIdx.x * 256 + threadIdx.x;  // one 16-byte piece of dst
+  if (i >= nvec) return;
+  const long long row = i / dst_c8;
+  const int c8 = (int)(i - row * dst_c8);
+  u32x4_t x = {0u, 0u, 0u, 0u};
+  if (c8 < src_c8) x = *reinterpret_cast<const u32x4_t*>(src + ((size_t)row * src_c8 + c8) * 8);
+  *reinterpret_cast<u32x4_t*>(dst + (size_t)i * 8) = x;
+}
+
+int launch_pad_channels(const void* src, void* dst, long long rows, int src_c, int dst_c, hipStream_t stream) {
+  if (src_c % 8 != 0 || dst_c % 8 != 0 || rows <= 0) return -95;
+  const long long nvec = rows * (dst_c / 8);
+  hipLaunchKernelGGL(pad_channels_kernel, dim3((unsigned)((nvec + 255) / 256)), dim3(256), 0, stream,
+                     (const uint16_t*)src, (uint16_t*)dst, nvec, src_c / 8, dst_c / 8);
+  return hipGetLastError() == hipSuccess ? 0 : -5;
+}
+
 }  // namespace vig
