@@ -124,8 +124,11 @@ __device__ __forceinline__ void issue_bwd_loads(const BwdNext& n, int w, int r, 
 // are out of range.
 template <bool FWD, bool LAST, int NG>
 __device__ __forceinline__ bool bwd_direction(const BwdSlab& sl, int L, int ntiles, int w, int lane, char* lds,
-                                              float s, f32x16_t (&dv)[2], BwdLoads<NG>& ld, const BwdNext& nxt,
-                                              bool first_slab) {
+                                              float s, f32x16_t (&dv)[2], u32x4_t (&keepq)[NG], u32x4_t (&keepk)[NG],
+                                              BwdLoads<NG>& ld, const BwdNext& nxt, bool first_slab) {
+  // where the first direction's dq, dk (bf16) wait for the second: in registers when the kernel has them to spare
+  // (Dk = 32), else parked in the output tensors
+  constexpr bool kKeepInRegs = NG == 2;
   constexpr bool stage_vdo = !LAST;
   constexpr int DK = 16 * NG;   // channels of q, k and the gates
   constexpr int HC = 8 * NG;    // channels per lane half
@@ -254,7 +257,11 @@ __device__ __forceinline__ bool bwd_direction(const BwdSlab& sl, int L, int ntil
   // the first direction parked its dq and dk (rounded to bf16) in the output tensors; fetch them under the loops
   const rsrc_t oq = chunk_rsrc(sl.dq + tk, rows, 2 * DK), okk = chunk_rsrc(sl.dk + tk, rows, 2 * DK);
   u32x4_t prevq[NG], prevk[NG];
-  if (LAST) {
+  if (LAST && kKeepInRegs) {
+#pragma unroll
+    for (int gq = 0; gq < NG; ++gq) prevq[gq] = keepq[gq], prevk[gq] = keepk[gq];
+  }
+  if (LAST && !kKeepInRegs) {
 #pragma unroll
     for (int gq = 0; gq < NG; ++gq) {
       const unsigned off = (unsigned)r * (2u * DK) + (2u * HC) * h + 16u * gq;
@@ -340,8 +347,13 @@ __device__ __forceinline__ bool bwd_direction(const BwdSlab& sl, int L, int ntil
         xk[m] = pack_bf16x2(b[0], b[1]);
       }
       const unsigned off = (unsigned)r * (2u * DK) + (2u * HC) * h + 16u * gq;
-      __builtin_amdgcn_raw_buffer_store_b128(xq, oq, off, 0, 0);
-      __builtin_amdgcn_raw_buffer_store_b128(xk, okk, off, 0, 0);
+      if (!LAST && kKeepInRegs) {
+        keepq[gq] = xq;
+        keepk[gq] = xk;
+      } else {
+        __builtin_amdgcn_raw_buffer_store_b128(xq, oq, off, 0, 0);
+        __builtin_amdgcn_raw_buffer_store_b128(xk, okk, off, 0, 0);
+      }
     }
   }
   VIG_BWD_STAMP(7);
@@ -433,11 +445,12 @@ __global__ __launch_bounds__(512) void gla_backward_mfma_kernel(
     const BwdSlab sn = slab_of(following < nslabs ? following : slab);
     const BwdNext second{sl, sl.gb, L}, next_first{sn, sn.gf, following < nslabs ? L : 0};
     f32x16_t dvacc[2] = {{0.f}, {0.f}};
+    u32x4_t keepq[NG], keepk[NG];
     const bool first_slab = slab == (int)blockIdx.x;
-    bool ok = bwd_direction<true, false, NG>(sl, L, ntiles, w, lane, lds, s, dvacc, ld, second, first_slab);
+    bool ok = bwd_direction<true, false, NG>(sl, L, ntiles, w, lane, lds, s, dvacc, keepq, keepk, ld, second, first_slab);
     if (ok) {
       lds_barrier();  // (5) the dg scratch of direction 1 is dead before q~, k~ of direction 2 are staged
-      ok = bwd_direction<false, true, NG>(sl, L, ntiles, w, lane, lds, s, dvacc, ld, next_first, first_slab);
+      ok = bwd_direction<false, true, NG>(sl, L, ntiles, w, lane, lds, s, dvacc, keepq, keepk, ld, next_first, first_slab);
     }
     // a direction that left early has not issued the loads of the slab that follows
     if (!ok) issue_bwd_loads<true, NG>(next_first, w, r, h, ld);
