@@ -54,7 +54,7 @@ const char* vig_gla_strerror(int code);
  * batch_bid_fused_chunk_gla (fla/ops/gla/chunk_fuse.py:574-596) and, with
  * g_bwd == NULL, fused_chunk_gla (chunk_fuse.py:554-572).
  *
- * Built shapes: Dk in {16, 32, 64, 128}, Dv in {32, 64}, any L >= 1.
+ * Built shapes: Dk in {16, 32, 64, 128}, Dv in {32, 64, 128}, any L >= 1.
  *
  * Numeric range of the matrix-core path (bf16 tensors and gates, Dk in {32, 64},
  * Dv = 64): the sum of |g| over any 64 consecutive tokens of one channel must

@@ -27,7 +27,7 @@ size_t gla_backward_workspace(int B, int H, int L, int Dk, int Dv, int bidir);
 
 static bool dtype_ok(int d) { return d == VIG_F32 || d == VIG_BF16; }
 static bool dk_ok(int d) { return d == 16 || d == 32 || d == 64 || d == 128; }
-static bool dv_ok(int d) { return d == 32 || d == 64; }
+static bool dv_ok(int d) { return d == 32 || d == 64 || d == 128; }
 
 extern "C" {
 
