@@ -147,8 +147,11 @@ def main():
     ap.add_argument("--sets", type=int, default=0, help="input sets to rotate (0 = enough to exceed 256 MB, >= 3)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--exact", action="store_true", help="time the fp32-arithmetic recurrent kernel instead")
-    ap.add_argument("--model", action="store_true", help="also time the full ViG-S eval forward (images/s)")
-    ap.add_argument("--backward", action="store_true", help="also time the backward of the op on the same workload")
+    ap.add_argument("--model", action="store_true",
+                    help="also time the full ViG-S eval forward (images/s); on by default for the headline workload")
+    ap.add_argument("--backward", action="store_true",
+                    help="also time the backward of the op on the same workload; on by default for the headline workload")
+    ap.add_argument("--op-only", action="store_true", help="no model forward and no backward, whatever the workload")
     ap.add_argument("--no-gemm-tuning", action="store_true",
                     help="with --model: leave torch's GEMM solution tuning off (clean kernel traces)")
     ap.add_argument("--unfused-gate", action="store_true",
@@ -296,9 +299,12 @@ def main():
         "roofline": {"bound": "hbm", "achieved": achieved_gbps, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                      "frac": achieved_gbps / HBM_PEAK_GBPS, "traffic": traffic},
     }
-    if args.backward:
+    # the headline run (config 1) also reports the other half of the metric (ViG-S images/s) and the backward
+    want_backward = (args.backward or args.config == 1) and not args.op_only and not args.exact
+    want_model = (args.model or args.config == 1) and not args.op_only and not args.exact
+    if want_backward:
         out["backward"] = backward_time(lib, sets, s, io_dt, scale, sp, stream, dev)
-    if args.model:
+    if want_model:
         out["vig_s_forward"] = model_throughput(dev, tune_gemm=not args.no_gemm_tuning)
     if not args.no_cpu:
         out["cpu_baseline"] = cpu_baseline(s, 1000 + args.config)
