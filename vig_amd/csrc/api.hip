@@ -18,6 +18,8 @@ int launch_split_heads(const void* qkv, void* q, void* k, void* v, int B, int L,
                        hipStream_t stream);
 int launch_swiglu(const void* in, void* out, long long rows, int I, int io_dtype, hipStream_t stream);
 int launch_pad_channels(const void* src, void* dst, long long rows, int src_c, int dst_c, hipStream_t stream);
+int launch_pad_channels_multi(const void* const* src, void* const* dst, const int* src_c, const int* dst_c, int n,
+                              long long rows, hipStream_t stream);
 int launch_gla_backward(const void* q, const void* k, const void* v, const void* g_fwd, const void* g_bwd,
                         const void* d_o, void* dq, void* dk, void* dv, void* dg_fwd, void* dg_bwd, void* workspace,
                         int B, int H, int L, int Dk, int Dv, float scale, float out_scale, int io_dtype,
@@ -106,11 +108,10 @@ int vig_gla_bidir_fwd(const void* q, const void* k, const void* v, const void* g
     uint16_t *qp = p, *kp = p + nqk, *gfp = p + 2 * nqk, *gbp = p + 3 * nqk, *vp = p + 4 * nqk, *op = vp + nv;
     const long long rows = (long long)B * H * L;
     hipStream_t st = (hipStream_t)stream;
-    int e = vig::launch_pad_channels(q, qp, rows, 16, 32, st);
-    if (!e) e = vig::launch_pad_channels(k, kp, rows, 16, 32, st);
-    if (!e) e = vig::launch_pad_channels(g_fwd, gfp, rows, 16, 32, st);
-    if (!e) e = vig::launch_pad_channels(g_bwd, gbp, rows, 16, 32, st);
-    if (!e) e = vig::launch_pad_channels(v, vp, rows, 32, 64, st);
+    const void* srcs[5] = {q, k, g_fwd, g_bwd, v};
+    void* dsts[5] = {qp, kp, gfp, gbp, vp};
+    const int src_c[5] = {16, 16, 16, 16, 32}, dst_c[5] = {32, 32, 32, 32, 64};
+    int e = vig::launch_pad_channels_multi(srcs, dsts, src_c, dst_c, 5, rows, st);
     if (e) return e;
     vig::GlaArgs b = a;
     b.q = qp, b.k = kp, b.v = vp, b.g_fwd = gfp, b.g_bwd = gbp, b.o = op;

@@ -229,6 +229,45 @@ __global__ __launch_bounds__(256) void pad_channels_kernel(const uint16_t* __res
   *reinterpret_cast<u32x4_t*>(dst + (size_t)i * 8) = x;
 }
 
+// Several tensors of the same row count in one launch (blockIdx.y = tensor).
+struct PadJobs {
+  const uint16_t* src[5];
+  uint16_t* dst[5];
+  int src_c8[5], dst_c8[5];
+};
+__global__ __launch_bounds__(256) void pad_channels_multi_kernel(PadJobs jobs, long long rows) {
+  const int j = blockIdx.y;
+  const int dst_c8 = jobs.dst_c8[j], src_c8 = jobs.src_c8[j];
+  const long long nvec = rows * dst_c8;
+  for (long long i = (long long)blockIdx.x * 256 + threadIdx.x; i < nvec; i += (long long)gridDim.x * 256) {
+    const long long row = i / dst_c8;
+    const int c8 = (int)(i - row * dst_c8);
+    u32x4_t x = {0u, 0u, 0u, 0u};
+    if (c8 < src_c8) x = *reinterpret_cast<const u32x4_t*>(jobs.src[j] + ((size_t)row * src_c8 + c8) * 8);
+    *reinterpret_cast<u32x4_t*>(jobs.dst[j] + (size_t)i * 8) = x;
+  }
+}
+
+int launch_pad_channels_multi(const void* const* src, void* const* dst, const int* src_c, const int* dst_c, int n,
+                              long long rows, hipStream_t stream) {
+  if (n < 1 || n > 5 || rows <= 0) return -95;
+  PadJobs jobs{};
+  int max_c8 = 0;
+  for (int j = 0; j < n; ++j) {
+    if (src_c[j] % 8 != 0 || dst_c[j] % 8 != 0) return -95;
+    jobs.src[j] = (const uint16_t*)src[j];
+    jobs.dst[j] = (uint16_t*)dst[j];
+    jobs.src_c8[j] = src_c[j] / 8;
+    jobs.dst_c8[j] = dst_c[j] / 8;
+    if (jobs.dst_c8[j] > max_c8) max_c8 = jobs.dst_c8[j];
+  }
+  const long long nvec = rows * max_c8;
+  const long long blocks = (nvec + 255) / 256;
+  hipLaunchKernelGGL(pad_channels_multi_kernel, dim3((unsigned)(blocks < 65536 ? blocks : 65536), n), dim3(256), 0,
+                     stream, jobs, rows);
+  return hipGetLastError() == hipSuccess ? 0 : -5;
+}
+
 int launch_pad_channels(const void* src, void* dst, long long rows, int src_c, int dst_c, hipStream_t stream) {
   if (src_c % 8 != 0 || dst_c % 8 != 0 || rows <= 0) return -95;
   const long long nvec = rows * (dst_c / 8);
