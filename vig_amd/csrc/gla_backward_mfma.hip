@@ -14,9 +14,10 @@
 // workgroup stages q~, k~ (and once v, do) as bf16 rows in LDS; then wave w accumulates dq of its tile over the key
 // tiles the direction keeps, and dk, dv of its tile over the query tiles: score tiles P, A come out of the matrix
 // cores in the register layout that feeds the next product directly (mfma_tiles.h), operands with tokens in the
-// contraction slots are read from the LDS rows as dwords.  The two directions take turns in LDS, so the work of a
-// tile pair (w, direction) and (w, other direction) adds up to the same for every wave.  dg needs a running sum over
-// tokens: the tile's q dq - k dk goes through LDS, lane = channel scans its 32 tokens, tile totals are exchanged.
+// contraction slots are read from the LDS rows as dwords.  The two directions take turns in LDS; a tile that is heavy
+// in one direction is light in the other, so over both every wave does the same amount of work.  dg needs a running
+// sum over tokens: the tile's q dq - k dk goes through LDS, lane = channel scans its 32 tokens, tile totals are
+// exchanged.  Loads of the next direction (or slab) are issued during that scan, the one phase with registers to spare.
 //
 // Slabs whose gate totals exceed the anchor's range (|G_total| / 2 * log2(e) > 60 in some channel) are not computed
 // here: the workgroup raises the slab's flag and the token-recurrent kernel, launched afterwards with that flag
@@ -120,8 +121,8 @@ __device__ __forceinline__ void issue_bwd_loads(const BwdNext& n, int w, int r, 
 
 // One direction of one slab, for wave w (tile w).  dv accumulates over both directions (raw, unscaled).  The first
 // direction (LAST = false) stages v and do and parks its dq and dk, rounded to bf16, in the output tensors; the second
-// adds its own to them and stores dq, dk, dv.  Returns false, for every wave alike and before it has stored anything, when the gates
-// are out of range.
+// adds its own to them and stores dq, dk, dv.  Returns false, for every wave alike and before it has stored anything,
+// when the gates are out of range.
 template <bool FWD, bool LAST, int NG>
 __device__ __forceinline__ bool bwd_direction(const BwdSlab& sl, int L, int ntiles, int w, int lane, char* lds,
                                               float s, f32x16_t (&dv)[2], u32x4_t (&keepq)[NG], u32x4_t (&keepk)[NG],
@@ -427,13 +428,6 @@ __global__ __launch_bounds__(512) void gla_backward_mfma_kernel(
     return BwdSlab{q + bk, k + bk, v + bv, gf + bk, gb + bk, d_o + bv, dq + bk, dk + bk, dv + bv, dgf + bk, dgb + bk};
   };
   const int r = lane & 31, h = lane >> 5;
-#ifdef VIG_BWD_STAGGER
-  // experiment: half of the workgroups start late, so that their memory phases meet the others' compute phases
-  if ((blockIdx.x >> 3) & 1) {
-    const unsigned long long t0 = wall_clock64();
-    while (wall_clock64() - t0 < (unsigned long long)(VIG_BWD_STAGGER) * 100ull) __builtin_amdgcn_s_sleep(16);
-  }
-#endif
   BwdLoads<NG> ld;
   if ((int)blockIdx.x < nslabs) {
     const BwdSlab s0 = slab_of(blockIdx.x);
