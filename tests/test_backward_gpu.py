@@ -150,3 +150,30 @@ def test_backward_mfma_strong_gates_fall_back_per_slab():
     want = O.bidir_gla_backward(f64(q), f64(k), f64(v), f64(gf), f64(gb), f64(do), out_scale=0.5)
     keep = ~strong[:, :, 0, 0].numpy()
     _check_mfma([g_.cpu()[keep] for g_ in got], [w_[keep] for w_ in want], q[keep])
+
+
+def test_random_shapes_matrix_core_paths_against_exact_paths():
+    """Forty random (B, H, L <= 256, Dk) shapes with gate strengths from ViG's /16 up to the reference tests'
+    clamp_min(-3): forward and backward on the matrix cores (out-of-range slabs included, which go to the recurrent
+    kernel slab by slab) against the fp32-arithmetic kernels on the same inputs."""
+    announce("random shapes, forward and backward, matrix-core paths against the exact paths")
+    rng = np.random.default_rng(7)
+    for it in range(40):
+        B, H, L = int(rng.integers(1, 9)), int(rng.integers(1, 7)), int(rng.integers(1, 257))
+        Dk = int(rng.choice([32, 64]))
+        gate_scale = float(rng.choice([1 / 16, 1 / 16, 0.25, 1.0]))
+        q, k, v, gf, gb = (t.cuda() for t in make_gla_inputs(B, H, L, Dk, 64, seed=1000 + it, dtype=torch.bfloat16,
+                                                             gate_scale=gate_scale))
+        gf, gb = gf.clamp_min(-3), gb.clamp_min(-3)
+        do = _do(v.shape, 2000 + it, torch.bfloat16).cuda()
+        case = f"B{B} H{H} L{L} Dk{Dk} gates x{gate_scale}"
+        o = vig_amd.gla_bidir_forward(q, k, v, gf, gb).float()
+        oe = vig_amd.gla_bidir_forward(q, k, v, gf, gb, exact=True).float()
+        assert bool(((o - oe).abs() <= 2e-2 + 2.0 ** -7 * oe.abs()).all()), case
+        got = vig_amd.gla_bidir_backward(q, k, v, gf, gb, do)
+        want = vig_amd.gla_bidir_backward(q, k, v, gf, gb, do, exact=True)
+        floor = float((q.float() * want[0].float()).abs().max())
+        for name, g_, w_ in zip(("dq", "dk", "dv", "dg_fwd", "dg_bwd"), got, want):
+            assert torch.isfinite(g_.float()).all(), (case, name)
+            den = max(float(w_.float().abs().max()), floor if name.startswith("dg") else 0.0, 1e-30)
+            assert float((g_.float() - w_.float()).abs().max()) / den <= MFMA_BWD_TOL, (case, name)
