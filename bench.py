@@ -69,7 +69,7 @@ def cpu_baseline(shape, seed, budget_s=20.0):
     }
 
 
-def model_throughput(dev, batch=256, warmup=10, iters=30, tune_gemm=True):
+def model_throughput(dev, batch=256, warmup=10, iters=30, tune_gemm=True, use_graph=True):
     """Full ViG-S eval forward (random init, synthetic images, bf16): images/s the way the reference's
     throughput() measures it (classification/main.py:389-406: timed forwards of one resident batch)."""
     import torch
@@ -96,8 +96,27 @@ def model_throughput(dev, batch=256, warmup=10, iters=30, tune_gemm=True):
     from vig_amd import evaluate
     ips = evaluate.throughput(model, images, warmup=warmup, iters=iters)
     dt = iters * batch / ips
-    return {"images_per_s": iters * batch / dt, "batch": batch, "dtype": "bf16", "iters": iters,
-            "ms_per_forward": dt / iters * 1e3, "gemm_solution_tuning": "torch.cuda.tunable" if tuned else None}
+    out = {"images_per_s": iters * batch / dt, "batch": batch, "dtype": "bf16", "iters": iters,
+           "ms_per_forward": dt / iters * 1e3, "gemm_solution_tuning": "torch.cuda.tunable" if tuned else None}
+    # the same forward as one HIP graph (one submission instead of ~190 launches), if it replays bit for bit
+    if use_graph:
+        if tuned:
+            torch.cuda.tunable.tuning_enable(False)  # every shape has its solution by now; none is tried under capture
+        graphed = evaluate.graphed_forward_checked(model, images)
+        if graphed is not None:
+            ips_g = evaluate.throughput(graphed, images, warmup=warmup, iters=iters)
+            out["hip_graph"] = {"images_per_s": ips_g, "ms_per_forward": batch / ips_g * 1e3,
+                                "replays_checked_against_eager": 4}
+        else:
+            out["hip_graph"] = None
+        # a small batch is bound by the ~190 launches, not by the kernels: there the graph is what counts
+        small = images[:16].contiguous()
+        ips_e = evaluate.throughput(model, small, warmup=warmup, iters=iters)
+        g16 = evaluate.graphed_forward_checked(model, small)
+        out["batch16_latency_ms"] = {"eager": 16 / ips_e * 1e3,
+                                     "hip_graph": 16 / evaluate.throughput(g16, small, warmup=warmup, iters=iters) * 1e3
+                                     if g16 is not None else None}
+    return out
 
 
 def backward_time(lib, sets, s, io_dt, scale, sp, stream, dev, iters=60):

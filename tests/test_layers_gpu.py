@@ -111,6 +111,31 @@ def test_evaluate_callers(tmp_path):
     assert ips > 0
 
 
+def test_graphed_forward_replays_match_eager():
+    """The eval forward captured as one HIP graph: every replay (with eager forwards, other inputs and
+    synchronisations in between) reproduces the eager logits bit for bit, also after the input buffer changes."""
+    import torch
+    from vig_amd import evaluate, layers
+
+    announce("evaluate.GraphedForward: 6 replays of a tiny ViG against the eager forward")
+    torch.manual_seed(0)
+    model = layers.ViG(img_size=64, depth=2, num_heads=3, embed_dim=96, num_classes=10).eval().cuda().to(torch.bfloat16)
+    g = torch.Generator().manual_seed(2)
+    batches = [torch.randn(8, 3, 64, 64, generator=g).cuda().to(torch.bfloat16) for _ in range(3)]
+    with torch.no_grad():
+        wants = [model(b).clone() for b in batches]
+    graphed = evaluate.graphed_forward_checked(model, batches[0], replays=2)
+    assert graphed is not None, "capture refused or a checked replay differed"
+    for i in range(6):
+        b = i % 3
+        got = graphed(batches[b]).clone()
+        torch.cuda.synchronize()
+        assert torch.equal(got, wants[b]), f"replay {i} differs from the eager forward"
+        with torch.no_grad():
+            model(batches[(b + 1) % 3] * 2.0)  # eager work between the replays
+        torch.cuda.synchronize()
+
+
 # ---- HierViG's GLA2D (classification/models/vig_h.py:338-606): Dk 16, Dv 32 at every stage ----
 def test_gla2d_parameter_names():
     m = layers.GLA2D(d_model=96, expand_k=0.5, expand_v=1.0, num_heads=3, use_act_in_conv=False, channel_first=True)

@@ -6,7 +6,7 @@ as used there; one process, one GPU (no reduce over ranks).  Forward only.
 from __future__ import annotations
 
 import time
-from typing import Iterable, Tuple
+from typing import Iterable, Optional, Tuple
 
 import torch
 import torch.nn.functional as F
@@ -62,7 +62,57 @@ def validate(model: torch.nn.Module, data_loader: Iterable, dtype: torch.dtype =
     return acc1_sum / n_total, acc5_sum / n_total, loss_sum / n_total
 
 
-@torch.no_grad()
+class GraphedForward:
+    """One eval forward of `model` on a fixed input shape, captured as a HIP graph and replayed: the ~190 kernel
+    launches of a ViG-S forward become one submission.  Everything the forward launches is a plain kernel on the
+    current stream (this library's entry points allocate nothing and never synchronise), so it captures as is; the
+    GEMM solution tuning, if on, has to have seen the shapes before (the warm-up forwards below do that)."""
+
+    def __init__(self, model: torch.nn.Module, example: torch.Tensor, warmup: int = 3):
+        self.model = model.eval()
+        self.static_in = example.clone()
+        side = torch.cuda.Stream(device=example.device)  # (default priority)
+        side.wait_stream(torch.cuda.current_stream(example.device))
+        with torch.cuda.stream(side), torch.no_grad():
+            for _ in range(warmup):
+                self.model(self.static_in)
+        torch.cuda.current_stream(example.device).wait_stream(side)
+        torch.cuda.synchronize(example.device)
+        self.graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(self.graph), torch.no_grad():
+            self.static_out = self.model(self.static_in)
+
+    def eval(self):
+        return self
+
+    def __call__(self, images: torch.Tensor) -> torch.Tensor:
+        if images.data_ptr() != self.static_in.data_ptr():
+            self.static_in.copy_(images)
+        self.graph.replay()
+        return self.static_out
+
+
+def graphed_forward_checked(model: torch.nn.Module, images: torch.Tensor, replays: int = 4) -> Optional[GraphedForward]:
+    """A GraphedForward that reproduced the eager logits bit for bit on `replays` replays with eager forwards and
+    synchronisations in between, or None (capture refused, or a replay differed: a library call inside the forward
+    may record nodes that do not replay faithfully)."""
+    try:
+        with torch.no_grad():
+            want = model(images).clone()
+        g = GraphedForward(model, images)
+        for i in range(replays):
+            got = g(images).clone()
+            torch.cuda.synchronize(images.device)
+            if not torch.equal(got, want):
+                return None
+            with torch.no_grad():
+                model(images + float(i + 1))  # eager work on other data between the replays
+            torch.cuda.synchronize(images.device)
+        return g
+    except Exception:  # noqa: BLE001 - capture is an optimisation; the eager forward is always there
+        return None
+
+
 def throughput(model: torch.nn.Module, images: torch.Tensor, warmup: int = 50, iters: int = 30) -> float:
     """Images per second of repeated forwards of one resident batch: `warmup` untimed and `iters` timed forwards
     between synchronisations (classification/main.py:388-406)."""

@@ -92,7 +92,6 @@ def gla_bidir_backward(q, k, v, g_fwd, g_bwd, d_o, scale: float = -1, out_scale:
                                    dgb.data_ptr() if dgb is not None else None, ws.data_ptr(), ws_bytes,
                                    B, H, L, Dk, Dv, float(scale), float(out_scale), _dt(q), _dt(g_fwd), _stream_ptr(q))
     _lib.check(rc, "vig_gla_bidir_bwd")
-    ws.record_stream(torch.cuda.current_stream(q.device))
     return dq, dk, dv, dgf, dgb
 
 
@@ -143,8 +142,6 @@ def _gla_bidir_forward_raw(q, k, v, g_fwd, g_bwd, scale, out_scale, exact, out):
                 ws.data_ptr() if ws is not None else None, ws_bytes,
                 B, H, L, Dk, Dv, float(scale), float(out_scale), io_dt, g_dt, _stream_ptr(q))
     _lib.check(rc, "vig_gla_bidir_fwd")
-    if ws is not None:
-        ws.record_stream(torch.cuda.current_stream(q.device))
     return out
 
 
