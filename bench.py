@@ -173,6 +173,8 @@ def main():
     ap.add_argument("--op-only", action="store_true", help="no model forward and no backward, whatever the workload")
     ap.add_argument("--no-gemm-tuning", action="store_true",
                     help="with --model: leave torch's GEMM solution tuning off (clean kernel traces)")
+    ap.add_argument("--no-graph", action="store_true",
+                    help="with --model: eager forwards only (no HIP graph capture, no batch-16 latency)")
     ap.add_argument("--unfused-gate", action="store_true",
                     help="workload 2: run the locality gate as a second kernel instead of inside the GLA kernel")
     ap.add_argument("--copy-calibration", action="store_true",
@@ -324,7 +326,7 @@ def main():
     if want_backward:
         out["backward"] = backward_time(lib, sets, s, io_dt, scale, sp, stream, dev)
     if want_model:
-        out["vig_s_forward"] = model_throughput(dev, tune_gemm=not args.no_gemm_tuning)
+        out["vig_s_forward"] = model_throughput(dev, tune_gemm=not args.no_gemm_tuning, use_graph=not args.no_graph)
     if not args.no_cpu:
         out["cpu_baseline"] = cpu_baseline(s, 1000 + args.config)
     else:

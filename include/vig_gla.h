@@ -137,6 +137,20 @@ int vig_dirgate_fwd(const void* gk_lin, void* g_out, int B, int L, int H, int Dk
                     int in_dtype, int out_dtype, void* stream);
 
 /*
+ * Direction-wise gate preparation with the second layer of the low-rank gate projection inside:
+ *   gk_low [B, L, rank] (token rows low_row_stride elements apart, 0 = packed), w_up [2*H*Dk, rank], b_up [2*H*Dk]
+ *   x = gk_low . w_up^T + b_up, rounded to in_dtype (what the separate layer would have stored);
+ *   g_out [2, B, H, L, Dk] as in vig_dirgate_fwd.  gk_low, w_up and b_up share in_dtype; rank must be 16; bases and
+ *   row strides in bytes must be multiples of 16.  The [B, L, 2*H*Dk] intermediate never goes to memory.
+ *
+ * Replaces: the second nn.Linear of gk_proj (classification/models/vig.py:296-297, applied at vig.py:432) together
+ * with vig.py:432-441.
+ */
+int vig_dirgate_lowrank_fwd(const void* gk_low, long long low_row_stride, const void* w_up, const void* b_up,
+                            void* g_out, int B, int L, int H, int Dk, int rank, float inv_normalizer, float clamp_min,
+                            int in_dtype, int out_dtype, void* stream);
+
+/*
  * 3x3 depthwise convolution on the token grid, channels-last, zero padding 1.
  *   x [B, L=h*w, C], weight [C, 3, 3] (f32), bias [C] (f32) or NULL -> y [B, L, C]
  *   optional SiLU on the result.
@@ -176,13 +190,15 @@ int vig_gla_bidir_locgate_fwd(const void* q, const void* k, const void* v, const
  *   y[b,l,hd*Dv+d] = rms(o[b,hd,l,:])*w_g * s + rms(local[b,l,hd,:])*w_l * (1-s),  s = sigmoid(g_lin[b,l,hd*Dv+d])
  *   rms(x) = x * rsqrt(mean(x^2) + eps); optional SiLU on y.
  * o [B,H,L,Dv]; local, g_lin, y [B, L, H*Dv]; w_g, w_l [Dv] f32.
+ * g_row_stride: elements between consecutive token rows of g_lin (0 = packed, H*Dv), so that g_lin may be a block
+ * of columns of a wider projection output; the base and the stride in bytes must be multiples of 16.
  *
  * Replaces: classification/models/vig.py:444-457 (two RMSNorm launches
  * fla/modules/rmsnorm.py:69-125, three rearranges, sigmoid blend, out_act).
  */
 int vig_locality_blend_fwd(const void* o, const void* local, const void* g_lin,
                            const float* w_g, const float* w_l, void* y,
-                           int B, int H, int L, int Dv, float eps, int silu_out,
+                           int B, int H, int L, int Dv, long long g_row_stride, float eps, int silu_out,
                            int io_dtype, void* stream);
 
 /*
@@ -201,12 +217,14 @@ int vig_rmsnorm_fwd(const void* x, const void* residual, const float* weight, vo
 /*
  * Head-major split of the fused q/k/v projection:
  *   qkv [B, L, H*Dk | H*Dk | H*Dv]  ->  q, k [B, H, L, Dk],  v [B, H, L, Dv]   (Dk, Dv multiples of 8)
+ * qkv_row_stride: elements between consecutive token rows of qkv (0 = packed), so that qkv may be the leading
+ * columns of a wider projection output; the base and the stride in bytes must be multiples of 16.
  *
  * Replaces: classification/models/vig.py:401-409 (torch.split and the three 'b l (h d) -> b h l d'
  * rearranges in front of the GLA op).
  */
 int vig_split_heads_fwd(const void* qkv, void* q, void* k, void* v, int B, int L, int H, int Dk, int Dv,
-                        int io_dtype, void* stream);
+                        long long qkv_row_stride, int io_dtype, void* stream);
 
 /*
  * SwiGLU product of the MLP:  gate_up [rows, 2*I] = (gate | up)  ->  out [rows, I] = gate * up / (1 + exp(-gate))

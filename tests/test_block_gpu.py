@@ -59,6 +59,21 @@ def test_split_heads_is_exact(dtype, B, L, H, Dk, Dv):
     assert np.array_equal(f64(q), wq) and np.array_equal(f64(k), wk) and np.array_equal(f64(v), wv)
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("B,L,H,Dk,Dv,W", [(2, 196, 6, 32, 64, 1280), (3, 7, 2, 16, 32, 136), (1, 50, 3, 64, 64, 588)])
+def test_split_heads_reads_a_column_block_in_place(dtype, B, L, H, Dk, Dv, W):
+    """qkv as the leading columns of a wider projection output: same result as on a packed copy; a row distance
+    that breaks the 16-byte alignment (the views that start at column 1, and W = 588 with bf16) is packed
+    by the wrapper."""
+    announce(f"split_heads strided {dtype} B{B} L{L} H{H} {Dk}/{Dv} W{W}")
+    n = H * (2 * Dk + Dv)
+    wide = _randn((B, L, W), 5, dtype).cuda()
+    for view in (wide[..., :n], wide[..., 8:8 + n], wide[..., 1:1 + n]):
+        q, k, v = vig_amd.ops.split_heads(view, H, Dk, Dv)
+        wq, wk, wv = O.split_heads_reference(f64(view), H, Dk, Dv)
+        assert np.array_equal(f64(q), wq) and np.array_equal(f64(k), wk) and np.array_equal(f64(v), wv)
+
+
 @pytest.mark.parametrize("dtype,tol", [(torch.float32, 2e-6), (torch.bfloat16, 2.0 ** -8)])
 @pytest.mark.parametrize("rows,I", [((2, 196), 1024), ((5,), 8), ((3, 4), 512)])
 def test_swiglu(dtype, tol, rows, I):

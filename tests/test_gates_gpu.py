@@ -31,6 +31,32 @@ def test_dirgate(dtype, tol, B, L, H, Dk):
     assert max_abs(gotc, wantc) <= tol
 
 
+@pytest.mark.parametrize("dtype,tol", [(torch.float32, 2e-6), (torch.bfloat16, 4e-3)])
+@pytest.mark.parametrize("B,L,H,Dk,wide", [(2, 196, 6, 32, 1280), (1, 197, 3, 64, 16), (3, 7, 2, 16, 24),
+                                           (2, 50, 12, 64, 40)])
+def test_dirgate_lowrank(dtype, tol, B, L, H, Dk, wide):
+    """The rank-16 up-projection inside the gate kernel against the fp64 restatement of the two steps (the
+    pre-activation rounded to the storage type in between, as the separate layer stores it): a pre-activation that
+    rounds the other way moves a gate by at most one storage ulp of the pre-activation / 16 (2^-9 for values in
+    [4, 8)), on top of the rounding of the output."""
+    announce(f"dirgate_lowrank {dtype} B{B} L{L} H{H} Dk{Dk} row width {wide}")
+    C2 = 2 * H * Dk
+    z = _randn((B, L, wide), 21, dtype)
+    w = _randn((C2, 16), 22, dtype, 0.5)
+    b = _randn((C2,), 23, dtype, 0.5)
+    low = z[..., wide - 16:]
+    pre = f64(low) @ f64(w).T + f64(b)
+    pre = f64(torch.from_numpy(pre).to(dtype))  # stored pre-activation
+    for clamp in (None, -0.03):
+        want = O.dirgate_reference(pre, H, 16.0, clamp_min=clamp)
+        got = vig_amd.ops.dirgate_lowrank(z.cuda()[..., wide - 16:], w.cuda(), b.cuda(), H, 16.0, clamp_min=clamp)
+        assert got.shape == want.shape
+        assert max_abs(f64(got), want) <= tol
+        # and against the two library steps it replaces
+        two = vig_amd.dirgate(torch.nn.functional.linear(low.cuda(), w.cuda(), b.cuda()), H, 16.0, clamp_min=clamp)
+        assert max_abs(f64(got), f64(two)) <= tol
+
+
 def test_dirgate_feeds_gla_layout():
     """g_out[0]/g_out[1] are directly the g_fwd/g_bwd operands (reference: cat([fw,bw],0) viewed as [2,B,...])."""
     announce("dirgate -> gla layout")
@@ -103,8 +129,13 @@ def test_locality_blend(dtype, tol, H, Dv, L):
     wl = _randn((Dv,), 14) * 0.1 + 1
     for silu in (False, True):
         want = O.locality_blend_reference(f64(o), f64(loc), f64(gl), f64(wg), f64(wl), 1e-6, silu)
-        got = f64(vig_amd.locality_blend(o.cuda(), loc.cuda(), gl.cuda(), wg.cuda(), wl.cuda(), 1e-6, silu))
-        assert max_abs(got, want) <= tol
+        got = vig_amd.locality_blend(o.cuda(), loc.cuda(), gl.cuda(), wg.cuda(), wl.cuda(), 1e-6, silu)
+        assert max_abs(f64(got), want) <= tol
+        # g_lin as a column block of a wider tensor is read in place: same bits as on the packed copy
+        wide = torch.zeros(B, L, H * Dv + 24, dtype=dtype).cuda()
+        wide[..., 16:16 + H * Dv] = gl.cuda()
+        got2 = vig_amd.locality_blend(o.cuda(), loc.cuda(), wide[..., 16:16 + H * Dv], wg.cuda(), wl.cuda(), 1e-6, silu)
+        assert torch.equal(got, got2)
 
 
 # ---- the locality gate fused into the GLA kernel (vig_gla_bidir_locgate_fwd) ----

@@ -17,6 +17,7 @@ _c_void_p = ctypes.c_void_p
 _c_int = ctypes.c_int
 _c_float = ctypes.c_float
 _c_size_t = ctypes.c_size_t
+_c_longlong = ctypes.c_longlong
 
 # name -> (restype, argtypes); mirrors include/vig_gla.h one to one.
 _GLA_SIG = [_c_void_p] * 6 + [_c_void_p, _c_size_t] + [_c_int] * 5 + [_c_float, _c_float, _c_int, _c_int, _c_void_p]
@@ -33,9 +34,10 @@ SIGNATURES = {
     "vig_dwconv3x3_fwd": (_c_int, [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_void_p]),
     "vig_gla_bidir_locgate_fwd": (_c_int, [_c_void_p] * 7 + [_c_int] * 7 + [_c_float, _c_float, _c_int, _c_int, _c_void_p]),
     "vig_locality_gate_fwd": (_c_int, [_c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_void_p]),
-    "vig_locality_blend_fwd": (_c_int, [_c_void_p] * 6 + [_c_int, _c_int, _c_int, _c_int, _c_float, _c_int, _c_int, _c_void_p]),
+    "vig_dirgate_lowrank_fwd": (_c_int, [_c_void_p, _c_longlong, _c_void_p, _c_void_p, _c_void_p] + [_c_int] * 5 + [_c_float, _c_float, _c_int, _c_int, _c_void_p]),
+    "vig_locality_blend_fwd": (_c_int, [_c_void_p] * 6 + [_c_int, _c_int, _c_int, _c_int, _c_longlong, _c_float, _c_int, _c_int, _c_void_p]),
     "vig_rmsnorm_fwd": (_c_int, [_c_void_p] * 5 + [ctypes.c_longlong, _c_int, _c_float, _c_int, _c_int, _c_void_p]),
-    "vig_split_heads_fwd": (_c_int, [_c_void_p] * 4 + [_c_int] * 6 + [_c_void_p]),
+    "vig_split_heads_fwd": (_c_int, [_c_void_p] * 4 + [_c_int] * 5 + [_c_longlong, _c_int, _c_void_p]),
     "vig_swiglu_fwd": (_c_int, [_c_void_p, _c_void_p, ctypes.c_longlong, _c_int, _c_int, _c_void_p]),
 }
 

@@ -8,14 +8,18 @@ int launch_dirgate(const void* in, void* out, int B, int L, int H, int Dk, float
                    int in_dtype, int out_dtype, hipStream_t stream);
 int launch_dwconv3x3(const void* x, const float* wt, const float* bias, void* y, int B, int h, int w, int C,
                      int silu, int io_dtype, hipStream_t stream);
+int launch_dirgate_lowrank(const void* low, long long ld, const void* w1, const void* b1, void* out, int B, int L,
+                           int H, int Dk, int rank, float inv_norm, float clamp_min, int in_dtype, int out_dtype,
+                           hipStream_t stream);
 int launch_locality_gate(const void* o, const float* wt, void* y, int B, int H, int h, int w, int Dv, int io_dtype,
                          hipStream_t stream);
 int launch_locality_blend(const void* o, const void* loc, const void* glin, const float* wg, const float* wl, void* y,
-                          int B, int H, int L, int Dv, float eps, int silu_out, int io_dtype, hipStream_t stream);
+                          int B, int H, int L, int Dv, long long ldg, float eps, int silu_out, int io_dtype,
+                          hipStream_t stream);
 int launch_rmsnorm(const void* x, const void* residual, const float* weight, void* y, void* residual_out, int rows,
                    int C, float eps, int round_sum, int io_dtype, hipStream_t stream);
-int launch_split_heads(const void* qkv, void* q, void* k, void* v, int B, int L, int H, int Dk, int Dv, int io_dtype,
-                       hipStream_t stream);
+int launch_split_heads(const void* qkv, void* q, void* k, void* v, int B, int L, int H, int Dk, int Dv, long long ld,
+                       int io_dtype, hipStream_t stream);
 int launch_swiglu(const void* in, void* out, long long rows, int I, int io_dtype, hipStream_t stream);
 int launch_pad_channels(const void* src, void* dst, long long rows, int src_c, int dst_c, hipStream_t stream);
 int launch_pad_channels_multi(const void* const* src, void* const* dst, const int* src_c, const int* dst_c, int n,
@@ -28,6 +32,12 @@ size_t gla_backward_workspace(int B, int H, int L, int Dk, int Dv, int bidir);
 }  // namespace vig
 
 static bool dtype_ok(int d) { return d == VIG_F32 || d == VIG_BF16; }
+
+// rows read with 16-byte vector loads: the base and the distance between rows have to keep that alignment
+static bool strided_rows_ok(const void* base, long long ld_elems, int dtype) {
+  const long long elem = dtype == VIG_BF16 ? 2 : 4;
+  return (reinterpret_cast<uintptr_t>(base) % 16) == 0 && (ld_elems * elem) % 16 == 0;
+}
 static bool dk_ok(int d) { return d == 16 || d == 32 || d == 64 || d == 128; }
 static bool dv_ok(int d) { return d == 32 || d == 64 || d == 128; }
 
@@ -170,6 +180,19 @@ int vig_dirgate_fwd(const void* gk_lin, void* g_out, int B, int L, int H, int Dk
                              (hipStream_t)stream);
 }
 
+int vig_dirgate_lowrank_fwd(const void* gk_low, long long low_row_stride, const void* w_up, const void* b_up,
+                            void* g_out, int B, int L, int H, int Dk, int rank, float inv_normalizer, float clamp_min,
+                            int in_dtype, int out_dtype, void* stream) {
+  if (!gk_low || !w_up || !b_up || !g_out || B <= 0 || L <= 0 || H <= 0 || Dk <= 0 || rank <= 0) return VIG_EINVAL;
+  if (!dtype_ok(in_dtype) || !dtype_ok(out_dtype) || (Dk % 8) != 0 || rank != 16) return VIG_ENOTSUP;
+  const long long ld = low_row_stride > 0 ? low_row_stride : rank;
+  if (ld < rank || !strided_rows_ok(gk_low, ld, in_dtype) || !strided_rows_ok(w_up, rank, in_dtype) ||
+      !strided_rows_ok(b_up, 8, in_dtype))
+    return VIG_EINVAL;
+  return vig::launch_dirgate_lowrank(gk_low, ld, w_up, b_up, g_out, B, L, H, Dk, rank, inv_normalizer, clamp_min,
+                                     in_dtype, out_dtype, (hipStream_t)stream);
+}
+
 int vig_dwconv3x3_fwd(const void* x, const float* weight, const float* bias, void* y, int B, int h, int w, int C,
                       int silu, int io_dtype, void* stream) {
   if (!x || !weight || !y || B <= 0 || h <= 0 || w <= 0 || C <= 0 || x == y) return VIG_EINVAL;
@@ -185,11 +208,13 @@ int vig_locality_gate_fwd(const void* o, const float* weight, void* y, int B, in
 }
 
 int vig_locality_blend_fwd(const void* o, const void* local, const void* g_lin, const float* w_g, const float* w_l,
-                           void* y, int B, int H, int L, int Dv, float eps, int silu_out, int io_dtype,
-                           void* stream) {
+                           void* y, int B, int H, int L, int Dv, long long g_row_stride, float eps, int silu_out,
+                           int io_dtype, void* stream) {
   if (!o || !local || !g_lin || !w_g || !w_l || !y || B <= 0 || H <= 0 || L <= 0) return VIG_EINVAL;
   if (!dtype_ok(io_dtype) || !(Dv == 32 || Dv == 64)) return VIG_ENOTSUP;
-  return vig::launch_locality_blend(o, local, g_lin, w_g, w_l, y, B, H, L, Dv, eps, silu_out, io_dtype,
+  const long long ldg = g_row_stride > 0 ? g_row_stride : (long long)H * Dv;
+  if (ldg < (long long)H * Dv || !strided_rows_ok(g_lin, ldg, io_dtype)) return VIG_EINVAL;
+  return vig::launch_locality_blend(o, local, g_lin, w_g, w_l, y, B, H, L, Dv, ldg, eps, silu_out, io_dtype,
                                     (hipStream_t)stream);
 }
 
@@ -202,10 +227,13 @@ int vig_rmsnorm_fwd(const void* x, const void* residual, const float* weight, vo
 }
 
 int vig_split_heads_fwd(const void* qkv, void* q, void* k, void* v, int B, int L, int H, int Dk, int Dv,
-                        int io_dtype, void* stream) {
+                        long long qkv_row_stride, int io_dtype, void* stream) {
   if (!qkv || !q || !k || !v || B <= 0 || L <= 0 || H <= 0 || Dk <= 0 || Dv <= 0) return VIG_EINVAL;
   if (!dtype_ok(io_dtype) || (Dk % 8) != 0 || (Dv % 8) != 0 || B > 65535) return VIG_ENOTSUP;
-  return vig::launch_split_heads(qkv, q, k, v, B, L, H, Dk, Dv, io_dtype, (hipStream_t)stream);
+  const long long packed = (long long)H * (2 * Dk + Dv);
+  const long long ld = qkv_row_stride > 0 ? qkv_row_stride : packed;
+  if (ld < packed || !strided_rows_ok(qkv, ld, io_dtype)) return VIG_EINVAL;
+  return vig::launch_split_heads(qkv, q, k, v, B, L, H, Dk, Dv, ld, io_dtype, (hipStream_t)stream);
 }
 
 int vig_swiglu_fwd(const void* gate_up, void* out, long long rows, int I, int io_dtype, void* stream) {

@@ -137,13 +137,14 @@ int launch_rmsnorm(const void* x, const void* residual, const float* weight, voi
 // ---------------------------------------------------------------------------
 // head-major split of the fused projection:
 //   qkv [B, L, H*Dk | H*Dk | H*Dv]  ->  q, k [B, H, L, Dk],  v [B, H, L, Dv]
+// A token's row may sit inside a wider row of `ld` elements (the columns of a larger projection).
 // One workgroup owns 32 consecutive tokens of one batch element: whole rows are read, and every (tensor, head)
 // receives a contiguous run of 32 tokens.
 // ---------------------------------------------------------------------------
 template <typename T>
 __global__ __launch_bounds__(256) void split_heads_kernel(const T* __restrict__ qkv, T* __restrict__ q,
                                                           T* __restrict__ k, T* __restrict__ v, int B, int L, int H,
-                                                          int Dk, int Dv) {
+                                                          int Dk, int Dv, long long ld) {
   const int K = H * Dk, V = H * Dv;
   const int row = 2 * K + V;
   const int nv = row >> 3;
@@ -158,28 +159,28 @@ __global__ __launch_bounds__(256) void split_heads_kernel(const T* __restrict__ 
     else if (ch < 2 * K) { dst = k; D = Dk; c = ch - K; }
     else { dst = v; D = Dv; c = ch - 2 * K; }
     const int hh = c / D, d = c - hh * D;
-    const T* src = qkv + ((size_t)b * L) * (size_t)row + ch;
+    const T* src = qkv + ((size_t)b * L) * (size_t)ld + ch;
     T* out = dst + (((size_t)b * H + hh) * L) * (size_t)D + d;
     for (int t = ty; t < 32; t += 4) {
       const int l = l0 + t;
       if (l >= L) break;
       float x[8];
-      Oct<T>::load(src + (size_t)l * row, x);
+      Oct<T>::load(src + (size_t)l * ld, x);
       Oct<T>::store(out + (size_t)l * D, x);
     }
   }
 }
 
-int launch_split_heads(const void* qkv, void* q, void* k, void* v, int B, int L, int H, int Dk, int Dv, int io_dtype,
-                       hipStream_t stream) {
+int launch_split_heads(const void* qkv, void* q, void* k, void* v, int B, int L, int H, int Dk, int Dv, long long ld,
+                       int io_dtype, hipStream_t stream) {
   if (Dk % 8 != 0 || Dv % 8 != 0 || B > 65535) return -95;
   const dim3 grid((L + 31) / 32, B), block(256);
   if (io_dtype == 1)
     hipLaunchKernelGGL(split_heads_kernel<uint16_t>, grid, block, 0, stream, (const uint16_t*)qkv, (uint16_t*)q,
-                       (uint16_t*)k, (uint16_t*)v, B, L, H, Dk, Dv);
+                       (uint16_t*)k, (uint16_t*)v, B, L, H, Dk, Dv, ld);
   else
     hipLaunchKernelGGL(split_heads_kernel<float>, grid, block, 0, stream, (const float*)qkv, (float*)q, (float*)k,
-                       (float*)v, B, L, H, Dk, Dv);
+                       (float*)v, B, L, H, Dk, Dv, ld);
   return hipGetLastError() == hipSuccess ? 0 : -5;
 }
 

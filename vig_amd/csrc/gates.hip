@@ -106,6 +106,183 @@ int launch_dirgate(const void* in, void* out, int B, int L, int H, int Dk, float
 }
 
 // ---------------------------------------------------------------------------
+// direction-wise gate preparation with the second (rank -> 2*H*Dk) layer of the gate projection inside:
+//   low [B, L, 16] (rows ld elements apart), w1 [2*H*Dk, 16], b1 [2*H*Dk]
+//   x = low . w1^T + b1, rounded to the storage type of `low` (what the separate layer would have stored),
+//   out [2, B, H, L, Dk] = logsigmoid(x) * inv_norm, clamp
+// The rank-16 product is 16 multiply-adds per output, far below what the output write costs, so the [B, L, 2*H*Dk]
+// intermediate never goes to memory.  One workgroup owns 32 consecutive tokens of one batch element; their low-rank
+// rows sit in LDS as f32; a thread keeps the 8x16 weights of one channel octet in registers for all its tokens.
+// ---------------------------------------------------------------------------
+constexpr int kGateRank = 16;
+
+template <typename T> struct Stored;  // value after a round trip through the storage type
+template <> struct Stored<float> { static __device__ __forceinline__ float of(float x) { return x; } };
+template <> struct Stored<uint16_t> {
+  static __device__ __forceinline__ float of(float x) { return bf16_to_f32(f32_to_bf16(x)); }
+};
+
+template <typename TI, typename TO>
+__global__ __launch_bounds__(256) void dirgate_lowrank_kernel(const TI* __restrict__ low, long long ld,
+                                                               const TI* __restrict__ w1, const TI* __restrict__ b1,
+                                                               TO* __restrict__ out, int B, int L, int H, int Dk,
+                                                               float inv_norm, float clamp_min, int use_clamp) {
+  constexpr int R = kGateRank, TOK = 32;
+  __shared__ float lowf[TOK][R];
+  const int nv = 2 * H * Dk / 8;  // channel octets per token row
+  const int dk8 = Dk >> 3;
+  const int b = blockIdx.y;
+  const int l0 = blockIdx.x * TOK;
+  if (threadIdx.x < TOK * (R / 8)) {
+    const int t = threadIdx.x / (R / 8), part = threadIdx.x % (R / 8);
+    float x[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+    if (l0 + t < L) Vec8<TI>::load(low + ((size_t)b * L + l0 + t) * (size_t)ld + part * 8, x);
+#pragma unroll
+    for (int j = 0; j < 8; ++j) lowf[t][part * 8 + j] = x[j];
+  }
+  __syncthreads();
+  const int per = nv < 256 ? nv : 256;  // threads side by side on one token
+  const int groups = 256 / per;         // tokens in flight
+  const int oc = threadIdx.x % per, tg = threadIdx.x / per;
+  if (tg >= groups) return;
+  for (int cv = oc; cv < nv; cv += per) {
+    float w[8][R], bias[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j)
+#pragma unroll
+      for (int p = 0; p < R / 8; ++p) {
+        float x[8];
+        Vec8<TI>::load(w1 + ((size_t)cv * 8 + j) * R + p * 8, x);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) w[j][p * 8 + i] = x[i];
+      }
+    Vec8<TI>::load(b1 + (size_t)cv * 8, bias);
+    const int d8 = cv % dk8, hh = (cv / dk8) % H, dir = cv / (dk8 * H);
+    TO* dst = out + ((((size_t)dir * B + b) * H + hh) * L) * (size_t)Dk + (size_t)d8 * 8;
+    for (int t = tg; t < TOK; t += groups) {
+      const int l = l0 + t;
+      if (l >= L) break;
+      float acc[8];
+#pragma unroll
+      for (int j = 0; j < 8; ++j) acc[j] = 0.f;
+#pragma unroll
+      for (int r = 0; r < R; ++r) {
+        const float xr = lowf[t][r];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) acc[j] = __builtin_fmaf(xr, w[j][r], acc[j]);
+      }
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        const float x = Stored<TI>::of(acc[j] + bias[j]);
+        float yv = fminf(x, 0.f) - __logf(1.f + __expf(-fabsf(x)));
+        yv *= inv_norm;
+        if (use_clamp) yv = fmaxf(yv, clamp_min);
+        acc[j] = yv;
+      }
+      Vec8<TO>::store(dst + (size_t)l * Dk, acc);
+    }
+  }
+}
+
+// The same for bf16 inputs on the matrix cores: one v_mfma_f32_32x32x16_bf16 is the whole rank-16 product of 32
+// channels x 32 tokens.  Operand A holds weight rows, operand B the tokens' low-rank rows, both read straight from
+// memory as one 16-byte load per lane (lane = (row r, contraction half h) supplies elements 8h..8h+7 of its row).
+// Accumulator register 4g+m of lane (r, h) holds matrix row 8g+4h+m of column r; matrix row i is given channel
+// 16*((i>>2)&1) + 4*(i>>3) + (i&3) of the tile, so that lane (r, h) ends up with channels 16h..16h+15 of token r:
+// 32 contiguous bytes of the head-major output.  Tokens are numbered over B*L; a workgroup owns 32 of them and its
+// four waves take the channel tiles in turn.  Needs Dk % 16 == 0 (a 16-channel run stays inside one head).
+template <typename TO>
+__global__ __launch_bounds__(256) void dirgate_lowrank_mfma_kernel(const uint16_t* __restrict__ low, long long ld,
+                                                                    const uint16_t* __restrict__ w1,
+                                                                    const uint16_t* __restrict__ b1,
+                                                                    TO* __restrict__ out, long long ntok, int B, int L,
+                                                                    int H, int Dk, float inv_norm, float clamp_min,
+                                                                    int use_clamp) {
+  constexpr int R = kGateRank;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int r = lane & 31, h = lane >> 5;
+  const long long tok = (long long)blockIdx.x * 32 + r;
+  const bool tok_ok = tok < ntok;
+  const long long tokc = tok_ok ? tok : ntok - 1;
+  const u32x4_t xb = *reinterpret_cast<const u32x4_t*>(low + (size_t)tokc * (size_t)ld + 8 * h);
+  const int b = (int)(tokc / L), l = (int)(tokc - (long long)b * L);
+  const int chan_of_row = 16 * ((r >> 2) & 1) + 4 * (r >> 3) + (r & 3);
+  const int ntiles = 2 * H * Dk / 32;
+  for (int tile = wave; tile < ntiles; tile += 4) {
+    const int c0 = tile * 32;
+    const u32x4_t wa = *reinterpret_cast<const u32x4_t*>(w1 + (size_t)(c0 + chan_of_row) * R + 8 * h);
+    float bias[16];
+    {
+      float x[8];
+      Vec8<uint16_t>::load(b1 + c0 + 16 * h, x);
+#pragma unroll
+      for (int j = 0; j < 8; ++j) bias[j] = x[j];
+      Vec8<uint16_t>::load(b1 + c0 + 16 * h + 8, x);
+#pragma unroll
+      for (int j = 0; j < 8; ++j) bias[8 + j] = x[j];
+    }
+    f32x16_t acc;
+#pragma unroll
+    for (int j = 0; j < 16; ++j) acc[j] = 0.f;
+    acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, wa), __builtin_bit_cast(bf16x8_t, xb),
+                                                  acc, 0, 0, 0);
+    float y[16];
+#pragma unroll
+    for (int j = 0; j < 16; ++j) {
+      const float x = Stored<uint16_t>::of(acc[j] + bias[j]);
+      float yv = fminf(x, 0.f) - __logf(1.f + __expf(-fabsf(x)));
+      yv *= inv_norm;
+      if (use_clamp) yv = fmaxf(yv, clamp_min);
+      y[j] = yv;
+    }
+    const int c = c0 + 16 * h;  // first of this lane's 16 channels
+    const int d = c % Dk, hh = (c / Dk) % H, dir = c / (Dk * H);
+    if (tok_ok) {
+      TO* dst = out + ((((size_t)dir * B + b) * H + hh) * L + l) * (size_t)Dk + d;
+      float lo[8], hi[8];
+#pragma unroll
+      for (int j = 0; j < 8; ++j) lo[j] = y[j], hi[j] = y[8 + j];
+      Vec8<TO>::store(dst, lo);
+      Vec8<TO>::store(dst + 8, hi);
+    }
+  }
+}
+
+template <typename TI, typename TO>
+static int launch_dirgate_lowrank_t(const void* low, long long ld, const void* w1, const void* b1, void* out, int B,
+                                    int L, int H, int Dk, float inv_norm, float clamp_min, hipStream_t stream) {
+  const int use_clamp = clamp_min == clamp_min;  // NaN disables
+  if (B > 65535) return -22;
+  hipLaunchKernelGGL((dirgate_lowrank_kernel<TI, TO>), dim3((L + 31) / 32, B), dim3(256), 0, stream, (const TI*)low, ld,
+                     (const TI*)w1, (const TI*)b1, (TO*)out, B, L, H, Dk, inv_norm, clamp_min, use_clamp);
+  return hipGetLastError() == hipSuccess ? 0 : -5;
+}
+
+int launch_dirgate_lowrank(const void* low, long long ld, const void* w1, const void* b1, void* out, int B, int L,
+                           int H, int Dk, int rank, float inv_norm, float clamp_min, int in_dtype, int out_dtype,
+                           hipStream_t stream) {
+  if (rank != kGateRank) return -95;
+  if (in_dtype == 1 && Dk % 16 == 0 && B <= 65535) {
+    const int use_clamp = clamp_min == clamp_min;  // NaN disables
+    const long long ntok = (long long)B * L;
+    const dim3 grid((unsigned)((ntok + 31) / 32)), block(256);
+    if (out_dtype == 1)
+      hipLaunchKernelGGL(dirgate_lowrank_mfma_kernel<uint16_t>, grid, block, 0, stream, (const uint16_t*)low, ld,
+                         (const uint16_t*)w1, (const uint16_t*)b1, (uint16_t*)out, ntok, B, L, H, Dk, inv_norm,
+                         clamp_min, use_clamp);
+    else
+      hipLaunchKernelGGL(dirgate_lowrank_mfma_kernel<float>, grid, block, 0, stream, (const uint16_t*)low, ld,
+                         (const uint16_t*)w1, (const uint16_t*)b1, (float*)out, ntok, B, L, H, Dk, inv_norm,
+                         clamp_min, use_clamp);
+    return hipGetLastError() == hipSuccess ? 0 : -5;
+  }
+  if (in_dtype == 0 && out_dtype == 0) return launch_dirgate_lowrank_t<float, float>(low, ld, w1, b1, out, B, L, H, Dk, inv_norm, clamp_min, stream);
+  if (in_dtype == 0 && out_dtype == 1) return launch_dirgate_lowrank_t<float, uint16_t>(low, ld, w1, b1, out, B, L, H, Dk, inv_norm, clamp_min, stream);
+  if (in_dtype == 1 && out_dtype == 0) return launch_dirgate_lowrank_t<uint16_t, float>(low, ld, w1, b1, out, B, L, H, Dk, inv_norm, clamp_min, stream);
+  return launch_dirgate_lowrank_t<uint16_t, uint16_t>(low, ld, w1, b1, out, B, L, H, Dk, inv_norm, clamp_min, stream);
+}
+
+// ---------------------------------------------------------------------------
 // 3x3 depthwise stencil on the token grid, channels-last.  One workgroup owns one image (or one head slab), a
 // group of 64 channels and a band of grid rows: it stages the band plus a one-cell halo all around in LDS, with
 // zeros where the halo leaves the grid (coalesced 16-byte loads, every input byte leaves L2 once, and no tap needs a
@@ -226,7 +403,8 @@ __global__ __launch_bounds__(256) void locality_blend_kernel(const T* __restrict
                                                               const T* __restrict__ glin,
                                                               const float* __restrict__ wg,
                                                               const float* __restrict__ wl, T* __restrict__ y,
-                                                              int H, int L, int Dv, float eps, int silu_out) {
+                                                              int H, int L, int Dv, long long ldg, float eps,
+                                                              int silu_out) {
   const int d8n = Dv >> 3;  // lanes per row: 4 (Dv=32) or 8 (Dv=64); divides 64, so groups never straddle a wave
   const int nv = H * d8n;   // channel octets per token row
   const int b = blockIdx.y;
@@ -243,6 +421,7 @@ __global__ __launch_bounds__(256) void locality_blend_kernel(const T* __restrict
     for (int j = 0; j < 8; ++j) w_g[j] = wg[d8 * 8 + j], w_l[j] = wl[d8 * 8 + j];
     const T* po = o + (((size_t)b * H + hd) * L) * (size_t)Dv + d8 * 8;
     const size_t row0 = ((size_t)b * L) * (size_t)(nv * 8) + (size_t)cvc * 8;
+    const T* pg = glin + ((size_t)b * L) * (size_t)ldg + (size_t)cvc * 8;  // g_lin rows are ldg elements apart
     for (int t = ty; t < 32; t += 4) {
       const int l = l0 + t;
       if (l >= L) break;  // uniform over the wave: a wave shares its token
@@ -250,7 +429,7 @@ __global__ __launch_bounds__(256) void locality_blend_kernel(const T* __restrict
       const size_t tok = row0 + (size_t)l * (nv * 8);
       Vec8<T>::load(po + (size_t)l * Dv, xo);
       Vec8<T>::load(loc + tok, xl);
-      Vec8<T>::load(glin + tok, xg);
+      Vec8<T>::load(pg + (size_t)l * ldg, xg);
       float so = 0.f, sl = 0.f;
 #pragma unroll
       for (int j = 0; j < 8; ++j) so += xo[j] * xo[j], sl += xl[j] * xl[j];
@@ -274,15 +453,16 @@ __global__ __launch_bounds__(256) void locality_blend_kernel(const T* __restrict
 }
 
 int launch_locality_blend(const void* o, const void* loc, const void* glin, const float* wg, const float* wl, void* y,
-                          int B, int H, int L, int Dv, float eps, int silu_out, int io_dtype, hipStream_t stream) {
+                          int B, int H, int L, int Dv, long long ldg, float eps, int silu_out, int io_dtype,
+                          hipStream_t stream) {
   if (B > 65535) return -22;
   const dim3 grid((L + 31) / 32, B), block(256);
   if (io_dtype == 0)
     hipLaunchKernelGGL((locality_blend_kernel<float>), grid, block, 0, stream, (const float*)o, (const float*)loc,
-                       (const float*)glin, wg, wl, (float*)y, H, L, Dv, eps, silu_out);
+                       (const float*)glin, wg, wl, (float*)y, H, L, Dv, ldg, eps, silu_out);
   else
     hipLaunchKernelGGL((locality_blend_kernel<uint16_t>), grid, block, 0, stream, (const uint16_t*)o,
-                       (const uint16_t*)loc, (const uint16_t*)glin, wg, wl, (uint16_t*)y, H, L, Dv, eps, silu_out);
+                       (const uint16_t*)loc, (const uint16_t*)glin, wg, wl, (uint16_t*)y, H, L, Dv, ldg, eps, silu_out);
   return hipGetLastError() == hipSuccess ? 0 : -5;
 }
 

@@ -99,6 +99,7 @@ class GatedLinearAttention(nn.Module):
         self.g_norm = RMSNorm(self.head_v_dim, eps=layernorm_eps)
         self.l_norm = RMSNorm(self.head_v_dim, eps=layernorm_eps)
         self.g_proj = nn.Linear(d_model, self.value_dim, bias=True)
+        self._in_cat = None  # (key, weight, bias) of the concatenated input projection, built on first use
         self.reset_parameters()
 
     def reset_parameters(self):
@@ -110,16 +111,43 @@ class GatedLinearAttention(nn.Module):
         nn.init.xavier_uniform_(self.gk_proj[0].weight, gain=gain)
         nn.init.xavier_uniform_(self.gk_proj[1].weight, gain=gain)
 
+    def _input_projections(self, xs):
+        """qkv_proj, g_proj and the first (low-rank) gk_proj layer all read xs: they run as ONE matrix product with
+        the three weights stacked (rows padded with zeros to a multiple of 128, which the GEMM tiles prefer), and the
+        consumers read their column blocks of the result in place.  Every output column is the same dot product (and
+        bias add) as in the separate layers.  The stacked copy follows the parameters: it is rebuilt when one of them
+        is replaced, moved, cast or written in place."""
+        srcs = (self.qkv_proj.weight, self.g_proj.weight, self.g_proj.bias, self.gk_proj[0].weight)
+        key = tuple((t.data_ptr(), t._version, t.dtype, t.device) for t in srcs)
+        if self._in_cat is None or self._in_cat[0] != key:
+            wq, wg, bg, wr = (t.detach() for t in srcs)
+            n = wq.shape[0] + wg.shape[0] + wr.shape[0]
+            w = wq.new_zeros((n + 127) // 128 * 128, wq.shape[1])
+            b = wq.new_zeros(w.shape[0])
+            w[:n] = torch.cat((wq, wg, wr), 0)
+            b[wq.shape[0]:wq.shape[0] + wg.shape[0]] = bg
+            self._in_cat = (key, w, b)
+        _, w, b = self._in_cat
+        z = F.linear(xs, w, b)
+        n0 = self.qkv_proj.weight.shape[0]
+        n1 = n0 + self.value_dim
+        return z[..., :n0], z[..., n0:n1], z[..., n1:n1 + self.gk_proj[0].weight.shape[0]]
+
     def _mix(self, x, hw, out_scale):
         """The token mixer on x [B, L, C] with L = h*w tokens in row-major grid order."""
         H = self.num_heads
         conv = self.in_proj[0]
         # local_out, already in the [B, L, C] layout the projections consume
         xs = ops.dwconv3x3(x, conv.weight, hw, bias=conv.bias, silu=self.use_act_in_conv)
-        q, k, v = ops.split_heads(self.qkv_proj(xs), H, self.head_qk_dim, self.head_v_dim)
-        gates = ops.dirgate(self.gk_proj(xs), H, self.gate_logit_normalizer, self.clamp_min)
+        qkv, g_lin, gk_low = self._input_projections(xs)
+        q, k, v = ops.split_heads(qkv, H, self.head_qk_dim, self.head_v_dim)
+        up = self.gk_proj[1]
+        if gk_low.shape[-1] == ops.GATE_RANK:  # the rank-16 up-projection runs inside the gate kernel
+            gates = ops.dirgate_lowrank(gk_low, up.weight, up.bias, H, self.gate_logit_normalizer, self.clamp_min)
+        else:
+            gates = ops.dirgate(up(gk_low), H, self.gate_logit_normalizer, self.clamp_min)
         o = ops.gla_bidir_forward(q, k, v, gates[0], gates[1], scale=-1, out_scale=out_scale)
-        y = ops.locality_blend(o, xs, self.g_proj(xs), self.g_norm._w32(), self.l_norm._w32(),
+        y = ops.locality_blend(o, xs, g_lin, self.g_norm._w32(), self.l_norm._w32(),
                                eps=self.layernorm_eps, silu_out=self.use_out_act)
         return self.o_proj(y)
 

@@ -225,6 +225,37 @@ def dirgate(gk_lin: torch.Tensor, num_heads: int, gate_logit_normalizer: float =
     return out
 
 
+GATE_RANK = 16  # the low-rank width vig_dirgate_lowrank_fwd is built for (gate_low_rank_dim of every shipped config)
+
+
+def dirgate_lowrank(gk_low: torch.Tensor, w_up: torch.Tensor, b_up: torch.Tensor, num_heads: int,
+                    gate_logit_normalizer: float = 16.0, clamp_min: Optional[float] = None,
+                    out_dtype: Optional[torch.dtype] = None) -> torch.Tensor:
+    """gk_low [B,L,16] (may be a column block of a wider tensor), w_up [2*H*Dk,16], b_up [2*H*Dk] ->
+    [2,B,H,L,Dk] = logsigmoid(gk_low @ w_up.T + b_up)/normalizer: the second gk_proj layer (vig.py:296-297) and
+    vig.py:432-441 in one kernel; the pre-activation is rounded to gk_low's dtype as the separate layer stores it."""
+    lib = _lib.load()
+    _check_cuda(gk_low, w_up, b_up)
+    gk_low, ld = _token_rows(gk_low)
+    B, L, R = gk_low.shape
+    w_up, b_up = w_up.detach().contiguous(), b_up.detach().contiguous()
+    C2 = w_up.shape[0]
+    if w_up.shape != (C2, R) or b_up.shape != (C2,) or C2 % (2 * num_heads):
+        raise ValueError("w_up must be [2*H*Dk, rank] and b_up [2*H*Dk]")
+    if w_up.dtype != gk_low.dtype or b_up.dtype != gk_low.dtype:
+        raise TypeError("gk_low, w_up and b_up must share a dtype")
+    Dk = C2 // (2 * num_heads)
+    out_dtype = out_dtype or gk_low.dtype
+    out = torch.empty(2, B, num_heads, L, Dk, dtype=out_dtype, device=gk_low.device)
+    with torch.cuda.device(gk_low.device):
+        rc = lib.vig_dirgate_lowrank_fwd(gk_low.data_ptr(), ld, w_up.data_ptr(), b_up.data_ptr(), out.data_ptr(),
+                                         B, L, num_heads, Dk, R, 1.0 / float(gate_logit_normalizer),
+                                         float("nan") if clamp_min is None else float(clamp_min),
+                                         _dt(gk_low), _DT[out_dtype], _stream_ptr(gk_low))
+    _lib.check(rc, "vig_dirgate_lowrank_fwd")
+    return out
+
+
 def dwconv3x3(x: torch.Tensor, weight: torch.Tensor, hw, bias: Optional[torch.Tensor] = None,
               silu: bool = False) -> torch.Tensor:
     """x [B,L,C] on the (h,w) token grid; weight [C,1,3,3] or [C,3,3]; returns [B,L,C]."""
@@ -298,12 +329,26 @@ def gla_bidir_locality_gate(q, k, v, g_fwd, g_bwd, weight: torch.Tensor, hw, sca
     return y
 
 
+def _token_rows(t: torch.Tensor):
+    """t [B, L, C] as (tensor, elements between token rows): a column block of a contiguous wider [B, L, W] tensor
+    is passed as it lies when its rows keep the 16-byte alignment of the vector loads, anything else is packed."""
+    if t.dim() == 3 and not t.is_contiguous():
+        B, L, C = t.shape
+        sb, sl, sc = t.stride()
+        if sc == 1 and sl >= C and sb == L * sl and (sl * t.element_size()) % 16 == 0 and t.data_ptr() % 16 == 0:
+            return t, sl
+    t = t.contiguous()
+    return t, t.shape[-1]
+
+
 def locality_blend(o: torch.Tensor, local: torch.Tensor, g_lin: torch.Tensor, w_g: torch.Tensor,
                    w_l: torch.Tensor, eps: float = 1e-6, silu_out: bool = False) -> torch.Tensor:
-    """Block epilogue (vig.py:444-457): o [B,H,L,Dv]; local, g_lin [B,L,H*Dv] -> y [B,L,H*Dv]."""
+    """Block epilogue (vig.py:444-457): o [B,H,L,Dv]; local, g_lin [B,L,H*Dv] -> y [B,L,H*Dv].
+    g_lin may be a block of columns of a wider [B, L, W] tensor (it is read in place)."""
     lib = _lib.load()
     _check_cuda(o, local, g_lin, w_g, w_l)
-    o, local, g_lin = o.contiguous(), local.contiguous(), g_lin.contiguous()
+    o, local = o.contiguous(), local.contiguous()
+    g_lin, ldg = _token_rows(g_lin)
     B, H, L, Dv = o.shape
     if local.shape != (B, L, H * Dv) or g_lin.shape != (B, L, H * Dv):
         raise ValueError("local and g_lin must be [B, L, H*Dv]")
@@ -314,7 +359,7 @@ def locality_blend(o: torch.Tensor, local: torch.Tensor, g_lin: torch.Tensor, w_
     wl = w_l.detach().float().contiguous()
     with torch.cuda.device(o.device):
         rc = lib.vig_locality_blend_fwd(o.data_ptr(), local.data_ptr(), g_lin.data_ptr(), wg.data_ptr(),
-                                        wl.data_ptr(), y.data_ptr(), B, H, L, Dv, float(eps), int(silu_out),
+                                        wl.data_ptr(), y.data_ptr(), B, H, L, Dv, ldg, float(eps), int(silu_out),
                                         _dt(o), _stream_ptr(o))
     _lib.check(rc, "vig_locality_blend_fwd")
     return y
@@ -353,10 +398,11 @@ def rmsnorm(x: torch.Tensor, weight: torch.Tensor, eps: float = 1e-6, residual: 
 
 
 def split_heads(qkv: torch.Tensor, num_heads: int, head_qk_dim: int, head_v_dim: int):
-    """qkv [B, L, H*Dk | H*Dk | H*Dv] -> q, k [B,H,L,Dk], v [B,H,L,Dv] (vig.py:401-409)."""
+    """qkv [B, L, H*Dk | H*Dk | H*Dv] -> q, k [B,H,L,Dk], v [B,H,L,Dv] (vig.py:401-409).
+    qkv may be a block of columns of a wider [B, L, W] tensor (it is read in place)."""
     lib = _lib.load()
     _check_cuda(qkv)
-    qkv = qkv.contiguous()
+    qkv, ld = _token_rows(qkv)
     B, L, W = qkv.shape
     H = num_heads
     if W != H * (2 * head_qk_dim + head_v_dim):
@@ -366,7 +412,7 @@ def split_heads(qkv: torch.Tensor, num_heads: int, head_qk_dim: int, head_v_dim:
     v = torch.empty(B, H, L, head_v_dim, dtype=qkv.dtype, device=qkv.device)
     with torch.cuda.device(qkv.device):
         rc = lib.vig_split_heads_fwd(qkv.data_ptr(), q.data_ptr(), k.data_ptr(), v.data_ptr(), B, L, H, head_qk_dim,
-                                     head_v_dim, _dt(qkv), _stream_ptr(qkv))
+                                     head_v_dim, ld, _dt(qkv), _stream_ptr(qkv))
     _lib.check(rc, "vig_split_heads_fwd")
     return q, k, v
 
