@@ -215,6 +215,18 @@ int vig_rmsnorm_fwd(const void* x, const void* residual, const float* weight, vo
                     long long rows, int C, float eps, int round_sum, int io_dtype, void* stream);
 
 /*
+ * LayerNorm over the last dimension (rows x C, C % 8 == 0, C <= 4096), optional SiLU behind it:
+ *   y = (x - mean) * rsqrt(var + eps) * weight + bias   (biased variance, fp32 arithmetic; weight, bias [C] f32)
+ *   silu != 0:  y = r * sigmoid(r) with r the normalised value rounded to the storage type
+ * x and y may be the same buffer.
+ *
+ * Replaces: LayerNorm2d of the v2 patch embedding on a channels-last feature map, and the swish that follows the
+ * first one (classification/models/vig.py:619-624, 650-655).
+ */
+int vig_layernorm_fwd(const void* x, const float* weight, const float* bias, void* y, long long rows, int C,
+                      float eps, int silu, int io_dtype, void* stream);
+
+/*
  * Head-major split of the fused q/k/v projection:
  *   qkv [B, L, H*Dk | H*Dk | H*Dv]  ->  q, k [B, H, L, Dk],  v [B, H, L, Dv]   (Dk, Dv multiples of 8)
  * qkv_row_stride: elements between consecutive token rows of qkv (0 = packed), so that qkv may be the leading

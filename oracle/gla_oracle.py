@@ -22,6 +22,8 @@ Pinning status (what fixes each function besides its own formula):
         index-by-index layout brute force.
   * locality_* / rmsnorm_reference       -- torch.nn.functional.conv2d and the
         reference's own closed formula; layout brute force.
+  * layernorm_reference                  -- torch.nn.functional.layer_norm (+ silu)
+        in float64, and the mean-0 / variance-1 invariant.
   * naive_recurrent_gla_f32              -- float32 torch port of the reference's
         CPU-runnable routine; pinned against gla_recurrent (fp64) to 1e-5.
 The reference holds no golden vectors for this path (its tests are GPU-only
@@ -328,6 +330,21 @@ def rmsnorm_reference(x, weight, eps=1e-6):
     x = np.asarray(x, dtype=np.float64)
     r = 1.0 / np.sqrt((x * x).mean(axis=-1, keepdims=True) + eps)
     return x * r * np.asarray(weight, dtype=np.float64)
+
+
+def layernorm_reference(x, weight, bias, eps=1e-5, silu=False, round_to=None):
+    """LayerNorm over the last axis, float64, biased variance (torch.nn.functional.layer_norm as called by
+    LayerNorm2d, classification/models/vig.py:619-624); silu applies x*sigmoid(x) to the result after round_to (a
+    function float64 array -> float64 array: the separate activation of vig.py:653 reads stored values)."""
+    x = np.asarray(x, dtype=np.float64)
+    mu = x.mean(axis=-1, keepdims=True)
+    var = ((x - mu) ** 2).mean(axis=-1, keepdims=True)
+    y = (x - mu) / np.sqrt(var + eps) * np.asarray(weight, dtype=np.float64) + np.asarray(bias, dtype=np.float64)
+    if silu:
+        if round_to is not None:
+            y = round_to(y)
+        y = y / (1.0 + np.exp(-y))
+    return y
 
 
 def rmsnorm_residual_reference(x, weight, eps=1e-6, residual=None, round_to=None):

@@ -49,6 +49,23 @@ def test_rmsnorm_residual_prenorm(dtype, tol, rows, C):
         assert _close(f64(got), want, tol)
 
 
+@pytest.mark.parametrize("dtype,tol", [(torch.float32, 5e-6), (torch.bfloat16, 2.0 ** -8)])
+@pytest.mark.parametrize("rows,C", [(1568, 192), (197, 384), (5, 8), (33, 264), (3, 768), (2, 2048), (1, 4096)])
+def test_layernorm(dtype, tol, rows, C):
+    """LayerNorm (+ SiLU on the stored value) against the fp64 oracle on the stored inputs; tolerance relative to
+    max(1, |want|): one rounding of the output."""
+    announce(f"layernorm {dtype} rows{rows} C{C}")
+    x = _randn((rows, C), 31, dtype) * 3 + 0.5
+    w = _randn((C,), 32) * 0.2 + 1
+    b = _randn((C,), 33) * 0.3
+    rnd = (lambda a: f64(torch.from_numpy(a).to(dtype)))
+    for silu in (False, True):
+        want = O.layernorm_reference(f64(x), f64(w), f64(b), 1e-5, silu=silu, round_to=rnd)
+        got = f64(vig_amd.ops.layernorm(x.cuda(), w.cuda(), b.cuda(), 1e-5, silu=silu))
+        err = np.abs(got - want) / np.maximum(1.0, np.abs(want))
+        assert err.max() <= (tol if not silu else 2 * tol), (silu, err.max())
+
+
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("B,L,H,Dk,Dv", [(2, 196, 6, 32, 64), (1, 197, 3, 64, 64), (3, 7, 2, 16, 32)])
 def test_split_heads_is_exact(dtype, B, L, H, Dk, Dv):

@@ -227,6 +227,18 @@ def test_block_row_ops_against_library_routines():
     # unit weight, eps -> 0: every row of the output has mean square 1
     y1, _ = O.rmsnorm_residual_reference(x, np.ones(24), 0.0)
     np.testing.assert_allclose((y1 ** 2).mean(-1), 1.0, rtol=1e-12)
+    # LayerNorm: torch's routine; unit weight, zero bias, eps -> 0 gives rows of mean 0 and variance 1
+    lw, lb = rng.standard_normal(24), rng.standard_normal(24)
+    tx = torch.from_numpy(x)
+    np.testing.assert_allclose(O.layernorm_reference(x, lw, lb, 1e-5),
+                               F.layer_norm(tx, (24,), torch.from_numpy(lw), torch.from_numpy(lb), 1e-5).numpy(),
+                               rtol=1e-12, atol=1e-12)
+    np.testing.assert_allclose(O.layernorm_reference(x, lw, lb, 1e-5, silu=True),
+                               F.silu(F.layer_norm(tx, (24,), torch.from_numpy(lw), torch.from_numpy(lb), 1e-5)).numpy(),
+                               rtol=1e-12, atol=1e-12)
+    y0 = O.layernorm_reference(x, np.ones(24), np.zeros(24), 0.0)
+    np.testing.assert_allclose(y0.mean(-1), 0.0, atol=1e-12)
+    np.testing.assert_allclose(y0.var(-1), 1.0, rtol=1e-12)
     gu = rng.standard_normal((5, 32))
     tg, tu = torch.from_numpy(gu).chunk(2, -1)
     np.testing.assert_allclose(O.swiglu_reference(gu), (F.silu(tg) * tu).numpy(), rtol=1e-12, atol=1e-12)

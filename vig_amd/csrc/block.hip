@@ -135,6 +135,100 @@ int launch_rmsnorm(const void* x, const void* residual, const float* weight, voi
 }
 
 // ---------------------------------------------------------------------------
+// LayerNorm over the last dimension with an optional SiLU behind it (the norms of the patch embedding, applied to
+// channels-last feature maps):  y = (x - mean) * rsqrt(var + eps) * weight + bias, var the biased variance; with
+// silu the normalised value is first rounded to the storage type (the separate activation reads stored values).
+// GROUP lanes own one row (GROUP = 32 for C <= 256: two rows per wave keep the lanes busy at small C), each lane
+// holds NV channel octets; mean and variance are two reductions over registers, as torch computes them.
+// ---------------------------------------------------------------------------
+template <int GROUP>
+__device__ __forceinline__ float group_sum(float v) {
+#pragma unroll
+  for (int off = GROUP / 2; off > 0; off >>= 1) v += __shfl_xor(v, off, 64);
+  return v;
+}
+
+template <typename T, int NV, int GROUP>
+__global__ __launch_bounds__(256) void layernorm_kernel(const T* __restrict__ x, const float* __restrict__ weight,
+                                                        const float* __restrict__ bias, T* __restrict__ y,
+                                                        long long rows, int C, float eps, int silu) {
+  constexpr int kRowsPerBlock = 256 / GROUP;
+  const int gl = threadIdx.x % GROUP;
+  const long long row = (long long)blockIdx.x * kRowsPerBlock + threadIdx.x / GROUP;
+  const bool row_ok = row < rows;  // lanes of a missing row still take part in the shuffles of their wave
+  const int nvec = C >> 3;
+  const size_t base = (size_t)(row_ok ? row : 0) * C;
+  float s[NV][8];
+  float sum = 0.f;
+#pragma unroll
+  for (int i = 0; i < NV; ++i) {
+    const int v = gl + GROUP * i;
+    if (v < nvec) {
+      Oct<T>::load(x + base + 8 * v, s[i]);
+#pragma unroll
+      for (int j = 0; j < 8; ++j) sum += s[i][j];
+    }
+  }
+  const float mean = group_sum<GROUP>(sum) / (float)C;
+  float ss = 0.f;
+#pragma unroll
+  for (int i = 0; i < NV; ++i) {
+    const int v = gl + GROUP * i;
+    if (v < nvec) {
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        s[i][j] -= mean;
+        ss = __builtin_fmaf(s[i][j], s[i][j], ss);
+      }
+    }
+  }
+  const float rstd = 1.0f / sqrtf(group_sum<GROUP>(ss) / (float)C + eps);
+  if (!row_ok) return;
+#pragma unroll
+  for (int i = 0; i < NV; ++i) {
+    const int v = gl + GROUP * i;
+    if (v < nvec) {
+      float w[8], b[8];
+      Oct<float>::load(weight + 8 * v, w);
+      Oct<float>::load(bias + 8 * v, b);
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        float r = __builtin_fmaf(s[i][j] * rstd, w[j], b[j]);
+        if (silu) {
+          r = Oct<T>::round(r);
+          r = r * sigmoidf_(r);
+        }
+        s[i][j] = r;
+      }
+      Oct<T>::store(y + base + 8 * v, s[i]);
+    }
+  }
+}
+
+template <typename T>
+static int launch_layernorm_t(const void* x, const float* weight, const float* bias, void* y, long long rows, int C,
+                              float eps, int silu, hipStream_t stream) {
+  const int nvec = C / 8;
+#define VIG_LN_CASE(NV, GROUP)                                                                                       \
+  hipLaunchKernelGGL((layernorm_kernel<T, NV, GROUP>), dim3((unsigned)((rows + 256 / GROUP - 1) / (256 / GROUP))), \
+                     dim3(256), 0, stream, (const T*)x, weight, bias, (T*)y, rows, C, eps, silu)
+  if (nvec <= 32) VIG_LN_CASE(1, 32);
+  else if (nvec <= 64) VIG_LN_CASE(1, 64);
+  else if (nvec <= 128) VIG_LN_CASE(2, 64);
+  else if (nvec <= 256) VIG_LN_CASE(4, 64);
+  else VIG_LN_CASE(8, 64);
+#undef VIG_LN_CASE
+  return hipGetLastError() == hipSuccess ? 0 : -5;
+}
+
+int launch_layernorm(const void* x, const float* weight, const float* bias, void* y, long long rows, int C, float eps,
+                     int silu, int io_dtype, hipStream_t stream) {
+  if (C % 8 != 0 || C > 4096 || (rows + 3) / 4 > 0x7fffffffLL) return -95;
+  return io_dtype == 1 ? launch_layernorm_t<uint16_t>(x, weight, bias, y, rows, C, eps, silu, stream)
+                       : launch_layernorm_t<float>(x, weight, bias, y, rows, C, eps, silu, stream);
+}
+
+// ---------------------------------------------------------------------------
 // head-major split of the fused projection:
 //   qkv [B, L, H*Dk | H*Dk | H*Dv]  ->  q, k [B, H, L, Dk],  v [B, H, L, Dv]
 // A token's row may sit inside a wider row of `ld` elements (the columns of a larger projection).

@@ -244,8 +244,13 @@ class GLABlock(nn.Module):
 
 
 class LayerNorm2d(nn.LayerNorm):
-    def forward(self, x):
-        return F.layer_norm(x.permute(0, 2, 3, 1), self.normalized_shape, self.weight, self.bias, self.eps).permute(0, 3, 1, 2)
+    """LayerNorm over the channels of a [B, C, H, W] map (vig.py:619-624).  The patch embedding keeps its maps in
+    channels-last memory, where the permuted view is a plain [B*H*W, C] row matrix for the row kernel; `silu`
+    folds the swish that follows the first norm (vig.py:653) into the same pass."""
+
+    def forward(self, x, silu: bool = False):
+        rows = x.permute(0, 2, 3, 1)  # a view; contiguous when x is channels-last
+        return ops.layernorm(rows, self.weight, self.bias, self.eps, silu=silu).permute(0, 3, 1, 2)
 
 
 class V2PatchEmbed(nn.Module):
@@ -260,10 +265,17 @@ class V2PatchEmbed(nn.Module):
             nn.SiLU(),
             nn.Conv2d(embed_dim // 2, embed_dim, kernel_size=3, stride=2, padding=1, bias=use_bias_in_patch),
             LayerNorm2d(embed_dim),
-        )
+        ).to(memory_format=torch.channels_last)  # conv weights stored the way the channels-last kernels read them
 
     def forward(self, x):
-        x = self.proj(x)
+        # channels-last throughout: the convolutions run in that layout, the norms see row matrices, and the final
+        # 'b c h w -> b (h w) c' is a view
+        conv1, norm1, act, conv2, norm2 = self.proj
+        x = conv1(x.contiguous(memory_format=torch.channels_last))
+        x = norm1(x, silu=isinstance(act, nn.SiLU))
+        if not isinstance(act, nn.SiLU):
+            x = act(x)
+        x = norm2(conv2(x))
         hw = tuple(x.shape[-2:])
         return x.flatten(2).transpose(1, 2), hw
 

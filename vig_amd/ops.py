@@ -397,6 +397,26 @@ def rmsnorm(x: torch.Tensor, weight: torch.Tensor, eps: float = 1e-6, residual: 
     return y
 
 
+def layernorm(x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor, eps: float = 1e-5,
+              silu: bool = False) -> torch.Tensor:
+    """LayerNorm over the last dimension of a contiguous tensor, optionally followed by SiLU on the stored value
+    (LayerNorm2d and the swish behind it, vig.py:619-624,650-655, on channels-last data)."""
+    lib = _lib.load()
+    _check_cuda(x, weight, bias)
+    x = x.contiguous()
+    C = x.shape[-1]
+    w = weight.detach().float().contiguous()
+    b = bias.detach().float().contiguous()
+    if w.shape != (C,) or b.shape != (C,):
+        raise ValueError("weight and bias must be [C]")
+    y = torch.empty_like(x)
+    with torch.cuda.device(x.device):
+        rc = lib.vig_layernorm_fwd(x.data_ptr(), w.data_ptr(), b.data_ptr(), y.data_ptr(), x.numel() // C, C,
+                                   float(eps), int(silu), _dt(x), _stream_ptr(x))
+    _lib.check(rc, "vig_layernorm_fwd")
+    return y
+
+
 def split_heads(qkv: torch.Tensor, num_heads: int, head_qk_dim: int, head_v_dim: int):
     """qkv [B, L, H*Dk | H*Dk | H*Dv] -> q, k [B,H,L,Dk], v [B,H,L,Dv] (vig.py:401-409).
     qkv may be a block of columns of a wider [B, L, W] tensor (it is read in place)."""
