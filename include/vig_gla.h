@@ -218,13 +218,19 @@ int vig_rmsnorm_fwd(const void* x, const void* residual, const float* weight, vo
  * LayerNorm over the last dimension (rows x C, C % 8 == 0, C <= 4096), optional SiLU behind it:
  *   y = (x - mean) * rsqrt(var + eps) * weight + bias   (biased variance, fp32 arithmetic; weight, bias [C] f32)
  *   silu != 0:  y = r * sigmoid(r) with r the normalised value rounded to the storage type
+ *   pre_bias [C] f32 or NULL: x + pre_bias, rounded to the storage type, is what gets normalised (the bias of the
+ *     convolution in front of the norm);
+ *   post_add [post_rows, C] (io dtype) or NULL: row r of the (rounded) result gets post_add[r % post_rows] added
+ *     (the position table behind the last norm, post_rows = tokens per image).
  * x and y may be the same buffer.
  *
- * Replaces: LayerNorm2d of the v2 patch embedding on a channels-last feature map, and the swish that follows the
- * first one (classification/models/vig.py:619-624, 650-655).
+ * Replaces: LayerNorm2d of the v2 patch embedding on a channels-last feature map with the bias add of the
+ * convolution before it, the swish that follows the first one (classification/models/vig.py:619-624, 650-655) and
+ * the position-table add behind the second (vig.py:858-865).
  */
 int vig_layernorm_fwd(const void* x, const float* weight, const float* bias, void* y, long long rows, int C,
-                      float eps, int silu, int io_dtype, void* stream);
+                      float eps, int silu, const float* pre_bias, const void* post_add, int post_rows, int io_dtype,
+                      void* stream);
 
 /*
  * Head-major split of the fused q/k/v projection:

@@ -64,6 +64,16 @@ def test_layernorm(dtype, tol, rows, C):
         got = f64(vig_amd.ops.layernorm(x.cuda(), w.cuda(), b.cuda(), 1e-5, silu=silu))
         err = np.abs(got - want) / np.maximum(1.0, np.abs(want))
         assert err.max() <= (tol if not silu else 2 * tol), (silu, err.max())
+    # a bias added in front (rounded sum, as a convolution would have stored it) and a row-periodic table behind
+    if rows % 7 == 0 or rows < 7:
+        period = 7 if rows % 7 == 0 else rows
+        pb = _randn((C,), 34) * 0.5
+        pa = _randn((period, C), 35, dtype)
+        xin = rnd(f64(x) + f64(pb))
+        want = rnd(O.layernorm_reference(xin, f64(w), f64(b), 1e-5)) + np.tile(f64(pa), (rows // period, 1))
+        got = f64(vig_amd.ops.layernorm(x.cuda(), w.cuda(), b.cuda(), 1e-5, pre_bias=pb.cuda(), post_add=pa.cuda()))
+        err = np.abs(got - want) / np.maximum(1.0, np.abs(want))
+        assert err.max() <= 3 * tol, err.max()
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])

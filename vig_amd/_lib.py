@@ -36,7 +36,7 @@ SIGNATURES = {
     "vig_locality_gate_fwd": (_c_int, [_c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_void_p]),
     "vig_dirgate_lowrank_fwd": (_c_int, [_c_void_p, _c_longlong, _c_void_p, _c_void_p, _c_void_p] + [_c_int] * 5 + [_c_float, _c_float, _c_int, _c_int, _c_void_p]),
     "vig_locality_blend_fwd": (_c_int, [_c_void_p] * 6 + [_c_int, _c_int, _c_int, _c_int, _c_longlong, _c_float, _c_int, _c_int, _c_void_p]),
-    "vig_layernorm_fwd": (_c_int, [_c_void_p] * 4 + [_c_longlong, _c_int, _c_float, _c_int, _c_int, _c_void_p]),
+    "vig_layernorm_fwd": (_c_int, [_c_void_p] * 4 + [_c_longlong, _c_int, _c_float, _c_int, _c_void_p, _c_void_p, _c_int, _c_int, _c_void_p]),
     "vig_rmsnorm_fwd": (_c_int, [_c_void_p] * 5 + [ctypes.c_longlong, _c_int, _c_float, _c_int, _c_int, _c_void_p]),
     "vig_split_heads_fwd": (_c_int, [_c_void_p] * 4 + [_c_int] * 5 + [_c_longlong, _c_int, _c_void_p]),
     "vig_swiglu_fwd": (_c_int, [_c_void_p, _c_void_p, ctypes.c_longlong, _c_int, _c_int, _c_void_p]),

@@ -19,7 +19,8 @@ int launch_locality_blend(const void* o, const void* loc, const void* glin, cons
 int launch_rmsnorm(const void* x, const void* residual, const float* weight, void* y, void* residual_out, int rows,
                    int C, float eps, int round_sum, int io_dtype, hipStream_t stream);
 int launch_layernorm(const void* x, const float* weight, const float* bias, void* y, long long rows, int C, float eps,
-                     int silu, int io_dtype, hipStream_t stream);
+                     int silu, const float* pre_bias, const void* post_add, int post_rows, int io_dtype,
+                     hipStream_t stream);
 int launch_split_heads(const void* qkv, void* q, void* k, void* v, int B, int L, int H, int Dk, int Dv, long long ld,
                        int io_dtype, hipStream_t stream);
 int launch_swiglu(const void* in, void* out, long long rows, int I, int io_dtype, hipStream_t stream);
@@ -229,10 +230,12 @@ int vig_rmsnorm_fwd(const void* x, const void* residual, const float* weight, vo
 }
 
 int vig_layernorm_fwd(const void* x, const float* weight, const float* bias, void* y, long long rows, int C,
-                      float eps, int silu, int io_dtype, void* stream) {
-  if (!x || !weight || !bias || !y || rows <= 0 || C <= 0) return VIG_EINVAL;
+                      float eps, int silu, const float* pre_bias, const void* post_add, int post_rows, int io_dtype,
+                      void* stream) {
+  if (!x || !weight || !bias || !y || rows <= 0 || C <= 0 || (post_add && post_rows <= 0)) return VIG_EINVAL;
   if (!dtype_ok(io_dtype) || (C % 8) != 0 || C > 4096) return VIG_ENOTSUP;
-  return vig::launch_layernorm(x, weight, bias, y, rows, C, eps, silu, io_dtype, (hipStream_t)stream);
+  return vig::launch_layernorm(x, weight, bias, y, rows, C, eps, silu, pre_bias, post_add, post_rows, io_dtype,
+                               (hipStream_t)stream);
 }
 
 int vig_split_heads_fwd(const void* qkv, void* q, void* k, void* v, int B, int L, int H, int Dk, int Dv,

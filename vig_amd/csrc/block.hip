@@ -138,6 +138,10 @@ int launch_rmsnorm(const void* x, const void* residual, const float* weight, voi
 // LayerNorm over the last dimension with an optional SiLU behind it (the norms of the patch embedding, applied to
 // channels-last feature maps):  y = (x - mean) * rsqrt(var + eps) * weight + bias, var the biased variance; with
 // silu the normalised value is first rounded to the storage type (the separate activation reads stored values).
+// Two neighbours ride along: pre_bias [C] is added to x first (the bias of the convolution in front, the sum rounded
+// to the storage type as that convolution would have stored it), and post_add [post_rows, C] is added to the result
+// of row r at its row r % post_rows (the position table behind the last norm; the normalised value is rounded to
+// the storage type first, as the separate add reads it).
 // GROUP lanes own one row (GROUP = 32 for C <= 256: two rows per wave keep the lanes busy at small C), each lane
 // holds NV channel octets; mean and variance are two reductions over registers, as torch computes them.
 // ---------------------------------------------------------------------------
@@ -151,7 +155,9 @@ __device__ __forceinline__ float group_sum(float v) {
 template <typename T, int NV, int GROUP>
 __global__ __launch_bounds__(256) void layernorm_kernel(const T* __restrict__ x, const float* __restrict__ weight,
                                                         const float* __restrict__ bias, T* __restrict__ y,
-                                                        long long rows, int C, float eps, int silu) {
+                                                        long long rows, int C, float eps, int silu,
+                                                        const float* __restrict__ pre_bias,
+                                                        const T* __restrict__ post_add, int post_rows) {
   constexpr int kRowsPerBlock = 256 / GROUP;
   const int gl = threadIdx.x % GROUP;
   const long long row = (long long)blockIdx.x * kRowsPerBlock + threadIdx.x / GROUP;
@@ -165,6 +171,12 @@ __global__ __launch_bounds__(256) void layernorm_kernel(const T* __restrict__ x,
     const int v = gl + GROUP * i;
     if (v < nvec) {
       Oct<T>::load(x + base + 8 * v, s[i]);
+      if (pre_bias) {
+        float pb[8];
+        Oct<float>::load(pre_bias + 8 * v, pb);
+#pragma unroll
+        for (int j = 0; j < 8; ++j) s[i][j] = Oct<T>::round(s[i][j] + pb[j]);
+      }
 #pragma unroll
       for (int j = 0; j < 8; ++j) sum += s[i][j];
     }
@@ -200,6 +212,12 @@ __global__ __launch_bounds__(256) void layernorm_kernel(const T* __restrict__ x,
         }
         s[i][j] = r;
       }
+      if (post_add) {
+        float pa[8];
+        Oct<T>::load(post_add + (size_t)(row % post_rows) * C + 8 * v, pa);
+#pragma unroll
+        for (int j = 0; j < 8; ++j) s[i][j] = Oct<T>::round(s[i][j]) + pa[j];
+      }
       Oct<T>::store(y + base + 8 * v, s[i]);
     }
   }
@@ -207,11 +225,13 @@ __global__ __launch_bounds__(256) void layernorm_kernel(const T* __restrict__ x,
 
 template <typename T>
 static int launch_layernorm_t(const void* x, const float* weight, const float* bias, void* y, long long rows, int C,
-                              float eps, int silu, hipStream_t stream) {
+                              float eps, int silu, const float* pre_bias, const void* post_add, int post_rows,
+                              hipStream_t stream) {
   const int nvec = C / 8;
 #define VIG_LN_CASE(NV, GROUP)                                                                                       \
   hipLaunchKernelGGL((layernorm_kernel<T, NV, GROUP>), dim3((unsigned)((rows + 256 / GROUP - 1) / (256 / GROUP))), \
-                     dim3(256), 0, stream, (const T*)x, weight, bias, (T*)y, rows, C, eps, silu)
+                     dim3(256), 0, stream, (const T*)x, weight, bias, (T*)y, rows, C, eps, silu, pre_bias,      \
+                     (const T*)post_add, post_rows)
   if (nvec <= 32) VIG_LN_CASE(1, 32);
   else if (nvec <= 64) VIG_LN_CASE(1, 64);
   else if (nvec <= 128) VIG_LN_CASE(2, 64);
@@ -222,10 +242,12 @@ static int launch_layernorm_t(const void* x, const float* weight, const float* b
 }
 
 int launch_layernorm(const void* x, const float* weight, const float* bias, void* y, long long rows, int C, float eps,
-                     int silu, int io_dtype, hipStream_t stream) {
+                     int silu, const float* pre_bias, const void* post_add, int post_rows, int io_dtype,
+                     hipStream_t stream) {
   if (C % 8 != 0 || C > 4096 || (rows + 3) / 4 > 0x7fffffffLL) return -95;
-  return io_dtype == 1 ? launch_layernorm_t<uint16_t>(x, weight, bias, y, rows, C, eps, silu, stream)
-                       : launch_layernorm_t<float>(x, weight, bias, y, rows, C, eps, silu, stream);
+  return io_dtype == 1
+             ? launch_layernorm_t<uint16_t>(x, weight, bias, y, rows, C, eps, silu, pre_bias, post_add, post_rows, stream)
+             : launch_layernorm_t<float>(x, weight, bias, y, rows, C, eps, silu, pre_bias, post_add, post_rows, stream);
 }
 
 // ---------------------------------------------------------------------------

@@ -248,9 +248,10 @@ class LayerNorm2d(nn.LayerNorm):
     channels-last memory, where the permuted view is a plain [B*H*W, C] row matrix for the row kernel; `silu`
     folds the swish that follows the first norm (vig.py:653) into the same pass."""
 
-    def forward(self, x, silu: bool = False):
+    def forward(self, x, silu: bool = False, pre_bias=None, post_add=None):
         rows = x.permute(0, 2, 3, 1)  # a view; contiguous when x is channels-last
-        return ops.layernorm(rows, self.weight, self.bias, self.eps, silu=silu).permute(0, 3, 1, 2)
+        return ops.layernorm(rows, self.weight, self.bias, self.eps, silu=silu, pre_bias=pre_bias,
+                             post_add=post_add).permute(0, 3, 1, 2)
 
 
 class V2PatchEmbed(nn.Module):
@@ -267,17 +268,26 @@ class V2PatchEmbed(nn.Module):
             LayerNorm2d(embed_dim),
         ).to(memory_format=torch.channels_last)  # conv weights stored the way the channels-last kernels read them
 
-    def forward(self, x):
+    def forward(self, x, pos_embed=None, pos_shape=None):
+        """pos_embed [1, h*w, C] on the grid pos_shape, if given, is added to the tokens (resized to the actual grid)
+        inside the last norm's kernel."""
         # channels-last throughout: the convolutions run in that layout, the norms see row matrices, and the final
-        # 'b c h w -> b (h w) c' is a view
+        # 'b c h w -> b (h w) c' is a view; each convolution's bias add rides in the norm kernel behind it
         conv1, norm1, act, conv2, norm2 = self.proj
-        x = conv1(x.contiguous(memory_format=torch.channels_last))
-        x = norm1(x, silu=isinstance(act, nn.SiLU))
+        x = self._conv_nobias(conv1, x.contiguous(memory_format=torch.channels_last))
+        x = norm1(x, silu=isinstance(act, nn.SiLU), pre_bias=conv1.bias)
         if not isinstance(act, nn.SiLU):
             x = act(x)
-        x = norm2(conv2(x))
+        x = self._conv_nobias(conv2, x)
         hw = tuple(x.shape[-2:])
+        if pos_embed is not None:
+            pos_embed = resize_pos_embed(pos_embed, pos_shape, hw).to(x.dtype)
+        x = norm2(x, pre_bias=conv2.bias, post_add=pos_embed)
         return x.flatten(2).transpose(1, 2), hw
+
+    @staticmethod
+    def _conv_nobias(conv, x):
+        return F.conv2d(x, conv.weight, None, conv.stride, conv.padding, conv.dilation, conv.groups)
 
 
 def resize_pos_embed(pos_embed, src_shape, dst_shape):
@@ -322,8 +332,7 @@ class ViG(nn.Module):
 
     def forward_features(self, x):
         B = x.shape[0]
-        x, hw = self.patch_embed(x)
-        x = x + resize_pos_embed(self.pos_embed, self.patch_resolution, hw)
+        x, hw = self.patch_embed(x, self.pos_embed, self.patch_resolution)
         branch, residual = x, None
         for blk in self.blocks:
             branch, residual = blk.forward_carry(branch, residual, patch_resolution=hw, token_position=None)

@@ -398,21 +398,37 @@ def rmsnorm(x: torch.Tensor, weight: torch.Tensor, eps: float = 1e-6, residual: 
 
 
 def layernorm(x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor, eps: float = 1e-5,
-              silu: bool = False) -> torch.Tensor:
+              silu: bool = False, pre_bias: Optional[torch.Tensor] = None,
+              post_add: Optional[torch.Tensor] = None) -> torch.Tensor:
     """LayerNorm over the last dimension of a contiguous tensor, optionally followed by SiLU on the stored value
-    (LayerNorm2d and the swish behind it, vig.py:619-624,650-655, on channels-last data)."""
+    (LayerNorm2d and the swish behind it, vig.py:619-624,650-655, on channels-last data).  pre_bias [C] is added to
+    x first (the bias of the convolution in front); post_add [P, C], P dividing the row count, is added to the
+    result row-periodically (the position table, vig.py:858-865)."""
     lib = _lib.load()
-    _check_cuda(x, weight, bias)
+    _check_cuda(x, weight, bias, pre_bias, post_add)
     x = x.contiguous()
     C = x.shape[-1]
+    rows = x.numel() // C
     w = weight.detach().float().contiguous()
     b = bias.detach().float().contiguous()
     if w.shape != (C,) or b.shape != (C,):
         raise ValueError("weight and bias must be [C]")
+    pb = None
+    if pre_bias is not None:
+        pb = pre_bias.detach().float().contiguous()
+        if pb.shape != (C,):
+            raise ValueError("pre_bias must be [C]")
+    pa, prow = None, 0
+    if post_add is not None:
+        pa = post_add.detach().reshape(-1, C).contiguous()
+        prow = pa.shape[0]
+        if pa.dtype != x.dtype or rows % prow:
+            raise ValueError("post_add must have x's dtype and a row count that divides x's")
     y = torch.empty_like(x)
     with torch.cuda.device(x.device):
-        rc = lib.vig_layernorm_fwd(x.data_ptr(), w.data_ptr(), b.data_ptr(), y.data_ptr(), x.numel() // C, C,
-                                   float(eps), int(silu), _dt(x), _stream_ptr(x))
+        rc = lib.vig_layernorm_fwd(x.data_ptr(), w.data_ptr(), b.data_ptr(), y.data_ptr(), rows, C,
+                                   float(eps), int(silu), pb.data_ptr() if pb is not None else None,
+                                   pa.data_ptr() if pa is not None else None, prow, _dt(x), _stream_ptr(x))
     _lib.check(rc, "vig_layernorm_fwd")
     return y
 
