@@ -29,6 +29,20 @@ import torch.nn.functional as F
 from . import ops
 
 
+def _f32(owner: nn.Module, tag: str, t: Optional[torch.Tensor], shape=None):
+    """fp32 contiguous copy of parameter `t` (the kernels take fp32 weights), kept on `owner` under `tag` and refreshed
+    when the parameter is replaced, moved, cast or written in place: no conversion kernel per forward."""
+    if t is None:
+        return None
+    key = (t.data_ptr(), t._version, t.dtype, t.device)
+    cache = owner.__dict__.setdefault("_f32_cache", {})
+    hit = cache.get(tag)
+    if hit is None or hit[0] != key:
+        v = t.detach().float()
+        cache[tag] = hit = (key, (v.reshape(shape) if shape is not None else v).contiguous())
+    return hit[1]
+
+
 class RMSNorm(nn.Module):
     """x * rsqrt(mean(x^2) + eps) * weight, arithmetic in fp32 (fla/modules/rmsnorm.py:38-52,491-512).
 
@@ -138,7 +152,8 @@ class GatedLinearAttention(nn.Module):
         H = self.num_heads
         conv = self.in_proj[0]
         # local_out, already in the [B, L, C] layout the projections consume
-        xs = ops.dwconv3x3(x, conv.weight, hw, bias=conv.bias, silu=self.use_act_in_conv)
+        xs = ops.dwconv3x3(x, _f32(self, "conv_w", conv.weight, (-1, 3, 3)), hw, bias=_f32(self, "conv_b", conv.bias),
+                           silu=self.use_act_in_conv)
         qkv, g_lin, gk_low = self._input_projections(xs)
         q, k, v = ops.split_heads(qkv, H, self.head_qk_dim, self.head_v_dim)
         up = self.gk_proj[1]
@@ -250,8 +265,8 @@ class LayerNorm2d(nn.LayerNorm):
 
     def forward(self, x, silu: bool = False, pre_bias=None, post_add=None):
         rows = x.permute(0, 2, 3, 1)  # a view; contiguous when x is channels-last
-        return ops.layernorm(rows, self.weight, self.bias, self.eps, silu=silu, pre_bias=pre_bias,
-                             post_add=post_add).permute(0, 3, 1, 2)
+        return ops.layernorm(rows, _f32(self, "w", self.weight), _f32(self, "b", self.bias), self.eps, silu=silu,
+                             pre_bias=pre_bias, post_add=post_add).permute(0, 3, 1, 2)
 
 
 class V2PatchEmbed(nn.Module):
@@ -275,14 +290,14 @@ class V2PatchEmbed(nn.Module):
         # 'b c h w -> b (h w) c' is a view; each convolution's bias add rides in the norm kernel behind it
         conv1, norm1, act, conv2, norm2 = self.proj
         x = self._conv_nobias(conv1, x.contiguous(memory_format=torch.channels_last))
-        x = norm1(x, silu=isinstance(act, nn.SiLU), pre_bias=conv1.bias)
+        x = norm1(x, silu=isinstance(act, nn.SiLU), pre_bias=_f32(self, "b1", conv1.bias))
         if not isinstance(act, nn.SiLU):
             x = act(x)
         x = self._conv_nobias(conv2, x)
         hw = tuple(x.shape[-2:])
         if pos_embed is not None:
             pos_embed = resize_pos_embed(pos_embed, pos_shape, hw).to(x.dtype)
-        x = norm2(x, pre_bias=conv2.bias, post_add=pos_embed)
+        x = norm2(x, pre_bias=_f32(self, "b2", conv2.bias), post_add=pos_embed)
         return x.flatten(2).transpose(1, 2), hw
 
     @staticmethod
