@@ -315,7 +315,7 @@ __global__ __launch_bounds__(256) void swiglu_kernel(const T* __restrict__ in, T
   Oct<T>::load(in + (size_t)row * 2 * I + c, g);
   Oct<T>::load(in + (size_t)row * 2 * I + I + c, u);
 #pragma unroll
-  for (int j = 0; j < 8; ++j) g[j] = g[j] * u[j] / (1.0f + __expf(-g[j]));
+  for (int j = 0; j < 8; ++j) g[j] = g[j] * u[j] * sigmoidf_(g[j]);
   Oct<T>::store(out + (size_t)row * I + c, g);
 }
 

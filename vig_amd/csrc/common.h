@@ -44,6 +44,14 @@ template <> struct Elem<uint16_t> {  // bf16 storage
 };
 
 // (hardware reciprocal, 1 ulp: a full-precision division costs ten instructions more per value)
-__device__ __forceinline__ float sigmoidf_(float x) { return __builtin_amdgcn_rcpf(1.0f + __expf(-x)); }
+// e^-|..| style arguments only need the bare hardware instructions (2^x and log2 x, 1 ulp): results below the
+// normal range flush to zero, which is exact enough next to 1, and the guards the library versions wrap around them
+// (range tests, rescaling) cost more than the instructions themselves.
+__device__ __forceinline__ float exp_fast(float x) { return __builtin_amdgcn_exp2f(x * 1.4426950408889634f); }
+__device__ __forceinline__ float sigmoidf_(float x) { return __builtin_amdgcn_rcpf(1.0f + exp_fast(-x)); }
+// log(sigmoid(x)) = min(x, 0) - log(1 + e^-|x|); the log's argument lies in [1, 2]
+__device__ __forceinline__ float logsigmoidf_(float x) {
+  return fminf(x, 0.f) - 0.6931471805599453f * __builtin_amdgcn_logf(1.f + exp_fast(-fabsf(x)));
+}
 
 }  // namespace vig

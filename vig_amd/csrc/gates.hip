@@ -77,7 +77,7 @@ __global__ __launch_bounds__(256) void dirgate_kernel(const TI* __restrict__ in,
 #pragma unroll
       for (int j = 0; j < 8; ++j) {
         // logsigmoid(x) = min(x,0) - log(1 + exp(-|x|)); hardware exp/log are accurate to ~1e-7 absolute here
-        float yv = fminf(x[j], 0.f) - __logf(1.f + __expf(-fabsf(x[j])));
+        float yv = logsigmoidf_(x[j]);
         yv *= inv_norm;
         if (use_clamp) yv = fmaxf(yv, clamp_min);
         x[j] = yv;
@@ -174,7 +174,7 @@ __global__ __launch_bounds__(256) void dirgate_lowrank_kernel(const TI* __restri
 #pragma unroll
       for (int j = 0; j < 8; ++j) {
         const float x = Stored<TI>::of(acc[j] + bias[j]);
-        float yv = fminf(x, 0.f) - __logf(1.f + __expf(-fabsf(x)));
+        float yv = logsigmoidf_(x);
         yv *= inv_norm;
         if (use_clamp) yv = fmaxf(yv, clamp_min);
         acc[j] = yv;
@@ -189,9 +189,9 @@ __global__ __launch_bounds__(256) void dirgate_lowrank_kernel(const TI* __restri
 // memory as one 16-byte load per lane (lane = (row r, contraction half h) supplies elements 8h..8h+7 of its row).
 // Accumulator register 4g+m of lane (r, h) holds matrix row 8g+4h+m of column r; matrix row i is given channel
 // 16*((i>>2)&1) + 4*(i>>3) + (i&3) of the tile, so that lane (r, h) ends up with channels 16h..16h+15 of token r:
-// 32 contiguous bytes of the head-major output.  Tokens are numbered over B*L; a workgroup owns 32 of them and its
-// four waves take the channel tiles in turn.  Needs Dk % 16 == 0 (a 16-channel run stays inside one head).
-template <typename TO>
+// 32 contiguous bytes of the head-major output.  Tokens are numbered over B*L; a workgroup owns NTG groups of 32 and
+// its four waves take the channel tiles in turn, each weight tile serving all the groups.  Needs Dk % 16 == 0 (a 16-channel run stays inside one head).
+template <typename TO, int NTG>
 __global__ __launch_bounds__(256) void dirgate_lowrank_mfma_kernel(const uint16_t* __restrict__ low, long long ld,
                                                                     const uint16_t* __restrict__ w1,
                                                                     const uint16_t* __restrict__ b1,
@@ -201,13 +201,22 @@ __global__ __launch_bounds__(256) void dirgate_lowrank_mfma_kernel(const uint16_
   constexpr int R = kGateRank;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int r = lane & 31, h = lane >> 5;
-  const long long tok = (long long)blockIdx.x * 32 + r;
-  const bool tok_ok = tok < ntok;
-  const long long tokc = tok_ok ? tok : ntok - 1;
-  const u32x4_t xb = *reinterpret_cast<const u32x4_t*>(low + (size_t)tokc * (size_t)ld + 8 * h);
-  const int b = (int)(tokc / L), l = (int)(tokc - (long long)b * L);
+  // NTG groups of 32 tokens per workgroup: their low-rank rows are fetched first, a weight tile serves all of them
+  u32x4_t xb[NTG];
+  bool tok_ok[NTG];
+  size_t row_off[NTG];  // (b*H*L + l) * Dk of the token: head hh adds hh*L*Dk
+#pragma unroll
+  for (int g = 0; g < NTG; ++g) {
+    const unsigned tok = (blockIdx.x * NTG + g) * 32u + r;  // the launch keeps B*L below 2^31
+    tok_ok[g] = tok < (unsigned)ntok;
+    const unsigned tokc = tok_ok[g] ? tok : (unsigned)ntok - 1;
+    xb[g] = *reinterpret_cast<const u32x4_t*>(low + (size_t)tokc * (size_t)ld + 8 * h);
+    const unsigned b = tokc / (unsigned)L, l = tokc - b * (unsigned)L;
+    row_off[g] = ((size_t)b * H * L + l) * (size_t)Dk;
+  }
   const int chan_of_row = 16 * ((r >> 2) & 1) + 4 * (r >> 3) + (r & 3);
   const int ntiles = 2 * H * Dk / 32;
+  const size_t dir_stride = (size_t)B * H * L * Dk;
   for (int tile = wave; tile < ntiles; tile += 4) {
     const int c0 = tile * 32;
     const u32x4_t wa = *reinterpret_cast<const u32x4_t*>(w1 + (size_t)(c0 + chan_of_row) * R + 8 * h);
@@ -221,29 +230,31 @@ __global__ __launch_bounds__(256) void dirgate_lowrank_mfma_kernel(const uint16_
 #pragma unroll
       for (int j = 0; j < 8; ++j) bias[8 + j] = x[j];
     }
-    f32x16_t acc;
-#pragma unroll
-    for (int j = 0; j < 16; ++j) acc[j] = 0.f;
-    acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, wa), __builtin_bit_cast(bf16x8_t, xb),
-                                                  acc, 0, 0, 0);
-    float y[16];
-#pragma unroll
-    for (int j = 0; j < 16; ++j) {
-      const float x = Stored<uint16_t>::of(acc[j] + bias[j]);
-      float yv = fminf(x, 0.f) - __logf(1.f + __expf(-fabsf(x)));
-      yv *= inv_norm;
-      if (use_clamp) yv = fmaxf(yv, clamp_min);
-      y[j] = yv;
-    }
     const int c = c0 + 16 * h;  // first of this lane's 16 channels
     const int d = c % Dk, hh = (c / Dk) % H, dir = c / (Dk * H);
-    if (tok_ok) {
-      TO* dst = out + ((((size_t)dir * B + b) * H + hh) * L + l) * (size_t)Dk + d;
+    TO* const dst0 = out + (size_t)dir * dir_stride + (size_t)hh * L * Dk + d;
+#pragma unroll
+    for (int g = 0; g < NTG; ++g) {
+      f32x16_t acc;
+#pragma unroll
+      for (int j = 0; j < 16; ++j) acc[j] = 0.f;
+      acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, wa),
+                                                    __builtin_bit_cast(bf16x8_t, xb[g]), acc, 0, 0, 0);
       float lo[8], hi[8];
 #pragma unroll
-      for (int j = 0; j < 8; ++j) lo[j] = y[j], hi[j] = y[8 + j];
-      Vec8<TO>::store(dst, lo);
-      Vec8<TO>::store(dst + 8, hi);
+      for (int j = 0; j < 16; ++j) {
+        const float x = Stored<uint16_t>::of(acc[j] + bias[j]);
+        float yv = logsigmoidf_(x);
+        yv *= inv_norm;
+        if (use_clamp) yv = fmaxf(yv, clamp_min);
+        if (j < 8) lo[j] = yv;
+        else hi[j - 8] = yv;
+      }
+      if (tok_ok[g]) {
+        TO* dst = dst0 + row_off[g];
+        Vec8<TO>::store(dst, lo);
+        Vec8<TO>::store(dst + 8, hi);
+      }
     }
   }
 }
@@ -262,16 +273,17 @@ int launch_dirgate_lowrank(const void* low, long long ld, const void* w1, const 
                            int H, int Dk, int rank, float inv_norm, float clamp_min, int in_dtype, int out_dtype,
                            hipStream_t stream) {
   if (rank != kGateRank) return -95;
-  if (in_dtype == 1 && Dk % 16 == 0 && B <= 65535) {
+  if (in_dtype == 1 && Dk % 16 == 0 && (long long)B * L < 0x7fffffffLL - 64) {
     const int use_clamp = clamp_min == clamp_min;  // NaN disables
     const long long ntok = (long long)B * L;
-    const dim3 grid((unsigned)((ntok + 31) / 32)), block(256);
+    constexpr int kGroups = 1;  // token groups of 32 per workgroup (two measured no faster)
+    const dim3 grid((unsigned)((ntok + 32 * kGroups - 1) / (32 * kGroups))), block(256);
     if (out_dtype == 1)
-      hipLaunchKernelGGL(dirgate_lowrank_mfma_kernel<uint16_t>, grid, block, 0, stream, (const uint16_t*)low, ld,
+      hipLaunchKernelGGL((dirgate_lowrank_mfma_kernel<uint16_t, kGroups>), grid, block, 0, stream, (const uint16_t*)low, ld,
                          (const uint16_t*)w1, (const uint16_t*)b1, (uint16_t*)out, ntok, B, L, H, Dk, inv_norm,
                          clamp_min, use_clamp);
     else
-      hipLaunchKernelGGL(dirgate_lowrank_mfma_kernel<float>, grid, block, 0, stream, (const uint16_t*)low, ld,
+      hipLaunchKernelGGL((dirgate_lowrank_mfma_kernel<float, kGroups>), grid, block, 0, stream, (const uint16_t*)low, ld,
                          (const uint16_t*)w1, (const uint16_t*)b1, (float*)out, ntok, B, L, H, Dk, inv_norm,
                          clamp_min, use_clamp);
     return hipGetLastError() == hipSuccess ? 0 : -5;
@@ -308,6 +320,22 @@ __global__ __launch_bounds__(256) void stencil3x3_kernel(const T* __restrict__ x
   const int L = h * w, pw = w + 2;
   const bool ch_ok = grp * kStencilGroup + oct * 8 < cgroup;  // channel tail of the last group
   const size_t base = (size_t)img * L * stride + (size_t)grp * kStencilGroup + oct * 8;
+  // ---- this thread's 8 x 9 weights: 72 consecutive floats, fetched (as 16-byte loads) ahead of the staging loop
+  // so that their latency runs under it ----
+  const int wch = (blockIdx.x / groups_per_image % wmod) * cgroup + grp * kStencilGroup + oct * 8;  // first weight channel
+  float wreg[8][9];
+  float breg[8];
+  if (ch_ok) {
+    float* wflat = &wreg[0][0];
+#pragma unroll
+    for (int i = 0; i < 18; ++i) {
+      const f32x4_t v = *reinterpret_cast<const f32x4_t*>(wt + (size_t)wch * 9 + 4 * i);
+#pragma unroll
+      for (int e = 0; e < 4; ++e) wflat[4 * i + e] = v[e];
+    }
+#pragma unroll
+    for (int j = 0; j < 8; ++j) breg[j] = (!GATE && bias) ? bias[wch + j] : 0.f;
+  }
   // ---- stage padded cells (pr, pc) <-> grid (r0 - 1 + pr, pc - 1) ----
   const int ncell = (r1 - r0 + 2) * pw;
   for (int t = tl; t < ncell; t += 32) {
@@ -319,15 +347,6 @@ __global__ __launch_bounds__(256) void stencil3x3_kernel(const T* __restrict__ x
   }
   __syncthreads();
   if (!ch_ok) return;
-  const int wch = (blockIdx.x / groups_per_image % wmod) * cgroup + grp * kStencilGroup + oct * 8;  // first weight channel
-  float wreg[8][9];
-#pragma unroll
-  for (int j = 0; j < 8; ++j)
-#pragma unroll
-    for (int t = 0; t < 9; ++t) wreg[j][t] = wt[(wch + j) * 9 + t];
-  float breg[8];
-#pragma unroll
-  for (int j = 0; j < 8; ++j) breg[j] = (!GATE && bias) ? bias[wch + j] : 0.f;
   const int nout = (r1 - r0) * w;
   for (int t = tl; t < nout; t += 32) {
     const int rl = t / w, c = t - rl * w;
