@@ -32,6 +32,41 @@ __device__ __forceinline__ uint32_t pack_bf16x2(float lo, float hi) {
 __device__ __forceinline__ float bf16lo_to_f32(uint32_t p) { return __uint_as_float(p << 16); }
 __device__ __forceinline__ float bf16hi_to_f32(uint32_t p) { return __uint_as_float(p & 0xffff0000u); }
 
+// eight channels as stored (no conversion): what a kernel that only moves them keeps in registers
+template <typename T> struct Raw8;
+template <> struct Raw8<uint16_t> {
+  u32x4_t a;
+  __device__ __forceinline__ void zero() { a = u32x4_t{0u, 0u, 0u, 0u}; }
+  __device__ __forceinline__ void load(const uint16_t* p) { a = *reinterpret_cast<const u32x4_t*>(p); }
+  __device__ __forceinline__ void store(uint16_t* p) const { *reinterpret_cast<u32x4_t*>(p) = a; }
+  __device__ __forceinline__ void unpack(float (&x)[8]) const {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      x[2 * i] = bf16lo_to_f32(a[i]);
+      x[2 * i + 1] = bf16hi_to_f32(a[i]);
+    }
+  }
+};
+template <> struct Raw8<float> {
+  f32x4_t a, b;
+  __device__ __forceinline__ void zero() { a = b = f32x4_t{0.f, 0.f, 0.f, 0.f}; }
+  __device__ __forceinline__ void load(const float* p) {
+    a = *reinterpret_cast<const f32x4_t*>(p);
+    b = *reinterpret_cast<const f32x4_t*>(p + 4);
+  }
+  __device__ __forceinline__ void store(float* p) const {
+    *reinterpret_cast<f32x4_t*>(p) = a;
+    *reinterpret_cast<f32x4_t*>(p + 4) = b;
+  }
+  __device__ __forceinline__ void unpack(float (&x)[8]) const {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      x[i] = a[i];
+      x[4 + i] = b[i];
+    }
+  }
+};
+
 // Typed element access used by the dtype-generic (non-MFMA) kernels.
 template <typename T> struct Elem;
 template <> struct Elem<float> {

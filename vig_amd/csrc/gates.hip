@@ -337,13 +337,25 @@ __global__ __launch_bounds__(256) void stencil3x3_kernel(const T* __restrict__ x
     for (int j = 0; j < 8; ++j) breg[j] = (!GATE && bias) ? bias[wch + j] : 0.f;
   }
   // ---- stage padded cells (pr, pc) <-> grid (r0 - 1 + pr, pc - 1) ----
+  // kBatch cells per thread are in flight at a time: the loads of a batch are issued before the first LDS store waits
+  constexpr int kBatch = sizeof(T) == 2 ? 8 : 4;
   const int ncell = (r1 - r0 + 2) * pw;
-  for (int t = tl; t < ncell; t += 32) {
-    const int pr = t / pw, pc = t - pr * pw;
-    const int r = r0 - 1 + pr, c = pc - 1;
-    float xv[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-    if (ch_ok && r >= 0 && r < h && c >= 0 && c < w) Vec8<T>::load(x + base + (size_t)(r * w + c) * stride, xv);
-    Vec8<T>::store(tile + t * kStencilGroup + oct * 8, xv);
+  for (int t0 = tl; t0 < ncell; t0 += 32 * kBatch) {
+    Raw8<T> cell[kBatch];
+#pragma unroll
+    for (int u = 0; u < kBatch; ++u) {
+      const int t = t0 + 32 * u;
+      const int pr = t / pw, pc = t - pr * pw;
+      const int r = r0 - 1 + pr, c = pc - 1;
+      cell[u].zero();
+      if (t < ncell && ch_ok && r >= 0 && r < h && c >= 0 && c < w)
+        cell[u].load(x + base + (size_t)(r * w + c) * stride);
+    }
+#pragma unroll
+    for (int u = 0; u < kBatch; ++u) {
+      const int t = t0 + 32 * u;
+      if (t < ncell) cell[u].store(tile + t * kStencilGroup + oct * 8);
+    }
   }
   __syncthreads();
   if (!ch_ok) return;
