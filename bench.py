@@ -51,7 +51,7 @@ def cpu_baseline(shape, seed, budget_s=20.0):
     O.bidir_naive_recurrent_gla_f32(q, k, v, gf, gb)  # warm-up
     ts = []
     t_begin = time.perf_counter()
-    while len(ts) < 3 or (time.perf_counter() - t_begin < budget_s / 2 and len(ts) < 50):
+    while len(ts) < 3 or (time.perf_counter() - t_begin < budget_s / 2 and len(ts) < 200):
         t0 = time.perf_counter()
         O.bidir_naive_recurrent_gla_f32(q, k, v, gf, gb)
         ts.append(time.perf_counter() - t0)
