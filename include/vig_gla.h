@@ -252,6 +252,21 @@ int vig_split_heads_fwd(const void* qkv, void* q, void* k, void* v, int B, int L
  */
 int vig_swiglu_fwd(const void* gate_up, void* out, long long rows, int I, int io_dtype, void* stream);
 
+/*
+ * First convolution of the v2 patch embedding, without its bias (vig_layernorm_fwd's pre_bias takes that):
+ *   x [B, Cin, H, W] (bf16, the layout images arrive in)  ->  y [B, OH, OW, Cout] (bf16, channels-last rows),
+ *   OH = (H + 2*padding - KH) / stride + 1, OW likewise.
+ *   w_packed [Cout, Cin*KH, 16] bf16: the kernel rows of the [Cout, Cin, KH, KW] weight, each padded with zeros to
+ *   16 columns.
+ * Built for the reference's stem: stride 8, padding 1, KW <= 16, Cin*KH = 27 (3 channels x 9 rows), W % 8 == 0,
+ * W <= 248, Cout a multiple of 32 from 64 to 256; anything else returns VIG_ENOTSUP (use a library convolution).
+ *
+ * Replaces: the first nn.Conv2d of V2PatchEmbed (classification/models/vig.py:651) and the layout change a
+ * channels-last convolution library needs in front of it.
+ */
+int vig_patch_conv_fwd(const void* x, const void* w_packed, void* y, int B, int Cin, int H, int W, int KH, int KW,
+                       int stride, int padding, int Cout, int io_dtype, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

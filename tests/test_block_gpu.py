@@ -76,6 +76,32 @@ def test_layernorm(dtype, tol, rows, C):
         assert err.max() <= 3 * tol, err.max()
 
 
+@pytest.mark.parametrize("B,H,W,KW,Cout", [(3, 224, 224, 9, 192), (2, 64, 64, 9, 96), (1, 40, 248, 9, 256),
+                                           (2, 17, 24, 9, 64), (1, 224, 224, 16, 64)])
+def test_patch_conv(B, H, W, KW, Cout):
+    """The stem convolution (kernel 9 rows x KW columns, stride 8, padding 1, 3 channels) against torch's conv2d in
+    fp64 on the stored bf16 inputs; one rounding of the output plus the fp32 accumulation of 243+ products."""
+    announce(f"patch_conv B{B} {H}x{W} KW{KW} Cout{Cout}")
+    x = _randn((B, 3, H, W), 41, torch.bfloat16)
+    w = _randn((Cout, 3, 9, KW), 42, torch.bfloat16) * 0.1
+    assert vig_amd.ops.patch_conv_supported(x.cuda(), w.cuda(), 8, 1)
+    got = vig_amd.ops.patch_conv(x.cuda(), vig_amd.ops.pack_patch_conv_weight(w.cuda()), (9, KW), 8, 1)
+    want = torch.nn.functional.conv2d(x.double(), w.double(), None, 8, 1).permute(0, 2, 3, 1)
+    assert tuple(got.shape) == tuple(want.shape)
+    err = (got.double().cpu() - want).abs() / want.abs().clamp_min(1.0)
+    assert err.max().item() <= 2.0 ** -8, err.max().item()
+
+
+def test_patch_conv_refuses_other_shapes():
+    x = torch.zeros(1, 3, 32, 36, dtype=torch.bfloat16).cuda()  # width not a multiple of 8
+    w = torch.zeros(32, 3, 9, 9, dtype=torch.bfloat16).cuda()
+    assert not vig_amd.ops.patch_conv_supported(x, w, 8, 1)
+    assert not vig_amd.ops.patch_conv_supported(x[..., :32], w, 4, 1)
+    assert not vig_amd.ops.patch_conv_supported(x[..., :32].float(), w.float(), 8, 1)
+    with pytest.raises(vig_amd._lib.VigGlaError):
+        vig_amd.ops.patch_conv(x, vig_amd.ops.pack_patch_conv_weight(w), (9, 9), 8, 1)
+
+
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("B,L,H,Dk,Dv", [(2, 196, 6, 32, 64), (1, 197, 3, 64, 64), (3, 7, 2, 16, 32)])
 def test_split_heads_is_exact(dtype, B, L, H, Dk, Dv):

@@ -24,6 +24,9 @@ int launch_layernorm(const void* x, const float* weight, const float* bias, void
 int launch_split_heads(const void* qkv, void* q, void* k, void* v, int B, int L, int H, int Dk, int Dv, long long ld,
                        int io_dtype, hipStream_t stream);
 int launch_swiglu(const void* in, void* out, long long rows, int I, int io_dtype, hipStream_t stream);
+bool patch_conv_supported(int Cin, int H, int W, int KH, int KW, int stride, int padding, int Cout);
+int launch_patch_conv(const void* x, const void* w_packed, void* y, int B, int Cin, int H, int W, int KH, int KW,
+                      int Cout, hipStream_t stream);
 int launch_pad_channels(const void* src, void* dst, long long rows, int src_c, int dst_c, hipStream_t stream);
 int launch_pad_channels_multi(const void* const* src, void* const* dst, const int* src_c, const int* dst_c, int n,
                               long long rows, hipStream_t stream);
@@ -246,6 +249,15 @@ int vig_split_heads_fwd(const void* qkv, void* q, void* k, void* v, int B, int L
   const long long ld = qkv_row_stride > 0 ? qkv_row_stride : packed;
   if (ld < packed || !strided_rows_ok(qkv, ld, io_dtype)) return VIG_EINVAL;
   return vig::launch_split_heads(qkv, q, k, v, B, L, H, Dk, Dv, ld, io_dtype, (hipStream_t)stream);
+}
+
+int vig_patch_conv_fwd(const void* x, const void* w_packed, void* y, int B, int Cin, int H, int W, int KH, int KW,
+                       int stride, int padding, int Cout, int io_dtype, void* stream) {
+  if (!x || !w_packed || !y || B <= 0 || Cin <= 0 || H <= 0 || W <= 0 || KH <= 0 || KW <= 0 || Cout <= 0) return VIG_EINVAL;
+  if (io_dtype != VIG_BF16 || !vig::patch_conv_supported(Cin, H, W, KH, KW, stride, padding, Cout)) return VIG_ENOTSUP;
+  if (!strided_rows_ok(x, W, io_dtype) || !strided_rows_ok(w_packed, 16, io_dtype) || !strided_rows_ok(y, Cout, io_dtype))
+    return VIG_EINVAL;
+  return vig::launch_patch_conv(x, w_packed, y, B, Cin, H, W, KH, KW, Cout, (hipStream_t)stream);
 }
 
 int vig_swiglu_fwd(const void* gate_up, void* out, long long rows, int I, int io_dtype, void* stream) {

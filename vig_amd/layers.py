@@ -289,7 +289,14 @@ class V2PatchEmbed(nn.Module):
         # channels-last throughout: the convolutions run in that layout, the norms see row matrices, and the final
         # 'b c h w -> b (h w) c' is a view; each convolution's bias add rides in the norm kernel behind it
         conv1, norm1, act, conv2, norm2 = self.proj
-        x = self._conv_nobias(conv1, x.contiguous(memory_format=torch.channels_last))
+        if (conv1.stride[0] == conv1.stride[1] and conv1.padding[0] == conv1.padding[1] and conv1.groups == 1
+                and conv1.dilation == (1, 1)
+                and ops.patch_conv_supported(x, conv1.weight, conv1.stride[0], conv1.padding[0])):
+            # the stem's shape: the library's implicit-GEMM kernel reads the images as they are and writes rows
+            x = ops.patch_conv(x, self._packed_w1(), conv1.kernel_size, conv1.stride[0], conv1.padding[0])
+            x = x.permute(0, 3, 1, 2)  # [B, C, H, W] view of channels-last memory
+        else:
+            x = self._conv_nobias(conv1, x.contiguous(memory_format=torch.channels_last))
         x = norm1(x, silu=isinstance(act, nn.SiLU), pre_bias=_f32(self, "b1", conv1.bias))
         if not isinstance(act, nn.SiLU):
             x = act(x)
@@ -299,6 +306,15 @@ class V2PatchEmbed(nn.Module):
             pos_embed = resize_pos_embed(pos_embed, pos_shape, hw).to(x.dtype)
         x = norm2(x, pre_bias=_f32(self, "b2", conv2.bias), post_add=pos_embed)
         return x.flatten(2).transpose(1, 2), hw
+
+    def _packed_w1(self):
+        """The first convolution's weight in the kernel's packed form, rebuilt when the parameter changes."""
+        w = self.proj[0].weight
+        key = (w.data_ptr(), w._version, w.dtype, w.device)
+        hit = self.__dict__.get("_w1_packed")
+        if hit is None or hit[0] != key:
+            self.__dict__["_w1_packed"] = hit = (key, ops.pack_patch_conv_weight(w))
+        return hit[1]
 
     @staticmethod
     def _conv_nobias(conv, x):

@@ -453,6 +453,42 @@ def split_heads(qkv: torch.Tensor, num_heads: int, head_qk_dim: int, head_v_dim:
     return q, k, v
 
 
+def pack_patch_conv_weight(weight: torch.Tensor) -> torch.Tensor:
+    """[Cout, Cin, KH, KW] -> [Cout, Cin*KH, 16]: kernel rows zero-padded to the 16 columns vig_patch_conv_fwd reads."""
+    Cout, Cin, KH, KW = weight.shape
+    if KW > 16:
+        raise ValueError("kernel width above 16")
+    return torch.nn.functional.pad(weight.detach(), (0, 16 - KW)).reshape(Cout, Cin * KH, 16).contiguous()
+
+
+def patch_conv_supported(x: torch.Tensor, weight: torch.Tensor, stride: int, padding: int) -> bool:
+    """Whether patch_conv takes this convolution (the reference's stem shape in bf16); else use torch's."""
+    Cout, Cin, KH, KW = weight.shape
+    return (x.dtype == torch.bfloat16 and x.is_cuda and x.dim() == 4 and stride == 8 and padding == 1 and KW <= 16
+            and Cin * KH == 27 and x.shape[1] == Cin and x.shape[3] % 8 == 0 and x.shape[3] <= 248
+            and Cout % 32 == 0 and 64 <= Cout <= 256 and (x.shape[3] + 2 - KW) // 8 + 1 <= 32)
+
+
+def patch_conv(x: torch.Tensor, w_packed: torch.Tensor, kernel_hw, stride: int = 8, padding: int = 1) -> torch.Tensor:
+    """x [B, Cin, H, W] bf16 -> [B, OH, OW, Cout] (channels-last rows) = conv2d without bias (vig.py:651);
+    w_packed from pack_patch_conv_weight."""
+    lib = _lib.load()
+    _check_cuda(x, w_packed)
+    x = x.contiguous()
+    B, Cin, H, W = x.shape
+    KH, KW = kernel_hw
+    Cout = w_packed.shape[0]
+    if w_packed.shape != (Cout, Cin * KH, 16) or w_packed.dtype != x.dtype or not w_packed.is_contiguous():
+        raise ValueError("w_packed must be the contiguous [Cout, Cin*KH, 16] tensor of pack_patch_conv_weight, in x's dtype")
+    OH, OW = (H + 2 * padding - KH) // stride + 1, (W + 2 * padding - KW) // stride + 1
+    y = torch.empty(B, OH, OW, Cout, dtype=x.dtype, device=x.device)
+    with torch.cuda.device(x.device):
+        rc = lib.vig_patch_conv_fwd(x.data_ptr(), w_packed.data_ptr(), y.data_ptr(), B, Cin, H, W, KH, KW, stride,
+                                    padding, Cout, _dt(x), _stream_ptr(x))
+    _lib.check(rc, "vig_patch_conv_fwd")
+    return y
+
+
 def swiglu(gate_up: torch.Tensor) -> torch.Tensor:
     """gate_up [..., 2*I] = (gate | up) -> gate * up / (1 + exp(-gate))  (fla/modules/activations.py:109-113)."""
     lib = _lib.load()
