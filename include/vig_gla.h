@@ -253,6 +253,19 @@ int vig_split_heads_fwd(const void* qkv, void* q, void* k, void* v, int B, int L
 int vig_swiglu_fwd(const void* gate_up, void* out, long long rows, int I, int io_dtype, void* stream);
 
 /*
+ * gate_proj and the SwiGLU product in one kernel, for a short contraction (K = 384 or 192, the hidden sizes of
+ * ViG-S / ViG-T), bf16, fp32 accumulation:
+ *   y [rows, I] = swiglu(gate, up) with (gate | up) = x [rows, K] . weight [2*I, K]^T, the product taken on gate and
+ *   up rounded to bf16 (what the separate layer stores); I % 32 == 0; x, weight and y packed row-major.
+ * Other K or dtypes return VIG_ENOTSUP (use a GEMM library and vig_swiglu_fwd).
+ *
+ * Replaces: gate_proj followed by swiglu (classification/models/vig.py:492-495,
+ * flash-linear-attention/fla/modules/activations.py:109-113) without the [rows, 2*I] intermediate.
+ */
+int vig_linear_swiglu_fwd(const void* x, const void* weight, void* y, long long rows, int K, int I, int io_dtype,
+                          void* stream);
+
+/*
  * First convolution of the v2 patch embedding, without its bias (vig_layernorm_fwd's pre_bias takes that):
  *   x [B, Cin, H, W] (bf16, the layout images arrive in)  ->  y [B, OH, OW, Cout] (bf16, channels-last rows),
  *   OH = (H + 2*padding - KH) / stride + 1, OW likewise.

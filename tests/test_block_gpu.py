@@ -76,6 +76,36 @@ def test_layernorm(dtype, tol, rows, C):
         assert err.max() <= 3 * tol, err.max()
 
 
+@pytest.mark.parametrize("rows,K,I", [(50176, 384, 1024), (1000, 384, 1024), (33, 384, 96), (1, 192, 32), (777, 192, 512),
+                                      (64, 384, 288)])
+def test_linear_swiglu(rows, K, I):
+    """gate_proj + SwiGLU in one kernel against (a) the fp64 oracle applied to the stored (bf16-rounded) gate and up
+    values of an fp64 product -- a gate or up that rounds the other way moves the output by one bf16 ulp of that factor,
+    hence the relative tolerance -- and (b) the two library steps it replaces (torch GEMM, then vig_swiglu_fwd)."""
+    announce(f"linear_swiglu rows{rows} K{K} I{I}")
+    x = _randn((rows, K), 51, torch.bfloat16)
+    w = _randn((2 * I, K), 52, torch.bfloat16) * (K ** -0.5)
+    got = vig_amd.ops.linear_swiglu(x.cuda(), w.cuda())
+    assert tuple(got.shape) == (rows, I)
+    gu = f64(x) @ f64(w).T
+    gu_stored = f64(torch.from_numpy(gu).to(torch.bfloat16))
+    want = O.swiglu_reference(gu_stored)
+    err = np.abs(f64(got) - want) / np.maximum(1.0, np.abs(want))
+    assert err.max() <= 3 * 2.0 ** -8, err.max()
+    two = vig_amd.ops.swiglu(torch.nn.functional.linear(x.cuda(), w.cuda()))
+    err2 = (got.double() - two.double()).abs() / two.double().abs().clamp_min(1.0)
+    assert err2.max().item() <= 3 * 2.0 ** -8, err2.max().item()
+
+
+def test_linear_swiglu_refuses_other_shapes():
+    x = torch.zeros(4, 256, dtype=torch.bfloat16).cuda()
+    w = torch.zeros(128, 256, dtype=torch.bfloat16).cuda()
+    assert not vig_amd.ops.linear_swiglu_supported(x, w)
+    assert not vig_amd.ops.linear_swiglu_supported(x.float()[:, :192], w.float()[:, :192])
+    with pytest.raises(vig_amd._lib.VigGlaError):
+        vig_amd.ops.linear_swiglu(x, w)
+
+
 @pytest.mark.parametrize("B,H,W,KW,Cout", [(3, 224, 224, 9, 192), (2, 64, 64, 9, 96), (1, 40, 248, 9, 256),
                                            (2, 17, 24, 9, 64), (1, 224, 224, 16, 64)])
 def test_patch_conv(B, H, W, KW, Cout):

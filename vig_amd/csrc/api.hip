@@ -24,6 +24,8 @@ int launch_layernorm(const void* x, const float* weight, const float* bias, void
 int launch_split_heads(const void* qkv, void* q, void* k, void* v, int B, int L, int H, int Dk, int Dv, long long ld,
                        int io_dtype, hipStream_t stream);
 int launch_swiglu(const void* in, void* out, long long rows, int I, int io_dtype, hipStream_t stream);
+bool linear_swiglu_supported(int K, int I);
+int launch_linear_swiglu(const void* A, const void* W, void* out, long long T, int K, int I, hipStream_t stream);
 bool patch_conv_supported(int Cin, int H, int W, int KH, int KW, int stride, int padding, int Cout);
 int launch_patch_conv(const void* x, const void* w_packed, void* y, int B, int Cin, int H, int W, int KH, int KW,
                       int Cout, hipStream_t stream);
@@ -258,6 +260,15 @@ int vig_patch_conv_fwd(const void* x, const void* w_packed, void* y, int B, int 
   if (!strided_rows_ok(x, W, io_dtype) || !strided_rows_ok(w_packed, 16, io_dtype) || !strided_rows_ok(y, Cout, io_dtype))
     return VIG_EINVAL;
   return vig::launch_patch_conv(x, w_packed, y, B, Cin, H, W, KH, KW, Cout, (hipStream_t)stream);
+}
+
+int vig_linear_swiglu_fwd(const void* x, const void* weight, void* y, long long rows, int K, int I, int io_dtype,
+                          void* stream) {
+  if (!x || !weight || !y || rows <= 0 || K <= 0 || I <= 0) return VIG_EINVAL;
+  if (io_dtype != VIG_BF16 || !vig::linear_swiglu_supported(K, I)) return VIG_ENOTSUP;
+  if (!strided_rows_ok(x, K, io_dtype) || !strided_rows_ok(weight, K, io_dtype) || !strided_rows_ok(y, I, io_dtype))
+    return VIG_EINVAL;
+  return vig::launch_linear_swiglu(x, weight, y, rows, K, I, (hipStream_t)stream);
 }
 
 int vig_swiglu_fwd(const void* gate_up, void* out, long long rows, int I, int io_dtype, void* stream) {

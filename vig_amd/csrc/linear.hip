@@ -1,0 +1,187 @@
+// gate_proj and the SwiGLU product of the block's MLP in one kernel, for contractions as short as the hidden size
+// (K = 16 * KS <= 384):
+//   out[t, c] = g * sigmoid(g) * u,   g = A[t, :] . W[c, :],   u = A[t, :] . W[I + c, :]      (W = [2*I, K])
+// bf16 operands, fp32 accumulation, bf16 out; the product is taken on g and u rounded to bf16, the values the
+// separate layer would have stored (flash-linear-attention/fla/modules/activations.py:109-113 on the two halves of
+// gate_proj's output, classification/models/vig.py:492-495), so the [T, 2*I] intermediate never exists.
+//
+// With K this short a wave's whole slice of W fits in registers: a wave keeps the 32 gate rows and the 32 matching
+// up rows of one channel tile as matrix-instruction A operands for the life of the workgroup, eight waves cover 256
+// channels, and the workgroup streams 32-token tiles of A through LDS (double-buffered, the next tile's global loads
+// in flight during the matrix instructions): every 16-byte LDS read feeds two v_mfma_f32_32x32x16_bf16.  Matrix rows
+// are assigned channels so that a lane ends with 16 consecutive channels of one token (32 contiguous bytes).
+// Workgroups of the same column group are spread over the token tiles; the column groups of one token tile run on the
+// same XCD (workers are a multiple of the XCD count apart in block index), so a tile of A leaves HBM once.
+#include "common.h"
+#include "launch.h"
+
+namespace vig {
+
+// Optional phase timing (development builds only: -DVIG_TIMING): cycles per phase, summed over the tiles of workgroup 0.
+#ifdef VIG_TIMING
+__device__ unsigned long long g_lin_stamp[8][8];
+#define VIG_LIN_T(i)                                             \
+  do {                                                           \
+    __builtin_amdgcn_sched_barrier(0);                           \
+    const unsigned long long now_ = __builtin_readcyclecounter(); \
+    ph[i] += now_ - last_;                                       \
+    last_ = now_;                                                \
+    __builtin_amdgcn_sched_barrier(0);                           \
+  } while (0)
+#else
+#define VIG_LIN_T(i) \
+  do {               \
+  } while (0)
+#endif
+
+namespace {
+
+constexpr int kLinWaves = 8;
+
+template <int KS>
+__global__ __launch_bounds__(64 * kLinWaves) void linear_swiglu_kernel(const uint16_t* __restrict__ A,
+                                                                       const uint16_t* __restrict__ W,
+                                                                       uint16_t* __restrict__ out, int T, int I,
+                                                                       int nworkers) {
+  constexpr int K = 16 * KS;
+  constexpr int kThreads = 64 * kLinWaves;
+  constexpr int kRow = K + 8;                                // LDS row stride in elements (conflict-free 16-byte reads)
+  constexpr int kChunks = 32 * K / 8;                        // 16-byte chunks of a 32-token tile
+  constexpr int kPer = (kChunks + kThreads - 1) / kThreads;  // chunks per thread
+  extern __shared__ __align__(16) char smem[];
+  uint16_t* buf = reinterpret_cast<uint16_t*>(smem);  // [2][32][kRow]
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int r = lane & 31, h = lane >> 5;
+  const int cg = blockIdx.x / nworkers, worker = blockIdx.x - cg * nworkers;
+  const int ct = cg * kLinWaves + wave;  // this wave's channel tile
+  const bool have = 32 * ct < I;
+  // matrix row i holds channel 16*((i>>2)&1) + 4*(i>>3) + (i&3) of the tile: lane (r, h) ends with channels 16h..16h+15
+  const int chan_of_row = 16 * ((r >> 2) & 1) + 4 * (r >> 3) + (r & 3);
+  u32x4_t wg[KS], wu[KS];
+  {
+    const uint16_t* pg = W + (size_t)(have ? 32 * ct + chan_of_row : 0) * K + 8 * h;
+    const uint16_t* pu = pg + (size_t)I * K;
+#pragma unroll
+    for (int t = 0; t < KS; ++t) {
+      wg[t] = *reinterpret_cast<const u32x4_t*>(pg + 16 * t);
+      wu[t] = *reinterpret_cast<const u32x4_t*>(pu + 16 * t);
+    }
+  }
+  const int ntiles_t = (T + 31) / 32;
+  // a 32-token tile of A is one contiguous run of 32*K elements: chunk c of it goes to row c / (K/8) of the buffer
+  int lds_off[kPer];
+#pragma unroll
+  for (int i = 0; i < kPer; ++i) {
+    const int c = tid + kThreads * i;
+    lds_off[i] = (c / (K / 8)) * kRow + (c % (K / 8)) * 8;
+  }
+  auto fetch = [&](int tile, u32x4_t (&v)[kPer]) {
+#pragma unroll
+    for (int i = 0; i < kPer; ++i) {
+      const int c = tid + kThreads * i;
+      v[i] = u32x4_t{0u, 0u, 0u, 0u};
+      if (tile < ntiles_t && c < kChunks && tile * 32 + c / (K / 8) < T)
+        v[i] = *reinterpret_cast<const u32x4_t*>(A + (size_t)tile * (32 * K) + (size_t)c * 8);
+    }
+  };
+  u32x4_t v[kPer];
+  fetch(worker, v);
+  int cur = 0;
+#ifdef VIG_TIMING
+  unsigned long long ph[6] = {0, 0, 0, 0, 0, 0}, last_ = __builtin_readcyclecounter();
+  const unsigned long long t_begin = last_;
+#endif
+  for (int tile = worker; tile < ntiles_t; tile += nworkers, cur ^= 1) {
+    uint16_t* mine = buf + cur * (32 * kRow);
+#pragma unroll
+    for (int i = 0; i < kPer; ++i)
+      if (tid + kThreads * i < kChunks) *reinterpret_cast<u32x4_t*>(mine + lds_off[i]) = v[i];
+    VIG_LIN_T(0);
+    __syncthreads();  // the tile is staged; the other buffer was last read before the previous barrier
+    VIG_LIN_T(1);
+    fetch(tile + nworkers, v);
+    VIG_LIN_T(2);
+    f32x16_t g, u;
+#pragma unroll
+    for (int j = 0; j < 16; ++j) g[j] = 0.f, u[j] = 0.f;
+    const uint16_t* xrow = mine + r * kRow + 8 * h;
+#pragma unroll
+    for (int t = 0; t < KS; ++t) {
+      const u32x4_t x = *reinterpret_cast<const u32x4_t*>(xrow + 16 * t);
+      g = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, wg[t]), __builtin_bit_cast(bf16x8_t, x),
+                                                  g, 0, 0, 0);
+      u = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, wu[t]), __builtin_bit_cast(bf16x8_t, x),
+                                                  u, 0, 0, 0);
+    }
+    VIG_LIN_T(3);
+    // (no run-time branch between the matrix instructions and the first read of their results)
+    u32x4_t lo, hi;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      float y[2];
+#pragma unroll
+      for (int e = 0; e < 2; ++e) {
+        const float gs = bf16_to_f32(f32_to_bf16(g[2 * j + e])), us = bf16_to_f32(f32_to_bf16(u[2 * j + e]));
+        y[e] = gs * us * sigmoidf_(gs);
+      }
+      const uint32_t pk = pack_bf16x2(y[0], y[1]);
+      if (j < 4) lo[j] = pk;
+      else hi[j - 4] = pk;
+    }
+    const int token = tile * 32 + r;
+    if (have && token < T) {
+      uint16_t* dst = out + (size_t)token * I + 32 * ct + 16 * h;
+      *reinterpret_cast<u32x4_t*>(dst) = lo;
+      *reinterpret_cast<u32x4_t*>(dst + 8) = hi;
+    }
+    VIG_LIN_T(4);
+  }
+#ifdef VIG_TIMING
+  if (blockIdx.x == 0 && lane == 0) {
+    for (int i = 0; i < 5; ++i) g_lin_stamp[wave][i] = ph[i];
+    g_lin_stamp[wave][5] = __builtin_readcyclecounter() - t_begin;
+  }
+#endif
+}
+
+template <int KS>
+int launch_linear_swiglu_t(const void* A, const void* W, void* out, long long T, int I, int num_cu, hipStream_t stream) {
+  constexpr int K = 16 * KS;
+  const size_t lds = (size_t)2 * 32 * (K + 8) * sizeof(uint16_t);
+  const int ncg = (I / 32 + kLinWaves - 1) / kLinWaves;
+  const long long ntiles_t = (T + 31) / 32;
+  // one workgroup a CU; workers a multiple of 8 so that the column groups of a token tile share an XCD
+  int nworkers = num_cu / ncg / 8 * 8;
+  if (nworkers < 8) nworkers = 8;
+  if (nworkers > ntiles_t) nworkers = (int)ntiles_t;
+  hipLaunchKernelGGL((linear_swiglu_kernel<KS>), dim3(ncg * nworkers), dim3(64 * kLinWaves), lds, stream,
+                     (const uint16_t*)A, (const uint16_t*)W, (uint16_t*)out, (int)T, I, nworkers);
+  return hipGetLastError() == hipSuccess ? 0 : -5;
+}
+
+}  // namespace
+
+bool linear_swiglu_supported(int K, int I) { return (K == 384 || K == 192) && I % 32 == 0 && I >= 32; }
+
+int launch_linear_swiglu(const void* A, const void* W, void* out, long long T, int K, int I, hipStream_t stream) {
+  if (!linear_swiglu_supported(K, I) || T <= 0 || T > 0x7fffffffLL - 64) return -95;
+  constexpr int kMaxDevices = 64;
+  static int num_cu_dev[kMaxDevices] = {};
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return -5;
+  if (num_cu_dev[dev] == 0) {
+    int n = 0;
+    if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess) return -5;
+    num_cu_dev[dev] = n > 0 ? n : 256;
+  }
+  return K == 384 ? launch_linear_swiglu_t<24>(A, W, out, T, I, num_cu_dev[dev], stream)
+                  : launch_linear_swiglu_t<12>(A, W, out, T, I, num_cu_dev[dev], stream);
+}
+
+}  // namespace vig
+
+#ifdef VIG_TIMING
+extern "C" int vig_debug_read_lin_stamps(unsigned long long* host_out) {
+  return hipMemcpyFromSymbol(host_out, HIP_SYMBOL(vig::g_lin_stamp), sizeof(vig::g_lin_stamp)) == hipSuccess ? 0 : -5;
+}
+#endif

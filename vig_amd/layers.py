@@ -223,6 +223,9 @@ class GLAMLP(nn.Module):
         self.down_proj = nn.Linear(intermediate_size, hidden_size, bias=False)
 
     def forward(self, x):
+        w = self.gate_proj.weight
+        if ops.linear_swiglu_supported(x, w):  # ViG-S / ViG-T widths in bf16: no [.., 2*I] intermediate
+            return self.down_proj(ops.linear_swiglu(x, w))
         return self.down_proj(ops.swiglu(self.gate_proj(x)))
 
 

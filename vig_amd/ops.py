@@ -489,6 +489,28 @@ def patch_conv(x: torch.Tensor, w_packed: torch.Tensor, kernel_hw, stride: int =
     return y
 
 
+def linear_swiglu_supported(x: torch.Tensor, weight: torch.Tensor) -> bool:
+    """Whether linear_swiglu takes this layer (bf16 on the GPU, contraction 384 or 192, 32-aligned halves)."""
+    return (x.is_cuda and x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16 and weight.dim() == 2
+            and weight.shape[1] in (384, 192) and x.shape[-1] == weight.shape[1] and weight.shape[0] % 64 == 0)
+
+
+def linear_swiglu(x: torch.Tensor, weight: torch.Tensor) -> torch.Tensor:
+    """swiglu(x @ weight.T) with weight [2*I, K] = (gate rows | up rows): gate_proj and the SwiGLU product
+    (vig.py:492-495) in one kernel, no [.., 2*I] intermediate."""
+    lib = _lib.load()
+    _check_cuda(x, weight)
+    x = x.contiguous()
+    w = weight.detach().contiguous()
+    K, I = w.shape[1], w.shape[0] // 2
+    y = torch.empty(*x.shape[:-1], I, dtype=x.dtype, device=x.device)
+    with torch.cuda.device(x.device):
+        rc = lib.vig_linear_swiglu_fwd(x.data_ptr(), w.data_ptr(), y.data_ptr(), x.numel() // K, K, I, _dt(x),
+                                       _stream_ptr(x))
+    _lib.check(rc, "vig_linear_swiglu_fwd")
+    return y
+
+
 def swiglu(gate_up: torch.Tensor) -> torch.Tensor:
     """gate_up [..., 2*I] = (gate | up) -> gate * up / (1 + exp(-gate))  (fla/modules/activations.py:109-113)."""
     lib = _lib.load()
