@@ -77,6 +77,22 @@ def test_vig_small_logits(dtype, tol):
     assert err <= tol
 
 
+@pytest.mark.parametrize("name,heads,kw", [("vig_tiny", 3, dict(out_act=True, act_in_conv=True)), ("vig_base", 12, {})])
+def test_vig_tiny_and_base_logits(name, heads, kw):
+    """The other two shipped widths in bf16 against the float64 restatement: ViG-T takes the hidden-size-192 forms of
+    the fused kernels (and SiLU after the depthwise conv and on the blend), ViG-B the library-GEMM paths."""
+    announce(f"{name} logits bf16")
+    torch.manual_seed(0)
+    model = getattr(layers, name)().eval()
+    images = torch.randn(1, 3, 224, 224)
+    want = R.vig_forward(model.state_dict(), images, num_heads=heads, depth=12, **kw).numpy()
+    got = model.to("cuda", torch.bfloat16)(images.to("cuda", torch.bfloat16)).double().cpu().numpy()
+    err = np.abs(got - want).max() / np.abs(want).max()
+    print(f"  logits max-rel err {err:.3e}  (max |logit| {np.abs(want).max():.3f})", flush=True)
+    assert got.shape == (1, 1000)
+    assert err <= 8e-2
+
+
 def test_evaluate_callers(tmp_path):
     """Checkpoint round trip (reference layout: weights under 'model'), accuracy, validate and throughput loops."""
     import torch
