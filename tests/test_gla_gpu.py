@@ -158,9 +158,12 @@ def test_bf16_mixed_gate_strength_many_items():
     assert max_abs(got, want) <= BF16_TOL
 
 
-def test_bf16_strong_gates_one_direction():
-    announce("bf16 default path, forward direction only, strong gates")
-    q, k, v, gf, _ = make_gla_inputs(2, 3, 300, 64, 64, seed=45, dtype=torch.bfloat16, gate_scale=1.0)
+@pytest.mark.parametrize("B,L", [(2, 300), (200, 196), (3, 64)])
+def test_bf16_strong_gates_one_direction(B, L):
+    """One direction only: half of the waves idle along and must keep the barrier count of the working half, also
+    through the segment that refuses the fp16 variant and is walked again (several slabs per workgroup at B = 200)."""
+    announce(f"bf16 default path, forward direction only, strong gates, B{B} L{L}")
+    q, k, v, gf, _ = make_gla_inputs(B, 3, L, 64, 64, seed=45, dtype=torch.bfloat16, gate_scale=1.0)
     gf = gf.clamp_min(-3)
     want = oracle_bidir(q, k, v, gf, None)
     got = f64(vig_amd.gla_bidir_forward(*dev(q, k, v, gf, None)))

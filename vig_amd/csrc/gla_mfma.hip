@@ -511,7 +511,7 @@ __device__ __forceinline__ bool direction_wave(const ChunkSrc& cur, const ChunkS
   VIG_STAMP(6);
   // same answer in every wave: the word is only written before this barrier and the variant is left once it is set
   const bool ok = !F16 || __builtin_amdgcn_readfirstlane(*veto) == 0;
-  if (F16 && !ok) o = chunk_rsrc(nullptr, 0, 0);  // nothing of this segment is stored
+  if (F16 && !ok) return false;  // every wave alike: the segment is walked again, barriers B and C are skipped by all
   // ---- state recurrence over the chunks of this direction, one slice (pv, NG/2 register quads) per wave ----
   {
     constexpr int NQ = NG / 2;
@@ -813,11 +813,13 @@ __global__ __launch_bounds__(512) void gla_mfma_kernel(const uint16_t* __restric
     const int* veto = reinterpret_cast<const int*>(lds + kLdsVeto);
     int item = blockIdx.x;
     for (; item < geo.nitems; item += gridDim.x) {
-      lds_barrier();
+      lds_barrier();  // (A)
       const bool refused = __builtin_amdgcn_readfirstlane(*veto) != 0;
-      lds_barrier();
-      lds_barrier();
-      lds_barrier();
+      if (!refused) {  // a refused segment leaves after barrier A
+        lds_barrier();
+        lds_barrier();
+      }
+      lds_barrier();  // (D)
       if (refused) break;
     }
     for (; item < geo.nitems; item += gridDim.x) {
