@@ -75,6 +75,22 @@ int vig_gla_bidir_fwd(const void* q, const void* k, const void* v,
 size_t vig_gla_bidir_fwd_workspace(int B, int H, int L, int Dk, int Dv, int io_dtype);
 
 /*
+ * Same contract, workspace and accuracy bar as vig_gla_bidir_fwd, for callers who know their gates to be strong.
+ * The matrix-core kernel computes scores on fp16 operands while a chunk's gate total stays within about 8 (natural
+ * log units) in every channel, and on split-bf16 operands beyond; it finds out per workgroup, on the first segment
+ * that refuses, and walks that segment twice.  This entry point starts with the split variant: about 10 % faster than
+ * finding out when every slab refuses and a workgroup has three slabs (nothing to gain at six or more), 25-30 %
+ * slower than the fp16 variant when none would have refused.  No counterpart
+ * in the reference, whose kernels have one arithmetic (fla/ops/gla/chunk_fuse.py:25-101,212-254).
+ */
+int vig_gla_bidir_fwd_wide(const void* q, const void* k, const void* v,
+                           const void* g_fwd, const void* g_bwd, void* o,
+                           void* workspace, size_t workspace_bytes,
+                           int B, int H, int L, int Dk, int Dv,
+                           float scale, float out_scale,
+                           int io_dtype, int gate_dtype, void* stream);
+
+/*
  * Same contract as vig_gla_bidir_fwd, but always runs the fp32-arithmetic
  * token-recurrent kernel whatever the dtypes (bf16 tensors are widened on load,
  * the state and all sums stay fp32).  This is the op-level counterpart of the

@@ -158,6 +158,21 @@ def test_bf16_mixed_gate_strength_many_items():
     assert max_abs(got, want) <= BF16_TOL
 
 
+@pytest.mark.parametrize("gate_scale,L,both", [(1.0, 196, True), (1.0 / 16, 196, True), (1.0, 700, True), (0.5, 130, False)])
+def test_bf16_wide_entry_point(gate_scale, L, both):
+    """vig_gla_bidir_fwd_wide (starts with the split-bf16 score variant): same accuracy bar on strong and on mild
+    gates, slab and long-sequence modes, one or two directions."""
+    announce(f"bf16 wide-range entry point, gates x{gate_scale} L={L} both={both}")
+    q, k, v, gf, gb = make_gla_inputs(40, 2, L, 64, 64, seed=46, dtype=torch.bfloat16, gate_scale=gate_scale)
+    gf, gb = gf.clamp_min(-3), gb.clamp_min(-3)
+    if not both:
+        gb = None
+    want = oracle_bidir(q, k, v, gf, gb)
+    got = f64(vig_amd.gla_bidir_forward(*dev(q, k, v, gf, gb), strong_gates=True))
+    assert np.isfinite(got).all()
+    assert max_abs(got, want) <= BF16_TOL
+
+
 @pytest.mark.parametrize("B,L", [(2, 300), (200, 196), (3, 64)])
 def test_bf16_strong_gates_one_direction(B, L):
     """One direction only: half of the waves idle along and must keep the barrier count of the working half, also

@@ -106,13 +106,14 @@ size_t vig_gla_bidir_fwd_workspace(int B, int H, int L, int Dk, int Dv, int io_d
   return need;
 }
 
-int vig_gla_bidir_fwd(const void* q, const void* k, const void* v, const void* g_fwd, const void* g_bwd, void* o,
-                      void* workspace, size_t workspace_bytes, int B, int H, int L, int Dk, int Dv, float scale,
-                      float out_scale, int io_dtype, int gate_dtype, void* stream) {
+static int gla_bidir_fwd(const void* q, const void* k, const void* v, const void* g_fwd, const void* g_bwd, void* o,
+                         void* workspace, size_t workspace_bytes, int B, int H, int L, int Dk, int Dv, float scale,
+                         float out_scale, int io_dtype, int gate_dtype, void* stream, int wide_gates) {
   vig::GlaArgs a;
   const int rc = fill_args(a, q, k, v, g_fwd, g_bwd, o, workspace, workspace_bytes, B, H, L, Dk, Dv, scale,
                            out_scale, io_dtype, gate_dtype, stream);
   if (rc != VIG_OK) return rc;
+  a.wide_gates = wide_gates;
   if (vig::gla_mfma_supported(a)) {
     if (vig::gla_mfma_workspace(B, H, L, Dk, Dv) > workspace_bytes) return VIG_ENOSPC;
     if (vig::gla_mfma_workspace(B, H, L, Dk, Dv) > 0 && !workspace) return VIG_EINVAL;
@@ -144,6 +145,21 @@ int vig_gla_bidir_fwd(const void* q, const void* k, const void* v, const void* g
   if (need > workspace_bytes) return VIG_ENOSPC;
   if (need > 0 && !workspace) return VIG_EINVAL;
   return vig::launch_gla_recurrent(a);
+}
+
+int vig_gla_bidir_fwd(const void* q, const void* k, const void* v, const void* g_fwd, const void* g_bwd, void* o,
+                      void* workspace, size_t workspace_bytes, int B, int H, int L, int Dk, int Dv, float scale,
+                      float out_scale, int io_dtype, int gate_dtype, void* stream) {
+  return gla_bidir_fwd(q, k, v, g_fwd, g_bwd, o, workspace, workspace_bytes, B, H, L, Dk, Dv, scale, out_scale,
+                       io_dtype, gate_dtype, stream, 0);
+}
+
+// Same contract and results to the same bar; for callers whose gates are known to be strong (see the header).
+int vig_gla_bidir_fwd_wide(const void* q, const void* k, const void* v, const void* g_fwd, const void* g_bwd, void* o,
+                           void* workspace, size_t workspace_bytes, int B, int H, int L, int Dk, int Dv, float scale,
+                           float out_scale, int io_dtype, int gate_dtype, void* stream) {
+  return gla_bidir_fwd(q, k, v, g_fwd, g_bwd, o, workspace, workspace_bytes, B, H, L, Dk, Dv, scale, out_scale,
+                       io_dtype, gate_dtype, stream, 1);
 }
 
 // vig_gla_bidir_fwd followed by vig_locality_gate_fwd in one kernel: y = o * sigmoid(conv3x3(o)) with o the rounded

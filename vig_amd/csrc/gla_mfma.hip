@@ -723,6 +723,7 @@ __device__ __forceinline__ bool direction_wave(const ChunkSrc& cur, const ChunkS
 struct Geometry {
   int L, nseg, seg_len, cw, nitems;
   int gw, gh, heads;  // fused locality gate only: token grid and heads per batch element
+  int wide_gates;     // nonzero: skip the fp16 score variant from the start
 };
 
 template <bool FWD, int MODE, int NG, bool F16, bool GATE>
@@ -782,8 +783,10 @@ template <bool FWD, int MODE, int NG, bool GATE>
 __device__ __forceinline__ void wave_items(const uint16_t* q, const uint16_t* k, const uint16_t* v, const uint16_t* g,
                                            uint16_t* o, const Geometry& geo, int c, int lane, char* lds, float oscale,
                                            bool bidir, float* state_ws, const float* gate_w) {
-  const int item = wave_loop<FWD, MODE, NG, true, GATE>(q, k, v, g, o, geo, (int)blockIdx.x, c, lane, lds, oscale,
-                                                        bidir, state_ws, gate_w);
+  int item = (int)blockIdx.x;
+  // (a caller that knows its gates to be strong starts with the split-bf16 variant: no segment is walked in vain)
+  if (!geo.wide_gates)
+    item = wave_loop<FWD, MODE, NG, true, GATE>(q, k, v, g, o, geo, item, c, lane, lds, oscale, bidir, state_ws, gate_w);
   wave_loop<FWD, MODE, NG, false, GATE>(q, k, v, g, o, geo, item, c, lane, lds, oscale, bidir, state_ws, gate_w);
 }
 
@@ -812,6 +815,7 @@ __global__ __launch_bounds__(512) void gla_mfma_kernel(const uint16_t* __restric
     // that is walked twice when the fp16 variant is refused
     const int* veto = reinterpret_cast<const int*>(lds + kLdsVeto);
     int item = blockIdx.x;
+    if (!geo.wide_gates)
     for (; item < geo.nitems; item += gridDim.x) {
       lds_barrier();  // (A)
       const bool refused = __builtin_amdgcn_readfirstlane(*veto) != 0;
@@ -910,6 +914,7 @@ static int launch_gla_mfma_t(const GlaArgs& a, int num_cu, int dev) {
     attr_done = true;
   }
   Geometry geo = make_geometry(a.B * a.H, a.L);
+  geo.wide_gates = a.wide_gates;
   int grid = geo.nitems < num_cu ? geo.nitems : num_cu;
 #ifdef VIG_TIMING
   if (const char* e = getenv("VIG_GRID")) grid = atoi(e);

@@ -22,6 +22,9 @@ struct GlaArgs {
   // stored instead of o; weights [H*Dv, 9] f32.  Null: plain output.
   const float* gate_w = nullptr;
   int gate_rows = 0, gate_cols = 0;
+  // bf16 MFMA path: the caller expects gates beyond the fp16 score variant's range (|chunk total| > ~8 nat in some
+  // channel): start with the split-bf16 variant instead of finding out on the first segment of every workgroup
+  int wide_gates = 0;
 };
 
 // fp32-arithmetic token-recurrent path (any supported dtype combination).

@@ -42,11 +42,14 @@ def _check_cuda(*ts):
 
 
 def gla_bidir_forward(q, k, v, g_fwd, g_bwd=None, scale: float = -1, out_scale: float = 1.0,
-                      exact: bool = False, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+                      exact: bool = False, out: Optional[torch.Tensor] = None,
+                      strong_gates: bool = False) -> torch.Tensor:
     """o = out_scale * (fwd(q,k,v,g_fwd) + bwd(q,k,v,g_bwd)), natural token order.
 
     q, k, g_*: [B,H,L,Dk]; v: [B,H,L,Dv].  g_bwd=None gives the causal op.
-    `exact=True` forces the fp32-arithmetic recurrent kernel.
+    `exact=True` forces the fp32-arithmetic recurrent kernel.  `strong_gates=True` (inference calls only) tells the
+    matrix-core kernel to start with its wide-range score variant (vig_gla_bidir_fwd_wide): worth it when most slabs
+    have a channel whose gates sum below about -8 over 64 tokens.
     Differentiable: when autograd is recording and an input requires grad, the backward runs vig_gla_bidir_bwd.
     """
     tensors = (q, k, v, g_fwd) + ((g_bwd,) if g_bwd is not None else ())
@@ -56,7 +59,7 @@ def gla_bidir_forward(q, k, v, g_fwd, g_bwd=None, scale: float = -1, out_scale: 
         if scale == -1 or scale is None:
             scale = q.shape[-1] ** -0.5
         return _GLABidirFunction.apply(q, k, v, g_fwd, g_bwd, float(scale), float(out_scale), bool(exact))
-    return _gla_bidir_forward_raw(q, k, v, g_fwd, g_bwd, scale, out_scale, exact, out)
+    return _gla_bidir_forward_raw(q, k, v, g_fwd, g_bwd, scale, out_scale, exact, out, strong_gates)
 
 
 def gla_bidir_backward(q, k, v, g_fwd, g_bwd, d_o, scale: float = -1, out_scale: float = 1.0,
@@ -112,7 +115,7 @@ class _GLABidirFunction(torch.autograd.Function):
         return dq, dk, dv, dgf, dgb, None, None, None
 
 
-def _gla_bidir_forward_raw(q, k, v, g_fwd, g_bwd, scale, out_scale, exact, out):
+def _gla_bidir_forward_raw(q, k, v, g_fwd, g_bwd, scale, out_scale, exact, out, strong_gates=False):
     lib = _lib.load()
     _check_cuda(q, k, v, g_fwd, g_bwd)
     q, k, v, g_fwd = (t.contiguous() for t in (q, k, v, g_fwd))
@@ -133,7 +136,7 @@ def _gla_bidir_forward_raw(q, k, v, g_fwd, g_bwd, scale, out_scale, exact, out):
         out = torch.empty(B, H, L, Dv, dtype=q.dtype, device=q.device)
     elif not (out.is_contiguous() and out.shape == (B, H, L, Dv) and out.dtype == q.dtype):
         raise ValueError("bad `out` tensor")
-    fn = lib.vig_gla_bidir_fwd_exact if exact else lib.vig_gla_bidir_fwd
+    fn = lib.vig_gla_bidir_fwd_exact if exact else (lib.vig_gla_bidir_fwd_wide if strong_gates else lib.vig_gla_bidir_fwd)
     ws_bytes = lib.vig_gla_bidir_fwd_workspace(B, H, L, Dk, Dv, io_dt)
     ws = torch.empty(ws_bytes, dtype=torch.uint8, device=q.device) if ws_bytes else None
     with torch.cuda.device(q.device):
