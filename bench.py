@@ -325,6 +325,12 @@ def main():
     want_model = (args.model or args.config == 1) and not args.op_only and not args.exact
     if want_backward:
         out["backward"] = backward_time(lib, sets, s, io_dt, scale, sp, stream, dev)
+        if out["backward"] is not None:
+            try:  # measured HBM bytes of the backward launch, where the profile summaries hold them
+                with open(os.path.join(ROOT, "profiles", "hbm_traffic.json")) as f:
+                    out["backward"]["traffic"] = json.load(f).get(s.name + ":backward", {}).get("bytes_per_launch")
+            except (OSError, ValueError):
+                out["backward"]["traffic"] = None
     if want_model:
         out["vig_s_forward"] = model_throughput(dev, tune_gemm=not args.no_gemm_tuning, use_graph=not args.no_graph)
     if not args.no_cpu:
