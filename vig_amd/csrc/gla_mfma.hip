@@ -148,6 +148,7 @@ __device__ __forceinline__ void make_pair16(const u32x4_t (&rawq)[NG], const u32
         const float q1 = bf16hi_to_f32(wq) * exp2_fast(x1);
         q16[g][m] = pack_f16x2(q0, q1);
         qb[g][m] = pack_bf16x2(q0, q1);
+        asm volatile("" : "+v"(qb[g][m]));  // packed here: the two floats must not stay alive until the pair is used
       }
     }
   }
