@@ -8,6 +8,8 @@
  *     freed or synchronised inside; work is enqueued on `stream`
  *     (a hipStream_t passed as void*; NULL = the null stream);
  *   - tensors are dense row-major with the innermost dimension contiguous;
+ *   - every tensor, weight vector and workspace starts on a 16-byte boundary
+ *     (the kernels move 16 bytes per access); a pointer off it is VIG_EINVAL;
  *   - return value: 0 on success, a negative VIG_E* code otherwise
  *     (vig_gla_strerror() gives the text); a failed call enqueues nothing;
  *   - dtype codes: VIG_F32 = 0, VIG_BF16 = 1.
@@ -27,7 +29,7 @@ extern "C" {
 #define VIG_BF16 1
 
 #define VIG_OK 0
-#define VIG_EINVAL (-22)  /* bad argument (null pointer, non-positive size) */
+#define VIG_EINVAL (-22)  /* bad argument (null or misaligned pointer, non-positive size) */
 #define VIG_ENOTSUP (-95) /* shape / dtype combination not built */
 #define VIG_ENOSPC (-28)  /* workspace too small */
 #define VIG_ELAUNCH (-5)  /* HIP reported a launch error */

@@ -234,3 +234,42 @@ def test_bf16_hiervig_head_shape_on_the_matrix_cores(B, H, L):
     exact = vig_amd.gla_bidir_forward(*dev(q, k, v, gf, gb), exact=True)
     assert np.all(np.abs(f64(got) - f64(exact)) <= BF16_TOL + 2.0 ** -7 * np.abs(want))
     assert not torch.equal(got, exact)  # (the two kernels round differently: proves the padded path ran)
+
+
+def test_pointers_off_a_16_byte_boundary():
+    """The library refuses a tensor that does not start on a 16-byte boundary (nothing is enqueued); the Python op
+    copies such a view first and gives the result of the aligned call."""
+    announce("misaligned views: C ABI refuses, Python op copies")
+    from vig_amd import _lib, ops
+    lib = _lib.load()
+    B, H, L, D = 2, 2, 70, 64
+    q, k, v, gf, gb = (t.bfloat16() for t in dev(*make_gla_inputs(B, H, L, D, D, seed=5)))
+    want = vig_amd.gla_bidir_forward(q, k, v, gf, gb)
+
+    def shifted(t):  # the same values in a view that starts one element into its storage
+        flat = torch.empty(t.numel() + 8, dtype=t.dtype, device=t.device)
+        flat[1:1 + t.numel()] = t.reshape(-1)
+        view = flat[1:1 + t.numel()].view(t.shape)
+        assert view.is_contiguous() and view.data_ptr() % 16 == 2
+        return view
+
+    got = vig_amd.gla_bidir_forward(shifted(q), k, shifted(v), gf, shifted(gb))
+    assert torch.equal(got, want)
+    out = torch.empty_like(v)
+    ws_bytes = lib.vig_gla_bidir_fwd_workspace(B, H, L, D, D, _lib.VIG_BF16)
+    ws = torch.empty(max(ws_bytes, 16), dtype=torch.uint8, device=q.device)
+    args = dict(q=q, k=k, v=v, gf=gf, gb=gb, out=out)
+    for name in args:
+        a = dict(args)
+        a[name] = shifted(args[name])
+        rc = lib.vig_gla_bidir_fwd(a["q"].data_ptr(), a["k"].data_ptr(), a["v"].data_ptr(), a["gf"].data_ptr(),
+                                   a["gb"].data_ptr(), a["out"].data_ptr(), ws.data_ptr(), ws_bytes, B, H, L, D, D,
+                                   D ** -0.5, 1.0, _lib.VIG_BF16, _lib.VIG_BF16, ops._stream_ptr(q))
+        assert rc == _lib.VIG_EINVAL, name
+    with pytest.raises(ValueError):
+        vig_amd.gla_bidir_forward(q, k, v, gf, gb, out=shifted(out))
+    x = shifted(torch.randn(40, 384, device="cuda").bfloat16())
+    w = torch.ones(384, device="cuda")
+    assert torch.equal(ops.rmsnorm(x, w), ops.rmsnorm(x.clone(), w))
+    assert lib.vig_rmsnorm_fwd(x.data_ptr(), None, w.data_ptr(), torch.empty_like(x).data_ptr(), None, 40, 384,
+                               1e-6, 0, _lib.VIG_BF16, ops._stream_ptr(x)) == _lib.VIG_EINVAL

@@ -12,6 +12,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "lib", "libvig_gla.so")
 
 VIG_F32, VIG_BF16 = 0, 1
+VIG_OK, VIG_EINVAL, VIG_ENOTSUP, VIG_ENOSPC, VIG_ELAUNCH = 0, -22, -95, -28, -5  # status codes of the C ABI
 
 _c_void_p = ctypes.c_void_p
 _c_int = ctypes.c_int

@@ -46,6 +46,11 @@ static bool strided_rows_ok(const void* base, long long ld_elems, int dtype) {
   const long long elem = dtype == VIG_BF16 ? 2 : 4;
   return (reinterpret_cast<uintptr_t>(base) % 16) == 0 && (ld_elems * elem) % 16 == 0;
 }
+// every tensor is moved 16 bytes per access: a pointer off that boundary is refused (null, for an optional tensor, passes)
+template <typename... P>
+static bool aligned16(P... p) {
+  return ((reinterpret_cast<uintptr_t>(static_cast<const void*>(p)) % 16 == 0) && ...);
+}
 static bool dk_ok(int d) { return d == 16 || d == 32 || d == 64 || d == 128; }
 static bool dv_ok(int d) { return d == 32 || d == 64 || d == 128; }
 
@@ -68,6 +73,7 @@ static int fill_args(vig::GlaArgs& a, const void* q, const void* k, const void* 
                      const void* g_bwd, void* o, void* workspace, size_t workspace_bytes, int B, int H, int L,
                      int Dk, int Dv, float scale, float out_scale, int io_dtype, int gate_dtype, void* stream) {
   if (!q || !k || !v || !g_fwd || !o) return VIG_EINVAL;
+  if (!aligned16(q, k, v, g_fwd, g_bwd, o, workspace)) return VIG_EINVAL;
   if (B <= 0 || H <= 0 || L <= 0) return VIG_EINVAL;
   if ((long long)B * H > 2147483647LL) return VIG_EINVAL;
   if (!dtype_ok(io_dtype) || !dtype_ok(gate_dtype)) return VIG_ENOTSUP;
@@ -172,6 +178,7 @@ int vig_gla_bidir_locgate_fwd(const void* q, const void* k, const void* v, const
                            gate_dtype, stream);
   if (rc != VIG_OK) return rc;
   if (!gate_weight || !g_bwd || grid_h <= 0 || grid_w <= 0 || (long long)grid_h * grid_w != L) return VIG_EINVAL;
+  if (!aligned16(gate_weight)) return VIG_EINVAL;
   if (!vig::gla_mfma_supported(a) || vig::gla_mfma_workspace(B, H, L, Dk, Dv) > 0 ||
       !vig::gla_mfma_gate_grid_ok(grid_h, grid_w))
     return VIG_ENOTSUP;
@@ -199,6 +206,7 @@ int vig_gla_bidir_fwd_exact(const void* q, const void* k, const void* v, const v
 int vig_dirgate_fwd(const void* gk_lin, void* g_out, int B, int L, int H, int Dk, float inv_normalizer,
                     float clamp_min, int in_dtype, int out_dtype, void* stream) {
   if (!gk_lin || !g_out || B <= 0 || L <= 0 || H <= 0 || Dk <= 0) return VIG_EINVAL;
+  if (!aligned16(gk_lin, g_out)) return VIG_EINVAL;
   if (!dtype_ok(in_dtype) || !dtype_ok(out_dtype) || (Dk % 8) != 0) return VIG_ENOTSUP;
   return vig::launch_dirgate(gk_lin, g_out, B, L, H, Dk, inv_normalizer, clamp_min, in_dtype, out_dtype,
                              (hipStream_t)stream);
@@ -211,7 +219,7 @@ int vig_dirgate_lowrank_fwd(const void* gk_low, long long low_row_stride, const 
   if (!dtype_ok(in_dtype) || !dtype_ok(out_dtype) || (Dk % 8) != 0 || rank != 16) return VIG_ENOTSUP;
   const long long ld = low_row_stride > 0 ? low_row_stride : rank;
   if (ld < rank || !strided_rows_ok(gk_low, ld, in_dtype) || !strided_rows_ok(w_up, rank, in_dtype) ||
-      !strided_rows_ok(b_up, 8, in_dtype))
+      !strided_rows_ok(b_up, 8, in_dtype) || !aligned16(g_out))
     return VIG_EINVAL;
   return vig::launch_dirgate_lowrank(gk_low, ld, w_up, b_up, g_out, B, L, H, Dk, rank, inv_normalizer, clamp_min,
                                      in_dtype, out_dtype, (hipStream_t)stream);
@@ -220,6 +228,7 @@ int vig_dirgate_lowrank_fwd(const void* gk_low, long long low_row_stride, const 
 int vig_dwconv3x3_fwd(const void* x, const float* weight, const float* bias, void* y, int B, int h, int w, int C,
                       int silu, int io_dtype, void* stream) {
   if (!x || !weight || !y || B <= 0 || h <= 0 || w <= 0 || C <= 0 || x == y) return VIG_EINVAL;
+  if (!aligned16(x, weight, bias, y)) return VIG_EINVAL;
   if (!dtype_ok(io_dtype) || (C % 8) != 0) return VIG_ENOTSUP;
   return vig::launch_dwconv3x3(x, weight, bias, y, B, h, w, C, silu, io_dtype, (hipStream_t)stream);
 }
@@ -227,6 +236,7 @@ int vig_dwconv3x3_fwd(const void* x, const float* weight, const float* bias, voi
 int vig_locality_gate_fwd(const void* o, const float* weight, void* y, int B, int H, int h, int w, int Dv,
                           int io_dtype, void* stream) {
   if (!o || !weight || !y || B <= 0 || H <= 0 || h <= 0 || w <= 0 || o == y) return VIG_EINVAL;
+  if (!aligned16(o, weight, y)) return VIG_EINVAL;
   if (!dtype_ok(io_dtype) || (Dv % 8) != 0 || Dv <= 0) return VIG_ENOTSUP;
   return vig::launch_locality_gate(o, weight, y, B, H, h, w, Dv, io_dtype, (hipStream_t)stream);
 }
@@ -235,6 +245,7 @@ int vig_locality_blend_fwd(const void* o, const void* local, const void* g_lin, 
                            void* y, int B, int H, int L, int Dv, long long g_row_stride, float eps, int silu_out,
                            int io_dtype, void* stream) {
   if (!o || !local || !g_lin || !w_g || !w_l || !y || B <= 0 || H <= 0 || L <= 0) return VIG_EINVAL;
+  if (!aligned16(o, local, w_g, w_l, y)) return VIG_EINVAL;
   if (!dtype_ok(io_dtype) || !(Dv == 32 || Dv == 64)) return VIG_ENOTSUP;
   const long long ldg = g_row_stride > 0 ? g_row_stride : (long long)H * Dv;
   if (ldg < (long long)H * Dv || !strided_rows_ok(g_lin, ldg, io_dtype)) return VIG_EINVAL;
@@ -245,6 +256,7 @@ int vig_locality_blend_fwd(const void* o, const void* local, const void* g_lin, 
 int vig_rmsnorm_fwd(const void* x, const void* residual, const float* weight, void* y, void* residual_out,
                     long long rows, int C, float eps, int round_sum, int io_dtype, void* stream) {
   if (!x || !weight || !y || rows <= 0 || C <= 0 || rows > 0x7fffffffLL) return VIG_EINVAL;
+  if (!aligned16(x, residual, weight, y, residual_out)) return VIG_EINVAL;
   if (!dtype_ok(io_dtype) || (C % 8) != 0 || C > 4096) return VIG_ENOTSUP;
   return vig::launch_rmsnorm(x, residual, weight, y, residual_out, (int)rows, C, eps, round_sum, io_dtype,
                              (hipStream_t)stream);
@@ -254,6 +266,7 @@ int vig_layernorm_fwd(const void* x, const float* weight, const float* bias, voi
                       float eps, int silu, const float* pre_bias, const void* post_add, int post_rows, int io_dtype,
                       void* stream) {
   if (!x || !weight || !bias || !y || rows <= 0 || C <= 0 || (post_add && post_rows <= 0)) return VIG_EINVAL;
+  if (!aligned16(x, weight, bias, y, pre_bias, post_add)) return VIG_EINVAL;
   if (!dtype_ok(io_dtype) || (C % 8) != 0 || C > 4096) return VIG_ENOTSUP;
   return vig::launch_layernorm(x, weight, bias, y, rows, C, eps, silu, pre_bias, post_add, post_rows, io_dtype,
                                (hipStream_t)stream);
@@ -262,6 +275,7 @@ int vig_layernorm_fwd(const void* x, const float* weight, const float* bias, voi
 int vig_split_heads_fwd(const void* qkv, void* q, void* k, void* v, int B, int L, int H, int Dk, int Dv,
                         long long qkv_row_stride, int io_dtype, void* stream) {
   if (!qkv || !q || !k || !v || B <= 0 || L <= 0 || H <= 0 || Dk <= 0 || Dv <= 0) return VIG_EINVAL;
+  if (!aligned16(q, k, v)) return VIG_EINVAL;
   if (!dtype_ok(io_dtype) || (Dk % 8) != 0 || (Dv % 8) != 0 || B > 65535) return VIG_ENOTSUP;
   const long long packed = (long long)H * (2 * Dk + Dv);
   const long long ld = qkv_row_stride > 0 ? qkv_row_stride : packed;
@@ -289,6 +303,7 @@ int vig_linear_swiglu_fwd(const void* x, const void* weight, void* y, long long 
 
 int vig_swiglu_fwd(const void* gate_up, void* out, long long rows, int I, int io_dtype, void* stream) {
   if (!gate_up || !out || rows <= 0 || I <= 0) return VIG_EINVAL;
+  if (!aligned16(gate_up, out)) return VIG_EINVAL;
   if (!dtype_ok(io_dtype) || (I % 8) != 0) return VIG_ENOTSUP;
   return vig::launch_swiglu(gate_up, out, rows, I, io_dtype, (hipStream_t)stream);
 }
@@ -309,6 +324,7 @@ static int gla_bidir_bwd(const void* q, const void* k, const void* v, const void
   if (!q || !k || !v || !g_fwd || !d_o || !dq || !dk || !dv || !dg_fwd || (g_bwd && !dg_bwd) || B <= 0 || H <= 0 ||
       L <= 0)
     return VIG_EINVAL;
+  if (!aligned16(q, k, v, g_fwd, g_bwd, d_o, dq, dk, dv, dg_fwd, dg_bwd, workspace)) return VIG_EINVAL;
   if (!dtype_ok(io_dtype) || !dtype_ok(gate_dtype) || !bwd_shape_ok(Dk, Dv)) return VIG_ENOTSUP;
   const size_t need = vig::gla_backward_workspace(B, H, L, Dk, Dv, g_bwd != nullptr);
   if (!workspace || workspace_bytes < need) return VIG_ENOSPC;

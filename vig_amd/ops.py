@@ -31,6 +31,13 @@ def _dt(t: torch.Tensor) -> int:
         raise TypeError(f"unsupported dtype {t.dtype}; float32 and bfloat16 are built") from None
 
 
+def _dense(t: torch.Tensor) -> torch.Tensor:
+    """t contiguous and on a 16-byte boundary (the kernels move 16 bytes per access and the library refuses
+    anything else): a view that starts in mid-row of its storage is copied."""
+    t = t.contiguous()
+    return t if t.data_ptr() % 16 == 0 else t.clone()
+
+
 def _check_cuda(*ts):
     for t in ts:
         if t is None:
@@ -71,9 +78,9 @@ def gla_bidir_backward(q, k, v, g_fwd, g_bwd, d_o, scale: float = -1, out_scale:
     """
     lib = _lib.load()
     _check_cuda(q, k, v, g_fwd, g_bwd, d_o)
-    q, k, v, g_fwd, d_o = (t.contiguous() for t in (q, k, v, g_fwd, d_o))
+    q, k, v, g_fwd, d_o = (_dense(t) for t in (q, k, v, g_fwd, d_o))
     if g_bwd is not None:
-        g_bwd = g_bwd.contiguous()
+        g_bwd = _dense(g_bwd)
     B, H, L, Dk = q.shape
     Dv = v.shape[-1]
     if d_o.shape != v.shape or d_o.dtype != q.dtype:
@@ -118,9 +125,9 @@ class _GLABidirFunction(torch.autograd.Function):
 def _gla_bidir_forward_raw(q, k, v, g_fwd, g_bwd, scale, out_scale, exact, out, strong_gates=False):
     lib = _lib.load()
     _check_cuda(q, k, v, g_fwd, g_bwd)
-    q, k, v, g_fwd = (t.contiguous() for t in (q, k, v, g_fwd))
+    q, k, v, g_fwd = (_dense(t) for t in (q, k, v, g_fwd))
     if g_bwd is not None:
-        g_bwd = g_bwd.contiguous()
+        g_bwd = _dense(g_bwd)
         if g_bwd.dtype != g_fwd.dtype or g_bwd.shape != g_fwd.shape:
             raise ValueError("g_bwd must match g_fwd in dtype and shape")
     B, H, L, Dk = q.shape
@@ -134,7 +141,8 @@ def _gla_bidir_forward_raw(q, k, v, g_fwd, g_bwd, scale, out_scale, exact, out, 
     io_dt, g_dt = _dt(q), _dt(g_fwd)
     if out is None:
         out = torch.empty(B, H, L, Dv, dtype=q.dtype, device=q.device)
-    elif not (out.is_contiguous() and out.shape == (B, H, L, Dv) and out.dtype == q.dtype):
+    elif not (out.is_contiguous() and out.data_ptr() % 16 == 0 and out.shape == (B, H, L, Dv)
+              and out.dtype == q.dtype):
         raise ValueError("bad `out` tensor")
     fn = lib.vig_gla_bidir_fwd_exact if exact else (lib.vig_gla_bidir_fwd_wide if strong_gates else lib.vig_gla_bidir_fwd)
     ws_bytes = lib.vig_gla_bidir_fwd_workspace(B, H, L, Dk, Dv, io_dt)
@@ -214,7 +222,7 @@ def dirgate(gk_lin: torch.Tensor, num_heads: int, gate_logit_normalizer: float =
     """gk_lin [B,L,2*H*Dk] -> [2,B,H,L,Dk] = logsigmoid/normalizer (vig.py:432-441)."""
     lib = _lib.load()
     _check_cuda(gk_lin)
-    gk_lin = gk_lin.contiguous()
+    gk_lin = _dense(gk_lin)
     B, L, C2 = gk_lin.shape
     Dk = C2 // (2 * num_heads)
     out_dtype = out_dtype or gk_lin.dtype
@@ -241,7 +249,7 @@ def dirgate_lowrank(gk_low: torch.Tensor, w_up: torch.Tensor, b_up: torch.Tensor
     _check_cuda(gk_low, w_up, b_up)
     gk_low, ld = _token_rows(gk_low)
     B, L, R = gk_low.shape
-    w_up, b_up = w_up.detach().contiguous(), b_up.detach().contiguous()
+    w_up, b_up = _dense(w_up.detach()), _dense(b_up.detach())
     C2 = w_up.shape[0]
     if w_up.shape != (C2, R) or b_up.shape != (C2,) or C2 % (2 * num_heads):
         raise ValueError("w_up must be [2*H*Dk, rank] and b_up [2*H*Dk]")
@@ -264,13 +272,13 @@ def dwconv3x3(x: torch.Tensor, weight: torch.Tensor, hw, bias: Optional[torch.Te
     """x [B,L,C] on the (h,w) token grid; weight [C,1,3,3] or [C,3,3]; returns [B,L,C]."""
     lib = _lib.load()
     _check_cuda(x, weight, bias)
-    x = x.contiguous()
+    x = _dense(x)
     B, L, C = x.shape
     h, w = hw
     if L != h * w:
         raise ValueError("L must equal h*w")
-    wt = weight.detach().reshape(C, 9).float().contiguous()
-    bs = bias.detach().float().contiguous() if bias is not None else None
+    wt = _dense(weight.detach().reshape(C, 9).float())
+    bs = _dense(bias.detach().float()) if bias is not None else None
     y = torch.empty_like(x)
     with torch.cuda.device(x.device):
         rc = lib.vig_dwconv3x3_fwd(x.data_ptr(), wt.data_ptr(), bs.data_ptr() if bs is not None else None,
@@ -283,12 +291,12 @@ def locality_gate(o: torch.Tensor, weight: torch.Tensor, hw) -> torch.Tensor:
     """y = o * sigmoid(dwconv3x3(o)) on [B,H,L,Dv] with channel = head*Dv + d."""
     lib = _lib.load()
     _check_cuda(o, weight)
-    o = o.contiguous()
+    o = _dense(o)
     B, H, L, Dv = o.shape
     h, w = hw
     if L != h * w:
         raise ValueError("L must equal h*w")
-    wt = weight.detach().reshape(H * Dv, 9).float().contiguous()
+    wt = _dense(weight.detach().reshape(H * Dv, 9).float())
     y = torch.empty_like(o)
     with torch.cuda.device(o.device):
         rc = lib.vig_locality_gate_fwd(o.data_ptr(), wt.data_ptr(), y.data_ptr(), B, H, h, w, Dv, _dt(o),
@@ -317,12 +325,12 @@ def gla_bidir_locality_gate(q, k, v, g_fwd, g_bwd, weight: torch.Tensor, hw, sca
                and Dv == 64 and L <= 256 and w + 2 <= 64 and h + 2 <= 8 * (64 // (w + 2)))
     if not fusable:
         return locality_gate(gla_bidir_forward(q, k, v, g_fwd, g_bwd, scale, out_scale), weight, hw)
-    q, k, v, g_fwd, g_bwd = (t.detach().contiguous() for t in (q, k, v, g_fwd, g_bwd))
+    q, k, v, g_fwd, g_bwd = (_dense(t.detach()) for t in (q, k, v, g_fwd, g_bwd))
     if k.shape != q.shape or g_fwd.shape != q.shape or g_bwd.shape != q.shape or v.shape[:3] != q.shape[:3]:
         raise ValueError("shape mismatch between q, k, v, g")
     if k.dtype != q.dtype or v.dtype != q.dtype or g_bwd.dtype != g_fwd.dtype:
         raise TypeError("q, k, v must share a dtype, and so must the gates")
-    wt = weight.detach().reshape(H * Dv, 9).float().contiguous()
+    wt = _dense(weight.detach().reshape(H * Dv, 9).float())
     y = torch.empty(B, H, L, Dv, dtype=q.dtype, device=q.device)
     with torch.cuda.device(q.device):
         rc = lib.vig_gla_bidir_locgate_fwd(q.data_ptr(), k.data_ptr(), v.data_ptr(), g_fwd.data_ptr(),
@@ -340,7 +348,7 @@ def _token_rows(t: torch.Tensor):
         sb, sl, sc = t.stride()
         if sc == 1 and sl >= C and sb == L * sl and (sl * t.element_size()) % 16 == 0 and t.data_ptr() % 16 == 0:
             return t, sl
-    t = t.contiguous()
+    t = _dense(t)
     return t, t.shape[-1]
 
 
@@ -350,7 +358,7 @@ def locality_blend(o: torch.Tensor, local: torch.Tensor, g_lin: torch.Tensor, w_
     g_lin may be a block of columns of a wider [B, L, W] tensor (it is read in place)."""
     lib = _lib.load()
     _check_cuda(o, local, g_lin, w_g, w_l)
-    o, local = o.contiguous(), local.contiguous()
+    o, local = _dense(o), _dense(local)
     g_lin, ldg = _token_rows(g_lin)
     B, H, L, Dv = o.shape
     if local.shape != (B, L, H * Dv) or g_lin.shape != (B, L, H * Dv):
@@ -358,8 +366,8 @@ def locality_blend(o: torch.Tensor, local: torch.Tensor, g_lin: torch.Tensor, w_
     if local.dtype != o.dtype or g_lin.dtype != o.dtype:
         raise TypeError("o, local, g_lin must share a dtype")
     y = torch.empty_like(local)
-    wg = w_g.detach().float().contiguous()
-    wl = w_l.detach().float().contiguous()
+    wg = _dense(w_g.detach().float())
+    wl = _dense(w_l.detach().float())
     with torch.cuda.device(o.device):
         rc = lib.vig_locality_blend_fwd(o.data_ptr(), local.data_ptr(), g_lin.data_ptr(), wg.data_ptr(),
                                         wl.data_ptr(), y.data_ptr(), B, H, L, Dv, ldg, float(eps), int(silu_out),
@@ -377,17 +385,16 @@ def rmsnorm(x: torch.Tensor, weight: torch.Tensor, eps: float = 1e-6, residual: 
     """
     lib = _lib.load()
     _check_cuda(x, weight)
-    x = x.contiguous()
+    x = _dense(x)
     C = x.shape[-1]
     rows = x.numel() // C
     if residual is not None:
         _check_cuda(residual)
-        residual = residual.contiguous()
+        residual = _dense(residual)
         if residual.shape != x.shape or residual.dtype != x.dtype:
             raise ValueError("residual must match x in shape and dtype")
     w = weight.detach()
-    if w.dtype != torch.float32 or not w.is_contiguous():
-        w = w.float().contiguous()
+    w = _dense(w.float())
     y = torch.empty_like(x)
     res_out = torch.empty_like(x) if (prenorm and residual is not None) else None
     with torch.cuda.device(x.device):
@@ -409,21 +416,21 @@ def layernorm(x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor, eps: fl
     result row-periodically (the position table, vig.py:858-865)."""
     lib = _lib.load()
     _check_cuda(x, weight, bias, pre_bias, post_add)
-    x = x.contiguous()
+    x = _dense(x)
     C = x.shape[-1]
     rows = x.numel() // C
-    w = weight.detach().float().contiguous()
-    b = bias.detach().float().contiguous()
+    w = _dense(weight.detach().float())
+    b = _dense(bias.detach().float())
     if w.shape != (C,) or b.shape != (C,):
         raise ValueError("weight and bias must be [C]")
     pb = None
     if pre_bias is not None:
-        pb = pre_bias.detach().float().contiguous()
+        pb = _dense(pre_bias.detach().float())
         if pb.shape != (C,):
             raise ValueError("pre_bias must be [C]")
     pa, prow = None, 0
     if post_add is not None:
-        pa = post_add.detach().reshape(-1, C).contiguous()
+        pa = _dense(post_add.detach().reshape(-1, C))
         prow = pa.shape[0]
         if pa.dtype != x.dtype or rows % prow:
             raise ValueError("post_add must have x's dtype and a row count that divides x's")
@@ -477,11 +484,12 @@ def patch_conv(x: torch.Tensor, w_packed: torch.Tensor, kernel_hw, stride: int =
     w_packed from pack_patch_conv_weight."""
     lib = _lib.load()
     _check_cuda(x, w_packed)
-    x = x.contiguous()
+    x = _dense(x)
     B, Cin, H, W = x.shape
     KH, KW = kernel_hw
     Cout = w_packed.shape[0]
-    if w_packed.shape != (Cout, Cin * KH, 16) or w_packed.dtype != x.dtype or not w_packed.is_contiguous():
+    if (w_packed.shape != (Cout, Cin * KH, 16) or w_packed.dtype != x.dtype or not w_packed.is_contiguous()
+            or w_packed.data_ptr() % 16):
         raise ValueError("w_packed must be the contiguous [Cout, Cin*KH, 16] tensor of pack_patch_conv_weight, in x's dtype")
     OH, OW = (H + 2 * padding - KH) // stride + 1, (W + 2 * padding - KW) // stride + 1
     y = torch.empty(B, OH, OW, Cout, dtype=x.dtype, device=x.device)
@@ -503,8 +511,8 @@ def linear_swiglu(x: torch.Tensor, weight: torch.Tensor) -> torch.Tensor:
     (vig.py:492-495) in one kernel, no [.., 2*I] intermediate."""
     lib = _lib.load()
     _check_cuda(x, weight)
-    x = x.contiguous()
-    w = weight.detach().contiguous()
+    x = _dense(x)
+    w = _dense(weight.detach())
     K, I = w.shape[1], w.shape[0] // 2
     y = torch.empty(*x.shape[:-1], I, dtype=x.dtype, device=x.device)
     with torch.cuda.device(x.device):
@@ -518,7 +526,7 @@ def swiglu(gate_up: torch.Tensor) -> torch.Tensor:
     """gate_up [..., 2*I] = (gate | up) -> gate * up / (1 + exp(-gate))  (fla/modules/activations.py:109-113)."""
     lib = _lib.load()
     _check_cuda(gate_up)
-    gate_up = gate_up.contiguous()
+    gate_up = _dense(gate_up)
     I = gate_up.shape[-1] // 2
     rows = gate_up.numel() // (2 * I)
     out = torch.empty(*gate_up.shape[:-1], I, dtype=gate_up.dtype, device=gate_up.device)
