@@ -30,10 +30,27 @@ def _ln2d(x, w, b, eps=1e-5):
     return F.layer_norm(x.permute(0, 2, 3, 1), (x.shape[1],), w, b, eps).permute(0, 3, 1, 2)
 
 
+def bidir_gla_torch(q, k, v, gf, gb, scale=None, out_scale=1.0):
+    """The bidirectional GLA as its unrolled double sum (the closed form of naive.py:33-41,48-56), in differentiable
+    torch operations: autograd through it gives the gradients the training path is checked against.  [B, H, L, D]
+    float64 tensors, moderate gate sums only (the decays are factored as e^{G_i} e^{-G_j}).  The forward is pinned
+    against the token recurrence in tests/test_oracle.py."""
+    L = q.shape[2]
+    scale = q.shape[-1] ** -0.5 if scale is None else scale
+    G = torch.cumsum(gf, dim=2)                                  # inclusive prefix sums: decay j -> i (j <= i) = G_i - G_j
+    Hs = torch.flip(torch.cumsum(torch.flip(gb, [2]), 2), [2])   # inclusive suffix sums: decay j -> i (j >= i) = H_i - H_j
+    lower = torch.tril(torch.ones(L, L, dtype=q.dtype))
+    a_f = torch.einsum("bhid,bhjd->bhij", q * torch.exp(G), k * torch.exp(-G)) * lower
+    a_b = torch.einsum("bhid,bhjd->bhij", q * torch.exp(Hs), k * torch.exp(-Hs)) * lower.T
+    return out_scale * scale * torch.einsum("bhij,bhjd->bhid", a_f + a_b, v)
+
+
 def gla_block_attn(sd, pre, x, hw, num_heads, eps=1e-6, act_in_conv=False, out_act=False, normalizer=16.0,
-                   second_halving=True):
+                   second_halving=True, differentiable=False):
     """Eval-mode GatedLinearAttention.forward on x [B, L, C] (float64).  second_halving=False gives HierViG's
-    GLA2D (classification/models/vig_h.py:536-606), whose `o /= 2` after the op is commented out (:579)."""
+    GLA2D (classification/models/vig_h.py:536-606), whose `o /= 2` after the op is commented out (:579), and the
+    training branch (vig.py:425-426: one average of the two directions).  differentiable=True runs the GLA as
+    bidir_gla_torch, so that autograd reaches x and the parameters."""
     B, L, C = x.shape
     h, w = hw
     x2 = x.reshape(B, h, w, C).permute(0, 3, 1, 2)
@@ -52,9 +69,12 @@ def gla_block_attn(sd, pre, x, hw, num_heads, eps=1e-6, act_in_conv=False, out_a
     heads = lambda t: t.reshape(B, L, H, -1).permute(0, 2, 1, 3)
     gf = F.logsigmoid(heads(fw)) / normalizer
     gb = F.logsigmoid(heads(bw)) / normalizer
-    o = O.bidir_gla_recurrent(heads(q).numpy(), heads(k).numpy(), heads(v).numpy(), gf.numpy(), gb.numpy(),
-                              out_scale=0.5)
-    o = torch.from_numpy(o)
+    if differentiable:
+        o = bidir_gla_torch(heads(q), heads(k), heads(v), gf, gb, out_scale=0.5)
+    else:
+        o = O.bidir_gla_recurrent(heads(q).numpy(), heads(k).numpy(), heads(v).numpy(), gf.numpy(), gb.numpy(),
+                                  out_scale=0.5)
+        o = torch.from_numpy(o)
     if second_halving:
         o = o / 2  # the second halving of the eval path (vig.py:443)
     o = o.permute(0, 2, 1, 3)  # b l h d
@@ -69,9 +89,11 @@ def gla_block_attn(sd, pre, x, hw, num_heads, eps=1e-6, act_in_conv=False, out_a
     return y @ sd[pre + "o_proj.weight"].T
 
 
-def vig_forward(state_dict, images, num_heads, depth, eps=1e-6, act_in_conv=False, out_act=False):
-    """Logits [B, num_classes] of the eval-mode ViG (v2 patch embedding, no class token, avgpool head)."""
-    sd = {k: v.detach().double().cpu() for k, v in state_dict.items()}
+def vig_forward(state_dict, images, num_heads, depth, eps=1e-6, act_in_conv=False, out_act=False, train=False):
+    """Logits [B, num_classes] of the eval-mode ViG (v2 patch embedding, no class token, avgpool head).
+    train=True follows the training branch instead (directions averaged once) and stays differentiable: the caller
+    passes float64 CPU leaf tensors and reads their .grad after a backward."""
+    sd = state_dict if train else {k: v.detach().double().cpu() for k, v in state_dict.items()}
     x = images.double().cpu()
     pe = "patch_embed.proj."
     x = F.conv2d(x, sd[pe + "0.weight"], sd.get(pe + "0.bias"), stride=sd[pe + "0.weight"].shape[-1] - 1, padding=1)
@@ -85,7 +107,8 @@ def vig_forward(state_dict, images, num_heads, depth, eps=1e-6, act_in_conv=Fals
         p = f"blocks.{i}."
         residual = x
         hsn = _rms(x, sd[p + "attn_norm.weight"], eps)
-        a = gla_block_attn(sd, p + "attn.", hsn, hw, num_heads, eps, act_in_conv, out_act)
+        a = gla_block_attn(sd, p + "attn.", hsn, hw, num_heads, eps, act_in_conv, out_act,
+                           second_halving=not train, differentiable=train)
         residual = a + residual
         hn = _rms(residual, sd[p + "mlp_norm.weight"], eps)
         gate, y = (hn @ sd[p + "mlp.gate_proj.weight"].T).chunk(2, -1)

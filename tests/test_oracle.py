@@ -295,3 +295,25 @@ def test_backward_against_finite_differences_and_autograd():
     (out * torch.tensor(do)).sum().backward()
     for grad, t in zip((dq, dk, dv, dgf, dgb), (tq, tk, tv, tgf, tgb)):
         np.testing.assert_allclose(grad, t.grad.numpy(), rtol=1e-10, atol=1e-12)
+
+
+def test_differentiable_model_restatement_gla():
+    """The torch double-sum GLA used by the differentiable block restatement: forward against the pinned token
+    recurrence, gradients against the pinned adjoint recurrences."""
+    import torch
+
+    from oracle import vig_model_ref as R
+
+    rng = np.random.default_rng(5)
+    B, H, L, Dk, Dv = 2, 2, 11, 4, 3
+    q, k = rng.standard_normal((B, H, L, Dk)), rng.standard_normal((B, H, L, Dk))
+    v, do = rng.standard_normal((B, H, L, Dv)), rng.standard_normal((B, H, L, Dv))
+    gf = -np.abs(rng.standard_normal((B, H, L, Dk))) * 0.3
+    gb = -np.abs(rng.standard_normal((B, H, L, Dk))) * 0.3
+    ts = [torch.tensor(a, requires_grad=True) for a in (q, k, v, gf, gb)]
+    out = R.bidir_gla_torch(*ts, out_scale=0.5)
+    np.testing.assert_allclose(out.detach().numpy(), O.bidir_gla_recurrent(q, k, v, gf, gb, out_scale=0.5),
+                               rtol=1e-11, atol=1e-12)
+    (out * torch.tensor(do)).sum().backward()
+    for want, t in zip(O.bidir_gla_backward(q, k, v, gf, gb, do, out_scale=0.5), ts):
+        np.testing.assert_allclose(t.grad.numpy(), want, rtol=1e-9, atol=1e-11)

@@ -1,0 +1,124 @@
+"""The differentiable (training-mode) path of the block and the model: outputs against the kernel path, gradients
+against autograd through the float64 CPU restatement (whose GLA is pinned in tests/test_oracle.py)."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import vig_model_ref as R
+from vig_amd import layers
+
+from .util import announce
+
+pytestmark = pytest.mark.gpu
+
+VARIANTS = {
+    # name: (d_model, heads, block options) -- head shapes Dk 32 / Dv 64 and Dk 16 / Dv 32
+    "s": (128, 2, dict(use_act_in_conv=False, use_out_act=False)),
+    "t": (96, 3, dict(use_act_in_conv=True, use_out_act=True)),
+}
+
+
+def _block(variant):
+    dim, H, kw = VARIANTS[variant]
+    torch.manual_seed(0)
+    m = layers.GatedLinearAttention(d_model=dim, expand_k=0.5, expand_v=1.0, num_heads=H, layernorm_eps=1e-6, **kw)
+    with torch.no_grad():
+        m.g_norm.weight.uniform_(0.5, 1.5)
+        m.l_norm.weight.uniform_(0.5, 1.5)
+        m.g_proj.bias.normal_(0, 0.5)
+        m.gk_proj[1].bias.normal_(0, 1.0)
+        for lin in (m.qkv_proj, m.g_proj, m.o_proj, m.gk_proj[0], m.gk_proj[1]):
+            lin.weight.mul_(8.0)  # the 2^-2.5 init makes everything tiny
+    return m, dim, H, kw
+
+
+def _rel(a, b):
+    a, b = np.asarray(a, dtype=np.float64), np.asarray(b, dtype=np.float64)
+    return np.abs(a - b).max() / max(np.abs(b).max(), 1e-30)
+
+
+@pytest.mark.parametrize("dtype,tol", [(torch.float32, 2e-4), (torch.bfloat16, 6e-2)])
+@pytest.mark.parametrize("variant", ["s", "t"])
+def test_training_forward_matches_kernel_forward(dtype, tol, variant):
+    announce(f"GatedLinearAttention train-mode forward, autograd path against kernel path, {variant}, {dtype}")
+    m, dim, H, kw = _block(variant)
+    m = m.to("cuda", dtype).train()
+    x = torch.randn(2, 49, dim, device="cuda", dtype=dtype)
+    y_graph = m(x, patch_resolution=(7, 7), token_position=None)
+    assert y_graph.requires_grad
+    with torch.no_grad():
+        y_kernel = m(x, patch_resolution=(7, 7), token_position=None)  # the library's kernels, training scale
+    assert not y_kernel.requires_grad
+    err = _rel(y_graph.detach().double().cpu(), y_kernel.double().cpu())
+    print(f"  max-rel difference {err:.3e}", flush=True)
+    assert err <= tol
+
+
+@pytest.mark.parametrize("dtype,tol", [(torch.float32, 2e-4), (torch.bfloat16, 8e-2)])
+@pytest.mark.parametrize("variant", ["s", "t"])
+def test_block_gradients(dtype, tol, variant):
+    announce(f"GatedLinearAttention gradients against the float64 restatement, {variant}, {dtype}")
+    m, dim, H, kw = _block(variant)
+    x = torch.randn(2, 49, dim)
+    cot = torch.randn(2, 49, dim)
+    sd = {k: v.detach().double().requires_grad_() for k, v in m.state_dict().items()}
+    x64 = x.double().requires_grad_()
+    want = R.gla_block_attn(sd, "", x64, (7, 7), H, 1e-6, kw["use_act_in_conv"], kw["use_out_act"],
+                            second_halving=False, differentiable=True)
+    (want * cot.double()).sum().backward()
+
+    md = m.to("cuda", dtype).train()
+    xg = x.to("cuda", dtype).requires_grad_()
+    got = md(xg, patch_resolution=(7, 7), token_position=None)
+    (got.float() * cot.cuda()).sum().backward()
+    err = _rel(got.detach().double().cpu(), want.detach())
+    print(f"  forward max-rel err {err:.3e}", flush=True)
+    assert err <= tol
+    worst = ("x", _rel(xg.grad.double().cpu(), x64.grad))
+    for name, p in md.named_parameters():
+        assert p.grad is not None, name
+        e = _rel(p.grad.double().cpu(), sd[name].grad)
+        if e > worst[1]:
+            worst = (name, e)
+    print(f"  worst gradient max-rel err {worst[1]:.3e} ({worst[0]})", flush=True)
+    assert worst[1] <= tol, worst
+
+
+def test_vig_training_step():
+    """A small ViG in training mode: logits and every parameter's gradient against the float64 restatement of the
+    training branch, then one SGD step lowers the loss."""
+    announce("ViG (64x64 images, depth 2, dim 96) training step, fp32")
+    torch.manual_seed(0)
+    kw = dict(img_size=64, depth=2, num_heads=3, embed_dim=96, num_classes=10)
+    model = layers.ViG(**kw)
+    with torch.no_grad():
+        for blk in model.blocks:
+            for lin in (blk.attn.qkv_proj, blk.attn.g_proj, blk.attn.o_proj, blk.attn.gk_proj[0], blk.attn.gk_proj[1]):
+                lin.weight.mul_(8.0)
+    images = torch.randn(3, 3, 64, 64)
+    target = torch.tensor([1, 7, 4])
+    sd = {k: v.detach().double().requires_grad_() for k, v in model.state_dict().items()}
+    want = R.vig_forward(sd, images.double(), num_heads=3, depth=2, train=True)
+    torch.nn.functional.cross_entropy(want, target).backward()
+
+    model = model.cuda().train()
+    logits = model(images.cuda())
+    loss = torch.nn.functional.cross_entropy(logits, target.cuda())
+    loss.backward()
+    e = _rel(logits.detach().double().cpu(), want.detach())
+    print(f"  logits max-rel err {e:.3e}", flush=True)
+    assert e <= 5e-4
+    worst = ("", 0.0)
+    for name, p in model.named_parameters():
+        assert p.grad is not None and torch.isfinite(p.grad).all(), name
+        e = _rel(p.grad.double().cpu(), sd[name].grad)
+        if e > worst[1]:
+            worst = (name, e)
+    print(f"  worst gradient max-rel err {worst[1]:.3e} ({worst[0]})", flush=True)
+    assert worst[1] <= 2e-3, worst
+    with torch.no_grad():
+        for p in model.parameters():
+            p -= 0.05 * p.grad
+    after = torch.nn.functional.cross_entropy(model(images.cuda()), target.cuda())
+    print(f"  loss {loss.item():.4f} -> {after.item():.4f}", flush=True)
+    assert after.item() < loss.item()

@@ -15,7 +15,12 @@ The surrounding ViG shell (patch embedding, MLP GEMMs, head) is plain torch and 
 vig.py:469-497,530-618,625-672,705-912 for the options the shipped configs use.  There is no CPU path: every
 library op raises on tensors that are not on the GPU.
 
-Forward (inference) only: the HIP ops carry no autograd graph.
+Two ways through every module.  In eval mode, or whenever gradients are not being recorded, the forward runs on the
+library's kernels and leaves no autograd graph.  In training mode with gradients enabled (`model.train()` outside
+`torch.no_grad()`) the same arithmetic is written in differentiable torch operations around the one op the training
+path spends its time in, the bidirectional GLA, whose forward and backward both run on the library's kernels
+(vig_gla_bidir_fwd / vig_gla_bidir_bwd through ops.gla_bidir_forward) -- the reference's training branch
+(vig.py:354-426) with the flips and concatenations folded into the op.
 """
 from __future__ import annotations
 
@@ -43,6 +48,11 @@ def _f32(owner: nn.Module, tag: str, t: Optional[torch.Tensor], shape=None):
     return hit[1]
 
 
+def _recording(module: nn.Module) -> bool:
+    """True when this call has to leave an autograd graph: training mode with gradients enabled."""
+    return module.training and torch.is_grad_enabled()
+
+
 class RMSNorm(nn.Module):
     """x * rsqrt(mean(x^2) + eps) * weight, arithmetic in fp32 (fla/modules/rmsnorm.py:38-52,491-512).
 
@@ -65,7 +75,20 @@ class RMSNorm(nn.Module):
         return self._w32_cache
 
     def forward(self, x, residual=None, prenorm: bool = False, round_sum: bool = False):
+        if _recording(self):
+            return self._forward_autograd(x, residual, prenorm, round_sum)
         return ops.rmsnorm(x, self._w32(), self.eps, residual=residual, prenorm=prenorm, round_sum=round_sum)
+
+    def _forward_autograd(self, x, residual, prenorm, round_sum):
+        """The kernel's arithmetic in differentiable torch operations: sum and norm in fp32, results in x's dtype."""
+        s, res_out = x.float(), x
+        if residual is not None:
+            s = s + residual.float()
+            res_out = s.to(x.dtype)
+            if round_sum:
+                s = res_out.float()
+        y = (s * torch.rsqrt(s.pow(2).mean(-1, keepdim=True) + self.eps) * self.weight.float()).to(x.dtype)
+        return (y, res_out) if prenorm else y
 
 
 class GatedLinearAttention(nn.Module):
@@ -166,13 +189,46 @@ class GatedLinearAttention(nn.Module):
                                eps=self.layernorm_eps, silu_out=self.use_out_act)
         return self.o_proj(y)
 
-    @torch.no_grad()
+    def _mix_autograd(self, x, hw, out_scale):
+        """_mix in differentiable torch operations around the differentiable GLA op (the reference's training branch,
+        vig.py:354-426,444-463: its flipped copies of q, k, v and of the backward gates are what the op's second
+        direction reads in place)."""
+        B, L, C = x.shape
+        H, Dv = self.num_heads, self.head_v_dim
+        local = self.in_proj(x.reshape(B, hw[0], hw[1], C).permute(0, 3, 1, 2))  # conv (+ SiLU), [B, C, h, w]
+        xs = local.flatten(2).transpose(1, 2)
+        q, k, v = torch.split(self.qkv_proj(xs), [self.key_dim, self.key_dim, self.value_dim], dim=2)
+
+        def heads(t):
+            return t.reshape(B, L, H, -1).transpose(1, 2)
+
+        def gate(t):
+            g = F.logsigmoid(heads(t).float()) / self.gate_logit_normalizer
+            if self.clamp_min is not None:
+                g = torch.clamp_min(g, self.clamp_min)
+            return g.to(q.dtype)
+
+        g_fwd, g_bwd = self.gk_proj(xs).chunk(2, dim=2)
+        o = ops.gla_bidir_forward(heads(q), heads(k), heads(v), gate(g_fwd), gate(g_bwd), scale=-1,
+                                  out_scale=out_scale)
+        o = self.g_norm(o.transpose(1, 2))  # [B, L, H, Dv]
+        loc = self.l_norm(xs.reshape(B, L, H, Dv))
+        g = torch.sigmoid(self.g_proj(xs)).reshape(B, L, H, Dv)
+        y = (o * g + loc * (1 - g)).reshape(B, L, H * Dv)
+        if self.use_out_act:
+            y = F.silu(y)
+        return self.o_proj(y)
+
     def forward(self, x, lower_bound=0, **kwargs):
         if kwargs.get("token_position", None) is not None:
             raise NotImplementedError("class-token splicing is not built (the shipped configs use IF_CLS_TOKEN False)")
         # training glue averages the directions (vig.py:425-426); the eval path halves twice
         # (recurrent_fuse.py:442, then vig.py:443)
-        return self._mix(x, tuple(kwargs["patch_resolution"]), 0.5 if self.training else 0.25)
+        hw = tuple(kwargs["patch_resolution"])
+        if _recording(self):
+            return self._mix_autograd(x, hw, 0.5)
+        with torch.no_grad():
+            return self._mix(x, hw, 0.5 if self.training else 0.25)
 
 
 class GLA2D(GatedLinearAttention):
@@ -194,14 +250,17 @@ class GLA2D(GatedLinearAttention):
         self.channel_first = channel_first
         self.d_group = 2
 
-    @torch.no_grad()
     def forward(self, x, **kwargs):
         if self.channel_first:
             B, C, H, W = x.shape
             x = x.permute(0, 2, 3, 1)
         else:
             B, H, W, C = x.shape
-        y = self._mix(x.reshape(B, H * W, C), (H, W), 0.5)
+        if _recording(self):
+            y = self._mix_autograd(x.reshape(B, H * W, C), (H, W), 0.5)
+        else:
+            with torch.no_grad():
+                y = self._mix(x.reshape(B, H * W, C), (H, W), 0.5)
         if self.channel_first:
             return y.permute(0, 2, 1).reshape(B, -1, H, W)
         return y.reshape(B, H, W, -1)
@@ -223,6 +282,9 @@ class GLAMLP(nn.Module):
         self.down_proj = nn.Linear(intermediate_size, hidden_size, bias=False)
 
     def forward(self, x):
+        if _recording(self):
+            gate, y = self.gate_proj(x).chunk(2, -1)
+            return self.down_proj(F.silu(gate) * y)
         w = self.gate_proj.weight
         if ops.linear_swiglu_supported(x, w):  # ViG-S / ViG-T widths in bf16: no [.., 2*I] intermediate
             return self.down_proj(ops.linear_swiglu(x, w))
@@ -268,6 +330,15 @@ class LayerNorm2d(nn.LayerNorm):
 
     def forward(self, x, silu: bool = False, pre_bias=None, post_add=None):
         rows = x.permute(0, 2, 3, 1)  # a view; contiguous when x is channels-last
+        if _recording(self):
+            if pre_bias is not None:
+                rows = rows + pre_bias.to(rows.dtype)
+            y = F.layer_norm(rows, (rows.shape[-1],), self.weight, self.bias, self.eps)
+            if silu:
+                y = F.silu(y)
+            if post_add is not None:
+                y = (y.flatten(1, 2) + post_add).reshape(y.shape)
+            return y.permute(0, 3, 1, 2)
         return ops.layernorm(rows, _f32(self, "w", self.weight), _f32(self, "b", self.bias), self.eps, silu=silu,
                              pre_bias=pre_bias, post_add=post_add).permute(0, 3, 1, 2)
 
@@ -291,6 +362,13 @@ class V2PatchEmbed(nn.Module):
         inside the last norm's kernel."""
         # channels-last throughout: the convolutions run in that layout, the norms see row matrices, and the final
         # 'b c h w -> b (h w) c' is a view; each convolution's bias add rides in the norm kernel behind it
+        if _recording(self):  # plain modules, differentiable (LayerNorm2d and the convolutions record their graph)
+            x = self.proj(x)
+            hw = tuple(x.shape[-2:])
+            x = x.flatten(2).transpose(1, 2)
+            if pos_embed is not None:
+                x = x + resize_pos_embed(pos_embed, pos_shape, hw).to(x.dtype)
+            return x, hw
         conv1, norm1, act, conv2, norm2 = self.proj
         if (conv1.stride[0] == conv1.stride[1] and conv1.padding[0] == conv1.padding[1] and conv1.groups == 1
                 and conv1.dilation == (1, 1)
@@ -373,9 +451,11 @@ class ViG(nn.Module):
         x = self.norm(branch, residual, round_sum=True) if residual is not None else self.norm(branch)
         return x.reshape(B, hw[0] * hw[1], -1).mean(dim=1)
 
-    @torch.no_grad()
     def forward(self, x):
-        return self.head(self.forward_features(x))
+        if _recording(self):
+            return self.head(self.forward_features(x))
+        with torch.no_grad():
+            return self.head(self.forward_features(x))
 
 
 def vig_small(**kw):
