@@ -119,6 +119,43 @@ def model_throughput(dev, batch=256, warmup=10, iters=30, tune_gemm=True, use_gr
     return out
 
 
+def train_step_throughput(dev, batch=128, warmup=3, iters=10):
+    """ViG-S training steps (forward, cross-entropy, backward, AdamW update) on synthetic images: the differentiable
+    path of the shell, whose GLA forward and backward run on the library's kernels.  fp32 as the reference's configs
+    train (vig-s.yaml: AMP off), and bf16 autocast."""
+    import torch
+
+    from vig_amd import layers
+
+    out = {"batch": batch, "iters": iters}
+    images = torch.randn(batch, 3, 224, 224, device=dev)
+    target = torch.randint(0, 1000, (batch,), device=dev)
+    for name, amp in (("fp32", False), ("bf16_autocast", True)):
+        torch.manual_seed(0)
+        model = layers.vig_small().to(dev).train()
+        opt = torch.optim.AdamW(model.parameters(), lr=1e-4)
+
+        def step():
+            opt.zero_grad(set_to_none=True)
+            with torch.autocast("cuda", dtype=torch.bfloat16, enabled=amp):
+                loss = torch.nn.functional.cross_entropy(model(images).float(), target)
+            loss.backward()
+            opt.step()
+            return loss
+
+        for _ in range(warmup):
+            step()
+        torch.cuda.synchronize(dev)
+        t0 = time.perf_counter()
+        for _ in range(iters):
+            loss = step()
+        torch.cuda.synchronize(dev)
+        dt = (time.perf_counter() - t0) / iters
+        out[name] = {"images_per_s": batch / dt, "ms_per_step": dt * 1e3, "loss": float(loss)}
+        del model, opt
+    return out
+
+
 def backward_time(lib, sets, s, io_dt, scale, sp, stream, dev, iters=60):
     """Event-bracketed time of vig_gla_bidir_bwd, rotating over the input sets like the forward loop does."""
     import torch
@@ -173,6 +210,8 @@ def main():
     ap.add_argument("--op-only", action="store_true", help="no model forward and no backward, whatever the workload")
     ap.add_argument("--no-gemm-tuning", action="store_true",
                     help="with --model: leave torch's GEMM solution tuning off (clean kernel traces)")
+    ap.add_argument("--train", action="store_true",
+                    help="also time ViG-S training steps (differentiable path of the shell; fp32 and bf16 autocast)")
     ap.add_argument("--no-graph", action="store_true",
                     help="with --model: eager forwards only (no HIP graph capture, no batch-16 latency)")
     ap.add_argument("--unfused-gate", action="store_true",
@@ -332,6 +371,8 @@ def main():
             except (OSError, ValueError):
                 out["backward"]["traffic"] = None
     if want_model:
+        if args.train:
+            out["vig_s_train_step"] = train_step_throughput(dev)
         out["vig_s_forward"] = model_throughput(dev, tune_gemm=not args.no_gemm_tuning, use_graph=not args.no_graph)
     if not args.no_cpu:
         out["cpu_baseline"] = cpu_baseline(s, 1000 + args.config)

@@ -199,3 +199,34 @@ def test_fused_locality_gate_other_shapes_take_two_calls():
     got = vig_amd.gla_bidir_locality_gate(*(t.cuda() for t in (q, k, v, gf, gb)), wt.cuda(), (7, 7))
     want = O.locality_sigmoid_gate_reference(oracle_bidir(q, k, v, gf, gb), f64(wt), (7, 7))
     assert max_abs(f64(got), want) <= 1e-4 * max(1.0, float(np.abs(want).max()))
+
+
+@pytest.mark.parametrize("silu", [False, True])
+@pytest.mark.parametrize("dtype,tol", [(torch.float32, 1e-5), (torch.bfloat16, 2e-2)])
+def test_dwconv3x3_gradients(dtype, tol, silu):
+    """Input, weight and bias gradients of the differentiable stencil op against autograd through torch's conv2d in
+    float64 (on the same rounded inputs)."""
+    announce(f"dwconv3x3 gradients {dtype} silu={silu}")
+    torch.manual_seed(3)
+    B, h, w, C = 3, 5, 7, 24
+    x = torch.randn(B, h * w, C).to(dtype)
+    wt = (torch.randn(C, 1, 3, 3) / 3).to(dtype)
+    bs = torch.randn(C).to(dtype)
+    cot = torch.randn(B, h * w, C)
+    x64, w64, b64 = (t.double().requires_grad_() for t in (x, wt, bs))
+    y64 = torch.nn.functional.conv2d(x64.reshape(B, h, w, C).permute(0, 3, 1, 2), w64, b64, padding=1, groups=C)
+    if silu:
+        y64 = torch.nn.functional.silu(y64)
+    y64 = y64.flatten(2).transpose(1, 2)
+    (y64 * cot.double()).sum().backward()
+    xg, wg, bg = (t.cuda().requires_grad_() for t in (x, wt, bs))
+    y = vig_amd.ops.dwconv3x3(xg, wg, (h, w), bias=bg, silu=silu)
+    (y.float() * cot.cuda()).sum().backward()
+
+    def rel(a, b):
+        return ((a.double().cpu() - b).abs().max() / b.abs().max()).item()
+
+    errs = dict(y=rel(y.detach(), y64.detach()), dx=rel(xg.grad, x64.grad), dw=rel(wg.grad, w64.grad),
+                db=rel(bg.grad, b64.grad))
+    print("  " + "  ".join(f"{k} {v:.2e}" for k, v in errs.items()), flush=True)
+    assert max(errs.values()) <= tol, errs

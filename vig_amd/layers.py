@@ -195,8 +195,10 @@ class GatedLinearAttention(nn.Module):
         direction reads in place)."""
         B, L, C = x.shape
         H, Dv = self.num_heads, self.head_v_dim
-        local = self.in_proj(x.reshape(B, hw[0], hw[1], C).permute(0, 3, 1, 2))  # conv (+ SiLU), [B, C, h, w]
-        xs = local.flatten(2).transpose(1, 2)
+        conv = self.in_proj[0]
+        if torch.is_autocast_enabled():  # what autocast would hand a convolution
+            x = x.to(torch.get_autocast_dtype("cuda"))
+        xs = ops.dwconv3x3(x, conv.weight, hw, bias=conv.bias, silu=self.use_act_in_conv)  # differentiable, [B, L, C]
         q, k, v = torch.split(self.qkv_proj(xs), [self.key_dim, self.key_dim, self.value_dim], dim=2)
 
         def heads(t):

@@ -269,7 +269,44 @@ def dirgate_lowrank(gk_low: torch.Tensor, w_up: torch.Tensor, b_up: torch.Tensor
 
 def dwconv3x3(x: torch.Tensor, weight: torch.Tensor, hw, bias: Optional[torch.Tensor] = None,
               silu: bool = False) -> torch.Tensor:
-    """x [B,L,C] on the (h,w) token grid; weight [C,1,3,3] or [C,3,3]; returns [B,L,C]."""
+    """x [B,L,C] on the (h,w) token grid; weight [C,1,3,3] or [C,3,3]; returns [B,L,C].
+    Differentiable: when autograd is recording and x, weight or bias requires grad, the input gradient is the same
+    stencil kernel run with the taps mirrored, the weight and bias gradients are reductions over batch and grid."""
+    if torch.is_grad_enabled() and any(t is not None and t.requires_grad for t in (x, weight, bias)):
+        y = _DWConv3x3Function.apply(x, weight, bias, tuple(hw))
+        return torch.nn.functional.silu(y) if silu else y
+    return _dwconv3x3_raw(x, weight, hw, bias, silu)
+
+
+class _DWConv3x3Function(torch.autograd.Function):
+    """Autograd node of the depthwise 3x3 convolution on the token grid (vig.py:291-294), without the activation."""
+
+    @staticmethod
+    def forward(ctx, x, weight, bias, hw):
+        ctx.save_for_backward(x, weight)
+        ctx.hw = hw
+        ctx.bias_dtype = bias.dtype if bias is not None else None
+        return _dwconv3x3_raw(x, weight, hw, bias, False)
+
+    @staticmethod
+    def backward(ctx, dy):
+        x, weight = ctx.saved_tensors
+        (h, w), (B, L, C) = ctx.hw, x.shape
+        dx = dw = db = None
+        if ctx.needs_input_grad[0]:
+            # dx[p] = sum_t w[t] dy[p - t]: the same stencil with the taps mirrored through the centre
+            dx = _dwconv3x3_raw(dy, weight.detach().reshape(C, 9).flip(-1), ctx.hw, None, False)
+        if ctx.needs_input_grad[1]:
+            d4 = dy.reshape(B, h, w, C).float()
+            xp = torch.nn.functional.pad(x.reshape(B, h, w, C).float(), (0, 0, 1, 1, 1, 1))
+            dw = torch.stack([(d4 * xp[:, ky:ky + h, kx:kx + w]).sum((0, 1, 2)) for ky in range(3) for kx in range(3)],
+                             dim=1).reshape(weight.shape).to(weight.dtype)
+        if ctx.bias_dtype is not None and ctx.needs_input_grad[2]:
+            db = dy.float().sum((0, 1)).to(ctx.bias_dtype)
+        return dx, dw, db, None
+
+
+def _dwconv3x3_raw(x, weight, hw, bias, silu):
     lib = _lib.load()
     _check_cuda(x, weight, bias)
     x = _dense(x)
