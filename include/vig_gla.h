@@ -271,6 +271,32 @@ int vig_split_heads_fwd(const void* qkv, void* q, void* k, void* v, int B, int L
 int vig_swiglu_fwd(const void* gate_up, void* out, long long rows, int I, int io_dtype, void* stream);
 
 /*
+ * Backward of vig_swiglu_fwd: d_gate_up [rows, 2*I] = (d_gate | d_up) from the forward's input and dy [rows, I]:
+ *   d_gate = dy * up * sig(gate) * (1 + gate * (1 - sig(gate))),  d_up = dy * gate * sig(gate).
+ *
+ * Replaces: swiglu_bwd (flash-linear-attention/fla/modules/activations.py:113-119, used by SwiGLUFunction :137-148).
+ */
+int vig_swiglu_bwd(const void* gate_up, const void* dy, void* d_gate_up, long long rows, int I, int io_dtype,
+                   void* stream);
+
+/*
+ * Backward of vig_rmsnorm_fwd.  `sum` [rows, C] is the tensor the forward normalised (x, or the x + residual it
+ * returned), dy the gradient of y, d_sum (may be NULL) the gradient that arrives at the returned sum:
+ *   r = rsqrt(mean(sum^2) + eps),  g = dy * weight,
+ *   ds = r * (g - sum * r^2 * mean(g * sum)) + d_sum     -- the gradient of x and of the residual alike
+ *   dweight[c] = sum over rows of dy[c] * sum[c] * r     -- fp32 [C]; NULL skips it (and needs no workspace)
+ * `workspace` holds vig_rmsnorm_bwd_workspace(rows, C) bytes of per-workgroup partial sums; the result does not
+ * depend on scheduling (no atomics).  C % 8 == 0, C <= 1024.
+ *
+ * Replaces: _layer_norm_bwd_kernel in its RMS mode with residual
+ * (flash-linear-attention/fla/modules/rmsnorm.py:203-296, driver :300-387).
+ */
+size_t vig_rmsnorm_bwd_workspace(long long rows, int C);
+int vig_rmsnorm_bwd(const void* sum, const float* weight, const void* dy, const void* d_sum, void* ds, float* dweight,
+                    void* workspace, size_t workspace_bytes, long long rows, int C, float eps, int io_dtype,
+                    void* stream);
+
+/*
  * gate_proj and the SwiGLU product in one kernel, for a short contraction (K = 384 or 192, the hidden sizes of
  * ViG-S / ViG-T), bf16, fp32 accumulation:
  *   y [rows, I] = swiglu(gate, up) with (gate | up) = x [rows, K] . weight [2*I, K]^T, the product taken on gate and

@@ -166,3 +166,60 @@ def test_swiglu(dtype, tol, rows, I):
     got = vig_amd.ops.swiglu(gu.cuda())
     assert got.shape == (*rows, I)
     assert _close(f64(got), want, tol)
+
+
+@pytest.mark.parametrize("dtype,tol", [(torch.float32, 2e-5), (torch.bfloat16, 2e-2)])
+@pytest.mark.parametrize("rows,C", [(37, 384), (300, 64), (9, 1024), (20000, 768), (5000, 192)])
+@pytest.mark.parametrize("residual", [False, True])
+def test_rmsnorm_gradients(dtype, tol, rows, C, residual):
+    """vig_rmsnorm_bwd through the op's autograd node against autograd through the float64 formula: gradients of x,
+    of the residual and of the weight, with a gradient arriving at the returned sum as well."""
+    announce(f"rmsnorm gradients rows={rows} C={C} residual={residual} {dtype}")
+    torch.manual_seed(rows + C)
+    x = torch.randn(rows, C).to(dtype)
+    r = torch.randn(rows, C).to(dtype) if residual else None
+    w = torch.rand(C) + 0.5
+    cot_y, cot_s = torch.randn(rows, C), torch.randn(rows, C)
+    x64, w64 = x.double().requires_grad_(), w.double().requires_grad_()
+    r64 = r.double().requires_grad_() if residual else None
+    s64 = x64 + r64 if residual else x64
+    if residual and dtype == torch.bfloat16:
+        # the op returns the sum rounded to bf16 and its backward recomputes from that stored sum
+        s64 = s64 + (s64.detach().to(dtype).double() - s64.detach())
+    y64 = s64 * torch.rsqrt(s64.pow(2).mean(-1, keepdim=True) + 1e-6) * w64
+    ((y64 * cot_y.double()).sum() + ((s64 * cot_s.double()).sum() if residual else 0)).backward()
+
+    xg, wg = x.cuda().requires_grad_(), w.cuda().requires_grad_()
+    rg = r.cuda().requires_grad_() if residual else None
+    if residual:
+        y, s = vig_amd.ops.rmsnorm(xg, wg, 1e-6, residual=rg, prenorm=True)
+        ((y.float() * cot_y.cuda()).sum() + (s.float() * cot_s.cuda()).sum()).backward()
+    else:
+        y = vig_amd.ops.rmsnorm(xg, wg, 1e-6)
+        (y.float() * cot_y.cuda()).sum().backward()
+
+    def rel(a, b):
+        return ((a.double().cpu() - b).abs().max() / b.abs().max()).item()
+
+    errs = dict(y=rel(y.detach(), y64.detach()), dx=rel(xg.grad, x64.grad), dw=rel(wg.grad, w64.grad))
+    if residual:
+        errs["dres"] = rel(rg.grad, r64.grad)
+    print("  " + "  ".join(f"{k} {v:.2e}" for k, v in errs.items()), flush=True)
+    assert max(errs.values()) <= tol, errs
+
+
+@pytest.mark.parametrize("dtype,tol", [(torch.float32, 1e-5), (torch.bfloat16, 2e-2)])
+def test_swiglu_gradients(dtype, tol):
+    announce(f"swiglu gradients {dtype}")
+    torch.manual_seed(2)
+    gu = (torch.randn(3, 50, 2 * 136) * 2).to(dtype)
+    cot = torch.randn(3, 50, 136)
+    g64 = gu.double().requires_grad_()
+    a, b = g64.chunk(2, -1)
+    ((torch.nn.functional.silu(a) * b) * cot.double()).sum().backward()
+    gg = gu.cuda().requires_grad_()
+    y = vig_amd.ops.swiglu(gg)
+    (y.float() * cot.cuda()).sum().backward()
+    err = ((gg.grad.double().cpu() - g64.grad).abs().max() / g64.grad.abs().max()).item()
+    print(f"  d_gate_up max-rel err {err:.2e}", flush=True)
+    assert err <= tol

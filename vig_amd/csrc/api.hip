@@ -24,6 +24,11 @@ int launch_layernorm(const void* x, const float* weight, const float* bias, void
 int launch_split_heads(const void* qkv, void* q, void* k, void* v, int B, int L, int H, int Dk, int Dv, long long ld,
                        int io_dtype, hipStream_t stream);
 int launch_swiglu(const void* in, void* out, long long rows, int I, int io_dtype, hipStream_t stream);
+int launch_swiglu_bwd(const void* in, const void* dy, void* din, long long rows, int I, int io_dtype,
+                      hipStream_t stream);
+size_t rmsnorm_bwd_workspace(long long rows, int C);
+int launch_rmsnorm_bwd(const void* s, const float* weight, const void* dy, const void* d_sum, void* ds, float* dweight,
+                       void* workspace, long long rows, int C, float eps, int io_dtype, hipStream_t stream);
 bool linear_swiglu_supported(int K, int I);
 int launch_linear_swiglu(const void* A, const void* W, void* out, long long T, int K, int I, hipStream_t stream);
 bool patch_conv_supported(int Cin, int H, int W, int KH, int KW, int stride, int padding, int Cout);
@@ -306,6 +311,30 @@ int vig_swiglu_fwd(const void* gate_up, void* out, long long rows, int I, int io
   if (!aligned16(gate_up, out)) return VIG_EINVAL;
   if (!dtype_ok(io_dtype) || (I % 8) != 0) return VIG_ENOTSUP;
   return vig::launch_swiglu(gate_up, out, rows, I, io_dtype, (hipStream_t)stream);
+}
+
+int vig_swiglu_bwd(const void* gate_up, const void* dy, void* d_gate_up, long long rows, int I, int io_dtype,
+                   void* stream) {
+  if (!gate_up || !dy || !d_gate_up || rows <= 0 || I <= 0) return VIG_EINVAL;
+  if (!aligned16(gate_up, dy, d_gate_up)) return VIG_EINVAL;
+  if (!dtype_ok(io_dtype) || (I % 8) != 0) return VIG_ENOTSUP;
+  return vig::launch_swiglu_bwd(gate_up, dy, d_gate_up, rows, I, io_dtype, (hipStream_t)stream);
+}
+
+size_t vig_rmsnorm_bwd_workspace(long long rows, int C) {
+  if (rows <= 0 || C <= 0) return 0;
+  return vig::rmsnorm_bwd_workspace(rows, C);
+}
+
+int vig_rmsnorm_bwd(const void* sum, const float* weight, const void* dy, const void* d_sum, void* ds, float* dweight,
+                    void* workspace, size_t workspace_bytes, long long rows, int C, float eps, int io_dtype,
+                    void* stream) {
+  if (!sum || !weight || !dy || !ds || rows <= 0 || C <= 0) return VIG_EINVAL;
+  if (!aligned16(sum, weight, dy, d_sum, ds, dweight, workspace)) return VIG_EINVAL;
+  if (!dtype_ok(io_dtype) || (C % 8) != 0 || C > 1024) return VIG_ENOTSUP;
+  if (dweight && (!workspace || workspace_bytes < vig::rmsnorm_bwd_workspace(rows, C))) return VIG_ENOSPC;
+  return vig::launch_rmsnorm_bwd(sum, weight, dy, d_sum, ds, dweight, workspace, rows, C, eps, io_dtype,
+                                 (hipStream_t)stream);
 }
 
 static bool bwd_shape_ok(int Dk, int Dv) {

@@ -331,6 +331,199 @@ int launch_swiglu(const void* in, void* out, long long rows, int I, int io_dtype
 }
 
 // ---------------------------------------------------------------------------
+// Backward of the SwiGLU product:  d_gate = dy * up * sig(gate) * (1 + gate * (1 - sig(gate))),
+// d_up = dy * gate * sig(gate), written as d_gate_up [rows, 2*I] = (d_gate | d_up).
+// ---------------------------------------------------------------------------
+template <typename T>
+__global__ __launch_bounds__(256) void swiglu_bwd_kernel(const T* __restrict__ in, const T* __restrict__ dy,
+                                                         T* __restrict__ din, long long nvec, int I8) {
+  const long long i = (long long)blockIdx.x * 256 + threadIdx.x;
+  if (i >= nvec) return;
+  const long long row = i / I8;
+  const int c = (int)(i - row * I8) * 8;
+  const size_t I = (size_t)I8 * 8;
+  float g[8], u[8], d[8];
+  Oct<T>::load(in + (size_t)row * 2 * I + c, g);
+  Oct<T>::load(in + (size_t)row * 2 * I + I + c, u);
+  Oct<T>::load(dy + (size_t)row * I + c, d);
+#pragma unroll
+  for (int j = 0; j < 8; ++j) {
+    const float sg = sigmoidf_(g[j]);
+    const float du = d[j] * g[j] * sg;
+    g[j] = d[j] * u[j] * sg * (1.f + g[j] * (1.f - sg));
+    u[j] = du;
+  }
+  Oct<T>::store(din + (size_t)row * 2 * I + c, g);
+  Oct<T>::store(din + (size_t)row * 2 * I + I + c, u);
+}
+
+int launch_swiglu_bwd(const void* in, const void* dy, void* din, long long rows, int I, int io_dtype,
+                      hipStream_t stream) {
+  if (I % 8 != 0) return -95;
+  const long long nvec = rows * (I / 8);
+  if ((nvec + 255) / 256 > 0x7fffffffLL) return -95;
+  const dim3 grid((unsigned)((nvec + 255) / 256)), block(256);
+  if (io_dtype == 1)
+    hipLaunchKernelGGL(swiglu_bwd_kernel<uint16_t>, grid, block, 0, stream, (const uint16_t*)in, (const uint16_t*)dy,
+                       (uint16_t*)din, nvec, I / 8);
+  else
+    hipLaunchKernelGGL(swiglu_bwd_kernel<float>, grid, block, 0, stream, (const float*)in, (const float*)dy,
+                       (float*)din, nvec, I / 8);
+  return hipGetLastError() == hipSuccess ? 0 : -5;
+}
+
+// ---------------------------------------------------------------------------
+// Backward of the residual-add + RMS norm.  s is the stored sum that was normalised (x, or x + residual as the
+// forward returned it), dy the gradient of y, d_sum (optional) the gradient arriving at the returned sum:
+//   r = rsqrt(mean(s^2) + eps),  g = dy * weight,
+//   ds = r * (g - s * r^2 * mean(g * s)) + d_sum         (the gradient of x and of the residual alike)
+//   dweight[c] = sum over rows of dy[c] * s[c] * r
+// One wave per row, sixteen waves a workgroup (eight a SIMD: the kernel is a chain of load -> reduce -> store per
+// row, and only occupancy hides it); workgroups walk the rows a grid apart and keep their share of dweight in
+// registers; the waves of a workgroup combine through LDS into one row of `partials` [gridDim.x, C], which a second
+// kernel sums (no atomics: the result does not depend on the order the workgroups finish in).
+// ---------------------------------------------------------------------------
+constexpr int kRmsBwdWaves = 16;
+
+template <typename T, int NV>
+__global__ __launch_bounds__(64 * kRmsBwdWaves) void rmsnorm_bwd_kernel(const T* __restrict__ s_in, const float* __restrict__ weight,
+                                                          const T* __restrict__ dy, const T* __restrict__ d_sum,
+                                                          T* __restrict__ ds, float* __restrict__ partials, int rows,
+                                                          int C, float eps) {
+  extern __shared__ __align__(16) float red[];  // [kRmsBwdWaves][C], only with partials
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int nvec = C >> 3;
+  float w[NV][8], dw[NV][8];
+#pragma unroll
+  for (int i = 0; i < NV; ++i) {
+    const int v = lane + 64 * i;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) dw[i][j] = 0.f, w[i][j] = 0.f;
+    if (v < nvec) Oct<float>::load(weight + 8 * v, w[i]);
+  }
+  const float inv_c = 1.0f / (float)C;
+  for (int row = blockIdx.x * kRmsBwdWaves + wave; row < rows; row += gridDim.x * kRmsBwdWaves) {
+    const size_t base = (size_t)row * C;
+    float s[NV][8], g[NV][8];
+    float ss = 0.f, gs = 0.f;
+#pragma unroll
+    for (int i = 0; i < NV; ++i) {
+      const int v = lane + 64 * i;
+#pragma unroll
+      for (int j = 0; j < 8; ++j) s[i][j] = 0.f, g[i][j] = 0.f;
+      if (v < nvec) {
+        Oct<T>::load(s_in + base + 8 * v, s[i]);
+        Oct<T>::load(dy + base + 8 * v, g[i]);
+      }
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        ss = __builtin_fmaf(s[i][j], s[i][j], ss);
+        gs = __builtin_fmaf(g[i][j] * w[i][j], s[i][j], gs);
+      }
+    }
+    ss = wave_sum(ss);
+    gs = wave_sum(gs);
+    const float rstd = 1.0f / sqrtf(ss * inv_c + eps);
+    const float coef = rstd * rstd * gs * inv_c;
+#pragma unroll
+    for (int i = 0; i < NV; ++i) {
+      const int v = lane + 64 * i;
+      if (v < nvec) {
+        float o[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+          dw[i][j] = __builtin_fmaf(g[i][j] * rstd, s[i][j], dw[i][j]);
+          o[j] = rstd * (g[i][j] * w[i][j] - s[i][j] * coef);
+        }
+        if (d_sum) {
+          float e[8];
+          Oct<T>::load(d_sum + base + 8 * v, e);
+#pragma unroll
+          for (int j = 0; j < 8; ++j) o[j] += e[j];
+        }
+        Oct<T>::store(ds + base + 8 * v, o);
+      }
+    }
+  }
+  if (!partials) return;  // uniform over the grid
+#pragma unroll
+  for (int i = 0; i < NV; ++i) {
+    const int v = lane + 64 * i;
+    if (v < nvec) Oct<float>::store(red + wave * C + 8 * v, dw[i]);
+  }
+  __syncthreads();
+  for (int c = threadIdx.x; c < C; c += 64 * kRmsBwdWaves) {
+    float acc = 0.f;
+#pragma unroll
+    for (int k = 0; k < kRmsBwdWaves; ++k) acc += red[k * C + c];
+    partials[(size_t)blockIdx.x * C + c] = acc;
+  }
+}
+
+// out[c] = sum over the n rows of partials [n, C]: a workgroup takes 64 columns, its 16 waves a sixteenth of the rows each
+__global__ __launch_bounds__(1024) void column_sum_kernel(const float* __restrict__ partials, float* __restrict__ out,
+                                                          int n, int C) {
+  __shared__ float red[16][64];
+  const int lane = threadIdx.x & 63, slice = threadIdx.x >> 6;
+  const int c = blockIdx.x * 64 + lane;
+  float acc[4] = {0.f, 0.f, 0.f, 0.f};
+  if (c < C) {
+    int i = slice;
+    for (; i + 48 < n; i += 64) {
+#pragma unroll
+      for (int k = 0; k < 4; ++k) acc[k] += partials[(size_t)(i + 16 * k) * C + c];
+    }
+    for (; i < n; i += 16) acc[0] += partials[(size_t)i * C + c];
+  }
+  red[slice][lane] = (acc[0] + acc[1]) + (acc[2] + acc[3]);
+  __syncthreads();
+  if (slice == 0 && c < C) {
+    float t = 0.f;
+#pragma unroll
+    for (int k = 0; k < 16; ++k) t += red[k][lane];
+    out[c] = t;
+  }
+}
+
+static int rmsnorm_bwd_grid(long long rows) {
+  const long long want = (rows + kRmsBwdWaves - 1) / kRmsBwdWaves;
+  return (int)(want < 512 ? want : 512);
+}
+
+size_t rmsnorm_bwd_workspace(long long rows, int C) { return (size_t)rmsnorm_bwd_grid(rows) * C * sizeof(float); }
+
+template <typename T>
+static int launch_rmsnorm_bwd_t(const void* s, const float* weight, const void* dy, const void* d_sum, void* ds,
+                                float* dweight, float* partials, int rows, int C, float eps, hipStream_t stream) {
+  const int grid = rmsnorm_bwd_grid(rows);
+  const size_t lds = dweight ? (size_t)kRmsBwdWaves * C * sizeof(float) : 0;
+  float* part = dweight ? partials : nullptr;
+  const int nvec = C / 8;
+#define VIG_RMSB_CASE(NV)                                                                                     \
+  hipLaunchKernelGGL((rmsnorm_bwd_kernel<T, NV>), dim3(grid), dim3(64 * kRmsBwdWaves), lds, stream, (const T*)s, \
+                     weight, (const T*)dy, (const T*)d_sum, (T*)ds, part, rows, C, eps)
+  if (nvec <= 64) VIG_RMSB_CASE(1);
+  else VIG_RMSB_CASE(2);
+#undef VIG_RMSB_CASE
+  if (hipGetLastError() != hipSuccess) return -5;
+  if (dweight) {
+    hipLaunchKernelGGL(column_sum_kernel, dim3((C + 63) / 64), dim3(1024), 0, stream, (const float*)partials, dweight,
+                       grid, C);
+    if (hipGetLastError() != hipSuccess) return -5;
+  }
+  return 0;
+}
+
+int launch_rmsnorm_bwd(const void* s, const float* weight, const void* dy, const void* d_sum, void* ds, float* dweight,
+                       void* workspace, long long rows, int C, float eps, int io_dtype, hipStream_t stream) {
+  if (C % 8 != 0 || C > 1024 || rows > 0x7fffffffLL - 8192) return -95;  // 16 rows of C floats in 64 KB of LDS
+  return io_dtype == 1 ? launch_rmsnorm_bwd_t<uint16_t>(s, weight, dy, d_sum, ds, dweight, (float*)workspace,
+                                                        (int)rows, C, eps, stream)
+                       : launch_rmsnorm_bwd_t<float>(s, weight, dy, d_sum, ds, dweight, (float*)workspace, (int)rows,
+                                                     C, eps, stream);
+}
+
+// ---------------------------------------------------------------------------
 // Channel padding / cropping of bf16 rows:  dst[row, c] = c < src_c ? src[row, c] : 0  for c < dst_c.
 // Used to run head shapes narrower than the matrix-core kernel's (Dk 16, Dv 32) on it: zero q, k and v channels
 // contribute nothing, zero log-gates mean no decay, and the surplus output channels are cropped.

@@ -75,20 +75,12 @@ class RMSNorm(nn.Module):
         return self._w32_cache
 
     def forward(self, x, residual=None, prenorm: bool = False, round_sum: bool = False):
-        if _recording(self):
-            return self._forward_autograd(x, residual, prenorm, round_sum)
+        if _recording(self):  # the op's autograd node: forward and backward on the library's kernels
+            if residual is not None and residual.dtype != x.dtype:  # autocast: a bf16 branch meets the fp32 stream
+                dt = torch.promote_types(x.dtype, residual.dtype)
+                x, residual = x.to(dt), residual.to(dt)
+            return ops.rmsnorm(x, self.weight, self.eps, residual=residual, prenorm=prenorm, round_sum=round_sum)
         return ops.rmsnorm(x, self._w32(), self.eps, residual=residual, prenorm=prenorm, round_sum=round_sum)
-
-    def _forward_autograd(self, x, residual, prenorm, round_sum):
-        """The kernel's arithmetic in differentiable torch operations: sum and norm in fp32, results in x's dtype."""
-        s, res_out = x.float(), x
-        if residual is not None:
-            s = s + residual.float()
-            res_out = s.to(x.dtype)
-            if round_sum:
-                s = res_out.float()
-        y = (s * torch.rsqrt(s.pow(2).mean(-1, keepdim=True) + self.eps) * self.weight.float()).to(x.dtype)
-        return (y, res_out) if prenorm else y
 
 
 class GatedLinearAttention(nn.Module):
@@ -284,9 +276,8 @@ class GLAMLP(nn.Module):
         self.down_proj = nn.Linear(intermediate_size, hidden_size, bias=False)
 
     def forward(self, x):
-        if _recording(self):
-            gate, y = self.gate_proj(x).chunk(2, -1)
-            return self.down_proj(F.silu(gate) * y)
+        if _recording(self):  # the SwiGLU product's autograd node runs on the library's kernels both ways
+            return self.down_proj(ops.swiglu(self.gate_proj(x)))
         w = self.gate_proj.weight
         if ops.linear_swiglu_supported(x, w):  # ViG-S / ViG-T widths in bf16: no [.., 2*I] intermediate
             return self.down_proj(ops.linear_swiglu(x, w))

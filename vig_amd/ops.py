@@ -420,6 +420,56 @@ def rmsnorm(x: torch.Tensor, weight: torch.Tensor, eps: float = 1e-6, residual: 
     Returns y, or (y, x + residual) with prenorm=True.  round_sum=True normalises the sum after rounding it to the
     storage dtype, i.e. what `norm(x + residual)` on stored tensors computes.
     """
+    if torch.is_grad_enabled() and any(t is not None and t.requires_grad for t in (x, residual, weight)):
+        if residual is None:
+            y = _RMSNormFunction.apply(x, None, weight, float(eps), False)
+            return (y, x) if prenorm else y
+        y, total = _RMSNormFunction.apply(x, residual, weight, float(eps), bool(round_sum))
+        return (y, total) if prenorm else y
+    return _rmsnorm_raw(x, weight, eps, residual, prenorm, round_sum)
+
+
+class _RMSNormFunction(torch.autograd.Function):
+    """Autograd node of the residual-add + RMS norm (LayerNormFn in its RMS mode, fla/modules/rmsnorm.py:390-471):
+    forward and backward on the library's kernels.  With a residual it returns (y, x + residual)."""
+
+    @staticmethod
+    def forward(ctx, x, residual, weight, eps, round_sum):
+        y, total = _rmsnorm_raw(x, weight, eps, residual, True, round_sum)
+        ctx.save_for_backward(total, weight)
+        ctx.eps, ctx.has_residual = eps, residual is not None
+        return y if residual is None else (y, total)
+
+    @staticmethod
+    def backward(ctx, dy, d_total=None):
+        total, weight = ctx.saved_tensors
+        lib = _lib.load()
+        C = total.shape[-1]
+        rows = total.numel() // C
+        dy = _dense(dy)
+        if d_total is not None:
+            d_total = _dense(d_total)
+        w = _dense(weight.detach().float())
+        ds = torch.empty_like(total)
+        dw = ws = None
+        ws_bytes = 0
+        if ctx.needs_input_grad[2]:
+            dw = torch.empty(C, dtype=torch.float32, device=total.device)
+            ws_bytes = lib.vig_rmsnorm_bwd_workspace(rows, C)
+            ws = torch.empty(ws_bytes, dtype=torch.uint8, device=total.device)
+        with torch.cuda.device(total.device):
+            rc = lib.vig_rmsnorm_bwd(total.data_ptr(), w.data_ptr(), dy.data_ptr(),
+                                     d_total.data_ptr() if d_total is not None else None, ds.data_ptr(),
+                                     dw.data_ptr() if dw is not None else None,
+                                     ws.data_ptr() if ws is not None else None, ws_bytes, rows, C, ctx.eps,
+                                     _dt(total), _stream_ptr(total))
+        _lib.check(rc, "vig_rmsnorm_bwd")
+        if dw is not None:
+            dw = dw.to(weight.dtype).reshape(weight.shape)
+        return ds, (ds if ctx.has_residual else None), dw, None, None
+
+
+def _rmsnorm_raw(x, weight, eps, residual, prenorm, round_sum):
     lib = _lib.load()
     _check_cuda(x, weight)
     x = _dense(x)
@@ -560,7 +610,38 @@ def linear_swiglu(x: torch.Tensor, weight: torch.Tensor) -> torch.Tensor:
 
 
 def swiglu(gate_up: torch.Tensor) -> torch.Tensor:
-    """gate_up [..., 2*I] = (gate | up) -> gate * up / (1 + exp(-gate))  (fla/modules/activations.py:109-113)."""
+    """gate_up [..., 2*I] = (gate | up) -> gate * up / (1 + exp(-gate))  (fla/modules/activations.py:109-113).
+    Differentiable (vig_swiglu_bwd) when autograd is recording and gate_up requires grad."""
+    if torch.is_grad_enabled() and gate_up.requires_grad:
+        return _SwiGLUFunction.apply(gate_up)
+    return _swiglu_raw(gate_up)
+
+
+class _SwiGLUFunction(torch.autograd.Function):
+    """Autograd node of the SwiGLU product (SwiGLUFunction, fla/modules/activations.py:137-148)."""
+
+    @staticmethod
+    def forward(ctx, gate_up):
+        gate_up = _dense(gate_up)
+        ctx.save_for_backward(gate_up)
+        return _swiglu_raw(gate_up)
+
+    @staticmethod
+    def backward(ctx, dy):
+        (gate_up,) = ctx.saved_tensors
+        lib = _lib.load()
+        dy = _dense(dy)
+        I = gate_up.shape[-1] // 2
+        rows = gate_up.numel() // (2 * I)
+        d_in = torch.empty_like(gate_up)
+        with torch.cuda.device(gate_up.device):
+            rc = lib.vig_swiglu_bwd(gate_up.data_ptr(), dy.data_ptr(), d_in.data_ptr(), rows, I, _dt(gate_up),
+                                    _stream_ptr(gate_up))
+        _lib.check(rc, "vig_swiglu_bwd")
+        return d_in
+
+
+def _swiglu_raw(gate_up: torch.Tensor) -> torch.Tensor:
     lib = _lib.load()
     _check_cuda(gate_up)
     gate_up = _dense(gate_up)
