@@ -220,6 +220,25 @@ int vig_locality_blend_fwd(const void* o, const void* local, const void* g_lin,
                            int io_dtype, void* stream);
 
 /*
+ * Backward of vig_locality_blend_fwd from the forward's inputs and dy [B, L, H*Dv]:
+ *   d_o [B, H, L, Dv], d_local and d_glin [B, L, H*Dv] (packed), dw fp32 [2, Dv] = (gradient of w_g | of w_l).
+ * With s = sigmoid(g_lin), on = rms(o) * w_g, ln = rms(local) * w_l, y0 = on * s + ln * (1 - s):
+ *   dy0 = dy * d(y)/d(y0) (SiLU derivative when silu_out), d_on = dy0 * s, d_ln = dy0 * (1 - s),
+ *   d_glin = dy0 * (on - ln) * s * (1 - s); d_o and d_local are the RMS-norm backward of d_on and d_ln per
+ *   (token, head) row; dw sums d_on * o * r_o and d_ln * local * r_l over batch, tokens and heads.
+ * `workspace` holds vig_locality_blend_bwd_workspace(B, L, Dv) bytes (per-workgroup partial sums of dw, added in a
+ * fixed order: no atomics).
+ *
+ * Replaces: what autograd derives for classification/models/vig.py:447-457 in the reference (two fused RMS-norm
+ * backward launches, rmsnorm.py:203-296, and the elementwise chain of the blend).
+ */
+size_t vig_locality_blend_bwd_workspace(int B, int L, int Dv);
+int vig_locality_blend_bwd(const void* o, const void* local, const void* g_lin, const float* w_g, const float* w_l,
+                           const void* dy, void* d_o, void* d_local, void* d_glin, float* dw, void* workspace,
+                           size_t workspace_bytes, int B, int H, int L, int Dv, long long g_row_stride, float eps,
+                           int silu_out, int io_dtype, void* stream);
+
+/*
  * Residual-add + RMS norm over the last dimension (rows x C, C % 8 == 0, C <= 4096):
  *   s = x (+ residual) in fp32;  residual_out = s (if not NULL);  y = s * rsqrt(mean(s^2) + eps) * weight
  * residual and residual_out may be NULL; weight [C] f32.  round_sum != 0 first rounds s to the storage

@@ -230,3 +230,42 @@ def test_dwconv3x3_gradients(dtype, tol, silu):
                 db=rel(bg.grad, b64.grad))
     print("  " + "  ".join(f"{k} {v:.2e}" for k, v in errs.items()), flush=True)
     assert max(errs.values()) <= tol, errs
+
+
+@pytest.mark.parametrize("silu_out", [False, True])
+@pytest.mark.parametrize("dtype,tol", [(torch.float32, 2e-5), (torch.bfloat16, 2e-2)])
+@pytest.mark.parametrize("B,H,L,Dv", [(2, 6, 49, 64), (1, 3, 70, 32), (2, 12, 33, 64)])
+def test_locality_blend_gradients(dtype, tol, silu_out, B, H, L, Dv):
+    """vig_locality_blend_bwd through the op's autograd node against autograd through the float64 expression of the
+    epilogue (vig.py:447-457), on the same rounded inputs: gradients of o, local, g_lin and both norm weights."""
+    announce(f"locality_blend gradients B{B} H{H} L{L} Dv{Dv} {dtype} silu_out={silu_out}")
+    torch.manual_seed(B * 100 + L)
+    C = H * Dv
+    o = torch.randn(B, H, L, Dv).to(dtype)
+    loc = torch.randn(B, L, C).to(dtype)
+    gl = torch.randn(B, L, C).to(dtype)
+    wg, wl = torch.rand(Dv) + 0.5, torch.rand(Dv) + 0.5
+    cot = torch.randn(B, L, C)
+    t64 = [t.double().requires_grad_() for t in (o, loc, gl, wg, wl)]
+
+    def rms(x, w):
+        return x * torch.rsqrt(x.pow(2).mean(-1, keepdim=True) + 1e-6) * w
+
+    on = rms(t64[0].permute(0, 2, 1, 3), t64[3])
+    ln = rms(t64[1].reshape(B, L, H, Dv), t64[4])
+    s = torch.sigmoid(t64[2]).reshape(B, L, H, Dv)
+    y64 = (on * s + ln * (1 - s)).reshape(B, L, C)
+    if silu_out:
+        y64 = torch.nn.functional.silu(y64)
+    (y64 * cot.double()).sum().backward()
+    tg = [t.cuda().requires_grad_() for t in (o, loc, gl, wg, wl)]
+    y = vig_amd.ops.locality_blend(*tg, eps=1e-6, silu_out=silu_out)
+    (y.float() * cot.cuda()).sum().backward()
+
+    def rel(a, b):
+        return ((a.double().cpu() - b).abs().max() / b.abs().max()).item()
+
+    errs = {n: rel(a.grad, b.grad) for n, a, b in zip(("do", "dlocal", "dglin", "dw_g", "dw_l"), tg, t64)}
+    errs["y"] = rel(y.detach(), y64.detach())
+    print("  " + "  ".join(f"{k} {v:.2e}" for k, v in errs.items()), flush=True)
+    assert max(errs.values()) <= tol, errs

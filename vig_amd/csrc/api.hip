@@ -16,6 +16,11 @@ int launch_locality_gate(const void* o, const float* wt, void* y, int B, int H, 
 int launch_locality_blend(const void* o, const void* loc, const void* glin, const float* wg, const float* wl, void* y,
                           int B, int H, int L, int Dv, long long ldg, float eps, int silu_out, int io_dtype,
                           hipStream_t stream);
+size_t locality_blend_bwd_workspace(int B, int L, int Dv);
+int launch_locality_blend_bwd(const void* o, const void* loc, const void* glin, const float* wg, const float* wl,
+                              const void* dy, void* d_o, void* d_loc, void* d_glin, float* dw, void* workspace, int B,
+                              int H, int L, int Dv, long long ldg, float eps, int silu_out, int io_dtype,
+                              hipStream_t stream);
 int launch_rmsnorm(const void* x, const void* residual, const float* weight, void* y, void* residual_out, int rows,
                    int C, float eps, int round_sum, int io_dtype, hipStream_t stream);
 int launch_layernorm(const void* x, const float* weight, const float* bias, void* y, long long rows, int C, float eps,
@@ -256,6 +261,27 @@ int vig_locality_blend_fwd(const void* o, const void* local, const void* g_lin, 
   if (ldg < (long long)H * Dv || !strided_rows_ok(g_lin, ldg, io_dtype)) return VIG_EINVAL;
   return vig::launch_locality_blend(o, local, g_lin, w_g, w_l, y, B, H, L, Dv, ldg, eps, silu_out, io_dtype,
                                     (hipStream_t)stream);
+}
+
+size_t vig_locality_blend_bwd_workspace(int B, int L, int Dv) {
+  if (B <= 0 || L <= 0 || !(Dv == 32 || Dv == 64)) return 0;
+  return vig::locality_blend_bwd_workspace(B, L, Dv);
+}
+
+int vig_locality_blend_bwd(const void* o, const void* local, const void* g_lin, const float* w_g, const float* w_l,
+                           const void* dy, void* d_o, void* d_local, void* d_glin, float* dw, void* workspace,
+                           size_t workspace_bytes, int B, int H, int L, int Dv, long long g_row_stride, float eps,
+                           int silu_out, int io_dtype, void* stream) {
+  if (!o || !local || !g_lin || !w_g || !w_l || !dy || !d_o || !d_local || !d_glin || !dw || B <= 0 || H <= 0 ||
+      L <= 0)
+    return VIG_EINVAL;
+  if (!aligned16(o, local, w_g, w_l, dy, d_o, d_local, d_glin, dw, workspace)) return VIG_EINVAL;
+  if (!dtype_ok(io_dtype) || !(Dv == 32 || Dv == 64)) return VIG_ENOTSUP;
+  const long long ldg = g_row_stride > 0 ? g_row_stride : (long long)H * Dv;
+  if (ldg < (long long)H * Dv || !strided_rows_ok(g_lin, ldg, io_dtype)) return VIG_EINVAL;
+  if (!workspace || workspace_bytes < vig::locality_blend_bwd_workspace(B, L, Dv)) return VIG_ENOSPC;
+  return vig::launch_locality_blend_bwd(o, local, g_lin, w_g, w_l, dy, d_o, d_local, d_glin, dw, workspace, B, H, L,
+                                        Dv, ldg, eps, silu_out, io_dtype, (hipStream_t)stream);
 }
 
 int vig_rmsnorm_fwd(const void* x, const void* residual, const float* weight, void* y, void* residual_out,

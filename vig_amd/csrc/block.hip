@@ -485,6 +485,11 @@ __global__ __launch_bounds__(1024) void column_sum_kernel(const float* __restric
   }
 }
 
+int launch_column_sum(const float* partials, float* out, int n, int C, hipStream_t stream) {
+  hipLaunchKernelGGL(column_sum_kernel, dim3((C + 63) / 64), dim3(1024), 0, stream, partials, out, n, C);
+  return hipGetLastError() == hipSuccess ? 0 : -5;
+}
+
 static int rmsnorm_bwd_grid(long long rows) {
   const long long want = (rows + kRmsBwdWaves - 1) / kRmsBwdWaves;
   return (int)(want < 512 ? want : 512);
@@ -507,9 +512,7 @@ static int launch_rmsnorm_bwd_t(const void* s, const float* weight, const void* 
 #undef VIG_RMSB_CASE
   if (hipGetLastError() != hipSuccess) return -5;
   if (dweight) {
-    hipLaunchKernelGGL(column_sum_kernel, dim3((C + 63) / 64), dim3(1024), 0, stream, (const float*)partials, dweight,
-                       grid, C);
-    if (hipGetLastError() != hipSuccess) return -5;
+    return launch_column_sum(partials, dweight, grid, C, stream);
   }
   return 0;
 }

@@ -497,4 +497,137 @@ int launch_locality_blend(const void* o, const void* loc, const void* glin, cons
   return hipGetLastError() == hipSuccess ? 0 : -5;
 }
 
+// ---------------------------------------------------------------------------
+// Backward of the RMS-norm blend epilogue, same thread layout as the forward.  With s = sig(g_lin),
+// on = rms(o) * w_g, ln = rms(local) * w_l, y0 = on * s + ln * (1 - s), y = silu_out ? y0 * sig(y0) : y0:
+//   dy0 = dy * d(y)/d(y0),  d_on = dy0 * s,  d_ln = dy0 * (1 - s),  d_glin = dy0 * (on - ln) * s * (1 - s),
+//   d_o = rms_backward(o, w_g, d_on),  d_local = rms_backward(local, w_l, d_ln)   (per (token, head) row of Dv),
+//   dw_g[d] = sum d_on * o * r_o,  dw_l[d] = sum d_ln * local * r_l   over batch, tokens and heads.
+// The weight gradients leave as one row of `partials` [workgroups, 2 * Dv] per workgroup (threads park their sums in
+// LDS and 2 * Dv threads add the ones of their channel, in a fixed order), which a column sum finishes.
+// ---------------------------------------------------------------------------
+template <typename T>
+__global__ __launch_bounds__(256) void locality_blend_bwd_kernel(
+    const T* __restrict__ o, const T* __restrict__ loc, const T* __restrict__ glin, const float* __restrict__ wg,
+    const float* __restrict__ wl, const T* __restrict__ dy, T* __restrict__ d_o, T* __restrict__ d_loc,
+    T* __restrict__ d_glin, float* __restrict__ partials, int H, int L, int Dv, long long ldg, float eps,
+    int silu_out) {
+  __shared__ float park[256][17];  // per thread: 8 dw_g + 8 dw_l sums of its channel octet (17: bank spread)
+  const int d8n = Dv >> 3;
+  const int nv = H * d8n;
+  const int b = blockIdx.y;
+  const int l0 = blockIdx.x * 32;
+  const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;
+  const float inv_dv = 1.0f / (float)Dv;
+  float total = 0.f;  // threads 0 .. 2*Dv-1: their channel's weight-gradient sum over the whole workgroup
+  for (int cv0 = 0; cv0 < nv; cv0 += 64) {
+    const int cv = cv0 + tx;
+    const bool has = cv < nv;
+    const int cvc = has ? cv : 0;
+    const int hd = cvc / d8n, d8 = cvc - hd * d8n;
+    float w_g[8], w_l[8], dwg[8], dwl[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) w_g[j] = wg[d8 * 8 + j], w_l[j] = wl[d8 * 8 + j], dwg[j] = 0.f, dwl[j] = 0.f;
+    const size_t head_off = (((size_t)b * H + hd) * L) * (size_t)Dv + d8 * 8;
+    const size_t row0 = ((size_t)b * L) * (size_t)(nv * 8) + (size_t)cvc * 8;
+    const T* pg = glin + ((size_t)b * L) * (size_t)ldg + (size_t)cvc * 8;
+    for (int t = ty; t < 32; t += 4) {
+      const int l = l0 + t;
+      if (l >= L) break;  // uniform over the wave
+      float xo[8], xl[8], xg[8], g[8];
+      const size_t tok = row0 + (size_t)l * (nv * 8);
+      Vec8<T>::load(o + head_off + (size_t)l * Dv, xo);
+      Vec8<T>::load(loc + tok, xl);
+      Vec8<T>::load(pg + (size_t)l * ldg, xg);
+      Vec8<T>::load(dy + tok, g);
+      float so = 0.f, sl = 0.f;
+#pragma unroll
+      for (int j = 0; j < 8; ++j) so += xo[j] * xo[j], sl += xl[j] * xl[j];
+      for (int m = 1; m < d8n; m <<= 1) {
+        so += __shfl_xor(so, m);
+        sl += __shfl_xor(sl, m);
+      }
+      const float ro = rsqrtf(so * inv_dv + eps);
+      const float rl = rsqrtf(sl * inv_dv + eps);
+      float don[8], dln[8], dgl[8];
+      float mo = 0.f, ml = 0.f;
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        const float s = sigmoidf_(xg[j]);
+        const float on = xo[j] * ro * w_g[j], ln = xl[j] * rl * w_l[j];
+        float dy0 = g[j];
+        if (silu_out) {
+          const float y0 = on * s + ln * (1.f - s);
+          const float sy = sigmoidf_(y0);
+          dy0 *= sy * (1.f + y0 * (1.f - sy));
+        }
+        don[j] = dy0 * s;
+        dln[j] = dy0 * (1.f - s);
+        dgl[j] = dy0 * (on - ln) * s * (1.f - s);
+        mo = __builtin_fmaf(don[j] * w_g[j], xo[j], mo);
+        ml = __builtin_fmaf(dln[j] * w_l[j], xl[j], ml);
+      }
+      for (int m = 1; m < d8n; m <<= 1) {
+        mo += __shfl_xor(mo, m);
+        ml += __shfl_xor(ml, m);
+      }
+      const float co = ro * ro * mo * inv_dv, cl = rl * rl * ml * inv_dv;
+      float eo[8], el[8];
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        eo[j] = ro * (don[j] * w_g[j] - xo[j] * co);
+        el[j] = rl * (dln[j] * w_l[j] - xl[j] * cl);
+        if (has) {
+          dwg[j] = __builtin_fmaf(don[j] * ro, xo[j], dwg[j]);
+          dwl[j] = __builtin_fmaf(dln[j] * rl, xl[j], dwl[j]);
+        }
+      }
+      if (has) {
+        Vec8<T>::store(d_o + head_off + (size_t)l * Dv, eo);
+        Vec8<T>::store(d_loc + tok, el);
+        Vec8<T>::store(d_glin + tok, dgl);
+      }
+    }
+    // combine the threads of one channel: thread (which, d) adds, in thread order, the parked sums of every thread
+    // whose octet holds channel d
+    __syncthreads();  // the previous round's readers are done
+#pragma unroll
+    for (int j = 0; j < 8; ++j) park[threadIdx.x][j] = dwg[j], park[threadIdx.x][8 + j] = dwl[j];
+    __syncthreads();
+    if (threadIdx.x < 2 * Dv) {
+      const int which = threadIdx.x / Dv, d = threadIdx.x - which * Dv;
+      const int want = d >> 3, slot = 8 * which + (d & 7);
+      // octet index of thread t in this round: ((cv0 + (t & 63)) % d8n), cv0 a multiple of 64 and d8n dividing 64
+      for (int t = want; t < 256; t += d8n) total += park[t][slot];
+    }
+  }
+  if (threadIdx.x < 2 * Dv)
+    partials[((size_t)blockIdx.y * gridDim.x + blockIdx.x) * (size_t)(2 * Dv) + threadIdx.x] = total;
+}
+
+int launch_column_sum(const float* partials, float* out, int n, int C, hipStream_t stream);
+
+size_t locality_blend_bwd_workspace(int B, int L, int Dv) {
+  return (size_t)B * ((L + 31) / 32) * 2 * Dv * sizeof(float);
+}
+
+int launch_locality_blend_bwd(const void* o, const void* loc, const void* glin, const float* wg, const float* wl,
+                              const void* dy, void* d_o, void* d_loc, void* d_glin, float* dw, void* workspace, int B,
+                              int H, int L, int Dv, long long ldg, float eps, int silu_out, int io_dtype,
+                              hipStream_t stream) {
+  if (B > 65535 || (long long)B * ((L + 31) / 32) > 0x7fffffffLL) return -22;
+  const dim3 grid((L + 31) / 32, B), block(256);
+  float* partials = static_cast<float*>(workspace);
+  if (io_dtype == 0)
+    hipLaunchKernelGGL((locality_blend_bwd_kernel<float>), grid, block, 0, stream, (const float*)o, (const float*)loc,
+                       (const float*)glin, wg, wl, (const float*)dy, (float*)d_o, (float*)d_loc, (float*)d_glin,
+                       partials, H, L, Dv, ldg, eps, silu_out);
+  else
+    hipLaunchKernelGGL((locality_blend_bwd_kernel<uint16_t>), grid, block, 0, stream, (const uint16_t*)o,
+                       (const uint16_t*)loc, (const uint16_t*)glin, wg, wl, (const uint16_t*)dy, (uint16_t*)d_o,
+                       (uint16_t*)d_loc, (uint16_t*)d_glin, partials, H, L, Dv, ldg, eps, silu_out);
+  if (hipGetLastError() != hipSuccess) return -5;
+  return launch_column_sum(partials, dw, (int)(grid.x * grid.y), 2 * Dv, stream);
+}
+
 }  // namespace vig

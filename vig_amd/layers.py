@@ -186,7 +186,7 @@ class GatedLinearAttention(nn.Module):
         vig.py:354-426,444-463: its flipped copies of q, k, v and of the backward gates are what the op's second
         direction reads in place)."""
         B, L, C = x.shape
-        H, Dv = self.num_heads, self.head_v_dim
+        H = self.num_heads
         conv = self.in_proj[0]
         if torch.is_autocast_enabled():  # what autocast would hand a convolution
             x = x.to(torch.get_autocast_dtype("cuda"))
@@ -205,12 +205,9 @@ class GatedLinearAttention(nn.Module):
         g_fwd, g_bwd = self.gk_proj(xs).chunk(2, dim=2)
         o = ops.gla_bidir_forward(heads(q), heads(k), heads(v), gate(g_fwd), gate(g_bwd), scale=-1,
                                   out_scale=out_scale)
-        o = self.g_norm(o.transpose(1, 2))  # [B, L, H, Dv]
-        loc = self.l_norm(xs.reshape(B, L, H, Dv))
-        g = torch.sigmoid(self.g_proj(xs)).reshape(B, L, H, Dv)
-        y = (o * g + loc * (1 - g)).reshape(B, L, H * Dv)
-        if self.use_out_act:
-            y = F.silu(y)
+        # both head norms, the sigmoid blend and the output activation: one kernel each way
+        y = ops.locality_blend(o, xs, self.g_proj(xs), self.g_norm.weight, self.l_norm.weight,
+                               eps=self.layernorm_eps, silu_out=self.use_out_act)
         return self.o_proj(y)
 
     def forward(self, x, lower_bound=0, **kwargs):

@@ -392,7 +392,44 @@ def _token_rows(t: torch.Tensor):
 def locality_blend(o: torch.Tensor, local: torch.Tensor, g_lin: torch.Tensor, w_g: torch.Tensor,
                    w_l: torch.Tensor, eps: float = 1e-6, silu_out: bool = False) -> torch.Tensor:
     """Block epilogue (vig.py:444-457): o [B,H,L,Dv]; local, g_lin [B,L,H*Dv] -> y [B,L,H*Dv].
-    g_lin may be a block of columns of a wider [B, L, W] tensor (it is read in place)."""
+    g_lin may be a block of columns of a wider [B, L, W] tensor (it is read in place).
+    Differentiable (vig_locality_blend_bwd) when autograd is recording and an input or a norm weight requires grad."""
+    if torch.is_grad_enabled() and any(t.requires_grad for t in (o, local, g_lin, w_g, w_l)):
+        return _LocalityBlendFunction.apply(o, local, g_lin, w_g, w_l, float(eps), bool(silu_out))
+    return _locality_blend_raw(o, local, g_lin, w_g, w_l, eps, silu_out)
+
+
+class _LocalityBlendFunction(torch.autograd.Function):
+    """Autograd node of the block epilogue: forward and backward each one kernel of the library."""
+
+    @staticmethod
+    def forward(ctx, o, local, g_lin, w_g, w_l, eps, silu_out):
+        o, local, g_lin = _dense(o), _dense(local), _dense(g_lin)
+        ctx.save_for_backward(o, local, g_lin, w_g, w_l)
+        ctx.eps, ctx.silu_out = eps, silu_out
+        return _locality_blend_raw(o, local, g_lin, w_g, w_l, eps, silu_out)
+
+    @staticmethod
+    def backward(ctx, dy):
+        o, local, g_lin, w_g, w_l = ctx.saved_tensors
+        lib = _lib.load()
+        B, H, L, Dv = o.shape
+        dy = _dense(dy)
+        d_o, d_local, d_glin = torch.empty_like(o), torch.empty_like(local), torch.empty_like(g_lin)
+        dw = torch.empty(2, Dv, dtype=torch.float32, device=o.device)
+        ws_bytes = lib.vig_locality_blend_bwd_workspace(B, L, Dv)
+        ws = torch.empty(ws_bytes, dtype=torch.uint8, device=o.device)
+        wg, wl = _dense(w_g.detach().float()), _dense(w_l.detach().float())
+        with torch.cuda.device(o.device):
+            rc = lib.vig_locality_blend_bwd(o.data_ptr(), local.data_ptr(), g_lin.data_ptr(), wg.data_ptr(),
+                                            wl.data_ptr(), dy.data_ptr(), d_o.data_ptr(), d_local.data_ptr(),
+                                            d_glin.data_ptr(), dw.data_ptr(), ws.data_ptr(), ws_bytes, B, H, L, Dv,
+                                            H * Dv, ctx.eps, int(ctx.silu_out), _dt(o), _stream_ptr(o))
+        _lib.check(rc, "vig_locality_blend_bwd")
+        return d_o, d_local, d_glin, dw[0].to(w_g.dtype), dw[1].to(w_l.dtype), None, None
+
+
+def _locality_blend_raw(o, local, g_lin, w_g, w_l, eps, silu_out):
     lib = _lib.load()
     _check_cuda(o, local, g_lin, w_g, w_l)
     o, local = _dense(o), _dense(local)
