@@ -155,6 +155,16 @@ int vig_dirgate_fwd(const void* gk_lin, void* g_out, int B, int L, int H, int Dk
                     int in_dtype, int out_dtype, void* stream);
 
 /*
+ * Backward of vig_dirgate_fwd: d_g [2, B, H, L, Dk] (type out_dtype) -> d_gk_lin [B, L, 2*H*Dk] (type in_dtype),
+ *   d_gk_lin = d_g * inv_normalizer * sigmoid(-gk_lin), zero where the forward clamped.
+ *
+ * Replaces: what autograd derives for classification/models/vig.py:368-371,411-414 (logsigmoid, division, clamp,
+ * the direction split and the head rearrange).
+ */
+int vig_dirgate_bwd(const void* gk_lin, const void* d_g, void* d_gk_lin, int B, int L, int H, int Dk,
+                    float inv_normalizer, float clamp_min, int in_dtype, int out_dtype, void* stream);
+
+/*
  * Direction-wise gate preparation with the second layer of the low-rank gate projection inside:
  *   gk_low [B, L, rank] (token rows low_row_stride elements apart, 0 = packed), w_up [2*H*Dk, rank], b_up [2*H*Dk]
  *   x = gk_low . w_up^T + b_up, rounded to in_dtype (what the separate layer would have stored);
@@ -280,6 +290,15 @@ int vig_layernorm_fwd(const void* x, const float* weight, const float* bias, voi
  */
 int vig_split_heads_fwd(const void* qkv, void* q, void* k, void* v, int B, int L, int H, int Dk, int Dv,
                         long long qkv_row_stride, int io_dtype, void* stream);
+
+/*
+ * Backward of vig_split_heads_fwd: dq, dk [B, H, L, Dk] and dv [B, H, L, Dv] gathered into d_qkv
+ * [B, L, H*(2*Dk+Dv)] (packed rows), one pass.
+ *
+ * Replaces: what autograd derives for classification/models/vig.py:401-409 (three rearranges back and a concat).
+ */
+int vig_split_heads_bwd(const void* dq, const void* dk, const void* dv, void* d_qkv, int B, int L, int H, int Dk,
+                        int Dv, int io_dtype, void* stream);
 
 /*
  * SwiGLU product of the MLP:  gate_up [rows, 2*I] = (gate | up)  ->  out [rows, I] = gate * up / (1 + exp(-gate))

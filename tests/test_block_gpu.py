@@ -223,3 +223,22 @@ def test_swiglu_gradients(dtype, tol):
     err = ((gg.grad.double().cpu() - g64.grad).abs().max() / g64.grad.abs().max()).item()
     print(f"  d_gate_up max-rel err {err:.2e}", flush=True)
     assert err <= tol
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_split_heads_gradients(dtype):
+    """vig_split_heads_bwd: the gradient of the split is the gather of the three head-major gradients (exact)."""
+    announce(f"split_heads gradients {dtype}")
+    torch.manual_seed(4)
+    B, L, H, Dk, Dv = 2, 37, 3, 16, 32
+    qkv = torch.randn(B, L, H * (2 * Dk + Dv), device="cuda").to(dtype).requires_grad_()
+    cq, ck = torch.randn(B, H, L, Dk, device="cuda").to(dtype), torch.randn(B, H, L, Dk, device="cuda").to(dtype)
+    cv = torch.randn(B, H, L, Dv, device="cuda").to(dtype)
+    q, k, v = vig_amd.ops.split_heads(qkv, H, Dk, Dv)
+    torch.autograd.backward((q, k, v), (cq, ck, cv))
+
+    def rows(t):
+        return t.permute(0, 2, 1, 3).reshape(B, L, -1)
+
+    want = torch.cat((rows(cq), rows(ck), rows(cv)), dim=-1)
+    assert torch.equal(qkv.grad, want)

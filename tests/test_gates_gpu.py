@@ -269,3 +269,26 @@ def test_locality_blend_gradients(dtype, tol, silu_out, B, H, L, Dv):
     errs["y"] = rel(y.detach(), y64.detach())
     print("  " + "  ".join(f"{k} {v:.2e}" for k, v in errs.items()), flush=True)
     assert max(errs.values()) <= tol, errs
+
+
+@pytest.mark.parametrize("clamp_min", [None, -0.05])
+@pytest.mark.parametrize("dtype,tol", [(torch.float32, 1e-5), (torch.bfloat16, 2e-2)])
+def test_dirgate_gradients(dtype, tol, clamp_min):
+    """vig_dirgate_bwd against autograd through logsigmoid / normalizer / clamp / split / rearrange in float64."""
+    announce(f"dirgate gradients {dtype} clamp_min={clamp_min}")
+    torch.manual_seed(1)
+    B, L, H, Dk = 2, 45, 3, 16
+    x = (torch.randn(B, L, 2 * H * Dk) * 2).to(dtype)
+    cot = torch.randn(2, B, H, L, Dk)
+    x64 = x.double().requires_grad_()
+    g64 = torch.nn.functional.logsigmoid(x64) / 16
+    if clamp_min is not None:
+        g64 = torch.clamp_min(g64, clamp_min)
+    g64 = g64.reshape(B, L, 2, H, Dk).permute(2, 0, 3, 1, 4)
+    (g64 * cot.double()).sum().backward()
+    xg = x.cuda().requires_grad_()
+    g = vig_amd.ops.dirgate(xg, H, 16.0, clamp_min)
+    (g.float() * cot.cuda()).sum().backward()
+    err = ((xg.grad.double().cpu() - x64.grad).abs().max() / x64.grad.abs().max()).item()
+    print(f"  d_gk_lin max-rel err {err:.2e}", flush=True)
+    assert err <= tol

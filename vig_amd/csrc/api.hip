@@ -6,6 +6,10 @@
 namespace vig {
 int launch_dirgate(const void* in, void* out, int B, int L, int H, int Dk, float inv_norm, float clamp_min,
                    int in_dtype, int out_dtype, hipStream_t stream);
+int launch_dirgate_bwd(const void* in, const void* d_out, void* d_in, int B, int L, int H, int Dk, float inv_norm,
+                       float clamp_min, int in_dtype, int out_dtype, hipStream_t stream);
+int launch_merge_heads(const void* dq, const void* dk, const void* dv, void* dqkv, int B, int L, int H, int Dk, int Dv,
+                       int io_dtype, hipStream_t stream);
 int launch_dwconv3x3(const void* x, const float* wt, const float* bias, void* y, int B, int h, int w, int C,
                      int silu, int io_dtype, hipStream_t stream);
 int launch_dirgate_lowrank(const void* low, long long ld, const void* w1, const void* b1, void* out, int B, int L,
@@ -220,6 +224,23 @@ int vig_dirgate_fwd(const void* gk_lin, void* g_out, int B, int L, int H, int Dk
   if (!dtype_ok(in_dtype) || !dtype_ok(out_dtype) || (Dk % 8) != 0) return VIG_ENOTSUP;
   return vig::launch_dirgate(gk_lin, g_out, B, L, H, Dk, inv_normalizer, clamp_min, in_dtype, out_dtype,
                              (hipStream_t)stream);
+}
+
+int vig_dirgate_bwd(const void* gk_lin, const void* d_g, void* d_gk_lin, int B, int L, int H, int Dk,
+                    float inv_normalizer, float clamp_min, int in_dtype, int out_dtype, void* stream) {
+  if (!gk_lin || !d_g || !d_gk_lin || B <= 0 || L <= 0 || H <= 0 || Dk <= 0) return VIG_EINVAL;
+  if (!aligned16(gk_lin, d_g, d_gk_lin)) return VIG_EINVAL;
+  if (!dtype_ok(in_dtype) || !dtype_ok(out_dtype) || (Dk % 8) != 0) return VIG_ENOTSUP;
+  return vig::launch_dirgate_bwd(gk_lin, d_g, d_gk_lin, B, L, H, Dk, inv_normalizer, clamp_min, in_dtype, out_dtype,
+                                 (hipStream_t)stream);
+}
+
+int vig_split_heads_bwd(const void* dq, const void* dk, const void* dv, void* d_qkv, int B, int L, int H, int Dk,
+                        int Dv, int io_dtype, void* stream) {
+  if (!dq || !dk || !dv || !d_qkv || B <= 0 || L <= 0 || H <= 0 || Dk <= 0 || Dv <= 0) return VIG_EINVAL;
+  if (!aligned16(dq, dk, dv, d_qkv)) return VIG_EINVAL;
+  if (!dtype_ok(io_dtype) || (Dk % 8) != 0 || (Dv % 8) != 0 || B > 65535) return VIG_ENOTSUP;
+  return vig::launch_merge_heads(dq, dk, dv, d_qkv, B, L, H, Dk, Dv, io_dtype, (hipStream_t)stream);
 }
 
 int vig_dirgate_lowrank_fwd(const void* gk_low, long long low_row_stride, const void* w_up, const void* b_up,

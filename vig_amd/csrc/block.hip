@@ -1,6 +1,8 @@
 // Row-wise kernels of the ViG block around the GLA op: residual-add + RMS norm, the head-major split of the
 // fused q/k/v projection and the SwiGLU product.  All are HBM-bound: every element is read once and written once
 // with 16-byte accesses, arithmetic in fp32.
+#include <type_traits>
+
 #include "common.h"
 #include "launch.h"
 
@@ -257,10 +259,12 @@ int launch_layernorm(const void* x, const float* weight, const float* bias, void
 // One workgroup owns 32 consecutive tokens of one batch element: whole rows are read, and every (tensor, head)
 // receives a contiguous run of 32 tokens.
 // ---------------------------------------------------------------------------
-template <typename T>
-__global__ __launch_bounds__(256) void split_heads_kernel(const T* __restrict__ qkv, T* __restrict__ q,
-                                                          T* __restrict__ k, T* __restrict__ v, int B, int L, int H,
-                                                          int Dk, int Dv, long long ld) {
+template <typename T, bool MERGE>  // MERGE: the backward, head-major gradients gathered into token-major rows
+__global__ __launch_bounds__(256) void split_heads_kernel(typename std::conditional<MERGE, T, const T>::type* __restrict__ qkv,
+                                                          typename std::conditional<MERGE, const T, T>::type* __restrict__ q,
+                                                          typename std::conditional<MERGE, const T, T>::type* __restrict__ k,
+                                                          typename std::conditional<MERGE, const T, T>::type* __restrict__ v,
+                                                          int B, int L, int H, int Dk, int Dv, long long ld) {
   const int K = H * Dk, V = H * Dv;
   const int row = 2 * K + V;
   const int nv = row >> 3;
@@ -269,20 +273,25 @@ __global__ __launch_bounds__(256) void split_heads_kernel(const T* __restrict__ 
   const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;
   for (int cv = tx; cv < nv; cv += 64) {
     const int ch = cv * 8;
-    T* dst;
+    typename std::conditional<MERGE, const T, T>::type* head;
     int D, c;
-    if (ch < K) { dst = q; D = Dk; c = ch; }
-    else if (ch < 2 * K) { dst = k; D = Dk; c = ch - K; }
-    else { dst = v; D = Dv; c = ch - 2 * K; }
+    if (ch < K) { head = q; D = Dk; c = ch; }
+    else if (ch < 2 * K) { head = k; D = Dk; c = ch - K; }
+    else { head = v; D = Dv; c = ch - 2 * K; }
     const int hh = c / D, d = c - hh * D;
-    const T* src = qkv + ((size_t)b * L) * (size_t)ld + ch;
-    T* out = dst + (((size_t)b * H + hh) * L) * (size_t)D + d;
+    auto* rows = qkv + ((size_t)b * L) * (size_t)ld + ch;
+    auto* slab = head + (((size_t)b * H + hh) * L) * (size_t)D + d;
     for (int t = ty; t < 32; t += 4) {
       const int l = l0 + t;
       if (l >= L) break;
       float x[8];
-      Oct<T>::load(src + (size_t)l * ld, x);
-      Oct<T>::store(out + (size_t)l * D, x);
+      if constexpr (MERGE) {
+        Oct<T>::load(slab + (size_t)l * D, x);
+        Oct<T>::store(rows + (size_t)l * ld, x);
+      } else {
+        Oct<T>::load(rows + (size_t)l * ld, x);
+        Oct<T>::store(slab + (size_t)l * D, x);
+      }
     }
   }
 }
@@ -292,11 +301,26 @@ int launch_split_heads(const void* qkv, void* q, void* k, void* v, int B, int L,
   if (Dk % 8 != 0 || Dv % 8 != 0 || B > 65535) return -95;
   const dim3 grid((L + 31) / 32, B), block(256);
   if (io_dtype == 1)
-    hipLaunchKernelGGL(split_heads_kernel<uint16_t>, grid, block, 0, stream, (const uint16_t*)qkv, (uint16_t*)q,
-                       (uint16_t*)k, (uint16_t*)v, B, L, H, Dk, Dv, ld);
+    hipLaunchKernelGGL((split_heads_kernel<uint16_t, false>), grid, block, 0, stream, (const uint16_t*)qkv,
+                       (uint16_t*)q, (uint16_t*)k, (uint16_t*)v, B, L, H, Dk, Dv, ld);
   else
-    hipLaunchKernelGGL(split_heads_kernel<float>, grid, block, 0, stream, (const float*)qkv, (float*)q, (float*)k,
-                       (float*)v, B, L, H, Dk, Dv, ld);
+    hipLaunchKernelGGL((split_heads_kernel<float, false>), grid, block, 0, stream, (const float*)qkv, (float*)q,
+                       (float*)k, (float*)v, B, L, H, Dk, Dv, ld);
+  return hipGetLastError() == hipSuccess ? 0 : -5;
+}
+
+// the backward of the split: dq, dk, dv (head-major) -> d_qkv [B, L, H*(2*Dk+Dv)] packed rows
+int launch_merge_heads(const void* dq, const void* dk, const void* dv, void* dqkv, int B, int L, int H, int Dk, int Dv,
+                       int io_dtype, hipStream_t stream) {
+  if (Dk % 8 != 0 || Dv % 8 != 0 || B > 65535) return -95;
+  const dim3 grid((L + 31) / 32, B), block(256);
+  const long long ld = (long long)H * (2 * Dk + Dv);
+  if (io_dtype == 1)
+    hipLaunchKernelGGL((split_heads_kernel<uint16_t, true>), grid, block, 0, stream, (uint16_t*)dqkv,
+                       (const uint16_t*)dq, (const uint16_t*)dk, (const uint16_t*)dv, B, L, H, Dk, Dv, ld);
+  else
+    hipLaunchKernelGGL((split_heads_kernel<float, true>), grid, block, 0, stream, (float*)dqkv, (const float*)dq,
+                       (const float*)dk, (const float*)dv, B, L, H, Dk, Dv, ld);
   return hipGetLastError() == hipSuccess ? 0 : -5;
 }
 

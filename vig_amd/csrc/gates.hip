@@ -87,6 +87,53 @@ __global__ __launch_bounds__(256) void dirgate_kernel(const TI* __restrict__ in,
   }
 }
 
+// Backward of the gate preparation: d_in[b, l, c] = d_out[dir, b, h, l, d] * inv_norm * sigmoid(-x), zero where the
+// forward clamped (x = in[b, l, c]; d/dx logsigmoid(x) = sigmoid(-x)).
+template <typename TI, typename TO>
+__global__ __launch_bounds__(256) void dirgate_bwd_kernel(const TI* __restrict__ in, const TO* __restrict__ d_out,
+                                                           TI* __restrict__ d_in, int B, int L, int H, int Dk,
+                                                           float inv_norm, float clamp_min, int use_clamp) {
+  const int nv = 2 * H * Dk / 8;
+  const int dk8 = Dk >> 3;
+  const int b = blockIdx.y;
+  const int l0 = blockIdx.x * 32;
+  const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;
+  for (int cv = tx; cv < nv; cv += 64) {
+    const int d8 = cv % dk8, hh = (cv / dk8) % H, dir = cv / (dk8 * H);
+    const size_t rows = ((size_t)b * L) * (size_t)(nv * 8) + (size_t)cv * 8;
+    const TO* grad = d_out + ((((size_t)dir * B + b) * H + hh) * L) * (size_t)Dk + (size_t)d8 * 8;
+    for (int t = ty; t < 32; t += 4) {
+      const int l = l0 + t;
+      if (l >= L) break;
+      float x[8], g[8];
+      Vec8<TI>::load(in + rows + (size_t)l * (nv * 8), x);
+      Vec8<TO>::load(grad + (size_t)l * Dk, g);
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        const bool clamped = use_clamp && logsigmoidf_(x[j]) * inv_norm < clamp_min;
+        x[j] = clamped ? 0.f : g[j] * inv_norm * sigmoidf_(-x[j]);
+      }
+      Vec8<TI>::store(d_in + rows + (size_t)l * (nv * 8), x);
+    }
+  }
+}
+
+int launch_dirgate_bwd(const void* in, const void* d_out, void* d_in, int B, int L, int H, int Dk, float inv_norm,
+                       float clamp_min, int in_dtype, int out_dtype, hipStream_t stream) {
+  const int use_clamp = clamp_min == clamp_min;  // NaN disables
+  if (B > 65535) return -22;
+  const dim3 grid((L + 31) / 32, B), block(256);
+#define VIG_DGB_CASE(TI, TO)                                                                                       \
+  hipLaunchKernelGGL((dirgate_bwd_kernel<TI, TO>), grid, block, 0, stream, (const TI*)in, (const TO*)d_out, (TI*)d_in, \
+                     B, L, H, Dk, inv_norm, clamp_min, use_clamp)
+  if (in_dtype == 0 && out_dtype == 0) VIG_DGB_CASE(float, float);
+  else if (in_dtype == 0 && out_dtype == 1) VIG_DGB_CASE(float, uint16_t);
+  else if (in_dtype == 1 && out_dtype == 0) VIG_DGB_CASE(uint16_t, float);
+  else VIG_DGB_CASE(uint16_t, uint16_t);
+#undef VIG_DGB_CASE
+  return hipGetLastError() == hipSuccess ? 0 : -5;
+}
+
 template <typename TI, typename TO>
 static int launch_dirgate_t(const void* in, void* out, int B, int L, int H, int Dk, float inv_norm,
                             float clamp_min, hipStream_t stream) {

@@ -16,11 +16,12 @@ vig.py:469-497,530-618,625-672,705-912 for the options the shipped configs use. 
 library op raises on tensors that are not on the GPU.
 
 Two ways through every module.  In eval mode, or whenever gradients are not being recorded, the forward runs on the
-library's kernels and leaves no autograd graph.  In training mode with gradients enabled (`model.train()` outside
-`torch.no_grad()`) the same arithmetic is written in differentiable torch operations around the one op the training
-path spends its time in, the bidirectional GLA, whose forward and backward both run on the library's kernels
-(vig_gla_bidir_fwd / vig_gla_bidir_bwd through ops.gla_bidir_forward) -- the reference's training branch
-(vig.py:354-426) with the flips and concatenations folded into the op.
+library's fused inference kernels and leaves no autograd graph.  In training mode with gradients enabled
+(`model.train()` outside `torch.no_grad()`) the block records one: the GEMMs and the patch embedding are torch's
+differentiable operations, and everything between them -- depthwise conv, head split, gate preparation, the
+bidirectional GLA, the norm/blend epilogue, the residual RMS norms and the SwiGLU product -- runs on the library's
+kernels in both directions through the autograd nodes of `ops` (the reference's training branch, vig.py:354-426,
+with its flips and concatenations folded into the op).
 """
 from __future__ import annotations
 
@@ -182,29 +183,19 @@ class GatedLinearAttention(nn.Module):
         return self.o_proj(y)
 
     def _mix_autograd(self, x, hw, out_scale):
-        """_mix in differentiable torch operations around the differentiable GLA op (the reference's training branch,
-        vig.py:354-426,444-463: its flipped copies of q, k, v and of the backward gates are what the op's second
-        direction reads in place)."""
-        B, L, C = x.shape
+        """_mix with an autograd graph (the reference's training branch, vig.py:354-426,444-463: its flipped copies of
+        q, k, v and of the backward gates are what the op's second direction reads in place).  The projections are
+        torch's differentiable GEMMs; everything between them is the library's kernels both ways, through the ops'
+        autograd nodes."""
         H = self.num_heads
         conv = self.in_proj[0]
         if torch.is_autocast_enabled():  # what autocast would hand a convolution
             x = x.to(torch.get_autocast_dtype("cuda"))
         xs = ops.dwconv3x3(x, conv.weight, hw, bias=conv.bias, silu=self.use_act_in_conv)  # differentiable, [B, L, C]
-        q, k, v = torch.split(self.qkv_proj(xs), [self.key_dim, self.key_dim, self.value_dim], dim=2)
-
-        def heads(t):
-            return t.reshape(B, L, H, -1).transpose(1, 2)
-
-        def gate(t):
-            g = F.logsigmoid(heads(t).float()) / self.gate_logit_normalizer
-            if self.clamp_min is not None:
-                g = torch.clamp_min(g, self.clamp_min)
-            return g.to(q.dtype)
-
-        g_fwd, g_bwd = self.gk_proj(xs).chunk(2, dim=2)
-        o = ops.gla_bidir_forward(heads(q), heads(k), heads(v), gate(g_fwd), gate(g_bwd), scale=-1,
-                                  out_scale=out_scale)
+        q, k, v = ops.split_heads(self.qkv_proj(xs), H, self.head_qk_dim, self.head_v_dim)
+        gates = ops.dirgate(self.gk_proj(xs), H, self.gate_logit_normalizer, self.clamp_min)
+        g_fwd, g_bwd = gates.unbind(0)
+        o = ops.gla_bidir_forward(q, k, v, g_fwd, g_bwd, scale=-1, out_scale=out_scale)
         # both head norms, the sigmoid blend and the output activation: one kernel each way
         y = ops.locality_blend(o, xs, self.g_proj(xs), self.g_norm.weight, self.l_norm.weight,
                                eps=self.layernorm_eps, silu_out=self.use_out_act)

@@ -219,7 +219,40 @@ def bid_fused_recurrent_gla(q, k, v, gk=None, gv=None, scale: int = -1, initial_
 
 def dirgate(gk_lin: torch.Tensor, num_heads: int, gate_logit_normalizer: float = 16.0,
             clamp_min: Optional[float] = None, out_dtype: Optional[torch.dtype] = None) -> torch.Tensor:
-    """gk_lin [B,L,2*H*Dk] -> [2,B,H,L,Dk] = logsigmoid/normalizer (vig.py:432-441)."""
+    """gk_lin [B,L,2*H*Dk] -> [2,B,H,L,Dk] = logsigmoid/normalizer (vig.py:432-441).
+    Differentiable (vig_dirgate_bwd) when autograd is recording and gk_lin requires grad."""
+    if torch.is_grad_enabled() and gk_lin.requires_grad:
+        return _DirGateFunction.apply(gk_lin, num_heads, float(gate_logit_normalizer), clamp_min, out_dtype)
+    return _dirgate_raw(gk_lin, num_heads, gate_logit_normalizer, clamp_min, out_dtype)
+
+
+class _DirGateFunction(torch.autograd.Function):
+    """Autograd node of the direction-wise gate preparation."""
+
+    @staticmethod
+    def forward(ctx, gk_lin, H, normalizer, clamp_min, out_dtype):
+        gk_lin = _dense(gk_lin)
+        ctx.save_for_backward(gk_lin)
+        ctx.args = (H, normalizer, clamp_min)
+        return _dirgate_raw(gk_lin, H, normalizer, clamp_min, out_dtype)
+
+    @staticmethod
+    def backward(ctx, d_g):
+        (gk_lin,) = ctx.saved_tensors
+        H, normalizer, clamp_min = ctx.args
+        lib = _lib.load()
+        d_g = _dense(d_g)
+        B, L, C2 = gk_lin.shape
+        d_in = torch.empty_like(gk_lin)
+        with torch.cuda.device(gk_lin.device):
+            rc = lib.vig_dirgate_bwd(gk_lin.data_ptr(), d_g.data_ptr(), d_in.data_ptr(), B, L, H, C2 // (2 * H),
+                                     1.0 / normalizer, float("nan") if clamp_min is None else float(clamp_min),
+                                     _dt(gk_lin), _dt(d_g), _stream_ptr(gk_lin))
+        _lib.check(rc, "vig_dirgate_bwd")
+        return d_in, None, None, None, None
+
+
+def _dirgate_raw(gk_lin, num_heads, gate_logit_normalizer=16.0, clamp_min=None, out_dtype=None):
     lib = _lib.load()
     _check_cuda(gk_lin)
     gk_lin = _dense(gk_lin)
@@ -569,7 +602,36 @@ def layernorm(x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor, eps: fl
 
 def split_heads(qkv: torch.Tensor, num_heads: int, head_qk_dim: int, head_v_dim: int):
     """qkv [B, L, H*Dk | H*Dk | H*Dv] -> q, k [B,H,L,Dk], v [B,H,L,Dv] (vig.py:401-409).
-    qkv may be a block of columns of a wider [B, L, W] tensor (it is read in place)."""
+    qkv may be a block of columns of a wider [B, L, W] tensor (it is read in place).
+    Differentiable (vig_split_heads_bwd) when autograd is recording and qkv requires grad."""
+    if torch.is_grad_enabled() and qkv.requires_grad:
+        return _SplitHeadsFunction.apply(qkv, num_heads, head_qk_dim, head_v_dim)
+    return _split_heads_raw(qkv, num_heads, head_qk_dim, head_v_dim)
+
+
+class _SplitHeadsFunction(torch.autograd.Function):
+    """Autograd node of the head split: the backward gathers dq, dk, dv into token-major rows in one pass."""
+
+    @staticmethod
+    def forward(ctx, qkv, H, Dk, Dv):
+        ctx.dims = (H, Dk, Dv)
+        return _split_heads_raw(qkv, H, Dk, Dv)
+
+    @staticmethod
+    def backward(ctx, dq, dk, dv):
+        lib = _lib.load()
+        H, Dk, Dv = ctx.dims
+        dq, dk, dv = _dense(dq), _dense(dk), _dense(dv)
+        B, _, L, _ = dq.shape
+        d_qkv = torch.empty(B, L, H * (2 * Dk + Dv), dtype=dq.dtype, device=dq.device)
+        with torch.cuda.device(dq.device):
+            rc = lib.vig_split_heads_bwd(dq.data_ptr(), dk.data_ptr(), dv.data_ptr(), d_qkv.data_ptr(), B, L, H, Dk,
+                                         Dv, _dt(dq), _stream_ptr(dq))
+        _lib.check(rc, "vig_split_heads_bwd")
+        return d_qkv, None, None, None
+
+
+def _split_heads_raw(qkv, num_heads, head_qk_dim, head_v_dim):
     lib = _lib.load()
     _check_cuda(qkv)
     qkv, ld = _token_rows(qkv)
