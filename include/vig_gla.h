@@ -190,6 +190,19 @@ int vig_dwconv3x3_fwd(const void* x, const float* weight, const float* bias, voi
                       int B, int h, int w, int C, int silu, int io_dtype, void* stream);
 
 /*
+ * Weight and bias gradients of vig_dwconv3x3_fwd (without its SiLU) from x and dy [B, h*w, C]:
+ *   dw_db fp32 [C*9 + C]: dw[c, ky, kx] = sum dy[b, y, x, c] * x[b, y+ky-1, x+kx-1, c], then db[c] = sum dy[b, y, x, c].
+ * The input gradient needs no entry point of its own: it is vig_dwconv3x3_fwd on dy with the nine taps of every
+ * channel mirrored through the centre.  `workspace` holds vig_dwconv3x3_bwd_weight_workspace(B, C) bytes
+ * (per-workgroup partial sums, added in a fixed order: no atomics).
+ *
+ * Replaces: the convolution library's depthwise weight-gradient call behind classification/models/vig.py:291-294.
+ */
+size_t vig_dwconv3x3_bwd_weight_workspace(int B, int C);
+int vig_dwconv3x3_bwd_weight(const void* x, const void* dy, float* dw_db, void* workspace, size_t workspace_bytes,
+                             int B, int h, int w, int C, int io_dtype, void* stream);
+
+/*
  * Synthetic locality gate of the ViG-B benchmark shape:
  *   y[b,hd,l,d] = o[b,hd,l,d] * sigmoid( dwconv3x3(o on the h x w grid, channel c = hd*Dv+d) )
  * o, y: [B, H, L=h*w, Dv]; weight [H*Dv, 3, 3] f32.  In-place (y == o) is NOT allowed.

@@ -203,12 +203,13 @@ def test_fused_locality_gate_other_shapes_take_two_calls():
 
 @pytest.mark.parametrize("silu", [False, True])
 @pytest.mark.parametrize("dtype,tol", [(torch.float32, 1e-5), (torch.bfloat16, 2e-2)])
-def test_dwconv3x3_gradients(dtype, tol, silu):
+@pytest.mark.parametrize("shape", [(3, 5, 7, 24), (2, 14, 14, 768), (1, 1, 40, 8)])
+def test_dwconv3x3_gradients(dtype, tol, silu, shape):
     """Input, weight and bias gradients of the differentiable stencil op against autograd through torch's conv2d in
     float64 (on the same rounded inputs)."""
-    announce(f"dwconv3x3 gradients {dtype} silu={silu}")
+    announce(f"dwconv3x3 gradients {shape} {dtype} silu={silu}")
     torch.manual_seed(3)
-    B, h, w, C = 3, 5, 7, 24
+    B, h, w, C = shape
     x = torch.randn(B, h * w, C).to(dtype)
     wt = (torch.randn(C, 1, 3, 3) / 3).to(dtype)
     bs = torch.randn(C).to(dtype)

@@ -46,6 +46,8 @@ SIGNATURES = {
     "vig_locality_blend_bwd_workspace": (_c_size_t, [_c_int] * 3),
     "vig_locality_blend_bwd": (_c_int, [_c_void_p] * 11 + [_c_size_t] + [_c_int] * 4 + [_c_longlong, _c_float, _c_int,
                                                                                         _c_int, _c_void_p]),
+    "vig_dwconv3x3_bwd_weight_workspace": (_c_size_t, [_c_int, _c_int]),
+    "vig_dwconv3x3_bwd_weight": (_c_int, [_c_void_p] * 4 + [_c_size_t] + [_c_int] * 5 + [_c_void_p]),
     "vig_dirgate_bwd": (_c_int, [_c_void_p] * 3 + [_c_int] * 4 + [_c_float, _c_float, _c_int, _c_int, _c_void_p]),
     "vig_split_heads_bwd": (_c_int, [_c_void_p] * 4 + [_c_int] * 6 + [_c_void_p]),
     "vig_swiglu_bwd": (_c_int, [_c_void_p] * 3 + [_c_longlong, _c_int, _c_int, _c_void_p]),

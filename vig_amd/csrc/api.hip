@@ -10,6 +10,9 @@ int launch_dirgate_bwd(const void* in, const void* d_out, void* d_in, int B, int
                        float clamp_min, int in_dtype, int out_dtype, hipStream_t stream);
 int launch_merge_heads(const void* dq, const void* dk, const void* dv, void* dqkv, int B, int L, int H, int Dk, int Dv,
                        int io_dtype, hipStream_t stream);
+size_t dwconv3x3_wgrad_workspace(int B, int C);
+int launch_dwconv3x3_wgrad(const void* x, const void* dy, float* dw_db, void* workspace, int B, int h, int w, int C,
+                           int io_dtype, hipStream_t stream);
 int launch_dwconv3x3(const void* x, const float* wt, const float* bias, void* y, int B, int h, int w, int C,
                      int silu, int io_dtype, hipStream_t stream);
 int launch_dirgate_lowrank(const void* low, long long ld, const void* w1, const void* b1, void* out, int B, int L,
@@ -262,6 +265,20 @@ int vig_dwconv3x3_fwd(const void* x, const float* weight, const float* bias, voi
   if (!aligned16(x, weight, bias, y)) return VIG_EINVAL;
   if (!dtype_ok(io_dtype) || (C % 8) != 0) return VIG_ENOTSUP;
   return vig::launch_dwconv3x3(x, weight, bias, y, B, h, w, C, silu, io_dtype, (hipStream_t)stream);
+}
+
+size_t vig_dwconv3x3_bwd_weight_workspace(int B, int C) {
+  if (B <= 0 || C <= 0) return 0;
+  return vig::dwconv3x3_wgrad_workspace(B, C);
+}
+
+int vig_dwconv3x3_bwd_weight(const void* x, const void* dy, float* dw_db, void* workspace, size_t workspace_bytes,
+                             int B, int h, int w, int C, int io_dtype, void* stream) {
+  if (!x || !dy || !dw_db || B <= 0 || h <= 0 || w <= 0 || C <= 0) return VIG_EINVAL;
+  if (!aligned16(x, dy, dw_db, workspace)) return VIG_EINVAL;
+  if (!dtype_ok(io_dtype) || (C % 8) != 0) return VIG_ENOTSUP;
+  if (!workspace || workspace_bytes < vig::dwconv3x3_wgrad_workspace(B, C)) return VIG_ENOSPC;
+  return vig::launch_dwconv3x3_wgrad(x, dy, dw_db, workspace, B, h, w, C, io_dtype, (hipStream_t)stream);
 }
 
 int vig_locality_gate_fwd(const void* o, const float* weight, void* y, int B, int H, int h, int w, int Dv,

@@ -545,6 +545,106 @@ int launch_locality_blend(const void* o, const void* loc, const void* glin, cons
 }
 
 // ---------------------------------------------------------------------------
+// Weight and bias gradients of the depthwise 3x3 convolution on token-major rows x, dy [B, h*w, C]:
+//   dw[c, ky, kx] = sum over b, y, x of dy[b, y, x, c] * x[b, y+ky-1, x+kx-1, c]   (zero padding),  db[c] = sum dy
+// A thread keeps one channel octet and walks every fourth token of its workgroup's share of one image with 9 * 8 + 8
+// sums in registers (the nine neighbour rows come from cache: every row is read by its nine neighbours); the four
+// token lanes combine through LDS in a fixed order and the workgroup leaves one row of `partials`
+// [workgroups, 10 * C] (columns c*9 + tap, then 9*C + c for the bias), which a column sum finishes.
+// ---------------------------------------------------------------------------
+constexpr int kWgradSplit = 4;  // workgroups per image
+
+template <typename T>
+__global__ __launch_bounds__(256) void dwconv3x3_wgrad_kernel(const T* __restrict__ x, const T* __restrict__ dy,
+                                                              float* __restrict__ partials, int h, int w, int C,
+                                                              int tiles_per_wg) {
+  __shared__ float red[64][81];
+  const int L = h * w, nv = C >> 3;
+  const int b = blockIdx.y;
+  const int tx = threadIdx.x & 63, ty = threadIdx.x >> 6;
+  const int ntiles = (L + 31) / 32;
+  const int tile0 = blockIdx.x * tiles_per_wg;
+  const int tile1 = tile0 + tiles_per_wg < ntiles ? tile0 + tiles_per_wg : ntiles;
+  float* prow = partials + ((size_t)b * gridDim.x + blockIdx.x) * ((size_t)C * 10);
+  for (int cv0 = 0; cv0 < nv; cv0 += 64) {
+    const int cv = cv0 + tx;
+    const bool has = cv < nv;
+    float acc[10][8];
+#pragma unroll
+    for (int k = 0; k < 10; ++k)
+#pragma unroll
+      for (int j = 0; j < 8; ++j) acc[k][j] = 0.f;
+    if (has) {
+      const T* px = x + (size_t)b * L * C + (size_t)cv * 8;
+      const T* pd = dy + (size_t)b * L * C + (size_t)cv * 8;
+      for (int tile = tile0; tile < tile1; ++tile) {
+        for (int t = ty; t < 32; t += 4) {
+          const int l = tile * 32 + t;
+          if (l >= L) break;
+          const int yy = l / w, xx = l - yy * w;
+          float g[8];
+          Vec8<T>::load(pd + (size_t)l * C, g);
+#pragma unroll
+          for (int j = 0; j < 8; ++j) acc[9][j] += g[j];
+#pragma unroll
+          for (int ky = 0; ky < 3; ++ky) {
+#pragma unroll
+            for (int kx = 0; kx < 3; ++kx) {
+              const int y2 = yy + ky - 1, x2 = xx + kx - 1;
+              if (y2 >= 0 && y2 < h && x2 >= 0 && x2 < w) {
+                float v[8];
+                Vec8<T>::load(px + (size_t)(y2 * w + x2) * C, v);
+#pragma unroll
+                for (int j = 0; j < 8; ++j) acc[ky * 3 + kx][j] = __builtin_fmaf(g[j], v[j], acc[ky * 3 + kx][j]);
+              }
+            }
+          }
+        }
+      }
+    }
+    for (int r = 0; r < 4; ++r) {  // the four token lanes add in turn
+      if (ty == r) {
+#pragma unroll
+        for (int k = 0; k < 10; ++k)
+#pragma unroll
+          for (int j = 0; j < 8; ++j) red[tx][k * 8 + j] = (r == 0 ? 0.f : red[tx][k * 8 + j]) + acc[k][j];
+      }
+      __syncthreads();
+    }
+    if (has) {
+      for (int k = ty * 20; k < ty * 20 + 20; ++k) {
+        const int tap = k >> 3, j = k & 7;
+        const size_t col = tap < 9 ? ((size_t)cv * 8 + j) * 9 + tap : (size_t)C * 9 + (size_t)cv * 8 + j;
+        prow[col] = red[tx][k];
+      }
+    }
+    __syncthreads();
+  }
+}
+
+int launch_column_sum(const float* partials, float* out, int n, int C, hipStream_t stream);
+
+size_t dwconv3x3_wgrad_workspace(int B, int C) { return (size_t)B * kWgradSplit * C * 10 * sizeof(float); }
+
+int launch_dwconv3x3_wgrad(const void* x, const void* dy, float* dw_db, void* workspace, int B, int h, int w, int C,
+                           int io_dtype, hipStream_t stream) {
+  if (B > 65535 || C % 8 != 0 || (long long)h * w > 0x7fffffffLL - 64 || (long long)C * 10 > 0x7fffffffLL) return -22;
+  const int ntiles = (h * w + 31) / 32;
+  const int split = ntiles < kWgradSplit ? ntiles : kWgradSplit;
+  const int tiles_per_wg = (ntiles + split - 1) / split;
+  const dim3 grid(split, B), block(256);
+  float* partials = static_cast<float*>(workspace);
+  if (io_dtype == 0)
+    hipLaunchKernelGGL((dwconv3x3_wgrad_kernel<float>), grid, block, 0, stream, (const float*)x, (const float*)dy,
+                       partials, h, w, C, tiles_per_wg);
+  else
+    hipLaunchKernelGGL((dwconv3x3_wgrad_kernel<uint16_t>), grid, block, 0, stream, (const uint16_t*)x,
+                       (const uint16_t*)dy, partials, h, w, C, tiles_per_wg);
+  if (hipGetLastError() != hipSuccess) return -5;
+  return launch_column_sum(partials, dw_db, split * B, C * 10, stream);
+}
+
+// ---------------------------------------------------------------------------
 // Backward of the RMS-norm blend epilogue, same thread layout as the forward.  With s = sig(g_lin),
 // on = rms(o) * w_g, ln = rms(local) * w_l, y0 = on * s + ln * (1 - s), y = silu_out ? y0 * sig(y0) : y0:
 //   dy0 = dy * d(y)/d(y0),  d_on = dy0 * s,  d_ln = dy0 * (1 - s),  d_glin = dy0 * (on - ln) * s * (1 - s),
@@ -651,8 +751,6 @@ __global__ __launch_bounds__(256) void locality_blend_bwd_kernel(
   if (threadIdx.x < 2 * Dv)
     partials[((size_t)blockIdx.y * gridDim.x + blockIdx.x) * (size_t)(2 * Dv) + threadIdx.x] = total;
 }
-
-int launch_column_sum(const float* partials, float* out, int n, int C, hipStream_t stream);
 
 size_t locality_blend_bwd_workspace(int B, int L, int Dv) {
   return (size_t)B * ((L + 31) / 32) * 2 * Dv * sizeof(float);

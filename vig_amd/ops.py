@@ -304,7 +304,7 @@ def dwconv3x3(x: torch.Tensor, weight: torch.Tensor, hw, bias: Optional[torch.Te
               silu: bool = False) -> torch.Tensor:
     """x [B,L,C] on the (h,w) token grid; weight [C,1,3,3] or [C,3,3]; returns [B,L,C].
     Differentiable: when autograd is recording and x, weight or bias requires grad, the input gradient is the same
-    stencil kernel run with the taps mirrored, the weight and bias gradients are reductions over batch and grid."""
+    stencil kernel run with the taps mirrored, the weight and bias gradients come from vig_dwconv3x3_bwd_weight."""
     if torch.is_grad_enabled() and any(t is not None and t.requires_grad for t in (x, weight, bias)):
         y = _DWConv3x3Function.apply(x, weight, bias, tuple(hw))
         return torch.nn.functional.silu(y) if silu else y
@@ -329,13 +329,20 @@ class _DWConv3x3Function(torch.autograd.Function):
         if ctx.needs_input_grad[0]:
             # dx[p] = sum_t w[t] dy[p - t]: the same stencil with the taps mirrored through the centre
             dx = _dwconv3x3_raw(dy, weight.detach().reshape(C, 9).flip(-1), ctx.hw, None, False)
-        if ctx.needs_input_grad[1]:
-            d4 = dy.reshape(B, h, w, C).float()
-            xp = torch.nn.functional.pad(x.reshape(B, h, w, C).float(), (0, 0, 1, 1, 1, 1))
-            dw = torch.stack([(d4 * xp[:, ky:ky + h, kx:kx + w]).sum((0, 1, 2)) for ky in range(3) for kx in range(3)],
-                             dim=1).reshape(weight.shape).to(weight.dtype)
-        if ctx.bias_dtype is not None and ctx.needs_input_grad[2]:
-            db = dy.float().sum((0, 1)).to(ctx.bias_dtype)
+        if ctx.needs_input_grad[1] or (ctx.bias_dtype is not None and ctx.needs_input_grad[2]):
+            lib = _lib.load()
+            x, dy = _dense(x), _dense(dy)
+            both = torch.empty(C * 10, dtype=torch.float32, device=x.device)
+            ws_bytes = lib.vig_dwconv3x3_bwd_weight_workspace(B, C)
+            ws = torch.empty(ws_bytes, dtype=torch.uint8, device=x.device)
+            with torch.cuda.device(x.device):
+                rc = lib.vig_dwconv3x3_bwd_weight(x.data_ptr(), dy.data_ptr(), both.data_ptr(), ws.data_ptr(), ws_bytes,
+                                                  B, h, w, C, _dt(x), _stream_ptr(x))
+            _lib.check(rc, "vig_dwconv3x3_bwd_weight")
+            if ctx.needs_input_grad[1]:
+                dw = both[:C * 9].reshape(weight.shape).to(weight.dtype)
+            if ctx.bias_dtype is not None and ctx.needs_input_grad[2]:
+                db = both[C * 9:].to(ctx.bias_dtype)
         return dx, dw, db, None
 
 
