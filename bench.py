@@ -151,7 +151,7 @@ def train_step_throughput(dev, batch=128, warmup=3, iters=10):
             loss = step()
         torch.cuda.synchronize(dev)
         dt = (time.perf_counter() - t0) / iters
-        out[name] = {"images_per_s": batch / dt, "ms_per_step": dt * 1e3, "loss": float(loss)}
+        out[name] = {"images_per_s": batch / dt, "ms_per_step": dt * 1e3, "loss": float(loss.detach())}
         del model, opt
     return out
 
@@ -212,6 +212,8 @@ def main():
                     help="with --model: leave torch's GEMM solution tuning off (clean kernel traces)")
     ap.add_argument("--train", action="store_true",
                     help="also time ViG-S training steps (differentiable path of the shell; fp32 and bf16 autocast)")
+    ap.add_argument("--train-only", action="store_true",
+                    help="time only the ViG-S training steps and print their JSON line (clean kernel traces)")
     ap.add_argument("--no-graph", action="store_true",
                     help="with --model: eager forwards only (no HIP graph capture, no batch-16 latency)")
     ap.add_argument("--unfused-gate", action="store_true",
@@ -239,6 +241,15 @@ def main():
     assert torch.cuda.is_available(), "bench.py needs a GPU"
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
+
+    if args.train_only:
+        res = train_step_throughput(dev)
+        print(json.dumps({"metric": "ViG-S training step images/sec @224^2 (forward + backward + AdamW)",
+                          "value": res["bf16_autocast"]["images_per_s"], "unit": "images/s", "n_gpus": 1,
+                          "ms_per_step": res["bf16_autocast"]["ms_per_step"], "higher_is_better": True,
+                          "dtype": "bf16 autocast", "data": "synthetic", "vs_baseline": None,
+                          "config": {"workload": "vig_s_train_step_B128_224"}, "detail": res}))
+        return
 
     s = CONFIGS[args.config]
     dt = torch_dtype(s.dtype)
