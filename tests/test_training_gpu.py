@@ -122,3 +122,39 @@ def test_vig_training_step():
     after = torch.nn.functional.cross_entropy(model(images.cuda()), target.cuda())
     print(f"  loss {loss.item():.4f} -> {after.item():.4f}", flush=True)
     assert after.item() < loss.item()
+
+
+@pytest.mark.parametrize("channel_first", [False, True])
+def test_gla2d_training_path(channel_first):
+    """HierViG's GLA2D in training mode: the recorded forward equals the kernel forward, and the input gradient equals
+    autograd through the float64 restatement."""
+    announce(f"GLA2D training path, channel_first={channel_first}")
+    torch.manual_seed(1)
+    dim, H, hw = 96, 3, (9, 13)
+    m = layers.GLA2D(d_model=dim, expand_k=0.5, expand_v=1.0, num_heads=H, layernorm_eps=1e-6,
+                     use_act_in_conv=False, use_out_act=False, channel_first=channel_first)
+    with torch.no_grad():
+        for lin in (m.qkv_proj, m.g_proj, m.o_proj, m.gk_proj[0], m.gk_proj[1]):
+            lin.weight.mul_(8.0)
+    x = torch.randn(2, dim, *hw) if channel_first else torch.randn(2, *hw, dim)
+    cot = torch.randn_like(x)
+    sd = {k: v.detach().double() for k, v in m.state_dict().items()}
+    x64 = x.double().requires_grad_()
+    rows = (x64.permute(0, 2, 3, 1) if channel_first else x64).reshape(2, hw[0] * hw[1], dim)
+    want = R.gla_block_attn(sd, "", rows, hw, H, 1e-6, False, False, second_halving=False, differentiable=True)
+    want = want.reshape(2, *hw, dim)
+    if channel_first:
+        want = want.permute(0, 3, 1, 2)
+    (want * cot.double()).sum().backward()
+
+    m = m.cuda().train()
+    xg = x.cuda().requires_grad_()
+    got = m(xg)
+    (got * cot.cuda()).sum().backward()
+    with torch.no_grad():
+        kernel = m(x.cuda())
+    assert _rel(got.detach().cpu(), kernel.cpu()) <= 2e-4
+    assert _rel(got.detach().cpu(), want.detach()) <= 2e-4
+    e = _rel(xg.grad.cpu(), x64.grad)
+    print(f"  input-gradient max-rel err {e:.3e}", flush=True)
+    assert e <= 2e-4
