@@ -242,3 +242,21 @@ def test_split_heads_gradients(dtype):
 
     want = torch.cat((rows(cq), rows(ck), rows(cv)), dim=-1)
     assert torch.equal(qkv.grad, want)
+
+
+def test_rmsnorm_gradients_with_an_unused_output():
+    """Only one of the two outputs of the residual form is used: the other's gradient arrives as None."""
+    announce("rmsnorm gradients, one output unused")
+    torch.manual_seed(0)
+    x, r = torch.randn(20, 64, device="cuda"), torch.randn(20, 64, device="cuda")
+    w = torch.rand(64, device="cuda") + 0.5
+    for use in ("y", "sum"):
+        xg, rg, wg = x.clone().requires_grad_(), r.clone().requires_grad_(), w.clone().requires_grad_()
+        y, s = vig_amd.ops.rmsnorm(xg, wg, 1e-6, residual=rg, prenorm=True)
+        (y if use == "y" else s).sum().backward()
+        x2, r2, w2 = x.clone().requires_grad_(), r.clone().requires_grad_(), w.clone().requires_grad_()
+        s2 = x2 + r2
+        y2 = s2 * torch.rsqrt(s2.pow(2).mean(-1, keepdim=True) + 1e-6) * w2
+        (y2 if use == "y" else s2).sum().backward()
+        assert torch.allclose(xg.grad, x2.grad, rtol=1e-4, atol=1e-5) and torch.equal(xg.grad, rg.grad)
+        assert torch.allclose(wg.grad, w2.grad if w2.grad is not None else torch.zeros_like(w), rtol=1e-4, atol=1e-5)

@@ -514,6 +514,7 @@ class _RMSNormFunction(torch.autograd.Function):
     def forward(ctx, x, residual, weight, eps, round_sum):
         y, total = _rmsnorm_raw(x, weight, eps, residual, True, round_sum)
         ctx.save_for_backward(total, weight)
+        ctx.set_materialize_grads(False)  # an unused output hands backward None instead of a tensor of zeros
         ctx.eps, ctx.has_residual = eps, residual is not None
         return y if residual is None else (y, total)
 
@@ -523,7 +524,7 @@ class _RMSNormFunction(torch.autograd.Function):
         lib = _lib.load()
         C = total.shape[-1]
         rows = total.numel() // C
-        dy = _dense(dy)
+        dy = _dense(dy) if dy is not None else torch.zeros_like(total)
         if d_total is not None:
             d_total = _dense(d_total)
         w = _dense(weight.detach().float())
