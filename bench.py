@@ -76,20 +76,7 @@ def model_throughput(dev, batch=256, warmup=10, iters=30, tune_gemm=True, use_gr
 
     from vig_amd import layers
 
-    # the block's GEMMs are hipBLASLt calls made by torch; let torch pick the fastest solution per shape
-    tuned = False
-    try:
-        if not tune_gemm:
-            raise RuntimeError("switched off")
-        import torch.cuda.tunable as tunable
-        import tempfile
-        tunable.enable(True)
-        tunable.tuning_enable(True)
-        tunable.set_max_tuning_duration(200)
-        tunable.set_filename(os.path.join(tempfile.gettempdir(), "vig_bench_gemm_solutions.csv"))
-        tuned = True
-    except Exception as e:  # noqa: BLE001 - tuning is optional plumbing
-        log(f"GEMM tuning unavailable: {e}")
+    tuned = _enable_gemm_tuning(tune_gemm)
     torch.manual_seed(0)
     model = layers.vig_small().eval().to(dev, torch.bfloat16)
     images = torch.randn(batch, 3, 224, 224, device=dev, dtype=torch.bfloat16)
@@ -119,15 +106,34 @@ def model_throughput(dev, batch=256, warmup=10, iters=30, tune_gemm=True, use_gr
     return out
 
 
-def train_step_throughput(dev, batch=128, warmup=3, iters=10):
+def _enable_gemm_tuning(tune_gemm):
+    """The GEMMs are hipBLASLt calls made by torch; let torch pick the fastest solution per shape."""
+    try:
+        if not tune_gemm:
+            raise RuntimeError("switched off")
+        import tempfile
+
+        import torch.cuda.tunable as tunable
+        tunable.enable(True)
+        tunable.tuning_enable(True)
+        tunable.set_max_tuning_duration(200)
+        tunable.set_filename(os.path.join(tempfile.gettempdir(), "vig_bench_gemm_solutions.csv"))
+        return True
+    except Exception as e:  # noqa: BLE001 - tuning is optional plumbing
+        log(f"GEMM tuning unavailable: {e}")
+        return False
+
+
+def train_step_throughput(dev, batch=128, warmup=3, iters=10, tune_gemm=True):
     """ViG-S training steps (forward, cross-entropy, backward, AdamW update) on synthetic images: the differentiable
-    path of the shell, whose GLA forward and backward run on the library's kernels.  fp32 as the reference's configs
-    train (vig-s.yaml: AMP off), and bf16 autocast."""
+    path of the shell, whose kernels between the GEMMs are the library's in both directions.  fp32 as the reference's
+    configs train (vig-s.yaml: AMP off), and bf16 autocast."""
     import torch
 
     from vig_amd import layers
 
-    out = {"batch": batch, "iters": iters}
+    tuned = _enable_gemm_tuning(tune_gemm)
+    out = {"batch": batch, "iters": iters, "gemm_solution_tuning": "torch.cuda.tunable" if tuned else None}
     images = torch.randn(batch, 3, 224, 224, device=dev)
     target = torch.randint(0, 1000, (batch,), device=dev)
     for name, amp in (("fp32", False), ("bf16_autocast", True)):
@@ -209,7 +215,7 @@ def main():
                     help="also time the backward of the op on the same workload; on by default for the headline workload")
     ap.add_argument("--op-only", action="store_true", help="no model forward and no backward, whatever the workload")
     ap.add_argument("--no-gemm-tuning", action="store_true",
-                    help="with --model: leave torch's GEMM solution tuning off (clean kernel traces)")
+                    help="with --model / --train: leave torch's GEMM solution tuning off (clean kernel traces)")
     ap.add_argument("--train", action="store_true",
                     help="also time ViG-S training steps (differentiable path of the shell; fp32 and bf16 autocast)")
     ap.add_argument("--train-only", action="store_true",
@@ -243,7 +249,7 @@ def main():
     torch.cuda.set_device(dev)
 
     if args.train_only:
-        res = train_step_throughput(dev)
+        res = train_step_throughput(dev, tune_gemm=not args.no_gemm_tuning)
         print(json.dumps({"metric": "ViG-S training step images/sec @224^2 (forward + backward + AdamW)",
                           "value": res["bf16_autocast"]["images_per_s"], "unit": "images/s", "n_gpus": 1,
                           "ms_per_step": res["bf16_autocast"]["ms_per_step"], "higher_is_better": True,
@@ -383,7 +389,7 @@ def main():
                 out["backward"]["traffic"] = None
     if want_model:
         if args.train:
-            out["vig_s_train_step"] = train_step_throughput(dev)
+            out["vig_s_train_step"] = train_step_throughput(dev, tune_gemm=not args.no_gemm_tuning)
         out["vig_s_forward"] = model_throughput(dev, tune_gemm=not args.no_gemm_tuning, use_graph=not args.no_graph)
     if not args.no_cpu:
         out["cpu_baseline"] = cpu_baseline(s, 1000 + args.config)
