@@ -92,7 +92,7 @@ def test_autograd_through_the_wrappers():
     assert _rel(f64(tq2.grad), want[0]) <= 1e-4
 
 
-# ---- the matrix-core backward (bf16 tensors and gates, Dk = Dv = 64, L <= 256, both directions) ----
+# ---- the matrix-core backward (bf16 tensors and gates, Dk in {32, 64}, Dv = 64, L <= 256) ----
 MFMA_BWD_TOL = 2e-2  # max |error| over the gradient's largest magnitude (bf16 operands, fp32 accumulation)
 
 
@@ -177,3 +177,21 @@ def test_random_shapes_matrix_core_paths_against_exact_paths():
             assert torch.isfinite(g_.float()).all(), (case, name)
             den = max(float(w_.float().abs().max()), floor if name.startswith("dg") else 0.0, 1e-30)
             assert float((g_.float() - w_.float()).abs().max()) / den <= MFMA_BWD_TOL, (case, name)
+
+
+@pytest.mark.parametrize("B,H,L,Dk", [(2, 2, 1, 64), (1, 3, 33, 64), (2, 6, 196, 64), (1, 2, 256, 64), (2, 3, 70, 32),
+                                      (3, 6, 196, 32), (80, 6, 196, 32)])
+def test_backward_mfma_causal(B, H, L, Dk):
+    """The one-direction (causal) op's backward on the matrix cores: the forward direction alone, against the adjoint
+    recurrence for small cases and against the fp32-arithmetic kernel for the many-slab case."""
+    announce(f"causal backward on the matrix cores B{B} H{H} L={L} Dk={Dk}")
+    q, k, v, gf, _ = make_gla_inputs(B, H, L, Dk, 64, seed=900 + L + B, dtype=torch.bfloat16)
+    do = _do(v.shape, 13, torch.bfloat16)
+    dev = [t.cuda() for t in (q, k, v, gf)]
+    got = vig_amd.gla_bidir_backward(*dev, None, do.cuda(), out_scale=1.0)
+    assert got[4] is None
+    if B * H <= 64:
+        want = O.gla_recurrent_backward(f64(q), f64(k), f64(v), f64(gf), f64(do))
+    else:
+        want = [f64(t) for t in vig_amd.gla_bidir_backward(*dev, None, do.cuda(), out_scale=1.0, exact=True)[:4]]
+    _check_mfma(got[:4], want, q)

@@ -274,7 +274,7 @@ int launch_gla_backward(const void* q, const void* k, const void* v, const void*
   GlaBwdArgs a{q, k, v, g_fwd, g_bwd, d_o, dq, dk, dv, dg_fwd, dg_bwd, workspace, B, H, L, Dk, Dv,
                scale, out_scale, io_dtype, gate_dtype, stream, nullptr};
   if (!exact && gla_backward_mfma_supported(L, Dk, Dv, io_dtype, gate_dtype, g_bwd != nullptr)) {
-    int* flags = reinterpret_cast<int*>((float*)workspace + recurrent_floats(B, H, L, Dk, Dv, 1));
+    int* flags = reinterpret_cast<int*>((float*)workspace + recurrent_floats(B, H, L, Dk, Dv, g_bwd != nullptr));
     const int rc = launch_gla_backward_mfma(q, k, v, g_fwd, g_bwd, d_o, dq, dk, dv, dg_fwd, dg_bwd, flags, B, H, L,
                                             Dk, scale * out_scale, stream);
     if (rc != 0) return rc;

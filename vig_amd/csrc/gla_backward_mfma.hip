@@ -120,17 +120,18 @@ __device__ __forceinline__ void issue_bwd_loads(const BwdNext& n, int w, int r, 
 }
 
 // One direction of one slab, for wave w (tile w).  dv accumulates over both directions (raw, unscaled).  The first
-// direction (LAST = false) stages v and do and parks its dq and dk, rounded to bf16, in the output tensors; the second
-// adds its own to them and stores dq, dk, dv.  Returns false, for every wave alike and before it has stored anything,
+// direction (FIRST, not LAST) stages v and do and parks its dq and dk, rounded to bf16, in the output tensors; the
+// second (LAST, not FIRST) adds its own to them and stores dq, dk, dv.  A one-direction (causal) launch runs a single
+// direction that is both.  Returns false, for every wave alike and before it has stored anything,
 // when the gates are out of range.
-template <bool FWD, bool LAST, int NG>
+template <bool FWD, bool FIRST, bool LAST, int NG>
 __device__ __forceinline__ bool bwd_direction(const BwdSlab& sl, int L, int ntiles, int w, int lane, char* lds,
                                               float s, f32x16_t (&dv)[2], u32x4_t (&keepq)[NG], u32x4_t (&keepk)[NG],
                                               BwdLoads<NG>& ld, const BwdNext& nxt, bool first_slab) {
   // where the first direction's dq, dk (bf16) wait for the second: in registers when the kernel has them to spare
   // (Dk = 32), else parked in the output tensors
   constexpr bool kKeepInRegs = NG == 2;
-  constexpr bool stage_vdo = !LAST;
+  constexpr bool stage_vdo = FIRST;
   constexpr int DK = 16 * NG;   // channels of q, k and the gates
   constexpr int HC = 8 * NG;    // channels per lane half
   asm volatile("" : "+v"(lane));  // per-lane constants are rebuilt per direction instead of living across the slab loop
@@ -258,11 +259,11 @@ __device__ __forceinline__ bool bwd_direction(const BwdSlab& sl, int L, int ntil
   // the first direction parked its dq and dk (rounded to bf16) in the output tensors; fetch them under the loops
   const rsrc_t oq = chunk_rsrc(sl.dq + tk, rows, 2 * DK), okk = chunk_rsrc(sl.dk + tk, rows, 2 * DK);
   u32x4_t prevq[NG], prevk[NG];
-  if (LAST && kKeepInRegs) {
+  if (!FIRST && kKeepInRegs) {
 #pragma unroll
     for (int gq = 0; gq < NG; ++gq) prevq[gq] = keepq[gq], prevk[gq] = keepk[gq];
   }
-  if (LAST && !kKeepInRegs) {
+  if (!FIRST && !kKeepInRegs) {
 #pragma unroll
     for (int gq = 0; gq < NG; ++gq) {
       const unsigned off = (unsigned)r * (2u * DK) + (2u * HC) * h + 16u * gq;
@@ -339,7 +340,7 @@ __device__ __forceinline__ bool bwd_direction(const BwdSlab& sl, int L, int ntil
           X[p][c] = s * (qt * dqc - kt * dkc);
           a[p] = s * exp2_fast(x[p][c]) * dqc;
           b[p] = s * exp2_fast(-x[p][c]) * dkc;
-          if (LAST) {
+          if (!FIRST) {
             a[p] += p ? bf16hi_to_f32(prevq[gq][m]) : bf16lo_to_f32(prevq[gq][m]);
             b[p] += p ? bf16hi_to_f32(prevk[gq][m]) : bf16lo_to_f32(prevk[gq][m]);
           }
@@ -412,7 +413,7 @@ __device__ __forceinline__ bool bwd_direction(const BwdSlab& sl, int L, int ntil
 
 }  // namespace
 
-template <int NG>
+template <int NG, bool BIDIR>
 __global__ __launch_bounds__(512) void gla_backward_mfma_kernel(
     const uint16_t* __restrict__ q, const uint16_t* __restrict__ k, const uint16_t* __restrict__ v,
     const uint16_t* __restrict__ gf, const uint16_t* __restrict__ gb, const uint16_t* __restrict__ d_o,
@@ -425,7 +426,8 @@ __global__ __launch_bounds__(512) void gla_backward_mfma_kernel(
   const int ntiles = (L + 31) / 32;
   auto slab_of = [&](int i) {
     const size_t bk = (size_t)i * L * (16 * NG), bv = (size_t)i * L * 64;
-    return BwdSlab{q + bk, k + bk, v + bv, gf + bk, gb + bk, d_o + bv, dq + bk, dk + bk, dv + bv, dgf + bk, dgb + bk};
+    return BwdSlab{q + bk, k + bk, v + bv, gf + bk, BIDIR ? gb + bk : nullptr, d_o + bv, dq + bk, dk + bk, dv + bv,
+                   dgf + bk, BIDIR ? dgb + bk : nullptr};
   };
   const int r = lane & 31, h = lane >> 5;
   BwdLoads<NG> ld;
@@ -441,10 +443,18 @@ __global__ __launch_bounds__(512) void gla_backward_mfma_kernel(
     f32x16_t dvacc[2] = {{0.f}, {0.f}};
     u32x4_t keepq[NG], keepk[NG];
     const bool first_slab = slab == (int)blockIdx.x;
-    bool ok = bwd_direction<true, false, NG>(sl, L, ntiles, w, lane, lds, s, dvacc, keepq, keepk, ld, second, first_slab);
-    if (ok) {
-      lds_barrier();  // (5) the dg scratch of direction 1 is dead before q~, k~ of direction 2 are staged
-      ok = bwd_direction<false, true, NG>(sl, L, ntiles, w, lane, lds, s, dvacc, keepq, keepk, ld, next_first, first_slab);
+    bool ok;
+    if constexpr (BIDIR) {
+      ok = bwd_direction<true, true, false, NG>(sl, L, ntiles, w, lane, lds, s, dvacc, keepq, keepk, ld, second,
+                                                first_slab);
+      if (ok) {
+        lds_barrier();  // (5) the dg scratch of direction 1 is dead before q~, k~ of direction 2 are staged
+        ok = bwd_direction<false, false, true, NG>(sl, L, ntiles, w, lane, lds, s, dvacc, keepq, keepk, ld, next_first,
+                                                   first_slab);
+      }
+    } else {  // the causal op: the forward direction alone, first and last at once
+      ok = bwd_direction<true, true, true, NG>(sl, L, ntiles, w, lane, lds, s, dvacc, keepq, keepk, ld, next_first,
+                                               first_slab);
     }
     // a direction that left early has not issued the loads of the slab that follows
     if (!ok) issue_bwd_loads<true, NG>(next_first, w, r, h, ld);
@@ -453,12 +463,6 @@ __global__ __launch_bounds__(512) void gla_backward_mfma_kernel(
   }
 }
 
-template __global__ void gla_backward_mfma_kernel<4>(const uint16_t*, const uint16_t*, const uint16_t*,
-                                                     const uint16_t*, const uint16_t*, const uint16_t*, uint16_t*,
-                                                     uint16_t*, uint16_t*, uint16_t*, uint16_t*, int*, int, int, float);
-template __global__ void gla_backward_mfma_kernel<2>(const uint16_t*, const uint16_t*, const uint16_t*,
-                                                     const uint16_t*, const uint16_t*, const uint16_t*, uint16_t*,
-                                                     uint16_t*, uint16_t*, uint16_t*, uint16_t*, int*, int, int, float);
 
 #ifdef VIG_TIMING
 extern "C" int vig_debug_read_bwd_stamps(unsigned long long* host_out) {
@@ -467,7 +471,8 @@ extern "C" int vig_debug_read_bwd_stamps(unsigned long long* host_out) {
 #endif
 
 bool gla_backward_mfma_supported(int L, int Dk, int Dv, int io_dtype, int gate_dtype, bool bidir) {
-  return bidir && io_dtype == 1 && gate_dtype == 1 && (Dk == 64 || Dk == 32) && Dv == 64 && L <= 32 * kBwdTiles;
+  (void)bidir;  // both the bidirectional and the causal op
+  return io_dtype == 1 && gate_dtype == 1 && (Dk == 64 || Dk == 32) && Dv == 64 && L <= 32 * kBwdTiles;
 }
 
 // flags: one int per (batch, head) slab, written by every launch: 1 = not computed here (gates out of range)
@@ -480,8 +485,10 @@ int launch_gla_backward_mfma(const void* q, const void* k, const void* v, const 
   int dev = 0;
   if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return -5;
   if (!attr_done_dev[dev]) {
-    const void* kernels[2] = {reinterpret_cast<const void*>(gla_backward_mfma_kernel<4>),
-                              reinterpret_cast<const void*>(gla_backward_mfma_kernel<2>)};
+    const void* kernels[4] = {reinterpret_cast<const void*>(gla_backward_mfma_kernel<4, true>),
+                              reinterpret_cast<const void*>(gla_backward_mfma_kernel<2, true>),
+                              reinterpret_cast<const void*>(gla_backward_mfma_kernel<4, false>),
+                              reinterpret_cast<const void*>(gla_backward_mfma_kernel<2, false>)};
     for (const void* kf : kernels)
       if (hipFuncSetAttribute(kf, hipFuncAttributeMaxDynamicSharedMemorySize, kBwdLdsTotal) != hipSuccess) return -5;
     int n = 0;
@@ -491,13 +498,18 @@ int launch_gla_backward_mfma(const void* q, const void* k, const void* v, const 
   }
   const int nslabs = B * H;
   const int grid = nslabs < num_cu_dev[dev] ? nslabs : num_cu_dev[dev];
-#define VIG_BWD_LAUNCH(NG)                                                                                          \
-  hipLaunchKernelGGL(gla_backward_mfma_kernel<NG>, dim3(grid), dim3(512), kBwdLdsTotal, stream, (const uint16_t*)q, \
-                     (const uint16_t*)k, (const uint16_t*)v, (const uint16_t*)gf, (const uint16_t*)gb,              \
-                     (const uint16_t*)d_o, (uint16_t*)dq, (uint16_t*)dk, (uint16_t*)dv, (uint16_t*)dgf,             \
-                     (uint16_t*)dgb, flags, nslabs, L, s)
-  if (Dk == 64) VIG_BWD_LAUNCH(4);
-  else VIG_BWD_LAUNCH(2);
+#define VIG_BWD_LAUNCH(NG, BIDIR)                                                                               \
+  hipLaunchKernelGGL((gla_backward_mfma_kernel<NG, BIDIR>), dim3(grid), dim3(512), kBwdLdsTotal, stream,         \
+                     (const uint16_t*)q, (const uint16_t*)k, (const uint16_t*)v, (const uint16_t*)gf,            \
+                     (const uint16_t*)gb, (const uint16_t*)d_o, (uint16_t*)dq, (uint16_t*)dk, (uint16_t*)dv,     \
+                     (uint16_t*)dgf, (uint16_t*)dgb, flags, nslabs, L, s)
+  if (gb) {
+    if (Dk == 64) VIG_BWD_LAUNCH(4, true);
+    else VIG_BWD_LAUNCH(2, true);
+  } else {
+    if (Dk == 64) VIG_BWD_LAUNCH(4, false);
+    else VIG_BWD_LAUNCH(2, false);
+  }
 #undef VIG_BWD_LAUNCH
   return hipGetLastError() == hipSuccess ? 0 : -5;
 }
