@@ -260,3 +260,31 @@ def test_rmsnorm_gradients_with_an_unused_output():
         (y2 if use == "y" else s2).sum().backward()
         assert torch.allclose(xg.grad, x2.grad, rtol=1e-4, atol=1e-5) and torch.equal(xg.grad, rg.grad)
         assert torch.allclose(wg.grad, w2.grad if w2.grad is not None else torch.zeros_like(w), rtol=1e-4, atol=1e-5)
+
+
+def test_backward_entry_points_validate_arguments():
+    """Null pointers, unsupported widths and short workspaces are refused with the documented codes before any launch."""
+    announce("argument validation of the block's backward entry points")
+    from vig_amd import _lib
+    lib = _lib.load()
+    x = torch.zeros(64, 384, device="cuda", dtype=torch.bfloat16)
+    w = torch.ones(384, device="cuda")
+    p, wp, st = x.data_ptr(), w.data_ptr(), torch.cuda.current_stream().cuda_stream
+    bf = _lib.VIG_BF16
+    assert lib.vig_swiglu_bwd(None, p, p, 64, 192, bf, st) == _lib.VIG_EINVAL
+    assert lib.vig_swiglu_bwd(p, p, p, 64, 190, bf, st) == _lib.VIG_ENOTSUP
+    assert lib.vig_rmsnorm_bwd(p, wp, None, None, p, None, None, 0, 64, 384, 1e-6, bf, st) == _lib.VIG_EINVAL
+    assert lib.vig_rmsnorm_bwd(p, wp, p, None, p, None, None, 0, 64, 2048, 1e-6, bf, st) == _lib.VIG_ENOTSUP
+    assert lib.vig_rmsnorm_bwd(p, wp, p, None, p, wp, p, 16, 64, 384, 1e-6, bf, st) == _lib.VIG_ENOSPC
+    assert lib.vig_rmsnorm_bwd_workspace(64, 384) == 4 * 384 * 4 and lib.vig_rmsnorm_bwd_workspace(0, 384) == 0
+    assert lib.vig_dirgate_bwd(p, None, p, 1, 64, 3, 64, 1 / 16, float("nan"), bf, bf, st) == _lib.VIG_EINVAL
+    assert lib.vig_dirgate_bwd(p, p, p, 1, 64, 3, 12, 1 / 16, float("nan"), bf, bf, st) == _lib.VIG_ENOTSUP
+    assert lib.vig_split_heads_bwd(p, p, None, p, 1, 64, 3, 32, 64, bf, st) == _lib.VIG_EINVAL
+    assert lib.vig_dwconv3x3_bwd_weight(p, p, wp, p, 16, 1, 8, 8, 384, bf, st) == _lib.VIG_ENOSPC
+    assert lib.vig_dwconv3x3_bwd_weight(p, p, wp, None, 0, 1, 8, 8, 380, bf, st) == _lib.VIG_ENOTSUP
+    assert lib.vig_locality_blend_bwd(p, p, p, wp, wp, p, p, p, p, wp, p, 16, 1, 6, 64, 64, 0, 1e-6, 0, bf,
+                                      st) == _lib.VIG_ENOSPC
+    assert lib.vig_locality_blend_bwd(p, p, p, wp, wp, p, p, p, p, wp, p, 1 << 20, 1, 6, 64, 48, 0, 1e-6, 0, bf,
+                                      st) == _lib.VIG_ENOTSUP
+    assert lib.vig_locality_blend_bwd_workspace(2, 64, 48) == 0
+    torch.cuda.synchronize()
