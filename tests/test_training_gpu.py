@@ -89,7 +89,7 @@ def test_vig_training_step():
     training branch, then one SGD step lowers the loss."""
     announce("ViG (64x64 images, depth 2, dim 96) training step, fp32")
     torch.manual_seed(0)
-    kw = dict(img_size=64, depth=2, num_heads=3, embed_dim=96, num_classes=10)
+    kw = dict(img_size=64, depth=2, num_heads=3, embed_dim=96, num_classes=10, drop_path_rate=0.0)
     model = layers.ViG(**kw)
     with torch.no_grad():
         for blk in model.blocks:
@@ -158,3 +158,30 @@ def test_gla2d_training_path(channel_first):
     e = _rel(xg.grad.cpu(), x64.grad)
     print(f"  input-gradient max-rel err {e:.3e}", flush=True)
     assert e <= 2e-4
+
+
+def test_drop_path():
+    """Stochastic depth of the block's branches (vig.py:533,606-608): per-sample masks scaled by 1/keep in training
+    mode with the linear rate rule over depth; identity in eval mode, so inference is unchanged."""
+    announce("DropPath: masks, scaling, rate rule, eval identity")
+    torch.manual_seed(0)
+    dp = layers.DropPath(0.25).train()
+    x = torch.ones(4000, 3, 5, device="cuda")
+    y = dp(x)
+    per_sample = y.reshape(4000, -1)
+    assert bool(((per_sample == 0).all(1) | (per_sample == 1 / 0.75).all(1)).all())  # whole samples, kept ones scaled
+    kept = float((per_sample[:, 0] != 0).float().mean())
+    assert abs(kept - 0.75) < 0.03
+    assert torch.equal(dp.eval()(x), x)
+    model = layers.ViG(img_size=64, depth=4, num_heads=3, embed_dim=96, num_classes=10, drop_path_rate=0.3)
+    rates = [getattr(b.drop_path, "drop_prob", 0.0) for b in model.blocks]
+    assert rates[0] == 0.0 and abs(rates[-1] - 0.3) < 1e-6 and abs(rates[1] - 0.1) < 1e-6
+    model = model.cuda()
+    images = torch.randn(8, 3, 64, 64, device="cuda")
+    a = model.eval()(images)
+    assert torch.equal(a, model(images))  # eval: deterministic
+    model.train()
+    b, c = model(images), model(images)
+    assert b.requires_grad and not torch.equal(b, c)  # training: masks differ from call to call
+    b.sum().backward()
+    assert all(p.grad is not None and torch.isfinite(p.grad).all() for p in model.parameters())

@@ -272,13 +272,36 @@ class GLAMLP(nn.Module):
         return self.down_proj(ops.swiglu(self.gate_proj(x)))
 
 
+class DropPath(nn.Module):
+    """Stochastic depth: in training mode a branch is dropped per sample with probability drop_prob and the kept
+    ones are scaled by 1 / (1 - drop_prob); identity otherwise (timm's DropPath as used at vig.py:533,606-608)."""
+
+    def __init__(self, drop_prob: float = 0.0, scale_by_keep: bool = True):
+        super().__init__()
+        self.drop_prob, self.scale_by_keep = float(drop_prob), scale_by_keep
+
+    def forward(self, x):
+        if self.drop_prob == 0.0 or not self.training:
+            return x
+        keep = 1.0 - self.drop_prob
+        mask = x.new_empty((x.shape[0],) + (1,) * (x.dim() - 1)).bernoulli_(keep)
+        if keep > 0.0 and self.scale_by_keep:
+            mask.div_(keep)
+        return x * mask
+
+    def extra_repr(self):
+        return f"drop_prob={self.drop_prob:0.3f}"
+
+
 class GLABlock(nn.Module):
-    """attn_norm -> GLA -> (residual add + mlp_norm, prenorm) -> MLP -> residual (vig.py:530-618), no layer scale."""
+    """attn_norm -> GLA -> (residual add + mlp_norm, prenorm) -> MLP -> residual (vig.py:530-618), no layer scale;
+    drop_path is the stochastic-depth rate of both branches (vig.py:533,606-608)."""
 
     def __init__(self, hidden_size: int, num_heads: int, expand_k: float, expand_v: float, eps: float = 1e-6,
                  use_out_act: bool = False, use_act_in_conv: bool = True, use_bias_in_dwconv: bool = False,
-                 intermediate_size: Optional[int] = None, mode: str = "fused_chunk"):
+                 intermediate_size: Optional[int] = None, mode: str = "fused_chunk", drop_path: float = 0.0):
         super().__init__()
+        self.drop_path = DropPath(drop_path) if drop_path > 0.0 else nn.Identity()
         self.attn_norm = RMSNorm(hidden_size, eps=eps)
         self.attn = GatedLinearAttention(d_model=hidden_size, expand_k=expand_k, expand_v=expand_v,
                                          num_heads=num_heads, layernorm_eps=eps, mode=mode, use_out_act=use_out_act,
@@ -289,8 +312,8 @@ class GLABlock(nn.Module):
     def forward(self, hidden_states, **kwargs):
         residual = hidden_states
         h = self.attn(self.attn_norm(hidden_states), **kwargs)
-        h, residual = self.mlp_norm(h, residual, True)
-        return (residual + self.mlp(h),)
+        h, residual = self.mlp_norm(self.drop_path(h), residual, True)
+        return (residual + self.drop_path(self.mlp(h)),)
 
     def forward_carry(self, branch, residual, **kwargs):
         """Same block, with the closing `residual + mlp(h)` of the previous block folded into this block's first norm:
@@ -300,8 +323,8 @@ class GLABlock(nn.Module):
         else:  # the explicit add stores a rounded sum and attn_norm normalises that (vig.py:598,606)
             h, hidden = self.attn_norm(branch, residual, True, round_sum=True)
         h = self.attn(h, **kwargs)
-        h, residual = self.mlp_norm(h, hidden, True)
-        return self.mlp(h), residual
+        h, residual = self.mlp_norm(self.drop_path(h), hidden, True)
+        return self.drop_path(self.mlp(h)), residual
 
 
 class LayerNorm2d(nn.LayerNorm):
@@ -399,17 +422,18 @@ class ViG(nn.Module):
 
     def __init__(self, img_size=224, patch_size=16, depth=12, num_heads=6, embed_dim=384, channels=3,
                  num_classes=1000, expand_k=0.5, expand_v=1.0, use_out_act=False, use_act_in_conv=False,
-                 use_bias_in_dwconv=False, rms_norm_eps=1e-6, initializer_range=0.02):
+                 use_bias_in_dwconv=False, rms_norm_eps=1e-6, initializer_range=0.02, drop_path_rate=0.1):
         super().__init__()
         self.embed_dim = embed_dim
+        dpr = [x.item() for x in torch.linspace(0, drop_path_rate, depth)]  # stochastic depth decay rule (vig.py:805)
         self.patch_embed = V2PatchEmbed(patch_size=patch_size, in_chans=channels, embed_dim=embed_dim)
         self.patch_resolution = (img_size // patch_size, img_size // patch_size)
         self.pos_embed = nn.Parameter(torch.zeros(1, self.patch_resolution[0] * self.patch_resolution[1], embed_dim))
         self.head = nn.Linear(embed_dim, num_classes)
         self.blocks = nn.ModuleList([
             GLABlock(embed_dim, num_heads, expand_k, expand_v, eps=rms_norm_eps, use_out_act=use_out_act,
-                     use_act_in_conv=use_act_in_conv, use_bias_in_dwconv=use_bias_in_dwconv)
-            for _ in range(depth)])
+                     use_act_in_conv=use_act_in_conv, use_bias_in_dwconv=use_bias_in_dwconv, drop_path=dpr[i])
+            for i in range(depth)])
         self.norm = RMSNorm(embed_dim, eps=rms_norm_eps)
         # init order of the reference (vig.py:825-837,332-349): every Linear N(0, 0.02) with zero bias, then the
         # GLA projections xavier-uniform with gain 2^-2.5; convs of the patch embedding keep torch's default
@@ -440,7 +464,8 @@ class ViG(nn.Module):
 
 
 def vig_small(**kw):
-    """vig-s.yaml: dim 384, 6 heads (Dk 32, Dv 64), depth 12."""
+    """vig-s.yaml: dim 384, 6 heads (Dk 32, Dv 64), depth 12, drop-path rate 0.2."""
+    kw.setdefault("drop_path_rate", 0.2)
     return ViG(depth=12, num_heads=6, embed_dim=384, use_out_act=False, use_act_in_conv=False, **kw)
 
 
@@ -450,5 +475,6 @@ def vig_tiny(**kw):
 
 
 def vig_base(**kw):
-    """vig-b.yaml: dim 768, 12 heads, depth 12."""
+    """vig-b.yaml: dim 768, 12 heads, depth 12, drop-path rate 0.5."""
+    kw.setdefault("drop_path_rate", 0.5)
     return ViG(depth=12, num_heads=12, embed_dim=768, use_out_act=False, use_act_in_conv=False, **kw)
