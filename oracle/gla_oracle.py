@@ -22,13 +22,16 @@ Pinning status (what fixes each function besides its own formula):
         index-by-index layout brute force.
   * locality_* / rmsnorm_reference       -- torch.nn.functional.conv2d and the
         reference's own closed formula; layout brute force.
+  * locality_sigmoid_gate_reference      -- tests/test_oracle_model.py: the library
+        convolution on an explicitly rearranged [B, C, h, w] tensor, an index-by-index
+        brute force on a 3 x 4 grid with H != Dv, zero / centre-tap / one-sided weights.
   * layernorm_reference                  -- torch.nn.functional.layer_norm (+ silu)
         in float64, and the mean-0 / variance-1 invariant.
   * naive_recurrent_gla_f32              -- float32 torch port of the reference's
         CPU-runnable routine; pinned against gla_recurrent (fp64) to 1e-5.
 The reference holds no golden vectors for this path (its tests are GPU-only
 kernel-vs-kernel comparisons), so nothing here is pinned by reference fixtures;
-the composed eval-mode model forward is "parity unpinned" and not restated here.
+the composed eval-mode model forward is restated in vig_model_ref.py and pinned there.
 """
 from __future__ import annotations
 

@@ -8,10 +8,15 @@ parameter names and follows the eval branch of the reference model:
   classification/models/vig.py:469-497  (GLAMLP, swiglu = silu(gate) * y)
   classification/models/vig.py:625-672  (V2PatchEmbed), :843-912 (forward_features, avgpool head)
   flash-linear-attention/fla/modules/rmsnorm.py:38-52 (RMS norm formula)
-PARITY UNPINNED: the reference cannot be imported here (missing timm / causal_conv1d / Triton-only
-modules), and it ships no golden logits, so the composed forward is pinned only by reading the source;
-each primitive it uses (conv2d, linear, logsigmoid, the GLA recurrence) is pinned separately in
-tests/test_oracle.py.
+The reference cannot be imported here (missing timm / causal_conv1d / Triton-only modules) and ships no
+golden logits.  Pinning: each primitive (conv2d, linear, logsigmoid, the GLA recurrence) is pinned in
+tests/test_oracle.py; the composition (op order, which norm takes which branch and weight, the channel map
+of 'b (h d) l -> b l h d', the second halving in front of g_norm, the un-normalised residual, the prenorm
+MLP input, row-major token order, pooling and head) by tests/test_oracle_model.py through special cases
+whose answers do not need the composed formula: saturated blend gates, zeroed output projections, eps = 0
+scale invariance against eps > 0 on small outputs, channel-constant biases in the stem, a single hot cell.
+What stays unpinned is only what no arithmetic check can reach: that the published checkpoints' keys mean
+what classification/models/vig.py says they mean (no weights are available offline).
 """
 from __future__ import annotations
 
