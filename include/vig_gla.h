@@ -60,8 +60,11 @@ const char* vig_gla_strerror(int code);
  *
  * Numeric range of the matrix-core path (bf16 tensors and gates, Dk in {32, 64},
  * Dv = 64): the sum of |g| over any 64 consecutive tokens of one channel must
- * stay below about 80, and |q|, |k| below about 1000 (beyond either, results
- * may be inf / NaN, never silently wrong finite numbers).  HierViG's head shape
+ * stay below about 80 (beyond it results may be inf / NaN, never silently wrong
+ * finite numbers).  q and k may hold any finite bf16 values: the kernel checks
+ * their magnitudes and the gate totals per chunk and takes its fp16-operand
+ * scores only where they are exact enough (|q|, |k| < 512, gate total of a chunk
+ * within about 8), split-bf16 scores otherwise.  HierViG's head shape
  * (bf16, Dk = 16, Dv = 32, both directions) takes the same path from L = 128 on,
  * zero-padded to Dk 32 / Dv 64 in the workspace (classification/models/vig_h.py:
  * 377-385 with EXPAND_K 0.5, EXPAND_V 1.0).  Other combinations run on the
@@ -74,7 +77,13 @@ int vig_gla_bidir_fwd(const void* q, const void* k, const void* v,
                       float scale, float out_scale,
                       int io_dtype, int gate_dtype, void* stream);
 
+/* Workspace that is enough for every gate dtype and for one or two directions (the largest over the kernels the
+ * call may dispatch to for this shape and io_dtype). */
 size_t vig_gla_bidir_fwd_workspace(int B, int H, int L, int Dk, int Dv, int io_dtype);
+/* Workspace of exactly the kernel vig_gla_bidir_fwd / _wide dispatch to for these arguments (bidirectional: g_bwd
+ * given): 0 for bf16 tensors and gates with Dk in {32, 64}, Dv = 64, L <= 256. */
+size_t vig_gla_bidir_fwd_workspace_for(int B, int H, int L, int Dk, int Dv, int io_dtype, int gate_dtype,
+                                       int bidirectional);
 
 /*
  * Same contract, workspace and accuracy bar as vig_gla_bidir_fwd, for callers who know their gates to be strong.

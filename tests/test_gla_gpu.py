@@ -158,6 +158,32 @@ def test_bf16_mixed_gate_strength_many_items():
     assert max_abs(got, want) <= BF16_TOL
 
 
+@pytest.mark.parametrize("qs,ks,L,Dk,everywhere", [(2000.0, 1.0, 196, 64, True), (1.0, 3000.0, 196, 64, True),
+                                                  (600.0, 600.0, 700, 64, True), (2000.0, 2000.0, 196, 32, True),
+                                                  (30000.0, 1.0, 196, 64, False), (1.0, 30000.0, 300, 64, False)])
+def test_bf16_large_magnitude_inputs(qs, ks, L, Dk, everywhere):
+    """|q| or |k| beyond what the fp16 score operands hold (raw value x 2^6 must stay below 65504): ordinary bf16
+    values, mild gates.  The kernel has to notice and take its split-bf16 scores; results finite and within the bf16
+    bar relative to the output scale.  `everywhere` False: a single large element in one slab of many."""
+    announce(f"bf16 default path, large inputs q x{qs} k x{ks} L={L} Dk={Dk} everywhere={everywhere}")
+    q, k, v, gf, gb = make_gla_inputs(5, 2, L, Dk, 64, seed=51, dtype=torch.bfloat16)
+    if everywhere:
+        q, k = (q.float() * qs).bfloat16(), (k.float() * ks).bfloat16()
+    else:
+        q, k = q.clone(), k.clone()
+        (q if qs > 1 else k)[3, 1, L // 2 + 7, 5] = max(qs, ks)
+    want = oracle_bidir(q, k, v, gf, gb)
+    got = f64(vig_amd.gla_bidir_forward(*dev(q, k, v, gf, gb)))
+    assert np.isfinite(got).all()
+    # the absolute bar of unit-scale inputs, scaled with the outputs (their bf16 grid alone is 2^-8 relative)
+    assert max_abs(got, want) <= BF16_TOL * max(1.0, np.abs(want).max() / 4.0)
+    if not everywhere:  # the slabs without the large element keep the plain absolute bar
+        ok = np.ones(5 * 2, dtype=bool)
+        ok[3 * 2 + 1] = False
+        d = np.abs(got - want).reshape(10, -1).max(axis=1)
+        assert (d[ok] <= BF16_TOL).all()
+
+
 @pytest.mark.parametrize("gate_scale,L,both", [(1.0, 196, True), (1.0 / 16, 196, True), (1.0, 700, True), (0.5, 130, False)])
 def test_bf16_wide_entry_point(gate_scale, L, both):
     """vig_gla_bidir_fwd_wide (starts with the split-bf16 score variant): same accuracy bar on strong and on mild

@@ -114,6 +114,20 @@ static size_t padded_workspace(int B, int H, int L) {
          vig::gla_mfma_workspace(B, H, L, 32, 64);
 }
 
+// What the path vig_gla_bidir_fwd dispatches to for exactly these arguments needs.
+static size_t fwd_workspace_exact(int B, int H, int L, int Dk, int Dv, int io_dtype, int gate_dtype, bool bidir) {
+  if (io_dtype == VIG_BF16 && gate_dtype == VIG_BF16 && (Dk == 64 || Dk == 32) && Dv == 64)
+    return vig::gla_mfma_workspace(B, H, L, Dk, Dv);
+  if (padded_shape(L, Dk, Dv, io_dtype, gate_dtype, bidir)) return padded_workspace(B, H, L);
+  return bidir ? vig::gla_recurrent_workspace(B, H, L, Dv, io_dtype) : 0;
+}
+
+size_t vig_gla_bidir_fwd_workspace_for(int B, int H, int L, int Dk, int Dv, int io_dtype, int gate_dtype,
+                                       int bidirectional) {
+  if (B <= 0 || H <= 0 || L <= 0 || !dtype_ok(io_dtype) || !dtype_ok(gate_dtype)) return 0;
+  return fwd_workspace_exact(B, H, L, Dk, Dv, io_dtype, gate_dtype, bidirectional != 0);
+}
+
 size_t vig_gla_bidir_fwd_workspace(int B, int H, int L, int Dk, int Dv, int io_dtype) {
   if (B <= 0 || H <= 0 || L <= 0) return 0;
   // The largest requirement over the paths the dispatcher may take for this shape.

@@ -19,8 +19,8 @@
 // bf16 once.  Loads for the next slab are issued before the swap.
 //
 // fp16 score operands need |G_end|/2 * log2(e) <= 6 in every channel of every chunk (ViG's
-// logsigmoid(.)/16 gates reach about 2.5) and inputs below 65504 / 64 in magnitude.  A
-// workgroup that meets a segment with stronger gates redoes it, and does all its later
+// logsigmoid(.)/16 gates reach about 2.5) and |q|, |k| below 512; every wave checks both for
+// its chunk.  A workgroup that meets a segment outside that range redoes it, and does all its later
 // segments, with bf16 hi + lo operands and three score terms per k-step (same algebra,
 // any gate total up to ~80 per chunk and channel).
 //
@@ -86,6 +86,24 @@ __device__ __forceinline__ uint32_t pack_f16x2(float lo, float hi) {
   f32x2_t x = {lo, hi};
   f16x2_t y = __builtin_convertvector(x, f16x2_t);  // round to nearest even
   return __builtin_bit_cast(uint32_t, y);
+}
+
+// Magnitude guard of the fp16 score variant.  Raw bf16 rows go through a 16x16x32 matrix instruction as both
+// operands: whatever the slot assignment, the result is a Gram matrix whose diagonal entries are sums of squares that
+// cover every value fed in and whose other entries are no larger than the largest diagonal one.  Eight passes and four
+// accumulator registers per step, no vector work until the one comparison at the end.
+typedef float f32x4acc_t __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ void gram_acc(const u32x4_t& raw, f32x4acc_t& acc) {
+  acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, raw), __builtin_bit_cast(bf16x8_t, raw), acc,
+                                                0, 0, 0);
+}
+// fp16 operands are raw * 2^x with |x| <= kFastHalfRange = 6: they stay finite while |raw| < 65504 / 64.  The guard
+// asks for every sum of squares below 2^18, i.e. every |raw| < 512 (inf or huge inputs fail it; NaN inputs give NaN
+// outputs on every path).
+constexpr float kFastMaxSquares = 262144.0f;
+__device__ __forceinline__ bool gram_too_large(const f32x4acc_t& acc) {
+  const float m = fmaxf(fmaxf(fabsf(acc[0]), fabsf(acc[1])), fmaxf(fabsf(acc[2]), fabsf(acc[3])));
+  return __builtin_amdgcn_ballot_w64(!(m < kFastMaxSquares)) != 0;
 }
 
 template <int NG>
@@ -255,8 +273,9 @@ constexpr int kStateFloats = 64 * 64 + 64;  // per (sequence, segment, direction
 // and V fragments are fetched while the first is worked on.
 //   F16: score operands are single fp16 roundings (valid while the chunk's gate totals keep them inside fp16 range);
 //   otherwise bf16 hi + lo pairs and three MFMA terms per k-step.
+// Returns (F16 only, wave-uniform) whether some raw q or k value of the chunk is too large for fp16 operands.
 template <bool FWD, int MODE, int NG, bool F16>
-__device__ __forceinline__ void tile_phase(const ChunkSrc& cur, const Prefetch<NG>& pf, const f32x16_t (&G)[2][2],
+__device__ __forceinline__ bool tile_phase(const ChunkSrc& cur, const Prefetch<NG>& pf, const f32x16_t (&G)[2][2],
                                            const float* gend2, uint16_t* kt, int r, int h, f32x16_t (&O)[2][2],
                                            u32x4_t (&qkeep)[2][NG], u32x4_t (&vfrag)[4][2]) {
   constexpr bool OUT = MODE != kModeState;
@@ -282,7 +301,14 @@ __device__ __forceinline__ void tile_phase(const ChunkSrc& cur, const Prefetch<N
     issue_raw_tile<NG>(cur.k, TB, r, h, rawk);
     issue_tdwords<2 * TB, 2, 4>(cur.v, r, h, vDb);
   };
+  bool too_large = false;
   if (F16) {
+    f32x4acc_t gram = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int g = 0; g < NG; ++g) {
+      gram_acc(pf.rawk[g], gram);
+      if (OUT) gram_acc(pf.rawq[g], gram);
+    }
     u32x4_t ka[NG], qb[NG];
     // the second tile's loads go out before the first tile's operands are built where registers allow it (measured:
     // earlier is better for whole slabs, later for the chained segments of long sequences)
@@ -299,6 +325,11 @@ __device__ __forceinline__ void tile_phase(const ChunkSrc& cur, const Prefetch<N
       if (OUT) apply_scores<MASK>(score_tile16<NG>(ka, qa), TA, r, h, vfrag, O[0][TA], O[1][TA]);
     }
     VIG_PHASE();
+#pragma unroll
+    for (int g = 0; g < NG; ++g) {
+      gram_acc(rawk[g], gram);
+      if (OUT) gram_acc(rawq[g], gram);
+    }
     u32x4_t kb[NG];
     {
       u32x4_t kbb[NG];
@@ -309,6 +340,7 @@ __device__ __forceinline__ void tile_phase(const ChunkSrc& cur, const Prefetch<N
     VIG_PHASE();
     set_vfrag(vDb, 2 * TB);
     if (OUT) apply_scores<MASK>(score_tile16<NG>(kb, qb), TB, r, h, vfrag, O[0][TB], O[1][TB]);
+    too_large = gram_too_large(gram);
   } else {
     HalfOps<NG> ka, qb;
     {
@@ -343,6 +375,7 @@ __device__ __forceinline__ void tile_phase(const ChunkSrc& cur, const Prefetch<N
       for (int ks = 0; ks < NG; ++ks) qkeep[TB][ks] = qb.h[ks];
     }
   }
+  return too_large;
 }
 
 
@@ -460,7 +493,7 @@ __device__ __forceinline__ bool direction_wave(const ChunkSrc& cur, const ChunkS
   f32x16_t O[2][2];
   u32x4_t qkeep[2][NG];
   u32x4_t vfrag[4][2];
-  tile_phase<FWD, MODE, NG, F16>(cur, pf, G, gend2, kt, r, h, O, qkeep, vfrag);
+  if (tile_phase<FWD, MODE, NG, F16>(cur, pf, G, gend2, kt, r, h, O, qkeep, vfrag)) fast = false;
   VIG_STAMP(3);
   wave_lds_sync();  // k~ rows of this wave visible to its other lanes
   VIG_STAMP(4);

@@ -5,8 +5,9 @@ Mirrors (same names, positional order, defaults and return convention):
   batch_bid_fused_chunk_gla    fla/ops/gla/chunk_fuse.py:574-596
   bid_fused_recurrent_gla      fla/ops/gla/recurrent_fuse.py:659-676
   fused_recurrent_gla          fla/ops/gla/recurrent_fuse.py:631-657
-Forward only: the outputs carry no autograd graph (the reference's own
-bidirectional backward is not functional, recurrent_fuse.py:443,456).
+The ops are differentiable: when autograd is recording and an input requires a
+gradient, the backward runs the library's backward kernels (the reference's own
+merged bidirectional op has no working backward, recurrent_fuse.py:443,456).
 """
 from __future__ import annotations
 
@@ -145,7 +146,10 @@ def _gla_bidir_forward_raw(q, k, v, g_fwd, g_bwd, scale, out_scale, exact, out, 
               and out.dtype == q.dtype):
         raise ValueError("bad `out` tensor")
     fn = lib.vig_gla_bidir_fwd_exact if exact else (lib.vig_gla_bidir_fwd_wide if strong_gates else lib.vig_gla_bidir_fwd)
-    ws_bytes = lib.vig_gla_bidir_fwd_workspace(B, H, L, Dk, Dv, io_dt)
+    if exact:  # the token-recurrent kernel parks the first direction's fp32 sums when the tensors are narrower
+        ws_bytes = B * H * L * Dv * 4 if (g_bwd is not None and io_dt != _lib.VIG_F32) else 0
+    else:
+        ws_bytes = lib.vig_gla_bidir_fwd_workspace_for(B, H, L, Dk, Dv, io_dt, g_dt, int(g_bwd is not None))
     ws = torch.empty(ws_bytes, dtype=torch.uint8, device=q.device) if ws_bytes else None
     with torch.cuda.device(q.device):
         rc = fn(q.data_ptr(), k.data_ptr(), v.data_ptr(), g_fwd.data_ptr(),
