@@ -102,6 +102,25 @@ int vig_gla_bidir_fwd_wide(const void* q, const void* k, const void* v,
                            int io_dtype, int gate_dtype, void* stream);
 
 /*
+ * vig_gla_bidir_fwd without a workspace argument, for callers that cannot allocate device memory: code under
+ * HIP graph capture, tight serving loops, harnesses that forbid hipMalloc.  Same tensors, dispatch, kernels and
+ * results (bit for bit) as vig_gla_bidir_fwd; the workspace is a device array inside the library,
+ * VIG_GLA_NOALLOC_SCRATCH_BYTES per GPU, held from the first call on that GPU until the process ends.  A shape whose
+ * vig_gla_bidir_fwd_workspace_for(...) exceeds that size returns VIG_ENOSPC and launches nothing (then use
+ * vig_gla_bidir_fwd with a workspace of the caller's).  Calls no hipMalloc / hipFree and nothing else that allocates.
+ * All calls on one GPU share the one array: calls that overlap in time on the same GPU (two streams, two threads)
+ * race on it; serialise them.  It has no counterpart in the reference, whose ops allocate their temporaries through
+ * torch (flash-linear-attention/fla/ops/gla/chunk_fuse.py:325-345).
+ */
+#define VIG_GLA_NOALLOC_SCRATCH_BYTES (16u << 20)
+int vig_gla_bidir_fwd_noalloc(const void* q, const void* k, const void* v,
+                              const void* g_fwd, const void* g_bwd, void* o,
+                              int B, int H, int L, int Dk, int Dv,
+                              float scale, float out_scale,
+                              int io_dtype, int gate_dtype, void* stream);
+size_t vig_gla_bidir_fwd_noalloc_max_workspace(void);
+
+/*
  * Same contract as vig_gla_bidir_fwd, but always runs the fp32-arithmetic
  * token-recurrent kernel whatever the dtypes (bf16 tensors are widened on load,
  * the state and all sums stay fp32).  This is the op-level counterpart of the

@@ -2,6 +2,7 @@
 // dispatch only.  Nothing here allocates, frees or synchronises.
 #include "../../include/vig_gla.h"
 #include "launch.h"
+#include <mutex>
 
 namespace vig {
 int launch_dirgate(const void* in, void* out, int B, int L, int H, int Dk, float inv_norm, float clamp_min,
@@ -197,6 +198,49 @@ int vig_gla_bidir_fwd_wide(const void* q, const void* k, const void* v, const vo
                            float out_scale, int io_dtype, int gate_dtype, void* stream) {
   return gla_bidir_fwd(q, k, v, g_fwd, g_bwd, o, workspace, workspace_bytes, B, H, L, Dk, Dv, scale, out_scale,
                        io_dtype, gate_dtype, stream, 1);
+}
+
+// ---- vig_gla_bidir_fwd for callers that cannot allocate: the workspace is a device array of this library ----
+// One copy per GPU, held from the first launch of the library on that GPU until the process ends.
+constexpr size_t kScratchBytes = VIG_GLA_NOALLOC_SCRATCH_BYTES;
+static __device__ __align__(256) unsigned char scratch[kScratchBytes];
+// The array's name is only a host-side handle: its address on each device is looked up once, with that device current.
+constexpr int kScratchMaxDevices = 64;
+static void* scratch_ptr[kScratchMaxDevices] = {};
+static std::mutex scratch_mutex;
+
+static int scratch_for_current_device(void** out) {
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kScratchMaxDevices) return VIG_ELAUNCH;
+  std::lock_guard<std::mutex> lock(scratch_mutex);
+  if (!scratch_ptr[dev]) {
+    void* p = nullptr;
+    if (hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)) != hipSuccess || !p) return VIG_ELAUNCH;
+    scratch_ptr[dev] = p;
+  }
+  *out = scratch_ptr[dev];
+  return VIG_OK;
+}
+
+size_t vig_gla_bidir_fwd_noalloc_max_workspace(void) { return kScratchBytes; }
+
+int vig_gla_bidir_fwd_noalloc(const void* q, const void* k, const void* v, const void* g_fwd, const void* g_bwd,
+                              void* o, int B, int H, int L, int Dk, int Dv, float scale, float out_scale,
+                              int io_dtype, int gate_dtype, void* stream) {
+  if (B <= 0 || H <= 0 || L <= 0) return VIG_EINVAL;
+  if (!dtype_ok(io_dtype) || !dtype_ok(gate_dtype)) return VIG_ENOTSUP;
+  // what the dispatched path of vig_gla_bidir_fwd needs; shapes whose need exceeds the array are refused, not shrunk
+  const size_t need = fwd_workspace_exact(B, H, L, Dk, Dv, io_dtype, gate_dtype, g_bwd != nullptr);
+  if (need > kScratchBytes) return VIG_ENOSPC;
+  void* ws = nullptr;
+  if (need > 0) {
+    const int rc = scratch_for_current_device(&ws);
+    if (rc != VIG_OK) return rc;
+  }
+  // Every kernel behind vig_gla_bidir_fwd writes the part of the workspace it later reads (segment states, padded
+  // copies, the reverse direction's partial outputs) before reading it: nothing has to start at zero.
+  return gla_bidir_fwd(q, k, v, g_fwd, g_bwd, o, ws, need, B, H, L, Dk, Dv, scale, out_scale, io_dtype, gate_dtype,
+                       stream, 0);
 }
 
 // vig_gla_bidir_fwd followed by vig_locality_gate_fwd in one kernel: y = o * sigmoid(conv3x3(o)) with o the rounded
