@@ -49,6 +49,19 @@ def test_argument_validation_without_gpu():
     assert rc == -28  # bf16 bidirectional exact path needs workspace
     assert lib.vig_gla_strerror(-28) == b"workspace too small"
     assert lib.vig_dirgate_fwd(one, one, 1, 1, 1, 12, 1.0, 0.0, 0, 0, None) == -95
+    # launch geometry is checked before anything is enqueued: B*H beyond int range, row counts beyond int range, and
+    # more (sequence, direction) pairs than the long-sequence scan's grid takes
+    assert lib.vig_gla_bidir_fwd(one, one, one, one, one, one, one, 1 << 40, 40000, 2, 300, 64, 64, 1.0, 1.0, 1, 1,
+                                 None) == -95
+    assert lib.vig_gla_bidir_fwd(one, one, one, one, None, one, one, 1 << 40, 40000, 1, 300, 64, 64, 1.0, 1.0, 1, 1,
+                                 None) != -95  # one direction: 40000 pairs fit (a workspace error or success path)
+    big = 1 << 40
+    assert lib.vig_gla_bidir_bwd(one, one, one, one, one, one, one, one, one, one, one, one, big, 70000, 70000, 8, 64,
+                                 64, 1.0, 1.0, 1, 1, None) == -22
+    assert lib.vig_rmsnorm_bwd(one, one, one, None, one, None, None, 0, 1 << 31, 384, 1e-6, 1, None) == -22
+    assert lib.vig_gla_bidir_fwd_workspace_for(128, 6, 196, 64, 64, 1, 1, 1) == 0
+    assert lib.vig_gla_bidir_fwd_workspace_for(128, 6, 196, 64, 64, 1, 0, 1) == 128 * 6 * 196 * 64 * 4
+    assert lib.vig_gla_bidir_fwd_workspace_for(2, 3, 197, 64, 64, 1, 0, 0) == 0
 
 
 def test_ops_refuse_cpu_tensors():

@@ -195,3 +195,19 @@ def test_backward_mfma_causal(B, H, L, Dk):
     else:
         want = [f64(t) for t in vig_amd.gla_bidir_backward(*dev, None, do.cuda(), out_scale=1.0, exact=True)[:4]]
     _check_mfma(got[:4], want, q)
+
+
+def test_autograd_keeps_the_exact_path():
+    """gla_bidir_forward(exact=True) under autograd: the backward runs the fp32-arithmetic kernel too, bit-equal to
+    gla_bidir_backward(exact=True) (and different from the matrix-core gradients of the default path)."""
+    announce("autograd with exact=True, bf16")
+    t = [x.cuda() for x in make_gla_inputs(2, 2, 196, 64, 64, seed=77, dtype=torch.bfloat16)]
+    leaves = [x.clone().requires_grad_() for x in t]
+    o = vig_amd.gla_bidir_forward(*leaves, exact=True)
+    d_o = torch.randn_like(o)
+    o.backward(d_o)
+    want = vig_amd.gla_bidir_backward(*t, d_o, exact=True)
+    other = vig_amd.gla_bidir_backward(*t, d_o, exact=False)
+    for leaf, w in zip(leaves, want):
+        assert torch.equal(leaf.grad, w)
+    assert any(not torch.equal(a, b) for a, b in zip(want, other))

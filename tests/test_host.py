@@ -64,3 +64,46 @@ def test_layers_mirror_the_reference_constructors():
     assert (m.head_qk_dim, m.head_v_dim, m.channel_first, m.d_group) == (16, 32, True, 2)
     mlp = layers.GLAMLP(384)
     assert mlp.intermediate_size == 1024  # 4 * 384 * 2 / 3 rounded up to a multiple of 256 (vig.py:480-483)
+
+
+def test_checkpoint_variants_and_cache_invalidation(tmp_path):
+    """'model' / 'model_ema' / bare state dicts / a 'module.' prefix (classification/utils/utils.py:17-103), and the
+    derived weight copies of the layers do not survive a load or a train()/eval() switch."""
+    from vig_amd import evaluate, layers
+
+    torch.manual_seed(0)
+    kw = dict(img_size=32, depth=1, num_heads=2, embed_dim=64, num_classes=5)
+    a, b = layers.ViG(**kw), layers.ViG(**kw)
+    with torch.no_grad():
+        for p in b.parameters():
+            p.add_(1.0)
+    path = str(tmp_path / "c.pth")
+    torch.save({"model": a.state_dict(), "model_ema": {"module." + k: v for k, v in b.state_dict().items()},
+                "max_accuracy": 1.0, "epoch": 2}, path)
+    m = layers.ViG(**kw)
+    evaluate.load_checkpoint(m, path)
+    assert all(torch.equal(x, y) for x, y in zip(m.state_dict().values(), a.state_dict().values()))
+    evaluate.load_checkpoint(m, path, use_ema=True)
+    assert all(torch.equal(x, y) for x, y in zip(m.state_dict().values(), b.state_dict().values()))
+    torch.save({"model": a.state_dict()}, path)          # no EMA copy in the file: 'model' serves (utils.py:73)
+    evaluate.load_checkpoint(m, path, use_ema=True)
+    assert all(torch.equal(x, y) for x, y in zip(m.state_dict().values(), a.state_dict().values()))
+    torch.save(b.state_dict(), path)                       # bare state dict
+    evaluate.load_checkpoint(m, path)
+    assert all(torch.equal(x, y) for x, y in zip(m.state_dict().values(), b.state_dict().values()))
+    # caches: filled by hand here (no GPU), gone after a load, after train()/eval() and after invalidate_caches
+    # (bf16 parameters, so that the fp32 copy is a tensor of its own)
+    m, a = m.to(torch.bfloat16), a.to(torch.bfloat16)
+    norm = m.blocks[0].attn_norm
+    norm._w32()
+    assert "_w32_cache" in norm.__dict__
+    m.load_state_dict(a.state_dict())
+    assert "_w32_cache" not in norm.__dict__
+    norm._w32()
+    m.train()
+    assert "_w32_cache" not in norm.__dict__
+    norm._w32()
+    norm.weight.data.mul_(2.0)  # behind the version counter: the stale copy would survive ...
+    assert torch.equal(norm._w32(), norm.weight.detach().float() / 2)
+    layers.invalidate_caches(m)  # ... until the caller says so
+    assert torch.equal(norm._w32(), norm.weight.detach().float())

@@ -21,7 +21,7 @@ def test_reference_parameter_names():
     assert m.head_qk_dim == 32 and m.head_v_dim == 64
 
 
-@pytest.mark.parametrize("dtype,tol", [(torch.float32, 2e-4), (torch.bfloat16, 6e-2)])
+@pytest.mark.parametrize("dtype,tol", [(torch.float32, 2e-4), (torch.bfloat16, 2e-2)])  # measured 6e-7 / 5.2e-3
 @pytest.mark.parametrize("variant", ["s", "t"])
 def test_gla_block_matches_restatement(dtype, tol, variant):
     announce(f"GatedLinearAttention eval forward, vig-{variant}, {dtype}")
@@ -62,7 +62,10 @@ def test_gla_block_train_mode_scale():
     assert torch.allclose(a, 2 * b, rtol=1e-6, atol=1e-7)
 
 
-@pytest.mark.parametrize("dtype,tol", [(torch.float32, 5e-4), (torch.bfloat16, 8e-2)])
+BF16_LOGITS_TOL = 2e-2  # bf16 model outputs: about three times what is measured (4e-3 .. 6.3e-3)
+
+
+@pytest.mark.parametrize("dtype,tol", [(torch.float32, 5e-4), (torch.bfloat16, BF16_LOGITS_TOL)])
 def test_vig_small_logits(dtype, tol):
     """Full ViG-S eval forward (random init, synthetic images) against the float64 restatement on the same state_dict."""
     announce(f"ViG-S logits {dtype}")
@@ -75,6 +78,36 @@ def test_vig_small_logits(dtype, tol):
     print(f"  logits max-rel err {err:.3e}  (max |logit| {np.abs(want).max():.3f})", flush=True)
     assert got.shape == (2, 1000)
     assert err <= tol
+
+
+def test_vig_small_full_batch_256():
+    """The named model workload at its full size: [256, 3, 224, 224] synthetic images in bf16 through ViG-S.  Samples
+    are independent, so four of the 256 logit rows are checked against the float64 restatement run on just those four
+    images; all 256 rows have to be finite, reproducible bit for bit, and equal to what the same images give in a
+    batch of their own (no leakage between samples)."""
+    announce("ViG-S logits, batch 256, bf16")
+    torch.manual_seed(0)
+    model = layers.vig_small().eval()
+    g = torch.Generator().manual_seed(1004)
+    images = torch.randn(256, 3, 224, 224, generator=g)
+    pick = [0, 77, 130, 255]
+    want = R.vig_forward(model.state_dict(), images[pick], num_heads=6, depth=12).numpy()
+    model = model.to("cuda", torch.bfloat16)
+    x = images.to("cuda", torch.bfloat16)
+    with torch.no_grad():
+        got = model(x)
+        again = model(x)
+        small = model(x[pick])
+    assert got.shape == (256, 1000) and torch.isfinite(got.float()).all()
+    assert torch.equal(got, again)
+    err = np.abs(got[pick].double().cpu().numpy() - want).max() / np.abs(want).max()
+    print(f"  logits max-rel err of 4 rows of the batch of 256: {err:.3e}", flush=True)
+    assert err <= BF16_LOGITS_TOL
+    # the library's kernels give every sample the same arithmetic whatever the batch; the GEMM library may pick other
+    # kernels for other row counts, so the two batches agree to bf16 rounding rather than bit for bit
+    d = (got[pick].float() - small.float()).abs().max().item() / np.abs(want).max()
+    print(f"  same images in a batch of 4: max-rel difference {d:.3e}", flush=True)
+    assert d <= BF16_LOGITS_TOL
 
 
 @pytest.mark.parametrize("name,heads,kw", [("vig_tiny", 3, dict(out_act=True, act_in_conv=True)), ("vig_base", 12, {})])
@@ -90,7 +123,7 @@ def test_vig_tiny_and_base_logits(name, heads, kw):
     err = np.abs(got - want).max() / np.abs(want).max()
     print(f"  logits max-rel err {err:.3e}  (max |logit| {np.abs(want).max():.3f})", flush=True)
     assert got.shape == (1, 1000)
-    assert err <= 8e-2
+    assert err <= BF16_LOGITS_TOL
 
 
 def test_evaluate_callers(tmp_path):

@@ -37,7 +37,7 @@ def _rel(a, b):
     return np.abs(a - b).max() / max(np.abs(b).max(), 1e-30)
 
 
-@pytest.mark.parametrize("dtype,tol", [(torch.float32, 2e-4), (torch.bfloat16, 6e-2)])
+@pytest.mark.parametrize("dtype,tol", [(torch.float32, 2e-4), (torch.bfloat16, 2e-2)])  # measured 2e-7 / 5.3e-3
 @pytest.mark.parametrize("variant", ["s", "t"])
 def test_training_forward_matches_kernel_forward(dtype, tol, variant):
     announce(f"GatedLinearAttention train-mode forward, autograd path against kernel path, {variant}, {dtype}")
@@ -54,7 +54,7 @@ def test_training_forward_matches_kernel_forward(dtype, tol, variant):
     assert err <= tol
 
 
-@pytest.mark.parametrize("dtype,tol", [(torch.float32, 2e-4), (torch.bfloat16, 8e-2)])
+@pytest.mark.parametrize("dtype,tol", [(torch.float32, 2e-4), (torch.bfloat16, 4e-2)])  # measured 7e-7 / 1.2e-2
 @pytest.mark.parametrize("variant", ["s", "t"])
 def test_block_gradients(dtype, tol, variant):
     announce(f"GatedLinearAttention gradients against the float64 restatement, {variant}, {dtype}")
@@ -122,6 +122,44 @@ def test_vig_training_step():
     after = torch.nn.functional.cross_entropy(model(images.cuda()), target.cuda())
     print(f"  loss {loss.item():.4f} -> {after.item():.4f}", flush=True)
     assert after.item() < loss.item()
+
+
+def test_vig_training_step_under_bf16_autocast():
+    """The same small ViG with fp32 parameters under torch.autocast(bfloat16) -- how the bf16 training-step figure is
+    measured: logits and every parameter gradient against the float64 restatement at the bf16 bar; the parameter
+    gradients stay fp32 and finite (the dtype glue: bf16 branches meeting the fp32 residual stream in the norm nodes,
+    the cast of the block input, gradient dtypes arriving at the library's autograd nodes)."""
+    announce("ViG (64x64 images, depth 2, dim 96) training step under bf16 autocast")
+    torch.manual_seed(0)
+    kw = dict(img_size=64, depth=2, num_heads=3, embed_dim=96, num_classes=10, drop_path_rate=0.0)
+    model = layers.ViG(**kw)
+    with torch.no_grad():
+        for blk in model.blocks:
+            for lin in (blk.attn.qkv_proj, blk.attn.g_proj, blk.attn.o_proj, blk.attn.gk_proj[0], blk.attn.gk_proj[1]):
+                lin.weight.mul_(8.0)
+    images = torch.randn(3, 3, 64, 64)
+    target = torch.tensor([1, 7, 4])
+    sd = {k: v.detach().double().requires_grad_() for k, v in model.state_dict().items()}
+    want = R.vig_forward(sd, images.double(), num_heads=3, depth=2, train=True)
+    torch.nn.functional.cross_entropy(want, target).backward()
+
+    model = model.cuda().train()
+    with torch.autocast("cuda", dtype=torch.bfloat16):
+        logits = model(images.cuda())
+        loss = torch.nn.functional.cross_entropy(logits.float(), target.cuda())
+    loss.backward()
+    e = _rel(logits.detach().double().cpu(), want.detach())
+    print(f"  logits max-rel err {e:.3e}", flush=True)
+    assert e <= 2e-2  # measured 4.1e-3
+    worst = ("", 0.0)
+    for name, p in model.named_parameters():
+        assert p.dtype == torch.float32 and p.grad is not None and p.grad.dtype == torch.float32, name
+        assert torch.isfinite(p.grad).all(), name
+        e = _rel(p.grad.double().cpu(), sd[name].grad)
+        if e > worst[1]:
+            worst = (name, e)
+    print(f"  worst gradient max-rel err {worst[1]:.3e} ({worst[0]})", flush=True)
+    assert worst[1] <= 6e-2, worst  # measured 1.7e-2
 
 
 @pytest.mark.parametrize("channel_first", [False, True])

@@ -153,6 +153,8 @@ static int gla_bidir_fwd(const void* q, const void* k, const void* v, const void
   if (rc != VIG_OK) return rc;
   a.wide_gates = wide_gates;
   if (vig::gla_mfma_supported(a)) {
+    // (the segment scan of long sequences puts sequence x direction on grid.y)
+    if (L > 256 && (long long)B * H * (g_bwd ? 2 : 1) > 65535) return VIG_ENOTSUP;
     if (vig::gla_mfma_workspace(B, H, L, Dk, Dv) > workspace_bytes) return VIG_ENOSPC;
     if (vig::gla_mfma_workspace(B, H, L, Dk, Dv) > 0 && !workspace) return VIG_EINVAL;
     return vig::launch_gla_mfma(a);
@@ -451,7 +453,7 @@ size_t vig_rmsnorm_bwd_workspace(long long rows, int C) {
 int vig_rmsnorm_bwd(const void* sum, const float* weight, const void* dy, const void* d_sum, void* ds, float* dweight,
                     void* workspace, size_t workspace_bytes, long long rows, int C, float eps, int io_dtype,
                     void* stream) {
-  if (!sum || !weight || !dy || !ds || rows <= 0 || C <= 0) return VIG_EINVAL;
+  if (!sum || !weight || !dy || !ds || rows <= 0 || C <= 0 || rows > 0x7fffffffLL) return VIG_EINVAL;
   if (!aligned16(sum, weight, dy, d_sum, ds, dweight, workspace)) return VIG_EINVAL;
   if (!dtype_ok(io_dtype) || (C % 8) != 0 || C > 1024) return VIG_ENOTSUP;
   if (dweight && (!workspace || workspace_bytes < vig::rmsnorm_bwd_workspace(rows, C))) return VIG_ENOSPC;
@@ -476,6 +478,7 @@ static int gla_bidir_bwd(const void* q, const void* k, const void* v, const void
       L <= 0)
     return VIG_EINVAL;
   if (!aligned16(q, k, v, g_fwd, g_bwd, d_o, dq, dk, dv, dg_fwd, dg_bwd, workspace)) return VIG_EINVAL;
+  if ((long long)B * H > 2147483647LL) return VIG_EINVAL;
   if (!dtype_ok(io_dtype) || !dtype_ok(gate_dtype) || !bwd_shape_ok(Dk, Dv)) return VIG_ENOTSUP;
   const size_t need = vig::gla_backward_workspace(B, H, L, Dk, Dv, g_bwd != nullptr);
   if (!workspace || workspace_bytes < need) return VIG_ENOSPC;

@@ -44,21 +44,6 @@ constexpr int kXStride = 68;  // floats per token row of the dg scratch (272 B: 
 static_assert(8 * 32 * kXStride * 4 <= 2 * kBwdMatBytes, "dg scratch overlays the q~ and k~ matrices");
 constexpr float kBwdHalfRange = 60.0f;
 
-// Optional phase timing (development builds only: -DVIG_TIMING): lane 0 of every wave of workgroup 0 records the
-// shader clock at the phase boundaries of the first slab, per direction.
-#ifdef VIG_TIMING
-__device__ unsigned long long g_bwd_stamp[2][8][16];
-#define VIG_BWD_STAMP(id)                                                                                   \
-  do {                                                                                                      \
-    __builtin_amdgcn_sched_barrier(0);                                                                      \
-    if (lane == 0 && blockIdx.x == 0 && first_slab) g_bwd_stamp[LAST ? 1 : 0][w][id] = __builtin_readcyclecounter(); \
-    __builtin_amdgcn_sched_barrier(0);                                                                      \
-  } while (0)
-#else
-#define VIG_BWD_STAMP(id) \
-  do {                    \
-  } while (0)
-#endif
 
 // fragment of 8 consecutive channels (k-step ks, lane half h) of a staged row: contraction over channels
 __device__ __forceinline__ u32x4_t row_frag(const uint16_t* mat, int row, int ks, int h) {
@@ -127,7 +112,7 @@ __device__ __forceinline__ void issue_bwd_loads(const BwdNext& n, int w, int r, 
 template <bool FWD, bool FIRST, bool LAST, int NG>
 __device__ __forceinline__ bool bwd_direction(const BwdSlab& sl, int L, int ntiles, int w, int lane, char* lds,
                                               float s, f32x16_t (&dv)[2], u32x4_t (&keepq)[NG], u32x4_t (&keepk)[NG],
-                                              BwdLoads<NG>& ld, const BwdNext& nxt, bool first_slab) {
+                                              BwdLoads<NG>& ld, const BwdNext& nxt) {
   // where the first direction's dq, dk (bf16) wait for the second: in registers when the kernel has them to spare
   // (Dk = 32), else parked in the output tensors
   constexpr bool kKeepInRegs = NG == 2;
@@ -146,7 +131,6 @@ __device__ __forceinline__ bool bwd_direction(const BwdSlab& sl, int L, int ntil
   const int rows = __builtin_amdgcn_readfirstlane(min(max(L - 32 * w, 0), 32));  // valid tokens of this wave's tile
   const size_t tk = (size_t)32 * w * DK, tv = (size_t)32 * w * 64;
 
-  VIG_BWD_STAMP(0);
   // ---- this tile's loads were issued a phase ago; v and do rows go to LDS once per slab ----
   if (stage_vdo) {
     store_kt<4>(V, 32 * w + r, h, ld.rawv);
@@ -178,7 +162,6 @@ __device__ __forceinline__ bool bwd_direction(const BwdSlab& sl, int L, int ntil
       tot[w * 64 + ch + 1] = G[1][c];
     }
   }
-  VIG_BWD_STAMP(1);
   lds_barrier();  // (1) tile totals (and v, do rows) visible; the previous direction's scratch is dead
   // lane = channel: gates before this tile in walking order, minus the anchor (half the slab total)
   bool out_of_range;
@@ -193,7 +176,6 @@ __device__ __forceinline__ bool bwd_direction(const BwdSlab& sl, int L, int ntil
     offs[lane] = pre - 0.5f * all;
     out_of_range = __builtin_amdgcn_ballot_w64(fabsf(all) * (0.5f * kLog2e) > kBwdHalfRange) != 0;
   }
-  VIG_BWD_STAMP(2);
   if (out_of_range) return false;  // same totals in every wave: the whole workgroup leaves together
   wave_lds_sync();
   // x = (G - a) * log2(e) per (token, channel): q~ = q 2^x, k~ = k 2^-x
@@ -223,9 +205,7 @@ __device__ __forceinline__ bool bwd_direction(const BwdSlab& sl, int L, int ntil
     store_kt<NG>(Q, 32 * w + r, h, qt);
     store_kt<NG>(K, 32 * w + r, h, kt);
   }
-  VIG_BWD_STAMP(3);
   lds_barrier();  // (2) q~, k~ of every tile visible
-  VIG_BWD_STAMP(4);
 
   // ---- dq of tile w: over the key tiles J the direction keeps ----
   f32x16_t dqh[2] = {{0.f}, {0.f}};
@@ -251,7 +231,6 @@ __device__ __forceinline__ bool bwd_direction(const BwdSlab& sl, int L, int ntil
       }
     }
   }
-  VIG_BWD_STAMP(5);
   // dq^ waits as bf16 pairs while the other accumulators are at work
   uint32_t dqp[16];
 #pragma unroll
@@ -308,7 +287,6 @@ __device__ __forceinline__ bool bwd_direction(const BwdSlab& sl, int L, int ntil
       }
     }
   }
-  VIG_BWD_STAMP(6);
   // ---- scale back; X = q dq - k dk = s (q~ dq^ - k~ dk^): the exponentials cancel, and the staged rows serve ----
   f32x16_t X[2];
   {
@@ -358,7 +336,6 @@ __device__ __forceinline__ bool bwd_direction(const BwdSlab& sl, int L, int ntil
       }
     }
   }
-  VIG_BWD_STAMP(7);
   lds_barrier();  // (3) nobody reads q~, k~ any more: their space becomes the dg scratch
   {
     float* xs = reinterpret_cast<float*>(lds + kBwdLdsQ) + w * 32 * kXStride;
@@ -379,9 +356,7 @@ __device__ __forceinline__ bool bwd_direction(const BwdSlab& sl, int L, int ntil
 #pragma unroll
     for (int t = 0; t < 32; ++t) acc += xs[t * kXStride + cl];
     if (lane < DK) dgtot[w * 64 + lane] = acc;
-    VIG_BWD_STAMP(8);
     lds_barrier();  // (4) tile totals of X visible
-    VIG_BWD_STAMP(9);
     float run = 0.f;
 #pragma unroll
     for (int t = 0; t < kBwdTiles; ++t) {
@@ -407,7 +382,6 @@ __device__ __forceinline__ bool bwd_direction(const BwdSlab& sl, int L, int ntil
       __builtin_amdgcn_raw_buffer_store_b128(out, rdg, (unsigned)r * (2u * DK) + (2u * HC) * h + 16u * gq, 0, 0);
     }
   }
-  VIG_BWD_STAMP(10);
   return true;
 }
 
@@ -442,19 +416,15 @@ __global__ __launch_bounds__(512) void gla_backward_mfma_kernel(
     const BwdNext second{sl, sl.gb, L}, next_first{sn, sn.gf, following < nslabs ? L : 0};
     f32x16_t dvacc[2] = {{0.f}, {0.f}};
     u32x4_t keepq[NG], keepk[NG];
-    const bool first_slab = slab == (int)blockIdx.x;
     bool ok;
     if constexpr (BIDIR) {
-      ok = bwd_direction<true, true, false, NG>(sl, L, ntiles, w, lane, lds, s, dvacc, keepq, keepk, ld, second,
-                                                first_slab);
+      ok = bwd_direction<true, true, false, NG>(sl, L, ntiles, w, lane, lds, s, dvacc, keepq, keepk, ld, second);
       if (ok) {
         lds_barrier();  // (5) the dg scratch of direction 1 is dead before q~, k~ of direction 2 are staged
-        ok = bwd_direction<false, false, true, NG>(sl, L, ntiles, w, lane, lds, s, dvacc, keepq, keepk, ld, next_first,
-                                                   first_slab);
+        ok = bwd_direction<false, false, true, NG>(sl, L, ntiles, w, lane, lds, s, dvacc, keepq, keepk, ld, next_first);
       }
     } else {  // the causal op: the forward direction alone, first and last at once
-      ok = bwd_direction<true, true, true, NG>(sl, L, ntiles, w, lane, lds, s, dvacc, keepq, keepk, ld, next_first,
-                                               first_slab);
+      ok = bwd_direction<true, true, true, NG>(sl, L, ntiles, w, lane, lds, s, dvacc, keepq, keepk, ld, next_first);
     }
     // a direction that left early has not issued the loads of the slab that follows
     if (!ok) issue_bwd_loads<true, NG>(next_first, w, r, h, ld);
@@ -464,11 +434,6 @@ __global__ __launch_bounds__(512) void gla_backward_mfma_kernel(
 }
 
 
-#ifdef VIG_TIMING
-extern "C" int vig_debug_read_bwd_stamps(unsigned long long* host_out) {
-  return hipMemcpyFromSymbol(host_out, HIP_SYMBOL(g_bwd_stamp), sizeof(g_bwd_stamp)) == hipSuccess ? 0 : -5;
-}
-#endif
 
 bool gla_backward_mfma_supported(int L, int Dk, int Dv, int io_dtype, int gate_dtype, bool bidir) {
   (void)bidir;  // both the bidirectional and the causal op

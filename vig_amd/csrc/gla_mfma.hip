@@ -39,9 +39,6 @@
 #include "common.h"
 #include "launch.h"
 #include "mfma_tiles.h"
-#ifdef VIG_TIMING
-#include <stdlib.h>
-#endif
 
 namespace vig {
 
@@ -50,21 +47,6 @@ namespace {
 // Scheduling fence: keeps the machine scheduler from hoisting the next phase's loads over this one's math.
 #define VIG_PHASE() __builtin_amdgcn_sched_barrier(0)
 
-// Optional phase timing (development builds only: -DVIG_TIMING): lane 0 of every wave of workgroup 0 records the
-// shader clock at phase boundaries of each slab it walks.
-#ifdef VIG_TIMING
-__device__ unsigned long long g_stamp[4][8][16];
-#define VIG_STAMP(id)                                                                                           \
-  do {                                                                                                          \
-    VIG_PHASE();                                                                                                \
-    if ((lane & 63) == 0 && blockIdx.x == 0 && iter < 4) g_stamp[iter][wi][id] = __builtin_readcyclecounter(); \
-    VIG_PHASE();                                                                                                \
-  } while (0)
-#else
-#define VIG_STAMP(id) \
-  do {                \
-  } while (0)
-#endif
 
 // fp16 score operands are used while |G_end|/2 * log2(e) <= this for every channel of the chunk: the scaled
 // operands then stay within 2^6 of the inputs' magnitudes (fp16 holds |x| < 65504 and full precision above 6e-5).
@@ -410,7 +392,7 @@ struct GateLayout {
 template <bool FWD, int MODE, int NG, bool F16, bool GATE>
 __device__ __forceinline__ bool direction_wave(const ChunkSrc& cur, const ChunkSrc& nxt, rsrc_t o, int c, int lane,
                                                char* lds, float oscale, bool bidir, float* state, Prefetch<NG>& pf,
-                                               int iter, const GateCtx& gate) {
+                                               const GateCtx& gate) {
   constexpr bool OUT = MODE != kModeState;  // produces outputs (needs q)
   int r = lane & 31, h = lane >> 5;
   const int wi = (FWD ? 0 : 4) + c;
@@ -420,7 +402,6 @@ __device__ __forceinline__ bool direction_wave(const ChunkSrc& cur, const ChunkS
   uint16_t* kt = reinterpret_cast<uint16_t*>(region);
   float* dvec_all = reinterpret_cast<float*>(lds + kLdsDvec);
   if (!FWD) issue_rows<FWD, OUT, NG>(cur, r, h, pf);
-  VIG_STAMP(0);
   // fused gate: the first 144 threads fetch the head's stencil weights now and park them in LDS before barrier A
   f32x4_t gate_w4 = {0.f, 0.f, 0.f, 0.f};
   const bool gate_w_mine = GATE && wi * 64 + lane < 64 * 9 / 4;
@@ -456,7 +437,6 @@ __device__ __forceinline__ bool direction_wave(const ChunkSrc& cur, const ChunkS
       G[FWD ? 1 : 0][p] = gb;
     }
   }
-  VIG_STAMP(1);
   // ---- anchor: half of the chunk total G_end (G at the last token forward / first token reverse), per channel, so
   // that q~ = q*exp(G - G_end/2) and k~ = k*exp(G_end/2 - G) share the exponent range [-|G_end|/2, |G_end|/2].
   // The anchors (x log2 e) and the half decays exp(G_end/2) go to LDS: the operand builders re-read the former per
@@ -488,15 +468,12 @@ __device__ __forceinline__ bool direction_wave(const ChunkSrc& cur, const ChunkS
     if (g < NG) dvec_all[wi * 64 + HC * h + 8 * g + 2 * m + p] = exp2_fast(an);
   }
   wave_lds_sync();
-  VIG_STAMP(2);
   // ---- intra-chunk scores, tile by tile ----
   f32x16_t O[2][2];
   u32x4_t qkeep[2][NG];
   u32x4_t vfrag[4][2];
   if (tile_phase<FWD, MODE, NG, F16>(cur, pf, G, gend2, kt, r, h, O, qkeep, vfrag)) fast = false;
-  VIG_STAMP(3);
   wave_lds_sync();  // k~ rows of this wave visible to its other lanes
-  VIG_STAMP(4);
   // ---- chunk state contribution U[pk][pv] = k~^T V; publish it (register-native fp32) ----
   {
     f32x16_t U[2][2];
@@ -532,7 +509,6 @@ __device__ __forceinline__ bool direction_wave(const ChunkSrc& cur, const ChunkS
   // descriptors are empty, which keeps branches off the loads.) ----
   if (FWD) issue_first_phase<FWD, OUT, NG>(nxt, r, h, pf);
   else issue_gates<NG>(nxt, r, h, pf);
-  VIG_STAMP(5);
   // lane-derived addresses of the exchange phases are rebuilt here instead of being carried (and spilled) across
   // the register-heavy tile phase
   asm volatile("" : "+v"(lane));
@@ -542,7 +518,6 @@ __device__ __forceinline__ bool direction_wave(const ChunkSrc& cur, const ChunkS
   if (F16 && !fast && lane == 0) *veto = 1;
   if (GATE && gate_w_mine) reinterpret_cast<f32x4_t*>(lds + kLdsGateW)[wi * 64 + lane] = gate_w4;
   lds_barrier();  // (A) published U's and decays visible
-  VIG_STAMP(6);
   // same answer in every wave: the word is only written before this barrier and the variant is left once it is set
   const bool ok = !F16 || __builtin_amdgcn_readfirstlane(*veto) == 0;
   if (F16 && !ok) return false;  // every wave alike: the segment is walked again, barriers B and C are skipped by all
@@ -612,9 +587,7 @@ __device__ __forceinline__ bool direction_wave(const ChunkSrc& cur, const ChunkS
       }
     }
   }
-  VIG_STAMP(7);
   lds_barrier();  // (B) incoming-state fragments of every chunk visible
-  VIG_STAMP(8);
   if (OUT) {
     // ---- O^T += (exp(G_end) * S_in) q~hi  for every chunk that has an incoming state ----
     if (MODE == kModeChain || (FWD ? (c > 0) : (c < 3))) {
@@ -627,7 +600,6 @@ __device__ __forceinline__ bool direction_wave(const ChunkSrc& cur, const ChunkS
           for (int it = 0; it < 2; ++it) O[pv][it] = mfma(sf, qkeep[it][ks], O[pv][it]);
         }
     }
-    VIG_STAMP(9);
     // ---- the output swap: each wave of a chunk keeps one 32-token tile ----
     constexpr int KEEP = FWD ? 0 : 1;
     constexpr int SEND = 1 - KEEP;
@@ -641,9 +613,7 @@ __device__ __forceinline__ bool direction_wave(const ChunkSrc& cur, const ChunkS
           *reinterpret_cast<f32x4_t*>(unit_ptr(region, pv * 4 + cq, lane)) = x;
         }
     }
-    VIG_STAMP(10);
     lds_barrier();  // (C) swapped output halves visible
-    VIG_STAMP(11);
     if (bidir) {
       char* partner = lds + ((FWD ? 4 : 0) + c) * kRegionBytes;
 #pragma unroll
@@ -748,7 +718,6 @@ __device__ __forceinline__ bool direction_wave(const ChunkSrc& cur, const ChunkS
   } else {
     lds_barrier();  // (C) keeps the barrier count of the output modes
   }
-  VIG_STAMP(12);
   return ok;
 }
 
@@ -790,8 +759,7 @@ __device__ __forceinline__ int wave_loop(const uint16_t* q, const uint16_t* k, c
     if (FWD) issue_first_phase<FWD, OUT, NG>(cur, lane & 31, lane >> 5, pf);
     else issue_gates<NG>(cur, lane & 31, lane >> 5, pf);
   }
-  int iter = 0;
-  for (; item < geo.nitems; item += gridDim.x, ++iter) {
+  for (; item < geo.nitems; item += gridDim.x) {
     ChunkSrc nxt;
     rsrc_t dst_next;
     locate(item + gridDim.x, nxt, dst_next);
@@ -803,7 +771,7 @@ __device__ __forceinline__ int wave_loop(const uint16_t* q, const uint16_t* k, c
       gate = GateCtx{gate_w + (size_t)(item % geo.heads) * (64 * 9), geo.gw, geo.gh, c * geo.cw, nvalid};
     }
     const bool ok =
-        direction_wave<FWD, MODE, NG, F16, GATE>(cur, nxt, dst, c, lane, lds, oscale, bidir, state, pf, iter, gate);
+        direction_wave<FWD, MODE, NG, F16, GATE>(cur, nxt, dst, c, lane, lds, oscale, bidir, state, pf, gate);
     lds_barrier();  // (D) the next item reuses the LDS regions
     if (F16 && !ok) break;  // this item again, and all that follow, with split-bf16 scores
     cur = nxt;
@@ -950,9 +918,6 @@ static int launch_gla_mfma_t(const GlaArgs& a, int num_cu, int dev) {
   Geometry geo = make_geometry(a.B * a.H, a.L);
   geo.wide_gates = a.wide_gates;
   int grid = geo.nitems < num_cu ? geo.nitems : num_cu;
-#ifdef VIG_TIMING
-  if (const char* e = getenv("VIG_GRID")) grid = atoi(e);
-#endif
   const uint16_t* q = (const uint16_t*)a.q;
   const uint16_t* k = (const uint16_t*)a.k;
   const uint16_t* v = (const uint16_t*)a.v;
@@ -1000,10 +965,5 @@ int launch_gla_mfma(const GlaArgs& a) {
   return a.Dk == 64 ? launch_gla_mfma_t<4>(a, num_cu, dev) : launch_gla_mfma_t<2>(a, num_cu, dev);
 }
 
-#ifdef VIG_TIMING
-extern "C" int vig_debug_read_stamps(unsigned long long* host_out) {
-  return hipMemcpyFromSymbol(host_out, HIP_SYMBOL(g_stamp), sizeof(g_stamp)) == hipSuccess ? 0 : -5;
-}
-#endif
 
 }  // namespace vig

@@ -11,16 +11,30 @@ from typing import Iterable, Optional, Tuple
 import torch
 import torch.nn.functional as F
 
-from .layers import resize_pos_embed
+from .layers import invalidate_caches, resize_pos_embed
 
 
-def load_checkpoint(model: torch.nn.Module, path: str, strict: bool = True):
-    """Loads a reference checkpoint (classification/utils/utils.py:22-24: the weights sit under 'model') or a bare
-    state_dict.  Tensors only (`weights_only=True`).  A position table of another grid is resized bicubically
-    (classification/models/vig.py:915-958) when the model knows its patch grid."""
+def load_checkpoint(model: torch.nn.Module, path: str, strict: bool = True, use_ema: bool = False):
+    """Loads a reference checkpoint or a bare state_dict.  The reference keeps the weights under 'model' and, when it
+    trained with an EMA copy, that copy's weights under 'model_ema' (classification/utils/utils.py:84-103);
+    `use_ema=True` takes the EMA weights the way load_pretrained_ema fills its EMA model (utils.py:70-79: 'model_ema'
+    if the file has it, else 'model').  Tensors only (`weights_only=True`): the reference's full training checkpoints
+    also pickle their config object, which this loader refuses -- load their 'best' files (weights only, utils.py:85-86)
+    or re-save the weights.  A position table of another grid is resized bicubically
+    (classification/models/vig.py:915-958) when the model knows its patch grid.  The fp32 / stacked weight copies the
+    layers keep are dropped, so the next forward reads the new values."""
     blob = torch.load(path, map_location="cpu", weights_only=True)
-    state = blob["model"] if isinstance(blob, dict) and "model" in blob and isinstance(blob["model"], dict) else blob
+    state = blob
+    if isinstance(blob, dict):
+        key = "model_ema" if (use_ema and isinstance(blob.get("model_ema"), dict)) else "model"
+        if isinstance(blob.get(key), dict):
+            state = blob[key]
+        elif use_ema and "model" not in blob and "model_ema" not in blob:
+            state = blob  # a bare state_dict has no EMA copy to prefer
     state = dict(state)
+    # timm's ModelEma wraps a deep copy of the model: same keys; a DataParallel-trained copy carries a 'module.' prefix
+    if state and all(k.startswith("module.") for k in state):
+        state = {k[len("module."):]: v for k, v in state.items()}
     own = model.state_dict()
     if "pos_embed" in state and "pos_embed" in own and state["pos_embed"].shape != own["pos_embed"].shape:
         n_src = state["pos_embed"].shape[1]
@@ -28,7 +42,9 @@ def load_checkpoint(model: torch.nn.Module, path: str, strict: bool = True):
         if side * side != n_src or not hasattr(model, "patch_resolution"):
             raise ValueError("cannot resize pos_embed: source grid is not square or the model has no patch_resolution")
         state["pos_embed"] = resize_pos_embed(state["pos_embed"], (side, side), tuple(model.patch_resolution))
-    return model.load_state_dict(state, strict=strict)
+    res = model.load_state_dict(state, strict=strict)
+    invalidate_caches(model)
+    return res
 
 
 def accuracy(output: torch.Tensor, target: torch.Tensor, topk: Tuple[int, ...] = (1,)):

@@ -49,12 +49,41 @@ def _f32(owner: nn.Module, tag: str, t: Optional[torch.Tensor], shape=None):
     return hit[1]
 
 
+_CACHE_ATTRS = ("_f32_cache", "_w32_key", "_w32_cache", "_w1_packed")
+
+
+def invalidate_caches(model: nn.Module) -> None:
+    """Drops the fp32, stacked and packed weight copies every module of `model` keeps for its kernels.  The copies are
+    refreshed by themselves when a parameter is replaced, moved, cast or written through torch's in-place operations;
+    a write through `.data` (p.data.mul_(..), module.weight.data[...] = ..) changes neither the pointer nor the version
+    counter they are keyed on, so code that writes that way calls this afterwards.  load_state_dict and train() /
+    eval() switches of these modules call it by themselves."""
+    for m in model.modules():
+        for a in _CACHE_ATTRS:
+            m.__dict__.pop(a, None)
+        if "_in_cat" in m.__dict__:
+            m.__dict__["_in_cat"] = None
+
+
+class _CacheMixin:
+    """For the modules that keep derived weight copies: the copies do not outlive a state-dict load or a switch
+    between training and evaluation (the usual places where weights change behind the version counter)."""
+
+    def train(self, mode: bool = True):
+        invalidate_caches(self)
+        return super().train(mode)
+
+    def _load_from_state_dict(self, *args, **kwargs):
+        invalidate_caches(self)
+        return super()._load_from_state_dict(*args, **kwargs)
+
+
 def _recording(module: nn.Module) -> bool:
     """True when this call has to leave an autograd graph: training mode with gradients enabled."""
     return module.training and torch.is_grad_enabled()
 
 
-class RMSNorm(nn.Module):
+class RMSNorm(_CacheMixin, nn.Module):
     """x * rsqrt(mean(x^2) + eps) * weight, arithmetic in fp32 (fla/modules/rmsnorm.py:38-52,491-512).
 
     forward(x, residual=None, prenorm=False): with a residual the sum is normalised and, with
@@ -84,7 +113,7 @@ class RMSNorm(nn.Module):
         return ops.rmsnorm(x, self._w32(), self.eps, residual=residual, prenorm=prenorm, round_sum=round_sum)
 
 
-class GatedLinearAttention(nn.Module):
+class GatedLinearAttention(_CacheMixin, nn.Module):
     """ViG's bidirectional GLA token mixer (classification/models/vig.py:241-464)."""
 
     def __init__(self, d_model: int = 1024, expand_v: float = 2.0, expand_k: float = 1.0, num_heads: int = 4,
@@ -327,7 +356,7 @@ class GLABlock(nn.Module):
         return self.drop_path(self.mlp(h)), residual
 
 
-class LayerNorm2d(nn.LayerNorm):
+class LayerNorm2d(_CacheMixin, nn.LayerNorm):
     """LayerNorm over the channels of a [B, C, H, W] map (vig.py:619-624).  The patch embedding keeps its maps in
     channels-last memory, where the permuted view is a plain [B*H*W, C] row matrix for the row kernel; `silu`
     folds the swish that follows the first norm (vig.py:653) into the same pass."""
@@ -347,7 +376,7 @@ class LayerNorm2d(nn.LayerNorm):
                              pre_bias=pre_bias, post_add=post_add).permute(0, 3, 1, 2)
 
 
-class V2PatchEmbed(nn.Module):
+class V2PatchEmbed(_CacheMixin, nn.Module):
     """Two strided convs with LayerNorm2d (vig.py:625-672), use_act_in_patch False."""
 
     def __init__(self, patch_size=16, in_chans=3, embed_dim=768, use_bias_in_patch=True):

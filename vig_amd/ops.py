@@ -113,13 +113,14 @@ class _GLABidirFunction(torch.autograd.Function):
     def forward(ctx, q, k, v, g_fwd, g_bwd, scale, out_scale, exact):
         o = _gla_bidir_forward_raw(q, k, v, g_fwd, g_bwd, scale, out_scale, exact, None)
         ctx.save_for_backward(q, k, v, g_fwd, g_bwd)
-        ctx.scale, ctx.out_scale = scale, out_scale
+        ctx.scale, ctx.out_scale, ctx.exact = scale, out_scale, exact
         return o
 
     @staticmethod
     def backward(ctx, d_o):
         q, k, v, g_fwd, g_bwd = ctx.saved_tensors
-        dq, dk, dv, dgf, dgb = gla_bidir_backward(q, k, v, g_fwd, g_bwd, d_o, ctx.scale, ctx.out_scale)
+        # (a caller that asked for fp32 arithmetic gets it in both directions of the graph)
+        dq, dk, dv, dgf, dgb = gla_bidir_backward(q, k, v, g_fwd, g_bwd, d_o, ctx.scale, ctx.out_scale, exact=ctx.exact)
         return dq, dk, dv, dgf, dgb, None, None, None
 
 
