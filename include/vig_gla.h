@@ -86,6 +86,35 @@ size_t vig_gla_bidir_fwd_workspace_for(int B, int H, int L, int Dk, int Dv, int 
                                        int bidirectional);
 
 /*
+ * The causal op (one direction) with a state carried in and / or out:
+ *   S_{-1} = initial_state (zero when NULL);  S_i = diag(exp(g_i)) S_{i-1} + k_i v_i^T;  o_i = out_scale * (scale*q_i)^T S_i;
+ *   final_state = S_{L-1} (not written when NULL).
+ * initial_state, final_state: fp32 [B, H, Dk, Dv], row-major (k channel, then v channel); same tensors, dtypes and
+ * shapes as vig_gla_bidir_fwd with g_bwd == NULL.  bf16 tensors and gates with Dk in {32, 64}, Dv = 64 run on the
+ * matrix cores as chained segments of up to 256 tokens (state contributions, a scan that starts from initial_state
+ * and ends in final_state, outputs); everything else on the fp32-arithmetic token-recurrent kernel.
+ * `workspace` must hold vig_gla_causal_state_fwd_workspace(...) bytes (may be NULL when that is 0).
+ *
+ * Replaces: fused_chunk_gla with initial_state / output_final_state (flash-linear-attention/fla/ops/gla/
+ * chunk_fuse.py:554-572; the state enters at :70-72 and leaves at :99-101) and fused_recurrent_gla with the same
+ * arguments (fla/ops/gla/recurrent_fuse.py:631-657, kernel :213-218,240-246).
+ */
+int vig_gla_causal_state_fwd(const void* q, const void* k, const void* v, const void* g, void* o,
+                             const float* initial_state, float* final_state,
+                             void* workspace, size_t workspace_bytes,
+                             int B, int H, int L, int Dk, int Dv,
+                             float scale, float out_scale,
+                             int io_dtype, int gate_dtype, void* stream);
+size_t vig_gla_causal_state_fwd_workspace(int B, int H, int L, int Dk, int Dv, int io_dtype, int gate_dtype);
+/* Same contract, always the fp32-arithmetic token-recurrent kernel whatever the dtypes (no workspace): the counterpart
+ * of fused_recurrent_gla's state arguments (fla/ops/gla/recurrent_fuse.py:631-657). */
+int vig_gla_causal_state_fwd_exact(const void* q, const void* k, const void* v, const void* g, void* o,
+                                   const float* initial_state, float* final_state,
+                                   int B, int H, int L, int Dk, int Dv,
+                                   float scale, float out_scale,
+                                   int io_dtype, int gate_dtype, void* stream);
+
+/*
  * Same contract, workspace and accuracy bar as vig_gla_bidir_fwd, for callers who know their gates to be strong.
  * The matrix-core kernel computes scores on fp16 operands while a chunk's gate total stays within about 8 (natural
  * log units) in every channel, and on split-bf16 operands beyond; it finds out per workgroup, on the first segment

@@ -76,8 +76,6 @@ def test_fp32_causal_only_and_wrappers():
     from oracle import gla_oracle as O
     assert max_rel(f64(orv), O.gla_recurrent(f64(q), f64(k), f64(v), f64(gf), reverse=True)) <= FP32_TOL
     assert max_rel(f64(of), O.gla_recurrent(f64(q), f64(k), f64(v), f64(gf))) <= FP32_TOL
-    with pytest.raises(NotImplementedError):
-        vig_amd.fused_chunk_gla(dq, dk_, dv_, dgf, output_final_state=True)
 
 
 def test_fp32_zero_gate_closed_form():
@@ -299,3 +297,47 @@ def test_pointers_off_a_16_byte_boundary():
     assert torch.equal(ops.rmsnorm(x, w), ops.rmsnorm(x.clone(), w))
     assert lib.vig_rmsnorm_fwd(x.data_ptr(), None, w.data_ptr(), torch.empty_like(x).data_ptr(), None, 40, 384,
                                1e-6, 0, _lib.VIG_BF16, ops._stream_ptr(x)) == _lib.VIG_EINVAL
+
+
+@pytest.mark.parametrize("dtype,L,Dk,Dv", [(torch.float32, 70, 32, 64), (torch.float32, 300, 64, 64), (torch.bfloat16, 196, 64, 64),
+                                           (torch.bfloat16, 64, 32, 64), (torch.bfloat16, 700, 64, 64), (torch.bfloat16, 1000, 32, 64),
+                                           (torch.bfloat16, 50, 16, 32)])
+def test_causal_op_with_initial_and_final_state(dtype, L, Dk, Dv):
+    """fused_chunk_gla(initial_state=, output_final_state=True) against the oracle's recurrence started from the same
+    state (chunk_fuse.py:70-72,99-101); also state passing: the second half of a sequence started from the first
+    half's final state reproduces the whole sequence (outputs and final state)."""
+    announce(f"causal op with states {dtype} L={L} Dk={Dk} Dv={Dv}")
+    from oracle import gla_oracle as O
+    B, H = 3, 2
+    q, k, v, gf, _ = make_gla_inputs(B, H, L, Dk, Dv, seed=61, dtype=dtype)
+    gen = torch.Generator().manual_seed(62)
+    s0 = torch.randn(B, H, Dk, Dv, generator=gen)
+    want_o, want_s = O.gla_recurrent(f64(q), f64(k), f64(v), f64(gf), initial_state=f64(s0), return_state=True)
+    o, s = vig_amd.fused_chunk_gla(*dev(q, k, v, gf), initial_state=s0.cuda(), output_final_state=True)
+    assert s.dtype == torch.float32 and tuple(s.shape) == (B, H, Dk, Dv)
+    if dtype == torch.float32:
+        assert max_rel(f64(o), want_o) <= FP32_TOL and max_rel(f64(s), want_s) <= FP32_TOL
+    else:
+        assert max_abs(f64(o), want_o) <= BF16_TOL * max(1.0, np.abs(want_o).max() / 4.0)
+        assert max_rel(f64(s), want_s) <= 1e-2  # the state accumulates bf16-rounded operands in fp32
+    # no state in: the plain causal op; final state only
+    o1, s1 = vig_amd.fused_chunk_gla(*dev(q, k, v, gf), output_final_state=True)
+    o_plain, none = vig_amd.fused_chunk_gla(*dev(q, k, v, gf))
+    assert none is None
+    tol = FP32_TOL if dtype == torch.float32 else 1e-2
+    assert max_rel(f64(o1), f64(o_plain)) <= tol
+    # state passing across a split of the sequence
+    cut = L // 2
+    a = [t[:, :, :cut].contiguous() for t in (q, k, v, gf)]
+    b = [t[:, :, cut:].contiguous() for t in (q, k, v, gf)]
+    oa, sa = vig_amd.fused_chunk_gla(*dev(*a), output_final_state=True)
+    ob, sb = vig_amd.fused_chunk_gla(*dev(*b), initial_state=sa, output_final_state=True)
+    whole = f64(o1)
+    assert max_rel(np.concatenate([f64(oa), f64(ob)], axis=2), whole) <= (FP32_TOL if dtype == torch.float32 else 2e-2)
+    assert max_rel(f64(sb), f64(s1)) <= (FP32_TOL if dtype == torch.float32 else 1e-2)
+    # the recurrent wrapper carries states too, in fp32 arithmetic
+    o2, s2 = vig_amd.fused_recurrent_gla(*dev(q, k, v, gf), initial_state=s0.cuda(), output_final_state=True)
+    if dtype == torch.float32:
+        assert max_rel(f64(o2), want_o) <= FP32_TOL and max_rel(f64(s2), want_s) <= FP32_TOL
+    else:
+        assert max_rel(f64(s2), want_s) <= 1e-5

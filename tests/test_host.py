@@ -43,11 +43,11 @@ def test_wrappers_reject_what_is_not_built():
 
     q = torch.zeros(1, 1, 4, 64)
     with pytest.raises(NotImplementedError):
-        vig_amd.fused_chunk_gla(q, q, q, q, output_final_state=True)
-    with pytest.raises(NotImplementedError):
-        vig_amd.fused_chunk_gla(q, q, q, q, initial_state=torch.zeros(1, 1, 64, 64))
-    with pytest.raises(NotImplementedError):
         vig_amd.fused_recurrent_gla(q, q, q, q, gv=q)
+    with pytest.raises(NotImplementedError):  # a state in or out belongs to the causal op (recurrent_fuse.py:650-652)
+        vig_amd.fused_recurrent_gla(q, q, q, q, output_final_state=True, causal=False)
+    with pytest.raises(NotImplementedError):
+        vig_amd.batch_bid_fused_chunk_gla(q, q, q, torch.cat([q, q]), initial_state=torch.zeros(1, 1, 64, 64))
     from vig_amd._lib import VigGlaError
     with pytest.raises(VigGlaError):  # CPU tensors: there is no CPU path, and the wrappers say so
         vig_amd.gla_bidir_locality_gate(q, q, q, q, q, torch.zeros(64, 1, 3, 3), (2, 2))

@@ -14,6 +14,7 @@ from .ops import (  # noqa: F401
     fused_recurrent_gla,
     gla_bidir_backward,
     gla_bidir_forward,
+    gla_causal_state_forward,
     gla_bidir_locality_gate,
     locality_blend,
     locality_gate,
@@ -24,5 +25,5 @@ from .ops import (  # noqa: F401
 
 __all__ = [
     "batch_bid_fused_chunk_gla", "bid_fused_recurrent_gla", "dirgate", "dwconv3x3", "fused_chunk_gla",
-    "fused_recurrent_gla", "gla_bidir_backward", "gla_bidir_forward", "gla_bidir_locality_gate", "locality_blend", "locality_gate", "rmsnorm", "split_heads", "swiglu",
+    "fused_recurrent_gla", "gla_bidir_backward", "gla_bidir_forward", "gla_causal_state_forward", "gla_bidir_locality_gate", "locality_blend", "locality_gate", "rmsnorm", "split_heads", "swiglu",
 ]

@@ -31,6 +31,9 @@ SIGNATURES = {
     "vig_gla_bidir_fwd_workspace": (_c_size_t, [_c_int] * 6),
     "vig_gla_bidir_fwd_noalloc": (_c_int, [_c_void_p] * 6 + [_c_int] * 5 + [_c_float, _c_float, _c_int, _c_int, _c_void_p]),
     "vig_gla_bidir_fwd_noalloc_max_workspace": (_c_size_t, []),
+    "vig_gla_causal_state_fwd": (_c_int, [_c_void_p] * 7 + [_c_void_p, _c_size_t] + [_c_int] * 5 + [_c_float, _c_float, _c_int, _c_int, _c_void_p]),
+    "vig_gla_causal_state_fwd_exact": (_c_int, [_c_void_p] * 7 + [_c_int] * 5 + [_c_float, _c_float, _c_int, _c_int, _c_void_p]),
+    "vig_gla_causal_state_fwd_workspace": (_c_size_t, [_c_int] * 7),
     "vig_gla_bidir_fwd_workspace_for": (_c_size_t, [_c_int] * 8),
     "vig_gla_bidir_bwd": (_c_int, [_c_void_p] * 11 + [_c_void_p, _c_size_t] + [_c_int] * 5 + [_c_float, _c_float, _c_int, _c_int, _c_void_p]),
     "vig_gla_bidir_bwd_exact": (_c_int, [_c_void_p] * 11 + [_c_void_p, _c_size_t] + [_c_int] * 5 + [_c_float, _c_float, _c_int, _c_int, _c_void_p]),

@@ -194,6 +194,55 @@ int vig_gla_bidir_fwd(const void* q, const void* k, const void* v, const void* g
                        io_dtype, gate_dtype, stream, 0);
 }
 
+// The causal op with a state carried in and / or out.
+static size_t causal_state_workspace(int B, int H, int L, int Dk, int Dv, int io_dtype, int gate_dtype) {
+  if (io_dtype == VIG_BF16 && gate_dtype == VIG_BF16 && (Dk == 64 || Dk == 32) && Dv == 64)
+    return vig::gla_mfma_state_workspace(B, H, L, Dk, Dv);
+  return 0;  // the token-recurrent kernel keeps the state in registers
+}
+
+size_t vig_gla_causal_state_fwd_workspace(int B, int H, int L, int Dk, int Dv, int io_dtype, int gate_dtype) {
+  if (B <= 0 || H <= 0 || L <= 0 || !dtype_ok(io_dtype) || !dtype_ok(gate_dtype)) return 0;
+  return causal_state_workspace(B, H, L, Dk, Dv, io_dtype, gate_dtype);
+}
+
+static int causal_state_fwd(const void* q, const void* k, const void* v, const void* g, void* o,
+                            const float* initial_state, float* final_state, void* workspace, size_t workspace_bytes,
+                            int B, int H, int L, int Dk, int Dv, float scale, float out_scale, int io_dtype,
+                            int gate_dtype, void* stream, bool exact) {
+  vig::GlaArgs a;
+  const int rc = fill_args(a, q, k, v, g, nullptr, o, workspace, workspace_bytes, B, H, L, Dk, Dv, scale, out_scale,
+                           io_dtype, gate_dtype, stream);
+  if (rc != VIG_OK) return rc;
+  if (!aligned16(initial_state, final_state)) return VIG_EINVAL;
+  a.init_state = initial_state;
+  a.final_state = final_state;
+  if (!exact && vig::gla_mfma_supported(a)) {
+    if ((long long)B * H > 65535) return VIG_ENOTSUP;  // (the segment scan puts the sequences on grid.y)
+    const size_t need = vig::gla_mfma_state_workspace(B, H, L, Dk, Dv);
+    if (need > workspace_bytes) return VIG_ENOSPC;
+    if (!workspace) return VIG_EINVAL;
+    return vig::launch_gla_mfma(a);
+  }
+  return vig::launch_gla_recurrent(a);
+}
+
+int vig_gla_causal_state_fwd(const void* q, const void* k, const void* v, const void* g, void* o,
+                             const float* initial_state, float* final_state, void* workspace, size_t workspace_bytes,
+                             int B, int H, int L, int Dk, int Dv, float scale, float out_scale, int io_dtype,
+                             int gate_dtype, void* stream) {
+  return causal_state_fwd(q, k, v, g, o, initial_state, final_state, workspace, workspace_bytes, B, H, L, Dk, Dv, scale,
+                          out_scale, io_dtype, gate_dtype, stream, false);
+}
+
+// Same contract, always the fp32-arithmetic token-recurrent kernel (no workspace).
+int vig_gla_causal_state_fwd_exact(const void* q, const void* k, const void* v, const void* g, void* o,
+                                   const float* initial_state, float* final_state, int B, int H, int L, int Dk, int Dv,
+                                   float scale, float out_scale, int io_dtype, int gate_dtype, void* stream) {
+  return causal_state_fwd(q, k, v, g, o, initial_state, final_state, nullptr, 0, B, H, L, Dk, Dv, scale, out_scale,
+                          io_dtype, gate_dtype, stream, true);
+}
+
 // Same contract and results to the same bar; for callers whose gates are known to be strong (see the header).
 int vig_gla_bidir_fwd_wide(const void* q, const void* k, const void* v, const void* g_fwd, const void* g_bwd, void* o,
                            void* workspace, size_t workspace_bytes, int B, int H, int L, int Dk, int Dv, float scale,

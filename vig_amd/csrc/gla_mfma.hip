@@ -841,7 +841,11 @@ __global__ __launch_bounds__(512) void gla_mfma_kernel(const uint16_t* __restric
 // decay D_s) is replaced by the state entering it,  S_in(s') = D_s * S_in(s) + U_s  with s' the next segment in the
 // direction's walk order.  One thread per state element; all accesses are coalesced (unit order is kept).  The
 // contributions and decays of eight segments are fetched together, so that the serial part is arithmetic only.
-__global__ __launch_bounds__(256) void gla_segment_scan_kernel(float* state_ws, int nseq, int nseg, int ndir, int ng) {
+// The causal op may start from a caller's state and hand the last one back (init / final: fp32 [nseq, Dk, Dv] row-major,
+// null: zero / not wanted; one direction only): the thread of state element e is also the one that knows its row
+// (k channel) and column (v channel).
+__global__ __launch_bounds__(256) void gla_segment_scan_kernel(float* state_ws, int nseq, int nseg, int ndir, int ng,
+                                                               const float* __restrict__ init, float* __restrict__ final) {
   const int e = blockIdx.x * 256 + threadIdx.x;  // element in unit order: ((u*64 + lane)*4 + m)
   const int seq = blockIdx.y / ndir, dir = blockIdx.y % ndir;
   if (seq >= nseq) return;
@@ -851,6 +855,10 @@ __global__ __launch_bounds__(256) void gla_segment_scan_kernel(float* state_ws, 
   const int ch = 8 * ng * h + 8 * cq + 2 * m + pk;
   constexpr int kBatch = 8;
   float S = 0.f;
+  // column of the state held by (lane, unit): the v channel the accumulator column r of output tile pv belongs to
+  const int vch = 2 * cpair<4>(lane & 31) + ((u >> 2) & 1);
+  const size_t rc = ((size_t)seq * (16 * ng) + ch) * 64 + vch;
+  if (init) S = init[rc];
   for (int i0 = 0; i0 < nseg; i0 += kBatch) {
     float us[kBatch], ds[kBatch];
 #pragma unroll
@@ -871,6 +879,7 @@ __global__ __launch_bounds__(256) void gla_segment_scan_kernel(float* state_ws, 
       }
     }
   }
+  if (final) final[rc] = S;
 }
 
 static Geometry make_geometry(int nseq, int L) {
@@ -895,6 +904,13 @@ bool gla_mfma_supported(const GlaArgs& a) {
 
 size_t gla_mfma_workspace(int B, int H, int L, int Dk, int Dv) {
   if ((Dk != 64 && Dk != 32) || Dv != 64 || L <= 256) return 0;
+  const Geometry g = make_geometry(B * H, L);
+  return (size_t)g.nitems * 2 * kStateFloats * sizeof(float);
+}
+
+// with an initial or final state every sequence goes through the segment passes, also a single-segment one
+size_t gla_mfma_state_workspace(int B, int H, int L, int Dk, int Dv) {
+  if ((Dk != 64 && Dk != 32) || Dv != 64) return 0;
   const Geometry g = make_geometry(B * H, L);
   return (size_t)g.nitems * 2 * kStateFloats * sizeof(float);
 }
@@ -936,16 +952,17 @@ static int launch_gla_mfma_t(const GlaArgs& a, int num_cu, int dev) {
     geo.heads = a.H;
     hipLaunchKernelGGL((gla_mfma_kernel<kModeSlab, NG, true>), dim3(grid), dim3(512), kLdsTotal, a.stream, q, k, v, gf,
                        gb, o, geo, oscale, (float*)nullptr, a.gate_w);
-  } else if (geo.nseg == 1) {
+  } else if (geo.nseg == 1 && !a.init_state && !a.final_state) {
     hipLaunchKernelGGL((gla_mfma_kernel<kModeSlab, NG>), dim3(grid), dim3(512), kLdsTotal, a.stream, q, k, v, gf, gb, o,
                        geo, oscale, (float*)nullptr, no_gate);
   } else {
+    if ((a.init_state || a.final_state) && gb) return -22;  // a state in or out belongs to the causal op
     float* ws = (float*)a.workspace;
     hipLaunchKernelGGL((gla_mfma_kernel<kModeState, NG>), dim3(grid), dim3(512), kLdsTotal, a.stream, q, k, v, gf, gb, o,
                        geo, oscale, ws, no_gate);
     const int ndir = gb ? 2 : 1;
     hipLaunchKernelGGL(gla_segment_scan_kernel, dim3(64 * 64 / 256, a.B * a.H * ndir), dim3(256), 0, a.stream, ws,
-                       a.B * a.H, geo.nseg, ndir, NG);
+                       a.B * a.H, geo.nseg, ndir, NG, a.init_state, a.final_state);
     hipLaunchKernelGGL((gla_mfma_kernel<kModeChain, NG>), dim3(grid), dim3(512), kLdsTotal, a.stream, q, k, v, gf, gb, o,
                        geo, oscale, ws, no_gate);
   }

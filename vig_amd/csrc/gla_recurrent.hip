@@ -21,7 +21,8 @@ template <typename TIO, typename TG, int DKG, int TB>
 __global__ __launch_bounds__(256) void gla_recurrent_kernel(
     const TIO* __restrict__ q, const TIO* __restrict__ k, const TIO* __restrict__ v,
     const TG* __restrict__ gf, const TG* __restrict__ gb, TIO* o,
-    float* acc, int L, int Dv, float scale, float out_scale) {
+    float* acc, int L, int Dv, float scale, float out_scale, const float* __restrict__ init_state,
+    float* __restrict__ final_state) {
   constexpr int DK = DKG * 4;
   __shared__ float sq[TB][DK];
   __shared__ float sk[TB][DK];
@@ -46,6 +47,11 @@ __global__ __launch_bounds__(256) void gla_recurrent_kernel(
     float S[DKG];
 #pragma unroll
     for (int j = 0; j < DKG; ++j) S[j] = 0.f;
+    // causal op: the state may start from a caller-supplied value (fla/ops/gla/chunk_fuse.py:70-72)
+    if (init_state && pass == 0 && dv_ok) {
+#pragma unroll
+      for (int j = 0; j < DKG; ++j) S[j] = init_state[((size_t)bh * DK + w * DKG + j) * Dv + dv];
+    }
 
     for (int ib = 0; ib < nblk; ++ib) {
       const int blk = pass ? (nblk - 1 - ib) : ib;
@@ -104,6 +110,11 @@ __global__ __launch_bounds__(256) void gla_recurrent_kernel(
       }
       __syncthreads();
     }
+    // ... and be handed back after the last token (chunk_fuse.py:99-101); padding tokens of the last block are no-ops
+    if (final_state && pass == 0 && dv_ok) {
+#pragma unroll
+      for (int j = 0; j < DKG; ++j) final_state[((size_t)bh * DK + w * DKG + j) * Dv + dv] = S[j];
+    }
   }
 }
 
@@ -118,7 +129,8 @@ static int launch_recurrent_t(const GlaArgs& a) {
 #define VIG_LAUNCH_REC(DKG)                                                                   \
   hipLaunchKernelGGL((gla_recurrent_kernel<TIO, TG, DKG, TB>), grid, block, 0, a.stream,      \
                      (const TIO*)a.q, (const TIO*)a.k, (const TIO*)a.v, (const TG*)a.g_fwd,   \
-                     (const TG*)a.g_bwd, (TIO*)a.o, acc, a.L, a.Dv, a.scale, a.out_scale)
+                     (const TG*)a.g_bwd, (TIO*)a.o, acc, a.L, a.Dv, a.scale, a.out_scale, a.init_state,   \
+                     a.final_state)
   switch (a.Dk) {
     case 16: VIG_LAUNCH_REC(4); break;
     case 32: VIG_LAUNCH_REC(8); break;

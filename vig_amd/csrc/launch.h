@@ -25,6 +25,9 @@ struct GlaArgs {
   // bf16 MFMA path: the caller expects gates beyond the fp16 score variant's range (|chunk total| > ~8 nat in some
   // channel): start with the split-bf16 variant instead of finding out on the first segment of every workgroup
   int wide_gates = 0;
+  // causal op only (g_bwd null): fp32 [B, H, Dk, Dv] state before the first token / after the last one; null: zero / not wanted
+  const float* init_state = nullptr;
+  float* final_state = nullptr;
 };
 
 // fp32-arithmetic token-recurrent path (any supported dtype combination).
@@ -36,6 +39,7 @@ bool gla_mfma_supported(const GlaArgs& a);
 int launch_gla_mfma(const GlaArgs& a);
 bool gla_mfma_gate_grid_ok(int rows, int cols);  // token grids the fused locality gate takes
 size_t gla_mfma_workspace(int B, int H, int L, int Dk, int Dv);
+size_t gla_mfma_state_workspace(int B, int H, int L, int Dk, int Dv);  // causal op with an initial / final state
 
 // bf16 matrix-core backward (whole-slab quadratic form); flags[b*H + h] = 1 marks slabs it left to the recurrent kernel
 bool gla_backward_mfma_supported(int L, int Dk, int Dv, int io_dtype, int gate_dtype, bool bidir);

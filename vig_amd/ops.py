@@ -168,11 +168,54 @@ def _split_bid_gates(q, g):
     return g[:B], g[B:]
 
 
+def gla_causal_state_forward(q, k, v, g, initial_state=None, output_final_state: bool = False, scale: float = -1,
+                             exact: bool = False):
+    """The causal op with a state carried in and / or out: (o, final_state or None).
+
+    initial_state [B,H,Dk,Dv] (any float dtype; used as fp32, detached as in chunk_fuse.py:565-566) is the state
+    before the first token; final_state is fp32 [B,H,Dk,Dv] (chunk_fuse.py:353-356).  Forward only: the library's
+    backward kernels start from a zero state, so a call that records a gradient is refused."""
+    lib = _lib.load()
+    _check_cuda(q, k, v, g, initial_state)
+    if torch.is_grad_enabled() and any(t.requires_grad for t in (q, k, v, g)):
+        raise NotImplementedError("initial_state / output_final_state are forward-only in the HIP path")
+    q, k, v, g = (_dense(t) for t in (q, k, v, g))
+    B, H, L, Dk = q.shape
+    Dv = v.shape[-1]
+    if k.shape != q.shape or g.shape != q.shape or v.shape[:3] != q.shape[:3]:
+        raise ValueError("shape mismatch between q, k, v, g")
+    if k.dtype != q.dtype or v.dtype != q.dtype:
+        raise TypeError("q, k, v must share a dtype")
+    if scale == -1 or scale is None:
+        scale = Dk ** -0.5
+    s0 = None
+    if initial_state is not None:
+        if tuple(initial_state.shape) != (B, H, Dk, Dv):
+            raise ValueError(f"initial_state must be [B,H,Dk,Dv] = {(B, H, Dk, Dv)}; got {tuple(initial_state.shape)}")
+        s0 = _dense(initial_state.detach().float())
+    final = torch.empty(B, H, Dk, Dv, dtype=torch.float32, device=q.device) if output_final_state else None
+    out = torch.empty(B, H, L, Dv, dtype=q.dtype, device=q.device)
+    io_dt, g_dt = _dt(q), _dt(g)
+    ptrs = (q.data_ptr(), k.data_ptr(), v.data_ptr(), g.data_ptr(), out.data_ptr(),
+            s0.data_ptr() if s0 is not None else None, final.data_ptr() if final is not None else None)
+    tail = (B, H, L, Dk, Dv, float(scale), 1.0, io_dt, g_dt, _stream_ptr(q))
+    with torch.cuda.device(q.device):
+        if exact:
+            rc = lib.vig_gla_causal_state_fwd_exact(*ptrs, *tail)
+        else:
+            ws_bytes = lib.vig_gla_causal_state_fwd_workspace(B, H, L, Dk, Dv, io_dt, g_dt)
+            ws = torch.empty(ws_bytes, dtype=torch.uint8, device=q.device) if ws_bytes else None
+            rc = lib.vig_gla_causal_state_fwd(*ptrs, ws.data_ptr() if ws is not None else None, ws_bytes, *tail)
+    _lib.check(rc, "vig_gla_causal_state_fwd")
+    return out, final
+
+
 def fused_chunk_gla(q, k, v, g, scale: int = -1, initial_state=None, output_final_state: bool = False
                     ) -> Tuple[torch.Tensor, Optional[torch.Tensor]]:
-    """Causal GLA on [B,H,L,D] tensors; returns (o, final_state=None)."""
+    """Causal GLA on [B,H,L,D] tensors; returns (o, final_state) with final_state None unless asked for
+    (chunk_fuse.py:554-572)."""
     if initial_state is not None or output_final_state:
-        raise NotImplementedError("initial_state / output_final_state are not built in the HIP path")
+        return gla_causal_state_forward(q, k, v, g, initial_state, output_final_state, scale)
     return gla_bidir_forward(q, k, v, g, None, scale, 1.0), None
 
 
@@ -181,10 +224,12 @@ def fused_recurrent_gla(q, k, v, gk=None, gv=None, scale: int = -1, initial_stat
     """Causal recurrent GLA (fp32 state arithmetic); causal=False returns [o, o_reversed] with shared gates."""
     if gv is not None:
         raise NotImplementedError("value gates (gv) are not used by ViG and not built")
-    if initial_state is not None or output_final_state:
-        raise NotImplementedError("initial_state / output_final_state are not built in the HIP path")
     if gk is None:
         gk = torch.zeros_like(q)
+    if initial_state is not None or output_final_state:
+        if not causal:  # (recurrent_fuse.py:650-652 asserts the same)
+            raise NotImplementedError("bidirectional GLA takes no initial/final state")
+        return gla_causal_state_forward(q, k, v, gk, initial_state, output_final_state, scale, exact=True)
     o = gla_bidir_forward(q, k, v, gk, None, scale, 1.0, exact=True)
     if causal:
         return o, None
