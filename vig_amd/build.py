@@ -50,5 +50,30 @@ def build_library(extra_flags: list[str] | None = None, verbose: bool = True) ->
     return LIB
 
 
+EXT = os.path.join(LIBDIR, "libvig_torch_ext.so")
+
+
+def build_torch_extension(verbose: bool = True) -> str:
+    """Builds vig_amd/lib/libvig_torch_ext.so: the PyTorch-ROCm operator library over the C ABI (csrc/torch_ext.cpp).
+    Host code only, compiled with the host compiler against torch's headers and linked to libvig_gla.so next to it."""
+    import torch
+    from torch.utils import cpp_extension as ce
+
+    os.makedirs(LIBDIR, exist_ok=True)
+    tlib = os.path.join(os.path.dirname(torch.__file__), "lib")
+    inc = [f"-I{p}" for p in ce.include_paths()] + ["-I/opt/rocm/include"]
+    cmd = [os.environ.get("CXX", "g++"), "-O2", "-std=c++17", "-fPIC", "-shared", "-D__HIP_PLATFORM_AMD__=1", "-DUSE_ROCM=1",
+           f"-D_GLIBCXX_USE_CXX11_ABI={int(torch.compiled_with_cxx11_abi())}", "-Wno-deprecated-declarations", *inc,
+           os.path.join(CSRC, "torch_ext.cpp"), "-o", EXT, f"-L{LIBDIR}", "-lvig_gla", f"-L{tlib}", "-lc10", "-lc10_hip",
+           "-ltorch_cpu", "-ltorch_hip", "-ltorch", "-Wl,-rpath,$ORIGIN", f"-Wl,-rpath,{tlib}"]
+    r = subprocess.run(cmd, capture_output=True, text=True)
+    if r.returncode != 0:
+        raise RuntimeError(f"torch extension build failed:\n{' '.join(cmd)}\n{r.stdout}\n{r.stderr}")
+    if verbose:
+        print(f"built {EXT}")
+    return EXT
+
+
 if __name__ == "__main__":
     build_library(sys.argv[1:])
+    build_torch_extension()

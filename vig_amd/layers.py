@@ -32,7 +32,7 @@ import torch
 import torch.nn as nn
 import torch.nn.functional as F
 
-from . import ops
+from . import _ext, ops
 
 
 def _f32(owner: nn.Module, tag: str, t: Optional[torch.Tensor], shape=None):
@@ -110,6 +110,12 @@ class RMSNorm(_CacheMixin, nn.Module):
                 dt = torch.promote_types(x.dtype, residual.dtype)
                 x, residual = x.to(dt), residual.to(dt)
             return ops.rmsnorm(x, self.weight, self.eps, residual=residual, prenorm=prenorm, round_sum=round_sum)
+        ext = _ext.load()
+        if (ext is not None and x.is_cuda and not _recording(self) and x.is_contiguous()
+                and (residual is None or (residual.is_contiguous() and residual.dtype == x.dtype))):
+            # (operator library: checks, allocation and launch in one C++ call)
+            y, total = ext.rmsnorm_fwd(x, residual, self._w32(), self.eps, round_sum)
+            return (y, x if total is None else total) if prenorm else y
         return ops.rmsnorm(x, self._w32(), self.eps, residual=residual, prenorm=prenorm, round_sum=round_sum)
 
 
@@ -176,6 +182,14 @@ class GatedLinearAttention(_CacheMixin, nn.Module):
         consumers read their column blocks of the result in place.  Every output column is the same dot product (and
         bias add) as in the separate layers.  The stacked copy follows the parameters: it is rebuilt when one of them
         is replaced, moved, cast or written in place."""
+        w, b = self._stacked_in()
+        z = F.linear(xs, w, b)
+        n0 = self.qkv_proj.weight.shape[0]
+        n1 = n0 + self.value_dim
+        return z[..., :n0], z[..., n0:n1], z[..., n1:n1 + self.gk_proj[0].weight.shape[0]]
+
+    def _stacked_in(self):
+        """(weight, bias) of the stacked input projection: rows qkv | g | low-rank gate, zero-padded to a multiple of 128."""
         srcs = (self.qkv_proj.weight, self.g_proj.weight, self.g_proj.bias, self.gk_proj[0].weight)
         key = tuple((t.data_ptr(), t._version, t.dtype, t.device) for t in srcs)
         if self._in_cat is None or self._in_cat[0] != key:
@@ -186,16 +200,23 @@ class GatedLinearAttention(_CacheMixin, nn.Module):
             w[:n] = torch.cat((wq, wg, wr), 0)
             b[wq.shape[0]:wq.shape[0] + wg.shape[0]] = bg
             self._in_cat = (key, w, b)
-        _, w, b = self._in_cat
-        z = F.linear(xs, w, b)
-        n0 = self.qkv_proj.weight.shape[0]
-        n1 = n0 + self.value_dim
-        return z[..., :n0], z[..., n0:n1], z[..., n1:n1 + self.gk_proj[0].weight.shape[0]]
+        return self._in_cat[1], self._in_cat[2]
 
     def _mix(self, x, hw, out_scale):
         """The token mixer on x [B, L, C] with L = h*w tokens in row-major grid order."""
         H = self.num_heads
         conv = self.in_proj[0]
+        ext = _ext.load()
+        if (ext is not None and x.is_cuda and x.is_contiguous() and self.gk_proj[0].weight.shape[0] == ops.GATE_RANK
+                and x.dtype == self.qkv_proj.weight.dtype):
+            # the whole mixer as one operator of the library (csrc/torch_ext.cpp: the same kernel sequence as below)
+            w_in, b_in = self._stacked_in()
+            up = self.gk_proj[1]
+            return ext.gla_block_mix(x, hw[0], hw[1], _f32(self, "conv_w_flat", conv.weight, (-1,)),
+                                     _f32(self, "conv_b", conv.bias), self.use_act_in_conv, w_in, b_in, H,
+                                     self.head_qk_dim, self.head_v_dim, up.weight, up.bias, self.gate_logit_normalizer,
+                                     self.clamp_min, self.g_norm._w32(), self.l_norm._w32(), self.layernorm_eps,
+                                     self.use_out_act, self.o_proj.weight, out_scale)
         # local_out, already in the [B, L, C] layout the projections consume
         xs = ops.dwconv3x3(x, _f32(self, "conv_w", conv.weight, (-1, 3, 3)), hw, bias=_f32(self, "conv_b", conv.bias),
                            silu=self.use_act_in_conv)
@@ -297,6 +318,9 @@ class GLAMLP(nn.Module):
             return self.down_proj(ops.swiglu(self.gate_proj(x)))
         w = self.gate_proj.weight
         if ops.linear_swiglu_supported(x, w):  # ViG-S / ViG-T widths in bf16: no [.., 2*I] intermediate
+            ext = _ext.load()
+            if ext is not None and x.is_contiguous():
+                return self.down_proj(ext.linear_swiglu_fwd(x, w))
             return self.down_proj(ops.linear_swiglu(x, w))
         return self.down_proj(ops.swiglu(self.gate_proj(x)))
 
@@ -347,6 +371,23 @@ class GLABlock(nn.Module):
     def forward_carry(self, branch, residual, **kwargs):
         """Same block, with the closing `residual + mlp(h)` of the previous block folded into this block's first norm:
         takes (branch, residual) with hidden_states = residual + branch and returns the next such pair."""
+        ext = _ext.load()
+        at = self.attn
+        if (ext is not None and not _recording(self) and not self.training and branch.is_cuda and branch.is_contiguous()
+                and type(at) is GatedLinearAttention and at.gk_proj[0].weight.shape[0] == ops.GATE_RANK
+                and branch.dtype == at.qkv_proj.weight.dtype and kwargs.get("token_position", None) is None
+                and (residual is None or (residual.is_contiguous() and residual.dtype == branch.dtype))):
+            # the whole block as one operator of the library (csrc/torch_ext.cpp: the same kernel sequence as below)
+            hw = tuple(kwargs["patch_resolution"])
+            conv, up = at.in_proj[0], at.gk_proj[1]
+            w_in, b_in = at._stacked_in()
+            with torch.no_grad():
+                return ext.gla_block_carry(
+                    branch, residual, self.attn_norm._w32(), self.attn_norm.eps, hw[0], hw[1],
+                    _f32(at, "conv_w_flat", conv.weight, (-1,)), _f32(at, "conv_b", conv.bias), at.use_act_in_conv, w_in,
+                    b_in, at.num_heads, at.head_qk_dim, at.head_v_dim, up.weight, up.bias, at.gate_logit_normalizer,
+                    at.clamp_min, at.g_norm._w32(), at.l_norm._w32(), at.layernorm_eps, at.use_out_act, at.o_proj.weight,
+                    0.25, self.mlp_norm._w32(), self.mlp.gate_proj.weight, self.mlp.down_proj.weight)
         if residual is None:
             h, hidden = self.attn_norm(branch), branch
         else:  # the explicit add stores a rounded sum and attn_norm normalises that (vig.py:598,606)
