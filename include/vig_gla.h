@@ -61,10 +61,11 @@ const char* vig_gla_strerror(int code);
  * Numeric range of the matrix-core path (bf16 tensors and gates, Dk in {32, 64},
  * Dv = 64): the sum of |g| over any 64 consecutive tokens of one channel must
  * stay below about 80 (beyond it results may be inf / NaN, never silently wrong
- * finite numbers).  q and k may hold any finite bf16 values: the kernel checks
- * their magnitudes and the gate totals per chunk and takes its fp16-operand
- * scores only where they are exact enough (|q|, |k| < 512, gate total of a chunk
- * within about 8), split-bf16 scores otherwise.  HierViG's head shape
+ * finite numbers).  q, k and v may hold any finite bf16 values: the kernel
+ * checks their magnitudes and the gate totals per chunk and takes its fp16
+ * operands (scaled q and k, scores, v) only where they are exact enough (rows
+ * with sums of squares below 2^15, i.e. elements below about 180; gate total of
+ * a chunk within about 8), bf16 hi + lo pairs otherwise.  HierViG's head shape
  * (bf16, Dk = 16, Dv = 32, both directions) takes the same path from L = 128 on,
  * zero-padded to Dk 32 / Dv 64 in the workspace (classification/models/vig_h.py:
  * 377-385 with EXPAND_K 0.5, EXPAND_V 1.0).  Other combinations run on the

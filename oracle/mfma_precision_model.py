@@ -7,10 +7,11 @@ chunk_fuse.py:76-97, here with the anchor at half the chunk total: q~ = q*exp(G 
 so state update and inter-chunk product carry exp(G_end/2) each.
 
 splits:  qk = score operands: "f16" (one fp16 rounding each), 1 (bf16 hi*hi) or 3 (+ lo*hi + hi*lo),
-         p = P terms in P V (1 or 2),  iq = q~ terms in the inter-chunk product, st = state terms,
-         u = k~ terms in the state update.
-The shipped kernel is qk="f16", p=2, iq=1, st=1, u=1 and falls back to qk=3 for chunks whose gate total leaves
-the fp16 range (FALLBACK).
+         p = P terms in P V: "f16" (P rounded once to fp16; V is exact in fp16), 1 or 2 (bf16 hi, hi + lo),
+         iq = q~ terms in the inter-chunk product, st = state terms,
+         u = k~ in the state update: "f16" (the score operand again), 1 or 2 bf16 terms.
+The shipped kernel is qk="f16", p="f16", iq=1, st=1, u="f16"; for chunks whose gate total or operand magnitudes leave
+the fp16 range it falls back to qk=3, p=2, u=1 (FALLBACK).
 """
 from __future__ import annotations
 
@@ -39,7 +40,7 @@ def f16_round(x):
     return np.asarray(x, dtype=np.float32).astype(np.float16).astype(np.float32)
 
 
-SHIPPED = dict(qk="f16", p=2, iq=1, st=1, u=1)
+SHIPPED = dict(qk="f16", p="f16", iq=1, st=1, u="f16")
 FALLBACK = dict(qk=3, p=2, iq=1, st=1, u=1)
 PLAIN = dict(qk=1, p=1, iq=1, st=1, u=1)
 
@@ -81,10 +82,13 @@ def emulate(q, k, v, gf, gb, chunk, splits=SHIPPED):
                 if splits["qk"] >= 3:
                     P += _mm(ql, T(kh)) + _mm(qh, T(kl))
             P *= tri
-            Ph, Pl = _split(P)
-            oc = _mm(Ph, vc)
-            if splits["p"] >= 2:
-                oc += _mm(Pl, vc)
+            if splits["p"] == "f16":
+                oc = _mm(f16_round(P), vc)
+            else:
+                Ph, Pl = _split(P)
+                oc = _mm(Ph, vc)
+                if splits["p"] >= 2:
+                    oc += _mm(Pl, vc)
             sd = T(np.exp(half).astype(np.float32))  # half decay per key channel
             Sd = S * sd
             Sh, Sl = _split(Sd)
@@ -94,8 +98,11 @@ def emulate(q, k, v, gf, gb, chunk, splits=SHIPPED):
             if splits["st"] >= 2:
                 oc += _mm(qh, Sl)
             o[:, sl] += s * oc
-            U = _mm(T(kh), vc)
-            if splits["u"] >= 2:
-                U += _mm(T(kl), vc)
+            if splits["u"] == "f16":
+                U = _mm(T(f16_round(kt)), vc)
+            else:
+                U = _mm(T(kh), vc)
+                if splits["u"] >= 2:
+                    U += _mm(T(kl), vc)
             S = (Sd + U) * sd
     return o

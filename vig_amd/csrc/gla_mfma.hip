@@ -19,7 +19,7 @@
 // bf16 once.  Loads for the next slab are issued before the swap.
 //
 // fp16 score operands need |G_end|/2 * log2(e) <= 6 in every channel of every chunk (ViG's
-// logsigmoid(.)/16 gates reach about 2.5) and |q|, |k| below 512; every wave checks both for
+// logsigmoid(.)/16 gates reach about 2.5) and rows of q, k, V with sums of squares below 2^15; every wave checks both for
 // its chunk.  A workgroup that meets a segment outside that range redoes it, and does all its later
 // segments, with bf16 hi + lo operands and three score terms per k-step (same algebra,
 // any gate total up to ~80 per chunk and channel).
@@ -79,10 +79,11 @@ __device__ __forceinline__ void gram_acc(const u32x4_t& raw, f32x4acc_t& acc) {
   acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, raw), __builtin_bit_cast(bf16x8_t, raw), acc,
                                                 0, 0, 0);
 }
-// fp16 operands are raw * 2^x with |x| <= kFastHalfRange = 6: they stay finite while |raw| < 65504 / 64.  The guard
-// asks for every sum of squares below 2^18, i.e. every |raw| < 512 (inf or huge inputs fail it; NaN inputs give NaN
-// outputs on every path).
-constexpr float kFastMaxSquares = 262144.0f;
+// The fp16 variant rounds q~ = q 2^x and k~ = k 2^-x (|x| <= kFastHalfRange = 6), the scores P = q~ . k~ and V to fp16.
+// With every row's sum of squares below 2^15 (the guard sums the rows of two tokens of q, k and V, which only makes it
+// stricter), elements stay below 182, the scaled operands below 182 * 64, and |P| <= |q_i| |k_j| below 2^15: all
+// inside fp16 range.  Inf or huge inputs fail the guard; NaN inputs give NaN outputs on every path.
+constexpr float kFastMaxSquares = 32768.0f;
 __device__ __forceinline__ bool gram_too_large(const f32x4acc_t& acc) {
   const float m = fmaxf(fmaxf(fabsf(acc[0]), fabsf(acc[1])), fmaxf(fabsf(acc[2]), fabsf(acc[3])));
   return __builtin_amdgcn_ballot_w64(!(m < kFastMaxSquares)) != 0;
@@ -122,12 +123,13 @@ __device__ __forceinline__ void make_half(const u32x4_t (&raw)[NG], const f32x16
 }
 
 // q~ and k~ of one 32-token tile for the fp16 score path: one exponent per element serves both (the factors are
-// reciprocal), each product is rounded once to fp16 (11-bit significand) for the scores and once to bf16 for the
-// state path (k~: state update through LDS; q~: inter-chunk product).
+// reciprocal), each product is rounded once to fp16 (11-bit significand): k~ serves the scores and, through LDS, the
+// state update (against V converted to fp16, which holds every bf16 value of ordinary magnitude exactly); q~ is
+// rounded a second time to bf16 for the inter-chunk product with the bf16 state fragments.
 template <bool WITH_Q, int NG>
 __device__ __forceinline__ void make_pair16(const u32x4_t (&rawq)[NG], const u32x4_t (&rawk)[NG],
                                             const f32x16_t (&G)[2], const float* gend2, u32x4_t (&q16)[NG],
-                                            u32x4_t (&k16)[NG], u32x4_t (&qb)[NG], u32x4_t (&kb)[NG]) {
+                                            u32x4_t (&k16)[NG], u32x4_t (&qb)[NG]) {
 #pragma unroll
   for (int g = 0; g < NG; ++g) {
     const f32x4_t a0 = *reinterpret_cast<const f32x4_t*>(gend2 + 4 * g);
@@ -141,7 +143,6 @@ __device__ __forceinline__ void make_pair16(const u32x4_t (&rawq)[NG], const u32
       const float k0 = bf16lo_to_f32(wk) * exp2_fast(-x0);
       const float k1 = bf16hi_to_f32(wk) * exp2_fast(-x1);
       k16[g][m] = pack_f16x2(k0, k1);
-      kb[g][m] = pack_bf16x2(k0, k1);
       if (WITH_Q) {
         const uint32_t wq = rawq[g][m];
         const float q0 = bf16lo_to_f32(wq) * exp2_fast(x0);
@@ -176,9 +177,10 @@ __device__ __forceinline__ f32x16_t score_tile(const HalfOps<NG>& kop, const Hal
   return acc;
 }
 
-// O^T[p] += V^T (k-steps 2*jt, 2*jt+1 of vfrag) x P^T tile, with P split hi + lo.
+// O^T[p] += V^T (k-steps 2*jt, 2*jt+1 of vfrag) x P^T tile, with P split into bf16 hi + lo against bf16 V, or (F16)
+// P as one fp16 operand against fp16 V.
 // MASK: 0 none, 1 keep j <= i (forward diagonal tile), 2 keep j >= i (reverse diagonal tile).
-template <int MASK>
+template <int MASK, bool F16 = false>
 __device__ __forceinline__ void apply_scores(f32x16_t P, int jt, int r, int h, const u32x4_t (&vfrag)[4][2],
                                              f32x16_t& O0, f32x16_t& O1) {
   if (MASK != 0) {
@@ -188,6 +190,21 @@ __device__ __forceinline__ void apply_scores(f32x16_t P, int jt, int r, int h, c
       const bool keep = MASK == 1 ? (j <= r) : (j >= r);
       P[c] = keep ? P[c] : 0.f;
     }
+  }
+  if (F16) {  // P rounded once to fp16 (11-bit significand) against fp16 V: one term
+#pragma unroll
+    for (int tl = 0; tl < 2; ++tl) {
+      u32x4_t ph;
+#pragma unroll
+      for (int x = 0; x < 4; ++x) {
+        const int c = 4 * (2 * tl + (x >> 1)) + 2 * (x & 1);
+        ph[x] = pack_f16x2(P[c], P[c + 1]);
+      }
+      const int t = 2 * jt + tl;
+      O0 = mfma_f16(vfrag[t][0], ph, O0);
+      O1 = mfma_f16(vfrag[t][1], ph, O1);
+    }
+    return;
   }
 #pragma unroll
   for (int tl = 0; tl < 2; ++tl) {
@@ -270,13 +287,21 @@ __device__ __forceinline__ bool tile_phase(const ChunkSrc& cur, const Prefetch<N
     for (int j = 0; j < 2; ++j) O[i][j] = f32x16_t{0.f};
   u32x4_t rawk[NG], rawq[NG];
   uint32_t vDb[2][8];
+  f32x4acc_t gram = {0.f, 0.f, 0.f, 0.f};  // (fp16 variant) magnitude guard over the chunk's q, k and V
   auto set_vfrag = [&](const uint32_t (&D)[2][8], int t0) {
     u32x4_t vf[2][2];
     finish_tfrags<2>(D, vf);
 #pragma unroll
     for (int tl = 0; tl < 2; ++tl)
 #pragma unroll
-      for (int p = 0; p < 2; ++p) vfrag[t0 + tl][p] = vf[tl][p];
+      for (int p = 0; p < 2; ++p) {
+        if (F16) {  // bf16 pairs -> fp16 pairs (exact for magnitudes the variant admits: the guard sees them first)
+          gram_acc(vf[tl][p], gram);
+#pragma unroll
+          for (int x = 0; x < 4; ++x) vf[tl][p][x] = pack_f16x2(bf16lo_to_f32(vf[tl][p][x]), bf16hi_to_f32(vf[tl][p][x]));
+        }
+        vfrag[t0 + tl][p] = vf[tl][p];
+      }
   };
   auto fetch_second = [&]() {
     if (OUT) issue_raw_tile<NG>(cur.q, TB, r, h, rawq);
@@ -285,7 +310,6 @@ __device__ __forceinline__ bool tile_phase(const ChunkSrc& cur, const Prefetch<N
   };
   bool too_large = false;
   if (F16) {
-    f32x4acc_t gram = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
     for (int g = 0; g < NG; ++g) {
       gram_acc(pf.rawk[g], gram);
@@ -298,13 +322,13 @@ __device__ __forceinline__ bool tile_phase(const ChunkSrc& cur, const Prefetch<N
     if (EARLY) fetch_second();
     VIG_PHASE();
     {
-      u32x4_t qa[NG], kab[NG];
-      make_pair16<OUT, NG>(pf.rawq, pf.rawk, G[TA], gend2, qa, ka, qkeep[TA], kab);
-      store_kt<NG>(kt, 32 * TA + r, h, kab);
+      u32x4_t qa[NG];
+      make_pair16<OUT, NG>(pf.rawq, pf.rawk, G[TA], gend2, qa, ka, qkeep[TA]);
+      store_kt<NG>(kt, 32 * TA + r, h, ka);
       VIG_PHASE();
       if (!EARLY) fetch_second();
       set_vfrag(pf.vD, 2 * TA);
-      if (OUT) apply_scores<MASK>(score_tile16<NG>(ka, qa), TA, r, h, vfrag, O[0][TA], O[1][TA]);
+      if (OUT) apply_scores<MASK, true>(score_tile16<NG>(ka, qa), TA, r, h, vfrag, O[0][TA], O[1][TA]);
     }
     VIG_PHASE();
 #pragma unroll
@@ -313,15 +337,12 @@ __device__ __forceinline__ bool tile_phase(const ChunkSrc& cur, const Prefetch<N
       if (OUT) gram_acc(rawq[g], gram);
     }
     u32x4_t kb[NG];
-    {
-      u32x4_t kbb[NG];
-      make_pair16<OUT, NG>(rawq, rawk, G[TB], gend2, qb, kb, qkeep[TB], kbb);
-      store_kt<NG>(kt, 32 * TB + r, h, kbb);
-    }
-    if (OUT) apply_scores<0>(score_tile16<NG>(ka, qb), TA, r, h, vfrag, O[0][TB], O[1][TB]);
+    make_pair16<OUT, NG>(rawq, rawk, G[TB], gend2, qb, kb, qkeep[TB]);
+    store_kt<NG>(kt, 32 * TB + r, h, kb);
+    if (OUT) apply_scores<0, true>(score_tile16<NG>(ka, qb), TA, r, h, vfrag, O[0][TB], O[1][TB]);
     VIG_PHASE();
     set_vfrag(vDb, 2 * TB);
-    if (OUT) apply_scores<MASK>(score_tile16<NG>(kb, qb), TB, r, h, vfrag, O[0][TB], O[1][TB]);
+    if (OUT) apply_scores<MASK, true>(score_tile16<NG>(kb, qb), TB, r, h, vfrag, O[0][TB], O[1][TB]);
     too_large = gram_too_large(gram);
   } else {
     HalfOps<NG> ka, qb;
@@ -488,7 +509,8 @@ __device__ __forceinline__ bool direction_wave(const ChunkSrc& cur, const ChunkS
 #pragma unroll
       for (int pk = 0; pk < 2; ++pk)
 #pragma unroll
-        for (int pv = 0; pv < 2; ++pv) U[pk][pv] = mfma(ktf[pk], vfrag[t][pv], U[pk][pv]);
+        for (int pv = 0; pv < 2; ++pv)
+          U[pk][pv] = F16 ? mfma_f16(ktf[pk], vfrag[t][pv], U[pk][pv]) : mfma(ktf[pk], vfrag[t][pv], U[pk][pv]);
     }
     // the chunk walked last is consumed by nobody inside the segment, unless the segment's own total is wanted
     if (MODE == kModeState || (FWD ? (c < 3) : (c > 0))) {
