@@ -171,9 +171,12 @@ int vig_gla_bidir_fwd_exact(const void* q, const void* k, const void* v,
  *   dg_fwd, dg_bwd [B, H, L, Dk] in gate_dtype (dg_bwd only when g_bwd != NULL).
  * `workspace` must hold vig_gla_bidir_bwd_workspace(...) bytes.
  * Built shapes: (Dk, Dv) in {(16,32), (32,32), (32,64), (64,32), (64,64)}, any L >= 1.
- * Dispatch: bf16 tensors + bf16 gates + Dk in {32, 64} + Dv = 64 + L <= 256 (both directions, or the causal op
- * with g_bwd == NULL) -> matrix-core kernel (bf16 operands, fp32 accumulation; gradients within ~1e-2 of their largest magnitude); a slab whose gate total exceeds
- * ~83 in some channel, and every other case -> fp32-arithmetic token-recurrent kernel.
+ * Dispatch: bf16 tensors + bf16 gates + Dk in {32, 64} + Dv = 64 (both directions, or the causal op with
+ * g_bwd == NULL) -> matrix-core kernel (bf16 operands, fp32 accumulation; gradients within ~1e-2 of their largest
+ * magnitude): one quadratic form per (batch, head) for L <= 256; a longer sequence as segments of <= 256 tokens linked
+ * by their states (two state passes of the forward kernel, a segment scan, then one quadratic form per segment;
+ * B*H*directions <= 65535).  A sequence with a segment whose gate total exceeds ~83 in some channel, and every other
+ * case -> fp32-arithmetic token-recurrent kernel.
  *
  * Replaces: FusedChunkGLAFunction.backward (flash-linear-attention/fla/ops/gla/chunk_fuse.py:413-518; gate
  * gradient :505-518) under the flip-concat glue of classification/models/vig.py:407-426, for both directions in

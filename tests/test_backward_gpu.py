@@ -197,6 +197,60 @@ def test_backward_mfma_causal(B, H, L, Dk):
     _check_mfma(got[:4], want, q)
 
 
+@pytest.mark.parametrize("B,H,L,Dk,bidir", [(2, 2, 257, 64, True), (1, 3, 300, 64, True), (2, 2, 512, 64, True),
+                                            (1, 2, 700, 64, True), (2, 3, 1030, 32, True), (1, 2, 300, 32, True),
+                                            (2, 2, 300, 64, False), (1, 3, 1000, 32, False)])
+def test_backward_mfma_long_sequences(B, H, L, Dk, bidir):
+    """L > 256: the sequence as chained segments on the matrix cores (state passes, segment scan, one quadratic form
+    per segment plus the products with the linking states), against the adjoint recurrences of the oracle."""
+    announce(f"segmented backward on the matrix cores B{B} H{H} L={L} Dk={Dk} bidirectional={bidir}")
+    q, k, v, gf, gb = make_gla_inputs(B, H, L, Dk, 64, seed=600 + L, dtype=torch.bfloat16)
+    do = _do(v.shape, 14, torch.bfloat16)
+    if bidir:
+        want = O.bidir_gla_backward(f64(q), f64(k), f64(v), f64(gf), f64(gb), f64(do), out_scale=0.5)
+        got = vig_amd.gla_bidir_backward(*(t.cuda() for t in (q, k, v, gf, gb, do)), out_scale=0.5)
+        _check_mfma(got, want, q)
+    else:
+        want = O.gla_recurrent_backward(f64(q), f64(k), f64(v), f64(gf), f64(do))
+        got = vig_amd.gla_bidir_backward(q.cuda(), k.cuda(), v.cuda(), gf.cuda(), None, do.cuda(), out_scale=1.0)
+        assert got[4] is None
+        _check_mfma(got[:4], want, q)
+
+
+def test_backward_mfma_long_sequences_many_segments_against_exact_path():
+    """More segments than workgroups and stronger gates (a state decays to nothing within a few segments), against the
+    fp32-arithmetic kernel on the same inputs; and a second call on the same workspace-sized problem gives the same bits."""
+    announce("segmented backward, 24 x 16 segments, against the recurrent kernel")
+    q, k, v, gf, gb = (t.cuda() for t in make_gla_inputs(8, 3, 4096, 64, 64, seed=78, dtype=torch.bfloat16))
+    do = _do(v.shape, 15, torch.bfloat16).cuda()
+    want = [f64(t) for t in vig_amd.gla_bidir_backward(q, k, v, gf, gb, do, out_scale=0.5, exact=True)]
+    got = vig_amd.gla_bidir_backward(q, k, v, gf, gb, do, out_scale=0.5)
+    _check_mfma(got, want, q.cpu())
+    again = vig_amd.gla_bidir_backward(q, k, v, gf, gb, do, out_scale=0.5)
+    for a, b in zip(got, again):
+        assert torch.equal(a, b)
+
+
+def test_backward_mfma_long_sequences_strong_gates_fall_back_per_sequence():
+    """One sequence of three has gates beyond the quadratic form's range in one of its segments: that whole sequence
+    comes from the recurrent kernel, bit for bit, the others from the matrix cores."""
+    announce("segmented backward, strong gates in one segment of one sequence")
+    B, H, L = 1, 3, 600
+    q, k, v, gf, gb = make_gla_inputs(B, H, L, 64, 64, seed=83, dtype=torch.bfloat16)
+    _, _, _, sf, sb = make_gla_inputs(B, H, L, 64, 64, seed=84, dtype=torch.bfloat16, gate_scale=2.0)
+    gf[:, 1, 400:], gb[:, 1, 400:] = sf[:, 1, 400:], sb[:, 1, 400:]
+    do = _do(v.shape, 16, torch.bfloat16)
+    dev = [t.cuda() for t in (q, k, v, gf, gb, do)]
+    exact = vig_amd.gla_bidir_backward(*dev, out_scale=0.5, exact=True)
+    got = vig_amd.gla_bidir_backward(*dev, out_scale=0.5)
+    for name, g_, e_ in zip(("dq", "dk", "dv", "dg_fwd", "dg_bwd"), got, exact):
+        assert torch.isfinite(g_.float()).all(), name
+        assert torch.equal(g_[:, 1], e_[:, 1]), name
+    want = O.bidir_gla_backward(f64(q), f64(k), f64(v), f64(gf), f64(gb), f64(do), out_scale=0.5)
+    keep = [0, 2]
+    _check_mfma([g_.cpu()[:, keep] for g_ in got], [w_[:, keep] for w_ in want], q[:, keep])
+
+
 def test_autograd_keeps_the_exact_path():
     """gla_bidir_forward(exact=True) under autograd: the backward runs the fp32-arithmetic kernel too, bit-equal to
     gla_bidir_backward(exact=True) (and different from the matrix-core gradients of the default path)."""

@@ -36,6 +36,13 @@ def test_workspace_sizes():
     n_qk, n_v = 2 * 3 * 50 * 64, 2 * 3 * 50 * 64
     assert wb(2, 3, 50, 64, 64, 1) == (3 * n_qk + n_v) * 4 + 2 * 3 * 4   # recurrent scratch + one flag per slab
     assert wb(2, 3, 50, 128, 64, 1) == 0                                  # no backward for Dk = 128
+    # L > 256 on the matrix cores: behind the 256-byte aligned scratch + flags, per (sequence, segment, direction) two
+    # state-pass slots, the S_in Q terms and carries (fp32) and three bf16 64 x 64 matrices
+    n_qk = n_v = 2 * 3 * 600 * 64
+    base = ((3 * n_qk + n_v) * 4 + 2 * 3 * 4 + 255) // 256 * 256
+    slots = 2 * 3 * 3 * 2
+    assert wb(2, 3, 600, 64, 64, 1) == base + slots * ((2 * (4096 + 64) + 4096 + 128) * 4 + 3 * 4096 * 2)
+    assert wb(2, 3, 600, 64, 32, 1) == (3 * n_qk + n_v // 2) * 4 + 2 * 3 * 4  # Dv = 32: recurrent kernel only
 
 
 def test_wrappers_reject_what_is_not_built():

@@ -263,8 +263,15 @@ static size_t recurrent_floats(int B, int H, int L, int Dk, int Dv, int bidir) {
   const size_t n_qk = (size_t)B * H * L * Dk, n_v = (size_t)B * H * L * Dv;
   return bidir ? 3 * n_qk + n_v : n_qk;
 }
+// ... and, 256-byte aligned behind the flags, what the matrix-core kernel needs for sequences longer than one slab
+static size_t flags_end(int B, int H, int L, int Dk, int Dv, int bidir) {
+  const size_t n = recurrent_floats(B, H, L, Dk, Dv, bidir) * sizeof(float) + (size_t)B * H * sizeof(int);
+  return (n + 255) / 256 * 256;
+}
 size_t gla_backward_workspace(int B, int H, int L, int Dk, int Dv, int bidir) {
-  return recurrent_floats(B, H, L, Dk, Dv, bidir) * sizeof(float) + (size_t)B * H * sizeof(int);
+  const size_t seg = gla_backward_mfma_workspace(B, H, L, Dk, Dv);
+  if (seg == 0) return recurrent_floats(B, H, L, Dk, Dv, bidir) * sizeof(float) + (size_t)B * H * sizeof(int);
+  return flags_end(B, H, L, Dk, Dv, bidir) + seg;
 }
 
 int launch_gla_backward(const void* q, const void* k, const void* v, const void* g_fwd, const void* g_bwd,
@@ -273,10 +280,11 @@ int launch_gla_backward(const void* q, const void* k, const void* v, const void*
                         int gate_dtype, bool exact, hipStream_t stream) {
   GlaBwdArgs a{q, k, v, g_fwd, g_bwd, d_o, dq, dk, dv, dg_fwd, dg_bwd, workspace, B, H, L, Dk, Dv,
                scale, out_scale, io_dtype, gate_dtype, stream, nullptr};
-  if (!exact && gla_backward_mfma_supported(L, Dk, Dv, io_dtype, gate_dtype, g_bwd != nullptr)) {
+  if (!exact && gla_backward_mfma_supported(B, H, L, Dk, Dv, io_dtype, gate_dtype, g_bwd != nullptr)) {
     int* flags = reinterpret_cast<int*>((float*)workspace + recurrent_floats(B, H, L, Dk, Dv, g_bwd != nullptr));
-    const int rc = launch_gla_backward_mfma(q, k, v, g_fwd, g_bwd, d_o, dq, dk, dv, dg_fwd, dg_bwd, flags, B, H, L,
-                                            Dk, scale * out_scale, stream);
+    void* seg_ws = (char*)workspace + flags_end(B, H, L, Dk, Dv, g_bwd != nullptr);
+    const int rc = launch_gla_backward_mfma(q, k, v, g_fwd, g_bwd, d_o, dq, dk, dv, dg_fwd, dg_bwd, flags, seg_ws, B,
+                                            H, L, Dk, scale * out_scale, stream);
     if (rc != 0) return rc;
     a.only_flagged = flags;  // slabs with gates beyond the matrix-core kernel's range
   }

@@ -1,5 +1,6 @@
-// Backward of the bidirectional GLA op on MFMA tiles (gfx950): bf16 tensors and gates, Dk in {32, 64}, Dv = 64,
-// L <= 256.
+// Backward of the bidirectional GLA op on MFMA tiles (gfx950): bf16 tensors and gates, Dk in {32, 64}, Dv = 64.
+// L <= 256 is one slab per (batch, head); a longer sequence is cut into the forward's segments (<= 256 tokens), each
+// handled like a slab plus three products with the states that link it to the other segments (see SEG below).
 //
 // Per direction the whole (batch, head) slab is one quadratic form (no chunk states): with G the inclusive
 // cumulative log-gate along the direction and the anchor a = G_total / 2,
@@ -76,7 +77,12 @@ __device__ __forceinline__ void mask_diag(f32x16_t& T, int r, int h, bool diag) 
 struct BwdSlab {
   const uint16_t *q, *k, *v, *gf, *gb, *d_o;
   uint16_t *dq, *dk, *dv, *dgf, *dgb;
+  // segments of a long sequence only (direction 1 follows direction 0 in each array):
+  const uint16_t *sp, *rp, *rpt;  // sqrt(D) S_in as [k channel][v], sqrt(D) R_out as [k channel][v] and as [v][k channel]
+  const float* carry;             // [2 directions][2 partial sums][64]: q dq - k dk summed over the segments walked later
+  int L;                          // tokens of this slab / segment
 };
+constexpr int kBwdStateElems = 64 * 64;
 
 // What a wave loads for one direction of one slab (its own 32-token tile), issued one phase ahead.
 template <int NG>
@@ -109,7 +115,12 @@ __device__ __forceinline__ void issue_bwd_loads(const BwdNext& n, int w, int r, 
 // second (LAST, not FIRST) adds its own to them and stores dq, dk, dv.  A one-direction (causal) launch runs a single
 // direction that is both.  Returns false, for every wave alike and before it has stored anything,
 // when the gates are out of range.
-template <bool FWD, bool FIRST, bool LAST, int NG>
+// SEG: the slab is a segment of a longer sequence.  With S_in the state entering it along the direction, R_out the
+// gradient of the state leaving it, a = half the segment's gate total and ' = times e^a per k channel:
+//   dq^_i += S_in' do_i,   dk^_j += R_out' v_j,   dv_j += R_out'^T k~_j
+// (the e^{G_i - a}, e^{a - G_j} factors applied to dq^, dk^ at the end turn e^a into e^{G_i}, e^{T - G_j}), and the
+// running sum of the gate gradient starts from the total of q dq - k dk over the segments walked later.
+template <bool FWD, bool FIRST, bool LAST, int NG, bool SEG>
 __device__ __forceinline__ bool bwd_direction(const BwdSlab& sl, int L, int ntiles, int w, int lane, char* lds,
                                               float s, f32x16_t (&dv)[2], u32x4_t (&keepq)[NG], u32x4_t (&keepk)[NG],
                                               BwdLoads<NG>& ld, const BwdNext& nxt) {
@@ -230,6 +241,19 @@ __device__ __forceinline__ bool bwd_direction(const BwdSlab& sl, int L, int ntil
         dqh[1] = mfma(kf[1], f[t], dqh[1]);
       }
     }
+    if (SEG) {  // the state entering the segment: rows = the k channels of this lane's accumulator rows, over v
+      const uint16_t* sp = sl.sp + (FWD ? 0 : kBwdStateElems);
+      const bool row_ok = row_has_channel<NG>(r);
+      const int row0 = row_ok ? 2 * cpair<NG>(r) : 0;
+#pragma unroll
+      for (int p = 0; p < 2; ++p)
+#pragma unroll
+        for (int ks = 0; ks < 4; ++ks) {
+          u32x4_t a = *reinterpret_cast<const u32x4_t*>(sp + (row0 + p) * 64 + 16 * ks + 8 * h);
+          if (NG != 4 && !row_ok) a = u32x4_t{0u, 0u, 0u, 0u};
+          dqh[p] = mfma(a, doB[ks], dqh[p]);
+        }
+    }
   }
   // dq^ waits as bf16 pairs while the other accumulators are at work
   uint32_t dqp[16];
@@ -285,6 +309,28 @@ __device__ __forceinline__ bool bwd_direction(const BwdSlab& sl, int L, int ntil
         dkh[0] = mfma(qf[0], af[t], dkh[0]);
         dkh[1] = mfma(qf[1], af[t], dkh[1]);
       }
+    }
+    if (SEG) {  // the gradient of the state leaving the segment, against this tile's k~ rows (dv) and v rows (dk)
+      const uint16_t* rpt = sl.rpt + (FWD ? 0 : kBwdStateElems);
+      const int vrow = 2 * cpair<4>(r);
+#pragma unroll
+      for (int p = 0; p < 2; ++p)
+#pragma unroll
+        for (int ks = 0; ks < NG; ++ks) {
+          const u32x4_t a = *reinterpret_cast<const u32x4_t*>(rpt + (vrow + p) * 64 + 16 * ks + 8 * h);
+          dv[p] = mfma(a, row_frag(K, 32 * w + r, ks, h), dv[p]);
+        }
+      const uint16_t* rp = sl.rp + (FWD ? 0 : kBwdStateElems);
+      const bool row_ok = row_has_channel<NG>(r);
+      const int row0 = row_ok ? 2 * cpair<NG>(r) : 0;
+#pragma unroll
+      for (int p = 0; p < 2; ++p)
+#pragma unroll
+        for (int ks = 0; ks < 4; ++ks) {
+          u32x4_t a = *reinterpret_cast<const u32x4_t*>(rp + (row0 + p) * 64 + 16 * ks + 8 * h);
+          if (NG != 4 && !row_ok) a = u32x4_t{0u, 0u, 0u, 0u};
+          dkh[p] = mfma(a, row_frag(V, 32 * w + r, ks, h), dkh[p]);
+        }
     }
   }
   // ---- scale back; X = q dq - k dk = s (q~ dq^ - k~ dk^): the exponentials cancel, and the staged rows serve ----
@@ -363,6 +409,10 @@ __device__ __forceinline__ bool bwd_direction(const BwdSlab& sl, int L, int ntil
       const float y = dgtot[t * 64 + cl];
       run += (FWD ? (t > w) : (t < w)) ? y : 0.f;
     }
+    if (SEG) {
+      const float* cy = sl.carry + (FWD ? 0 : 128) + cl;
+      run += s * (cy[0] + cy[64]);
+    }
 #pragma unroll
     for (int i = 0; i < 32; ++i) {
       const int t = FWD ? 31 - i : i;
@@ -387,73 +437,181 @@ __device__ __forceinline__ bool bwd_direction(const BwdSlab& sl, int L, int ntil
 
 }  // namespace
 
-template <int NG, bool BIDIR>
+// What the segments of long sequences read besides the tensors (see bwd_direction, SEG): per (sequence, segment) the
+// two directions' matrices, written by gla_backward_segment_scan_kernel.
+struct BwdSegments {
+  const uint16_t *sp, *rp, *rpt;
+  const float* carry;
+  int nseg, seg_len;
+};
+
+template <int NG, bool BIDIR, bool SEG>
 __global__ __launch_bounds__(512) void gla_backward_mfma_kernel(
     const uint16_t* __restrict__ q, const uint16_t* __restrict__ k, const uint16_t* __restrict__ v,
     const uint16_t* __restrict__ gf, const uint16_t* __restrict__ gb, const uint16_t* __restrict__ d_o,
     uint16_t* __restrict__ dq, uint16_t* __restrict__ dk, uint16_t* __restrict__ dv, uint16_t* __restrict__ dgf,
-    uint16_t* __restrict__ dgb, int* __restrict__ flags, int nslabs, int L, float s) {
+    uint16_t* __restrict__ dgb, int* __restrict__ flags, int nslabs, int L, float s, BwdSegments sg) {
   extern __shared__ __align__(16) char lds[];
   const int tid = threadIdx.x;
   const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int lane = tid & 63;
-  const int ntiles = (L + 31) / 32;
+  // slab i: a whole sequence, or (SEG) segment i % nseg of sequence i / nseg
   auto slab_of = [&](int i) {
-    const size_t bk = (size_t)i * L * (16 * NG), bv = (size_t)i * L * 64;
-    return BwdSlab{q + bk, k + bk, v + bv, gf + bk, BIDIR ? gb + bk : nullptr, d_o + bv, dq + bk, dk + bk, dv + bv,
-                   dgf + bk, BIDIR ? dgb + bk : nullptr};
+    size_t t0 = (size_t)i * L;
+    int len = L;
+    BwdSlab sl{};
+    if (SEG) {
+      const int seq = i / sg.nseg, seg = i - seq * sg.nseg;
+      t0 = (size_t)seq * L + (size_t)seg * sg.seg_len;
+      len = min(sg.seg_len, L - seg * sg.seg_len);
+      sl.sp = sg.sp + (size_t)i * 2 * kBwdStateElems;
+      sl.rp = sg.rp + (size_t)i * 2 * kBwdStateElems;
+      sl.rpt = sg.rpt + (size_t)i * 2 * kBwdStateElems;
+      sl.carry = sg.carry + (size_t)i * 256;
+    }
+    const size_t bk = t0 * (16 * NG), bv = t0 * 64;
+    sl.q = q + bk, sl.k = k + bk, sl.v = v + bv, sl.gf = gf + bk, sl.gb = BIDIR ? gb + bk : nullptr, sl.d_o = d_o + bv;
+    sl.dq = dq + bk, sl.dk = dk + bk, sl.dv = dv + bv, sl.dgf = dgf + bk, sl.dgb = BIDIR ? dgb + bk : nullptr;
+    sl.L = len;
+    return sl;
   };
   const int r = lane & 31, h = lane >> 5;
   BwdLoads<NG> ld;
   if ((int)blockIdx.x < nslabs) {
     const BwdSlab s0 = slab_of(blockIdx.x);
-    issue_bwd_loads<true, NG>(BwdNext{s0, s0.gf, L}, w, r, h, ld);
+    issue_bwd_loads<true, NG>(BwdNext{s0, s0.gf, s0.L}, w, r, h, ld);
   }
   for (int slab = blockIdx.x; slab < nslabs; slab += gridDim.x) {
     const BwdSlab sl = slab_of(slab);
+    const int ntiles = (sl.L + 31) / 32;
     const int following = slab + (int)gridDim.x;
     const BwdSlab sn = slab_of(following < nslabs ? following : slab);
-    const BwdNext second{sl, sl.gb, L}, next_first{sn, sn.gf, following < nslabs ? L : 0};
+    const BwdNext second{sl, sl.gb, sl.L}, next_first{sn, sn.gf, following < nslabs ? sn.L : 0};
     f32x16_t dvacc[2] = {{0.f}, {0.f}};
     u32x4_t keepq[NG], keepk[NG];
     bool ok;
     if constexpr (BIDIR) {
-      ok = bwd_direction<true, true, false, NG>(sl, L, ntiles, w, lane, lds, s, dvacc, keepq, keepk, ld, second);
+      ok = bwd_direction<true, true, false, NG, SEG>(sl, sl.L, ntiles, w, lane, lds, s, dvacc, keepq, keepk, ld, second);
       if (ok) {
         lds_barrier();  // (5) the dg scratch of direction 1 is dead before q~, k~ of direction 2 are staged
-        ok = bwd_direction<false, false, true, NG>(sl, L, ntiles, w, lane, lds, s, dvacc, keepq, keepk, ld, next_first);
+        ok = bwd_direction<false, false, true, NG, SEG>(sl, sl.L, ntiles, w, lane, lds, s, dvacc, keepq, keepk, ld,
+                                                        next_first);
       }
     } else {  // the causal op: the forward direction alone, first and last at once
-      ok = bwd_direction<true, true, true, NG>(sl, L, ntiles, w, lane, lds, s, dvacc, keepq, keepk, ld, next_first);
+      ok = bwd_direction<true, true, true, NG, SEG>(sl, sl.L, ntiles, w, lane, lds, s, dvacc, keepq, keepk, ld,
+                                                    next_first);
     }
     // a direction that left early has not issued the loads of the slab that follows
     if (!ok) issue_bwd_loads<true, NG>(next_first, w, r, h, ld);
-    if (tid == 0) flags[slab] = ok ? 0 : 1;
+    if (SEG) {  // one flag per sequence, cleared by the segment scan: any segment out of range gives the sequence away
+      if (tid == 0 && !ok) flags[slab / sg.nseg] = 1;
+    } else if (tid == 0) {
+      flags[slab] = ok ? 0 : 1;
+    }
     lds_barrier();  // the next slab restages everything
   }
 }
 
-
-
-bool gla_backward_mfma_supported(int L, int Dk, int Dv, int io_dtype, int gate_dtype, bool bidir) {
-  (void)bidir;  // both the bidirectional and the causal op
-  return io_dtype == 1 && gate_dtype == 1 && (Dk == 64 || Dk == 32) && Dv == 64 && L <= 32 * kBwdTiles;
+// Links the segments of every (sequence, direction) for the backward.  Per segment s (walked in the direction's order)
+// it reads the forward's state pass (contribution U_s, decay D_s) and the gradient state pass (Q_s = sum over the
+// segment's tokens of (q e^{G})^T do, unscaled), and leaves
+//   sp   = sqrt(D_s) S_in(s),     S_in(s') = D_s S_in(s) + U_s   for the segment s' walked next,
+//   rp   = sqrt(D_s) R_out(s),    R_out(s) = Q_{s'} + D_{s'} R_out(s'),  zero for the segment walked last,
+//   rpt  = rp transposed,
+//   carry(s) = sum over the segments walked after s of rowsum_v(S_in Q - R_out U): what q dq - k dk adds up to there
+// (bf16 matrices in plain row-major order; carry as two partial sums per channel, one per half of the v columns).
+// One thread per state element in the passes' register order; `term` holds S_in Q between the two sweeps.
+__global__ __launch_bounds__(256) void gla_backward_segment_scan_kernel(
+    const float* __restrict__ ws_fwd, const float* __restrict__ ws_grad, float* __restrict__ term, uint16_t* __restrict__ sp,
+    uint16_t* __restrict__ rp, uint16_t* __restrict__ rpt, float* __restrict__ carry, int* __restrict__ flags, int nseq,
+    int nseg, int ndir, int ng) {
+  __shared__ float red[256];
+  const int tid = threadIdx.x;
+  const int e = blockIdx.x * 256 + tid;  // element in register order: ((u*64 + lane)*4 + m)
+  const int seq = blockIdx.y / ndir, dir = blockIdx.y % ndir;
+  if (blockIdx.x == 0 && tid == 0 && dir == 0) flags[seq] = 0;
+  const int m = e & 3, lane = (e >> 2) & 63, u = e >> 8;
+  const int pk = u >> 3, pv = (u >> 2) & 1, cq = u & 3, h = lane >> 5;
+  const bool live = cq < ng;  // register quads beyond Dk/16 carry no channel (uniform per block)
+  const int ch = live ? 8 * ng * h + 8 * cq + 2 * m + pk : 0;
+  const int vch = 2 * cpair<4>(lane & 31) + pv;
+  auto slot = [&](int seg, int d) { return (((size_t)seq * nseg + seg) * 2 + d); };
+  // the gradient state pass ran with the directions' roles exchanged (see launch_gla_backward_mfma)
+  const int gdir = 1 - dir;
+  float S = 0.f;
+  if (live) {
+    for (int i = 0; i < nseg; ++i) {
+      const int seg = dir == 0 ? i : nseg - 1 - i;
+      const float* f = ws_fwd + slot(seg, dir) * kGlaStateFloats;
+      const float U = f[e], D = f[64 * 64 + ch];
+      const float Q = ws_grad[slot(seg, gdir) * kGlaStateFloats + e];
+      sp[slot(seg, dir) * kBwdStateElems + ch * 64 + vch] = f32_to_bf16(__builtin_sqrtf(D) * S);
+      term[slot(seg, dir) * kBwdStateElems + e] = S * Q;
+      S = __builtin_fmaf(D, S, U);
+    }
+  }
+  float R = 0.f, later = 0.f;
+  for (int i = nseg - 1; i >= 0; --i) {
+    const int seg = dir == 0 ? i : nseg - 1 - i;
+    float U = 0.f, D = 0.f, Q = 0.f, t1 = 0.f;
+    if (live) {
+      const float* f = ws_fwd + slot(seg, dir) * kGlaStateFloats;
+      U = f[e], D = f[64 * 64 + ch];
+      Q = ws_grad[slot(seg, gdir) * kGlaStateFloats + e];
+      t1 = term[slot(seg, dir) * kBwdStateElems + e];
+      const uint16_t x = f32_to_bf16(__builtin_sqrtf(D) * R);
+      rp[slot(seg, dir) * kBwdStateElems + ch * 64 + vch] = x;
+      rpt[slot(seg, dir) * kBwdStateElems + vch * 64 + ch] = x;
+    }
+    // the block holds 8 channels (lane half h, register m) x the 32 v columns of its half: sum them in a fixed order
+    red[tid] = later;
+    __syncthreads();
+    if (tid < 8 && live) {
+      const int hh = tid >> 2, mm = tid & 3;
+      float acc = 0.f;
+      for (int x = 0; x < 32; ++x) acc += red[(32 * hh + x) * 4 + mm];
+      carry[slot(seg, dir) * 128 + pv * 64 + 8 * ng * hh + 8 * cq + 2 * mm + pk] = acc;
+    }
+    __syncthreads();
+    later += t1 - R * U;
+    R = __builtin_fmaf(D, R, Q);
+  }
 }
 
-// flags: one int per (batch, head) slab, written by every launch: 1 = not computed here (gates out of range)
+static bool seg_grid_ok(int B, int H, bool bidir) { return (long long)B * H * (bidir ? 2 : 1) <= 65535; }
+
+bool gla_backward_mfma_supported(int B, int H, int L, int Dk, int Dv, int io_dtype, int gate_dtype, bool bidir) {
+  if (!(io_dtype == 1 && gate_dtype == 1 && (Dk == 64 || Dk == 32) && Dv == 64)) return false;
+  return L <= 32 * kBwdTiles || seg_grid_ok(B, H, true);
+}
+
+// Long sequences: two state passes (kGlaStateFloats floats per sequence, segment and direction each), the S_in Q terms
+// and the carries (fp32), then the three bf16 matrices the segments read.
+static size_t seg_slots(int B, int H, int L) { return (size_t)B * H * gla_segments(L) * 2; }
+size_t gla_backward_mfma_workspace(int B, int H, int L, int Dk, int Dv) {
+  if (L <= 32 * kBwdTiles || !(Dk == 64 || Dk == 32) || Dv != 64) return 0;
+  const size_t n = seg_slots(B, H, L);
+  return n * ((2 * (size_t)kGlaStateFloats + kBwdStateElems + 128) * sizeof(float) + 3 * (size_t)kBwdStateElems * 2);
+}
+
+// flags: one int per (batch, head) sequence, written by every launch: 1 = not computed here (gates out of range)
 int launch_gla_backward_mfma(const void* q, const void* k, const void* v, const void* gf, const void* gb,
-                             const void* d_o, void* dq, void* dk, void* dv, void* dgf, void* dgb, int* flags, int B,
-                             int H, int L, int Dk, float s, hipStream_t stream) {
+                             const void* d_o, void* dq, void* dk, void* dv, void* dgf, void* dgb, int* flags,
+                             void* seg_workspace, int B, int H, int L, int Dk, float s, hipStream_t stream) {
   constexpr int kMaxDevices = 64;
   static bool attr_done_dev[kMaxDevices] = {};
   static int num_cu_dev[kMaxDevices] = {};
   int dev = 0;
   if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return -5;
   if (!attr_done_dev[dev]) {
-    const void* kernels[4] = {reinterpret_cast<const void*>(gla_backward_mfma_kernel<4, true>),
-                              reinterpret_cast<const void*>(gla_backward_mfma_kernel<2, true>),
-                              reinterpret_cast<const void*>(gla_backward_mfma_kernel<4, false>),
-                              reinterpret_cast<const void*>(gla_backward_mfma_kernel<2, false>)};
+    const void* kernels[8] = {reinterpret_cast<const void*>(gla_backward_mfma_kernel<4, true, false>),
+                              reinterpret_cast<const void*>(gla_backward_mfma_kernel<2, true, false>),
+                              reinterpret_cast<const void*>(gla_backward_mfma_kernel<4, false, false>),
+                              reinterpret_cast<const void*>(gla_backward_mfma_kernel<2, false, false>),
+                              reinterpret_cast<const void*>(gla_backward_mfma_kernel<4, true, true>),
+                              reinterpret_cast<const void*>(gla_backward_mfma_kernel<2, true, true>),
+                              reinterpret_cast<const void*>(gla_backward_mfma_kernel<4, false, true>),
+                              reinterpret_cast<const void*>(gla_backward_mfma_kernel<2, false, true>)};
     for (const void* kf : kernels)
       if (hipFuncSetAttribute(kf, hipFuncAttributeMaxDynamicSharedMemorySize, kBwdLdsTotal) != hipSuccess) return -5;
     int n = 0;
@@ -461,20 +619,59 @@ int launch_gla_backward_mfma(const void* q, const void* k, const void* v, const 
     num_cu_dev[dev] = n > 0 ? n : 256;
     attr_done_dev[dev] = true;
   }
-  const int nslabs = B * H;
+  const bool seg = L > 32 * kBwdTiles;
+  BwdSegments sg{};
+  int nslabs = B * H;
+  if (seg) {
+    if (!seg_workspace || !seg_grid_ok(B, H, gb != nullptr)) return -22;
+    const size_t n = seg_slots(B, H, L);
+    float* ws_fwd = (float*)seg_workspace;
+    float* ws_grad = ws_fwd + n * kGlaStateFloats;
+    float* term = ws_grad + n * kGlaStateFloats;
+    float* carry = term + n * kBwdStateElems;
+    uint16_t* sp = (uint16_t*)(carry + n * 128);
+    uint16_t* rp = sp + n * kBwdStateElems;
+    uint16_t* rpt = rp + n * kBwdStateElems;
+    // the forward's state pass: contributions k~^T v and decays of every segment, both directions
+    GlaArgs a{};
+    a.q = q, a.k = k, a.v = v, a.g_fwd = gf, a.g_bwd = gb, a.o = nullptr, a.workspace = ws_fwd;
+    a.B = B, a.H = H, a.L = L, a.Dk = Dk, a.Dv = 64, a.scale = 1.f, a.out_scale = 1.f, a.io_dtype = 1, a.gate_dtype = 1;
+    a.stream = stream, a.state_pass = 1;
+    int rc = launch_gla_mfma(a);
+    if (rc != 0) return rc;
+    // the gradient states: the same pass on (q for k, do for v) with each token's own gate included in its weight.
+    // A state pass anchors a token at the END of its walk (the weight of token j is the decay from j to the last
+    // token walked); the gradient state needs the decay from the FIRST token walked to i, i.e. the walk of the other
+    // direction over the same gates: the forward gates go to the reverse waves and the reverse gates to the forward
+    // waves, and slot d of this pass belongs to direction 1 - d.
+    a.k = q, a.v = d_o, a.g_fwd = gb ? gb : gf, a.g_bwd = gf, a.workspace = ws_grad, a.state_pass = 2;
+    rc = launch_gla_mfma(a);
+    if (rc != 0) return rc;
+    const int ndir = gb ? 2 : 1;
+    hipLaunchKernelGGL(gla_backward_segment_scan_kernel, dim3(64 * 64 / 256, B * H * ndir), dim3(256), 0, stream, ws_fwd,
+                       ws_grad, term, sp, rp, rpt, carry, flags, B * H, gla_segments(L), ndir, Dk / 16);
+    sg = BwdSegments{sp, rp, rpt, carry, gla_segments(L), gla_segment_len(L)};
+    nslabs = B * H * sg.nseg;
+  }
   const int grid = nslabs < num_cu_dev[dev] ? nslabs : num_cu_dev[dev];
-#define VIG_BWD_LAUNCH(NG, BIDIR)                                                                               \
-  hipLaunchKernelGGL((gla_backward_mfma_kernel<NG, BIDIR>), dim3(grid), dim3(512), kBwdLdsTotal, stream,         \
+#define VIG_BWD_LAUNCH(NG, BIDIR, SEG)                                                                          \
+  hipLaunchKernelGGL((gla_backward_mfma_kernel<NG, BIDIR, SEG>), dim3(grid), dim3(512), kBwdLdsTotal, stream,    \
                      (const uint16_t*)q, (const uint16_t*)k, (const uint16_t*)v, (const uint16_t*)gf,            \
                      (const uint16_t*)gb, (const uint16_t*)d_o, (uint16_t*)dq, (uint16_t*)dk, (uint16_t*)dv,     \
-                     (uint16_t*)dgf, (uint16_t*)dgb, flags, nslabs, L, s)
+                     (uint16_t*)dgf, (uint16_t*)dgb, flags, nslabs, L, s, sg)
+#define VIG_BWD_LAUNCH_SEG(NG, BIDIR) \
+  do {                                \
+    if (seg) VIG_BWD_LAUNCH(NG, BIDIR, true); \
+    else VIG_BWD_LAUNCH(NG, BIDIR, false);    \
+  } while (0)
   if (gb) {
-    if (Dk == 64) VIG_BWD_LAUNCH(4, true);
-    else VIG_BWD_LAUNCH(2, true);
+    if (Dk == 64) VIG_BWD_LAUNCH_SEG(4, true);
+    else VIG_BWD_LAUNCH_SEG(2, true);
   } else {
-    if (Dk == 64) VIG_BWD_LAUNCH(4, false);
-    else VIG_BWD_LAUNCH(2, false);
+    if (Dk == 64) VIG_BWD_LAUNCH_SEG(4, false);
+    else VIG_BWD_LAUNCH_SEG(2, false);
   }
+#undef VIG_BWD_LAUNCH_SEG
 #undef VIG_BWD_LAUNCH
   return hipGetLastError() == hipSuccess ? 0 : -5;
 }

@@ -264,8 +264,12 @@ __device__ __forceinline__ void issue_first_phase(const ChunkSrc& src, int r, in
 //               contribution and total decay are written to the workspace (no outputs);
 //   kModeChain  pass 2 of a long sequence: the state entering the segment (from the left for the forward direction,
 //               from the right for the reverse one) is read from the workspace and outputs are produced.
-constexpr int kModeSlab = 0, kModeState = 1, kModeChain = 2;
-constexpr int kStateFloats = 64 * 64 + 64;  // per (sequence, segment, direction): state in unit order, then 64 decays
+//   kModeStateStrict  kModeState with the cumulative gates taken exclusive of a token's own gate (so that the weight of
+//               a token reaches back to and includes it): the backward of a long sequence builds its per-segment
+//               gradient states with this pass, fed q for k and the output gradient for v.
+constexpr int kModeSlab = 0, kModeState = 1, kModeChain = 2, kModeStateStrict = 3;
+constexpr bool is_state_mode(int mode) { return mode == kModeState || mode == kModeStateStrict; }
+constexpr int kStateFloats = kGlaStateFloats;  // per (sequence, segment, direction): state in unit order, then 64 decays
 
 // Intra-chunk part of one wave: scores of the three tile pairs of its chunk, applied to V; k~ (bf16) goes to the
 // wave's LDS scratch for the state update, q~ (bf16) is kept for the inter-chunk product.  The second tile's rows
@@ -277,7 +281,7 @@ template <bool FWD, int MODE, int NG, bool F16>
 __device__ __forceinline__ bool tile_phase(const ChunkSrc& cur, const Prefetch<NG>& pf, const f32x16_t (&G)[2][2],
                                            const float* gend2, uint16_t* kt, int r, int h, f32x16_t (&O)[2][2],
                                            u32x4_t (&qkeep)[2][NG], u32x4_t (&vfrag)[4][2]) {
-  constexpr bool OUT = MODE != kModeState;
+  constexpr bool OUT = !is_state_mode(MODE);
   constexpr int TA = FWD ? 0 : 1;  // tile walked first
   constexpr int TB = FWD ? 1 : 0;
   constexpr int MASK = FWD ? 1 : 2;
@@ -414,7 +418,7 @@ template <bool FWD, int MODE, int NG, bool F16, bool GATE>
 __device__ __forceinline__ bool direction_wave(const ChunkSrc& cur, const ChunkSrc& nxt, rsrc_t o, int c, int lane,
                                                char* lds, float oscale, bool bidir, float* state, Prefetch<NG>& pf,
                                                const GateCtx& gate) {
-  constexpr bool OUT = MODE != kModeState;  // produces outputs (needs q)
+  constexpr bool OUT = !is_state_mode(MODE);  // produces outputs (needs q)
   int r = lane & 31, h = lane >> 5;
   const int wi = (FWD ? 0 : 4) + c;
   constexpr int TA = FWD ? 0 : 1;  // tile walked first
@@ -435,7 +439,8 @@ __device__ __forceinline__ bool direction_wave(const ChunkSrc& cur, const ChunkS
     u32x4_t gfrag[4][2];
     finish_tfrags<4>(pf.gD, gfrag);
     const u32x4_t ones = {0x3F803F80u, 0x3F803F80u, 0x3F803F80u, 0x3F803F80u};
-    const u32x4_t tri0 = tri_frag<FWD>(0, 0, r, h), tri1 = tri_frag<FWD>(1, 0, r, h);
+    constexpr bool STRICT = MODE == kModeStateStrict;
+    const u32x4_t tri0 = tri_frag<FWD, STRICT>(0, 0, r, h), tri1 = tri_frag<FWD, STRICT>(1, 0, r, h);
     // k-steps of the tile walked first / second (the triangular operand depends on (k-step, tile) only through
     // their offset, so two fragments serve both tiles)
     constexpr int A0 = FWD ? 0 : 2, B0 = FWD ? 2 : 0;
@@ -513,7 +518,7 @@ __device__ __forceinline__ bool direction_wave(const ChunkSrc& cur, const ChunkS
           U[pk][pv] = F16 ? mfma_f16(ktf[pk], vfrag[t][pv], U[pk][pv]) : mfma(ktf[pk], vfrag[t][pv], U[pk][pv]);
     }
     // the chunk walked last is consumed by nobody inside the segment, unless the segment's own total is wanted
-    if (MODE == kModeState || (FWD ? (c < 3) : (c > 0))) {
+    if (is_state_mode(MODE) || (FWD ? (c < 3) : (c > 0))) {
 #pragma unroll
       for (int pk = 0; pk < 2; ++pk)
 #pragma unroll
@@ -569,7 +574,7 @@ __device__ __forceinline__ bool direction_wave(const ChunkSrc& cur, const ChunkS
     for (int i = (MODE == kModeChain ? 0 : 1); i < 4; ++i) {
       const int wc = W0 + STEP * i;  // consumer chunk: needs exp(G_end(wc)/2) * S as fragments
       char* creg = dirbase + wc * kRegionBytes;
-      const bool add_u = MODE == kModeState || i < 3;
+      const bool add_u = is_state_mode(MODE) || i < 3;
 #pragma unroll
       for (int j = 0; j < NQ; ++j) {
         const int cq = cqa + j;
@@ -596,7 +601,7 @@ __device__ __forceinline__ bool direction_wave(const ChunkSrc& cur, const ChunkS
         if (OUT) *reinterpret_cast<u32x4_t*>(unit_ptr(creg, pv * 4 + cq, lane)) = fr;
       }
     }
-    if (MODE == kModeState && ok) {
+    if (is_state_mode(MODE) && ok) {
       // the segment's end-anchored contribution (unit order) and its total decay per channel
 #pragma unroll
       for (int pk = 0; pk < 2; ++pk)
@@ -755,7 +760,7 @@ template <bool FWD, int MODE, int NG, bool F16, bool GATE>
 __device__ __forceinline__ int wave_loop(const uint16_t* q, const uint16_t* k, const uint16_t* v, const uint16_t* g,
                                          uint16_t* o, const Geometry& geo, int item, int c, int lane, char* lds,
                                          float oscale, bool bidir, float* state_ws, const float* gate_w) {
-  constexpr bool OUT = MODE != kModeState;
+  constexpr bool OUT = !is_state_mode(MODE);
   constexpr int DK = 16 * NG;
   // descriptors of this wave's chunk of an item; past the last item (or for a chunk with no tokens) they are empty
   auto locate = [&](int it, ChunkSrc& src, rsrc_t& dst) {
@@ -907,8 +912,8 @@ __global__ __launch_bounds__(256) void gla_segment_scan_kernel(float* state_ws, 
 static Geometry make_geometry(int nseq, int L) {
   Geometry g{};
   g.L = L;
-  g.nseg = (L + 255) / 256;
-  g.seg_len = (L + g.nseg - 1) / g.nseg;
+  g.nseg = gla_segments(L);
+  g.seg_len = gla_segment_len(L);
   g.cw = (g.seg_len + 3) / 4;
   g.nitems = nseq * g.nseg;
   return g;
@@ -945,10 +950,11 @@ static int launch_gla_mfma_t(const GlaArgs& a, int num_cu, int dev) {
   static bool attr_done_dev[kMaxDevices] = {};
   bool& attr_done = attr_done_dev[dev];
   if (!attr_done) {
-    const void* kernels[4] = {reinterpret_cast<const void*>(gla_mfma_kernel<kModeSlab, NG>),
+    const void* kernels[5] = {reinterpret_cast<const void*>(gla_mfma_kernel<kModeSlab, NG>),
                               reinterpret_cast<const void*>(gla_mfma_kernel<kModeState, NG>),
                               reinterpret_cast<const void*>(gla_mfma_kernel<kModeChain, NG>),
-                              reinterpret_cast<const void*>(gla_mfma_kernel<kModeSlab, NG, true>)};
+                              reinterpret_cast<const void*>(gla_mfma_kernel<kModeSlab, NG, true>),
+                              reinterpret_cast<const void*>(gla_mfma_kernel<kModeStateStrict, NG>)};
     for (const void* kf : kernels)
       if (hipFuncSetAttribute(kf, hipFuncAttributeMaxDynamicSharedMemorySize, kLdsTotal) != hipSuccess) return -5;
     attr_done = true;
@@ -964,7 +970,15 @@ static int launch_gla_mfma_t(const GlaArgs& a, int num_cu, int dev) {
   uint16_t* o = (uint16_t*)a.o;
   const float oscale = a.scale * a.out_scale;
   const float* no_gate = nullptr;
-  if (a.gate_w) {
+  if (a.state_pass) {
+    // one state pass alone: contributions and decays of every (sequence, segment, direction), no scan, no outputs
+    if (a.state_pass == 2)
+      hipLaunchKernelGGL((gla_mfma_kernel<kModeStateStrict, NG>), dim3(grid), dim3(512), kLdsTotal, a.stream, q, k, v,
+                         gf, gb, o, geo, oscale, (float*)a.workspace, no_gate);
+    else
+      hipLaunchKernelGGL((gla_mfma_kernel<kModeState, NG>), dim3(grid), dim3(512), kLdsTotal, a.stream, q, k, v, gf, gb,
+                         o, geo, oscale, (float*)a.workspace, no_gate);
+  } else if (a.gate_w) {
     // fused locality gate: whole-sequence slabs, both directions, the padded token grid must fit the staging cells
     if (geo.nseg != 1 || !gb || a.gate_cols <= 0 || a.gate_rows <= 0 || a.gate_cols * a.gate_rows != a.L ||
         !gla_mfma_gate_grid_ok(a.gate_rows, a.gate_cols))

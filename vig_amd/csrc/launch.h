@@ -28,7 +28,17 @@ struct GlaArgs {
   // causal op only (g_bwd null): fp32 [B, H, Dk, Dv] state before the first token / after the last one; null: zero / not wanted
   const float* init_state = nullptr;
   float* final_state = nullptr;
+  // bf16 MFMA path, any L: run one state pass alone into `workspace` (1: plain, 2: with the cumulative gates exclusive
+  // of each token's own gate): per (sequence, segment, direction) kGlaStateFloats floats, no scan, no outputs
+  int state_pass = 0;
 };
+
+// Per (sequence, segment, direction) slot of a state pass: the 64 x 64 state contribution in the matrix cores' register
+// order (element ((u*64 + lane)*4 + m): unit u = (pk*2 + pv)*4 + cq), then the segment's 64 per-channel decays.
+constexpr int kGlaStateFloats = 64 * 64 + 64;
+// Segments of a long sequence: ceil(L / 256) of them, ceil(L / nseg) tokens each (the last one possibly fewer).
+inline int gla_segments(int L) { return (L + 255) / 256; }
+inline int gla_segment_len(int L) { return (L + gla_segments(L) - 1) / gla_segments(L); }
 
 // fp32-arithmetic token-recurrent path (any supported dtype combination).
 int launch_gla_recurrent(const GlaArgs& a);
@@ -41,10 +51,13 @@ bool gla_mfma_gate_grid_ok(int rows, int cols);  // token grids the fused locali
 size_t gla_mfma_workspace(int B, int H, int L, int Dk, int Dv);
 size_t gla_mfma_state_workspace(int B, int H, int L, int Dk, int Dv);  // causal op with an initial / final state
 
-// bf16 matrix-core backward (whole-slab quadratic form); flags[b*H + h] = 1 marks slabs it left to the recurrent kernel
-bool gla_backward_mfma_supported(int L, int Dk, int Dv, int io_dtype, int gate_dtype, bool bidir);
+// bf16 matrix-core backward (quadratic form per slab, or per <= 256-token segment of a longer sequence with the
+// segments chained through states); flags[b*H + h] = 1 marks sequences it left to the recurrent kernel.
+// seg_workspace: gla_backward_mfma_workspace() bytes, used for L > 256 only.
+bool gla_backward_mfma_supported(int B, int H, int L, int Dk, int Dv, int io_dtype, int gate_dtype, bool bidir);
+size_t gla_backward_mfma_workspace(int B, int H, int L, int Dk, int Dv);
 int launch_gla_backward_mfma(const void* q, const void* k, const void* v, const void* gf, const void* gb,
-                             const void* d_o, void* dq, void* dk, void* dv, void* dgf, void* dgb, int* flags, int B,
-                             int H, int L, int Dk, float s, hipStream_t stream);
+                             const void* d_o, void* dq, void* dk, void* dv, void* dgf, void* dgb, int* flags,
+                             void* seg_workspace, int B, int H, int L, int Dk, float s, hipStream_t stream);
 
 }  // namespace vig

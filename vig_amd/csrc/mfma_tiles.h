@@ -118,16 +118,17 @@ __device__ __forceinline__ void load_tfrag_lds(const uint16_t* kt, int t, int r,
   }
 }
 
-// B operand of the cumulative-sum MFMA: ones where token slot j is on the kept side of column token i.
-template <bool FWD>
+// B operand of the cumulative-sum MFMA: ones where token slot j is on the kept side of column token i (STRICT: the
+// token itself is not kept).
+template <bool FWD, bool STRICT = false>
 __device__ __forceinline__ u32x4_t tri_frag(int t, int it, int r, int h) {
   const int i = 32 * it + r;
   u32x4_t f;
 #pragma unroll
   for (int x = 0; x < 4; ++x) {
     const int j0 = jmap(t, h, 2 * x), j1 = jmap(t, h, 2 * x + 1);
-    const bool b0 = FWD ? (j0 <= i) : (j0 >= i);
-    const bool b1 = FWD ? (j1 <= i) : (j1 >= i);
+    const bool b0 = STRICT ? (FWD ? (j0 < i) : (j0 > i)) : (FWD ? (j0 <= i) : (j0 >= i));
+    const bool b1 = STRICT ? (FWD ? (j1 < i) : (j1 > i)) : (FWD ? (j1 <= i) : (j1 >= i));
     f[x] = (b0 ? 0x00003F80u : 0u) | (b1 ? 0x3F800000u : 0u);
   }
   return f;

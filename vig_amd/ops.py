@@ -74,7 +74,8 @@ def gla_bidir_backward(q, k, v, g_fwd, g_bwd, d_o, scale: float = -1, out_scale:
                        exact: bool = False):
     """Gradients of gla_bidir_forward contracted with d_o: (dq, dk, dv, dg_fwd, dg_bwd or None).
 
-    bf16 tensors and gates with Dk in {32, 64}, Dv = 64 and L <= 256 run on the matrix cores, bidirectional or causal (bf16 operands,
+    bf16 tensors and gates with Dk in {32, 64} and Dv = 64 run on the matrix cores, bidirectional or causal, any L (sequences
+    longer than 256 tokens as segments chained through their states; bf16 operands,
     fp32 accumulation); everything else, and `exact=True`, on the fp32-arithmetic token-recurrent kernel.
     """
     lib = _lib.load()
