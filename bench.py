@@ -193,11 +193,13 @@ def backward_time(lib, sets, s, io_dt, scale, sp, stream, dev, iters=60):
     torch.cuda.synchronize()
     us = sum(a.elapsed_time(b) for a, b in evs) / iters * 1e3
     esz = 4 if s.dtype == "f32" else 2
-    mfma = s.dtype != "f32" and s.Dk in (32, 64) and s.Dv == 64 and s.L <= 256
+    mfma = s.dtype != "f32" and s.Dk in (32, 64) and s.Dv == 64
     alg = s.tokens * esz * ((2 * s.Dk + 2 * s.Dv) + 2 * s.Dk + (2 * s.Dk + s.Dv) + 2 * s.Dk)
     return {"us": us, "algorithmic_bytes": alg, "algorithmic_GBps": alg / (us * 1e-6) / 1e9,
             "frac_of_hbm_peak": alg / (us * 1e-6) / 1e9 / HBM_PEAK_GBPS,
-            "kernel": "matrix cores (whole-slab quadratic form), bf16 operands" if mfma else "fp32 token-recurrent"}
+            "kernel": ("fp32 token-recurrent" if not mfma else
+                       "matrix cores (whole-slab quadratic form), bf16 operands" if s.L <= 256 else
+                       "matrix cores (segments of <= 256 tokens linked by states), bf16 operands")}
 
 
 def main():

@@ -525,7 +525,6 @@ __global__ __launch_bounds__(256) void gla_backward_segment_scan_kernel(
     const float* __restrict__ ws_fwd, const float* __restrict__ ws_grad, float* __restrict__ term, uint16_t* __restrict__ sp,
     uint16_t* __restrict__ rp, uint16_t* __restrict__ rpt, float* __restrict__ carry, int* __restrict__ flags, int nseq,
     int nseg, int ndir, int ng) {
-  __shared__ float red[256];
   const int tid = threadIdx.x;
   const int e = blockIdx.x * 256 + tid;  // element in register order: ((u*64 + lane)*4 + m)
   const int seq = blockIdx.y / ndir, dir = blockIdx.y % ndir;
@@ -538,43 +537,76 @@ __global__ __launch_bounds__(256) void gla_backward_segment_scan_kernel(
   auto slot = [&](int seg, int d) { return (((size_t)seq * nseg + seg) * 2 + d); };
   // the gradient state pass ran with the directions' roles exchanged (see launch_gla_backward_mfma)
   const int gdir = 1 - dir;
+  // Both sweeps fetch eight segments at a time, so that the serial part is arithmetic only.
+  constexpr int kBatch = 8;
   float S = 0.f;
   if (live) {
-    for (int i = 0; i < nseg; ++i) {
-      const int seg = dir == 0 ? i : nseg - 1 - i;
-      const float* f = ws_fwd + slot(seg, dir) * kGlaStateFloats;
-      const float U = f[e], D = f[64 * 64 + ch];
-      const float Q = ws_grad[slot(seg, gdir) * kGlaStateFloats + e];
-      sp[slot(seg, dir) * kBwdStateElems + ch * 64 + vch] = f32_to_bf16(__builtin_sqrtf(D) * S);
-      term[slot(seg, dir) * kBwdStateElems + e] = S * Q;
-      S = __builtin_fmaf(D, S, U);
+    for (int i0 = 0; i0 < nseg; i0 += kBatch) {
+      float U[kBatch], D[kBatch], Q[kBatch];
+#pragma unroll
+      for (int j = 0; j < kBatch; ++j) {
+        const int i = min(i0 + j, nseg - 1);
+        const int seg = dir == 0 ? i : nseg - 1 - i;
+        const float* f = ws_fwd + slot(seg, dir) * kGlaStateFloats;
+        U[j] = f[e], D[j] = f[64 * 64 + ch];
+        Q[j] = ws_grad[slot(seg, gdir) * kGlaStateFloats + e];
+      }
+#pragma unroll
+      for (int j = 0; j < kBatch; ++j) {
+        const int i = i0 + j;
+        if (i < nseg) {
+          const int seg = dir == 0 ? i : nseg - 1 - i;
+          sp[slot(seg, dir) * kBwdStateElems + ch * 64 + vch] = f32_to_bf16(__builtin_sqrtf(D[j]) * S);
+          term[slot(seg, dir) * kBwdStateElems + e] = S * Q[j];
+          S = __builtin_fmaf(D[j], S, U[j]);
+        }
+      }
     }
   }
+  __shared__ float red[kBatch][256];
   float R = 0.f, later = 0.f;
-  for (int i = nseg - 1; i >= 0; --i) {
-    const int seg = dir == 0 ? i : nseg - 1 - i;
-    float U = 0.f, D = 0.f, Q = 0.f, t1 = 0.f;
-    if (live) {
-      const float* f = ws_fwd + slot(seg, dir) * kGlaStateFloats;
-      U = f[e], D = f[64 * 64 + ch];
-      Q = ws_grad[slot(seg, gdir) * kGlaStateFloats + e];
-      t1 = term[slot(seg, dir) * kBwdStateElems + e];
-      const uint16_t x = f32_to_bf16(__builtin_sqrtf(D) * R);
-      rp[slot(seg, dir) * kBwdStateElems + ch * 64 + vch] = x;
-      rpt[slot(seg, dir) * kBwdStateElems + vch * 64 + ch] = x;
+  for (int i0 = nseg - 1; i0 >= 0; i0 -= kBatch) {  // segments i0, i0 - 1, ... in this batch
+    float U[kBatch], D[kBatch], Q[kBatch], T1[kBatch];
+#pragma unroll
+    for (int j = 0; j < kBatch; ++j) {
+      const int i = max(i0 - j, 0);
+      const int seg = dir == 0 ? i : nseg - 1 - i;
+      U[j] = D[j] = Q[j] = T1[j] = 0.f;
+      if (live) {
+        const float* f = ws_fwd + slot(seg, dir) * kGlaStateFloats;
+        U[j] = f[e], D[j] = f[64 * 64 + ch];
+        Q[j] = ws_grad[slot(seg, gdir) * kGlaStateFloats + e];
+        T1[j] = term[slot(seg, dir) * kBwdStateElems + e];
+      }
     }
-    // the block holds 8 channels (lane half h, register m) x the 32 v columns of its half: sum them in a fixed order
-    red[tid] = later;
+#pragma unroll
+    for (int j = 0; j < kBatch; ++j) {
+      const int i = i0 - j;
+      red[j][tid] = later;
+      if (i >= 0) {
+        if (live) {
+          const int seg = dir == 0 ? i : nseg - 1 - i;
+          const uint16_t x = f32_to_bf16(__builtin_sqrtf(D[j]) * R);
+          rp[slot(seg, dir) * kBwdStateElems + ch * 64 + vch] = x;
+          rpt[slot(seg, dir) * kBwdStateElems + vch * 64 + ch] = x;
+        }
+        later += T1[j] - R * U[j];
+        R = __builtin_fmaf(D[j], R, Q[j]);
+      }
+    }
+    // the block holds 8 channels (lane half h, register m) x the 32 v columns of its half: summed in a fixed order
     __syncthreads();
-    if (tid < 8 && live) {
-      const int hh = tid >> 2, mm = tid & 3;
-      float acc = 0.f;
-      for (int x = 0; x < 32; ++x) acc += red[(32 * hh + x) * 4 + mm];
-      carry[slot(seg, dir) * 128 + pv * 64 + 8 * ng * hh + 8 * cq + 2 * mm + pk] = acc;
+    if (tid < 8 * kBatch && live) {
+      const int j = tid >> 3, hh = (tid >> 2) & 1, mm = tid & 3;
+      const int i = i0 - j;
+      if (i >= 0) {
+        const int seg = dir == 0 ? i : nseg - 1 - i;
+        float acc = 0.f;
+        for (int x = 0; x < 32; ++x) acc += red[j][(32 * hh + x) * 4 + mm];
+        carry[slot(seg, dir) * 128 + pv * 64 + 8 * ng * hh + 8 * cq + 2 * mm + pk] = acc;
+      }
     }
     __syncthreads();
-    later += t1 - R * U;
-    R = __builtin_fmaf(D, R, Q);
   }
 }
 
