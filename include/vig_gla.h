@@ -192,6 +192,16 @@ int vig_gla_bidir_bwd(const void* q, const void* k, const void* v,
 
 size_t vig_gla_bidir_bwd_workspace(int B, int H, int L, int Dk, int Dv, int bidirectional);
 
+/*
+ * Workspace of the path vig_gla_bidir_bwd takes for exactly these dtypes.  It differs from the query above for
+ * HierViG's head shape (Dk 16, Dv 32; classification/models/vig_h.py:521-527) with bf16 tensors and gates, both
+ * directions and L >= 128: given this many bytes, the backward runs zero-padded to 32 / 64 channels on the matrix-core
+ * kernels (inputs padded, gradients cropped; 20x faster than the token-recurrent kernel at L = 3136); given only the
+ * smaller amount of the query above, it runs on the token-recurrent kernel.
+ */
+size_t vig_gla_bidir_bwd_workspace_for(int B, int H, int L, int Dk, int Dv, int io_dtype, int gate_dtype,
+                                       int bidirectional);
+
 /* Same contract as vig_gla_bidir_bwd, always the fp32-arithmetic token-recurrent kernel (the exact path). */
 int vig_gla_bidir_bwd_exact(const void* q, const void* k, const void* v,
                             const void* g_fwd, const void* g_bwd, const void* d_o,

@@ -251,6 +251,35 @@ def test_backward_mfma_long_sequences_strong_gates_fall_back_per_sequence():
     _check_mfma([g_.cpu()[:, keep] for g_ in got], [w_[:, keep] for w_ in want], q[:, keep])
 
 
+@pytest.mark.parametrize("B,H,L", [(2, 3, 128), (2, 3, 196), (1, 6, 784), (1, 3, 3136)])
+def test_backward_hiervig_head_shape_on_the_matrix_cores(B, H, L):
+    """HierViG's head shape (Dk 16, Dv 32, vig_h.py:521-527): the backward zero-padded to 32 / 64 channels on the
+    matrix-core kernels (one slab for L <= 256, linked segments beyond), against the adjoint recurrences; a caller
+    that sizes the workspace for the recurrent kernel only still gets that kernel (the exact path, bit for bit)."""
+    announce(f"backward of the Dk16/Dv32 head shape B{B} H{H} L={L}")
+    q, k, v, gf, gb = make_gla_inputs(B, H, L, 16, 32, seed=700 + L, dtype=torch.bfloat16)
+    do = _do(v.shape, 17, torch.bfloat16)
+    dev = [t.cuda() for t in (q, k, v, gf, gb, do)]
+    want = O.bidir_gla_backward(f64(q), f64(k), f64(v), f64(gf), f64(gb), f64(do), out_scale=0.5)
+    got = vig_amd.gla_bidir_backward(*dev, out_scale=0.5)
+    _check_mfma(got, want, q)
+    exact = vig_amd.gla_bidir_backward(*dev, out_scale=0.5, exact=True)
+    assert any(not torch.equal(a, b) for a, b in zip(got, exact))  # (it did take the other path)
+    # through the C ABI with the smaller workspace: the recurrent kernel
+    from vig_amd import _lib
+    lib = _lib.load()
+    small = lib.vig_gla_bidir_bwd_workspace(B, H, L, 16, 32, 1)
+    assert small < lib.vig_gla_bidir_bwd_workspace_for(B, H, L, 16, 32, _lib.VIG_BF16, _lib.VIG_BF16, 1)
+    ws = torch.empty(small, dtype=torch.uint8, device="cuda")
+    outs = [torch.empty_like(t) for t in (dev[0], dev[1], dev[2], dev[3], dev[4])]
+    rc = lib.vig_gla_bidir_bwd(*(t.data_ptr() for t in dev), *(t.data_ptr() for t in outs), ws.data_ptr(), small,
+                               B, H, L, 16, 32, 16 ** -0.5, 0.5, _lib.VIG_BF16, _lib.VIG_BF16, None)
+    assert rc == 0
+    torch.cuda.synchronize()
+    for a, b in zip(outs, exact):
+        assert torch.equal(a, b)
+
+
 def test_autograd_keeps_the_exact_path():
     """gla_bidir_forward(exact=True) under autograd: the backward runs the fp32-arithmetic kernel too, bit-equal to
     gla_bidir_backward(exact=True) (and different from the matrix-core gradients of the default path)."""

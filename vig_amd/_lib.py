@@ -38,6 +38,7 @@ SIGNATURES = {
     "vig_gla_bidir_bwd": (_c_int, [_c_void_p] * 11 + [_c_void_p, _c_size_t] + [_c_int] * 5 + [_c_float, _c_float, _c_int, _c_int, _c_void_p]),
     "vig_gla_bidir_bwd_exact": (_c_int, [_c_void_p] * 11 + [_c_void_p, _c_size_t] + [_c_int] * 5 + [_c_float, _c_float, _c_int, _c_int, _c_void_p]),
     "vig_gla_bidir_bwd_workspace": (_c_size_t, [_c_int] * 6),
+    "vig_gla_bidir_bwd_workspace_for": (_c_size_t, [_c_int] * 8),
     "vig_dirgate_fwd": (_c_int, [_c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_float, _c_float, _c_int, _c_int, _c_void_p]),
     "vig_dwconv3x3_fwd": (_c_int, [_c_void_p, _c_void_p, _c_void_p, _c_void_p, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_void_p]),
     "vig_gla_bidir_locgate_fwd": (_c_int, [_c_void_p] * 7 + [_c_int] * 7 + [_c_float, _c_float, _c_int, _c_int, _c_void_p]),

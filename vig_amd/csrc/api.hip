@@ -519,6 +519,23 @@ size_t vig_gla_bidir_bwd_workspace(int B, int H, int L, int Dk, int Dv, int bidi
   return vig::gla_backward_workspace(B, H, L, Dk, Dv, bidirectional);
 }
 
+// The backward of HierViG's head shape rides the matrix-core kernels the way its forward does: q, k, both gates and
+// their four gradients padded to 32 channels, v, d_o and dv to 64, then the backward's own workspace at 32 / 64.
+static size_t padded_bwd_tensors(int B, int H, int L) {
+  const size_t n = (8 * padded_elems_qk(B, H, L) + 3 * padded_elems_v(B, H, L)) * sizeof(uint16_t);
+  return (n + 255) / 256 * 256;
+}
+static size_t padded_bwd_workspace(int B, int H, int L) {
+  return padded_bwd_tensors(B, H, L) + vig::gla_backward_workspace(B, H, L, 32, 64, 1);
+}
+
+size_t vig_gla_bidir_bwd_workspace_for(int B, int H, int L, int Dk, int Dv, int io_dtype, int gate_dtype,
+                                       int bidirectional) {
+  if (B <= 0 || H <= 0 || L <= 0 || !bwd_shape_ok(Dk, Dv) || !dtype_ok(io_dtype) || !dtype_ok(gate_dtype)) return 0;
+  if (padded_shape(L, Dk, Dv, io_dtype, gate_dtype, bidirectional != 0)) return padded_bwd_workspace(B, H, L);
+  return vig::gla_backward_workspace(B, H, L, Dk, Dv, bidirectional);
+}
+
 static int gla_bidir_bwd(const void* q, const void* k, const void* v, const void* g_fwd, const void* g_bwd,
                          const void* d_o, void* dq, void* dk, void* dv, void* dg_fwd, void* dg_bwd, void* workspace,
                          size_t workspace_bytes, int B, int H, int L, int Dk, int Dv, float scale, float out_scale,
@@ -529,6 +546,31 @@ static int gla_bidir_bwd(const void* q, const void* k, const void* v, const void
   if (!aligned16(q, k, v, g_fwd, g_bwd, d_o, dq, dk, dv, dg_fwd, dg_bwd, workspace)) return VIG_EINVAL;
   if ((long long)B * H > 2147483647LL) return VIG_EINVAL;
   if (!dtype_ok(io_dtype) || !dtype_ok(gate_dtype) || !bwd_shape_ok(Dk, Dv)) return VIG_ENOTSUP;
+  if (!exact && padded_shape(L, Dk, Dv, io_dtype, gate_dtype, g_bwd != nullptr) && workspace &&
+      workspace_bytes >= padded_bwd_workspace(B, H, L)) {
+    // (a caller that sized the workspace with vig_gla_bidir_bwd_workspace gets the recurrent kernel below)
+    const size_t nqk = padded_elems_qk(B, H, L), nv = padded_elems_v(B, H, L);
+    uint16_t* p = static_cast<uint16_t*>(workspace);
+    uint16_t *qp = p, *kp = p + nqk, *gfp = p + 2 * nqk, *gbp = p + 3 * nqk, *dqp = p + 4 * nqk, *dkp = p + 5 * nqk,
+             *dgfp = p + 6 * nqk, *dgbp = p + 7 * nqk, *vp = p + 8 * nqk, *dop = vp + nv, *dvp = dop + nv;
+    const long long rows = (long long)B * H * L;
+    hipStream_t st = (hipStream_t)stream;
+    {
+      const void* srcs[6] = {q, k, g_fwd, g_bwd, v, d_o};
+      void* dsts[6] = {qp, kp, gfp, gbp, vp, dop};
+      const int src_c[6] = {16, 16, 16, 16, 32, 32}, dst_c[6] = {32, 32, 32, 32, 64, 64};
+      const int e = vig::launch_pad_channels_multi(srcs, dsts, src_c, dst_c, 6, rows, st);
+      if (e) return e;
+    }
+    const int e = vig::launch_gla_backward(qp, kp, vp, gfp, gbp, dop, dqp, dkp, dvp, dgfp, dgbp,
+                                           (char*)workspace + padded_bwd_tensors(B, H, L), B, H, L, 32, 64, scale,
+                                           out_scale, io_dtype, gate_dtype, false, st);
+    if (e) return e;
+    const void* srcs[5] = {dqp, dkp, dgfp, dgbp, dvp};
+    void* dsts[5] = {dq, dk, dg_fwd, dg_bwd, dv};
+    const int src_c[5] = {32, 32, 32, 32, 64}, dst_c[5] = {16, 16, 16, 16, 32};
+    return vig::launch_pad_channels_multi(srcs, dsts, src_c, dst_c, 5, rows, st);
+  }
   const size_t need = vig::gla_backward_workspace(B, H, L, Dk, Dv, g_bwd != nullptr);
   if (!workspace || workspace_bytes < need) return VIG_ENOSPC;
   return vig::launch_gla_backward(q, k, v, g_fwd, g_bwd, d_o, dq, dk, dv, dg_fwd, dg_bwd, workspace, B, H, L, Dk, Dv,

@@ -567,10 +567,11 @@ __global__ __launch_bounds__(256) void pad_channels_kernel(const uint16_t* __res
 }
 
 // Several tensors of the same row count in one launch (blockIdx.y = tensor).
+constexpr int kMaxPadJobs = 6;
 struct PadJobs {
-  const uint16_t* src[5];
-  uint16_t* dst[5];
-  int src_c8[5], dst_c8[5];
+  const uint16_t* src[kMaxPadJobs];
+  uint16_t* dst[kMaxPadJobs];
+  int src_c8[kMaxPadJobs], dst_c8[kMaxPadJobs];
 };
 __global__ __launch_bounds__(256) void pad_channels_multi_kernel(PadJobs jobs, long long rows) {
   const int j = blockIdx.y;
@@ -587,7 +588,7 @@ __global__ __launch_bounds__(256) void pad_channels_multi_kernel(PadJobs jobs, l
 
 int launch_pad_channels_multi(const void* const* src, void* const* dst, const int* src_c, const int* dst_c, int n,
                               long long rows, hipStream_t stream) {
-  if (n < 1 || n > 5 || rows <= 0) return -95;
+  if (n < 1 || n > kMaxPadJobs || rows <= 0) return -95;
   PadJobs jobs{};
   int max_c8 = 0;
   for (int j = 0; j < n; ++j) {

@@ -168,7 +168,8 @@ std::tuple<Tensor, Tensor, Tensor, Tensor, optional<Tensor>> gla_bidir_bwd(const
   Tensor dq = at::empty_like(q), dk = at::empty_like(k), dv = at::empty_like(v), dgf = at::empty_like(g_fwd);
   optional<Tensor> dgb;
   if (g_bwd) dgb = at::empty_like(*g_bwd);
-  const size_t need = vig_gla_bidir_bwd_workspace(d.B, d.H, d.L, d.Dk, d.Dv, g_bwd ? 1 : 0);
+  const size_t need = exact ? vig_gla_bidir_bwd_workspace(d.B, d.H, d.L, d.Dk, d.Dv, g_bwd ? 1 : 0)
+                            : vig_gla_bidir_bwd_workspace_for(d.B, d.H, d.L, d.Dk, d.Dv, dt(q), dt(g_fwd), g_bwd ? 1 : 0);
   TORCH_CHECK(need > 0, "vig_gla_bidir_bwd: shape Dk=", d.Dk, ", Dv=", d.Dv, " is not built");
   Tensor ws = workspace(need, q);
   auto fn = exact ? vig_gla_bidir_bwd_exact : vig_gla_bidir_bwd;

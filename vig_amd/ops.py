@@ -92,7 +92,10 @@ def gla_bidir_backward(q, k, v, g_fwd, g_bwd, d_o, scale: float = -1, out_scale:
     dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
     dgf = torch.empty_like(g_fwd)
     dgb = torch.empty_like(g_bwd) if g_bwd is not None else None
-    ws_bytes = lib.vig_gla_bidir_bwd_workspace(B, H, L, Dk, Dv, int(g_bwd is not None))
+    if exact:
+        ws_bytes = lib.vig_gla_bidir_bwd_workspace(B, H, L, Dk, Dv, int(g_bwd is not None))
+    else:  # the workspace of the dispatched path (HierViG's head shape rides the matrix cores zero-padded)
+        ws_bytes = lib.vig_gla_bidir_bwd_workspace_for(B, H, L, Dk, Dv, _dt(q), _dt(g_fwd), int(g_bwd is not None))
     if ws_bytes == 0:
         raise _lib.VigGlaError(f"vig_gla_bidir_bwd: shape Dk={Dk}, Dv={Dv} is not built")
     ws = torch.empty(ws_bytes, dtype=torch.uint8, device=q.device)
