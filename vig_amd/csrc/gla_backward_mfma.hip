@@ -519,91 +519,128 @@ __global__ __launch_bounds__(512) void gla_backward_mfma_kernel(
 //   rp   = sqrt(D_s) R_out(s),    R_out(s) = Q_{s'} + D_{s'} R_out(s'),  zero for the segment walked last,
 //   rpt  = rp transposed,
 //   carry(s) = sum over the segments walked after s of rowsum_v(S_in Q - R_out U): what q dq - k dk adds up to there
-// (bf16 matrices in plain row-major order; carry as two partial sums per channel, one per half of the v columns).
-// One thread per state element in the passes' register order; `term` holds S_in Q between the two sweeps.
+// (bf16 matrices in plain row-major order; carry in the first of two slots per channel, the second zero).
+// A thread holds the four state elements (k channels c, c+1) x (v columns x, x+1) of the passes' register order
+// (units pk = 0, 1 and pv = 0, 1 of one register quad cq, lane, register m), so that its bf16 results leave as
+// 4-byte words: whole 128-byte rows of sp and rp per 32 lanes, 16-byte pieces of rpt per four threads.  `term` holds
+// S_in Q between the two sweeps.  Both sweeps fetch eight segments at a time: the serial part is arithmetic only.
 __global__ __launch_bounds__(256) void gla_backward_segment_scan_kernel(
     const float* __restrict__ ws_fwd, const float* __restrict__ ws_grad, float* __restrict__ term, uint16_t* __restrict__ sp,
     uint16_t* __restrict__ rp, uint16_t* __restrict__ rpt, float* __restrict__ carry, int* __restrict__ flags, int nseq,
     int nseg, int ndir, int ng) {
+  constexpr int kBatch = 8;
+  __shared__ float red[kBatch][2][256];
   const int tid = threadIdx.x;
-  const int e = blockIdx.x * 256 + tid;  // element in register order: ((u*64 + lane)*4 + m)
+  const int cq = blockIdx.x;  // register quad: 4 blocks per (sequence, direction)
   const int seq = blockIdx.y / ndir, dir = blockIdx.y % ndir;
-  if (blockIdx.x == 0 && tid == 0 && dir == 0) flags[seq] = 0;
-  const int m = e & 3, lane = (e >> 2) & 63, u = e >> 8;
-  const int pk = u >> 3, pv = (u >> 2) & 1, cq = u & 3, h = lane >> 5;
-  const bool live = cq < ng;  // register quads beyond Dk/16 carry no channel (uniform per block)
-  const int ch = live ? 8 * ng * h + 8 * cq + 2 * m + pk : 0;
-  const int vch = 2 * cpair<4>(lane & 31) + pv;
+  if (cq == 0 && tid == 0 && dir == 0) flags[seq] = 0;
+  if (cq >= ng) return;  // register quads beyond Dk/16 carry no channel (whole blocks)
+  const int m = tid & 3, lane = tid >> 2, h = lane >> 5;
+  const int ch0 = 8 * ng * h + 8 * cq + 2 * m;  // k channels ch0 (pk = 0), ch0 + 1 (pk = 1)
+  const int v0 = 2 * cpair<4>(lane & 31);         // v columns v0 (pv = 0), v0 + 1 (pv = 1)
+  // element (pk, pv) of this thread in register order: unit u = (pk*2 + pv)*4 + cq
+  int e[2][2];
+#pragma unroll
+  for (int pk = 0; pk < 2; ++pk)
+#pragma unroll
+    for (int pv = 0; pv < 2; ++pv) e[pk][pv] = ((((pk * 2 + pv) * 4 + cq) * 64 + lane) << 2) + m;
   auto slot = [&](int seg, int d) { return (((size_t)seq * nseg + seg) * 2 + d); };
   // the gradient state pass ran with the directions' roles exchanged (see launch_gla_backward_mfma)
   const int gdir = 1 - dir;
-  // Both sweeps fetch eight segments at a time, so that the serial part is arithmetic only.
-  constexpr int kBatch = 8;
-  float S = 0.f;
-  if (live) {
-    for (int i0 = 0; i0 < nseg; i0 += kBatch) {
-      float U[kBatch], D[kBatch], Q[kBatch];
+  float S[2][2] = {{0.f, 0.f}, {0.f, 0.f}};
+  for (int i0 = 0; i0 < nseg; i0 += kBatch) {
+    float U[kBatch][2][2], Q[kBatch][2][2], D[kBatch][2];
 #pragma unroll
-      for (int j = 0; j < kBatch; ++j) {
-        const int i = min(i0 + j, nseg - 1);
-        const int seg = dir == 0 ? i : nseg - 1 - i;
-        const float* f = ws_fwd + slot(seg, dir) * kGlaStateFloats;
-        U[j] = f[e], D[j] = f[64 * 64 + ch];
-        Q[j] = ws_grad[slot(seg, gdir) * kGlaStateFloats + e];
+    for (int j = 0; j < kBatch; ++j) {
+      const int i = min(i0 + j, nseg - 1);
+      const int seg = dir == 0 ? i : nseg - 1 - i;
+      const float* f = ws_fwd + slot(seg, dir) * kGlaStateFloats;
+      const float* g = ws_grad + slot(seg, gdir) * kGlaStateFloats;
+#pragma unroll
+      for (int pk = 0; pk < 2; ++pk) {
+        D[j][pk] = f[64 * 64 + ch0 + pk];
+#pragma unroll
+        for (int pv = 0; pv < 2; ++pv) U[j][pk][pv] = f[e[pk][pv]], Q[j][pk][pv] = g[e[pk][pv]];
       }
+    }
 #pragma unroll
-      for (int j = 0; j < kBatch; ++j) {
-        const int i = i0 + j;
-        if (i < nseg) {
-          const int seg = dir == 0 ? i : nseg - 1 - i;
-          sp[slot(seg, dir) * kBwdStateElems + ch * 64 + vch] = f32_to_bf16(__builtin_sqrtf(D[j]) * S);
-          term[slot(seg, dir) * kBwdStateElems + e] = S * Q[j];
-          S = __builtin_fmaf(D[j], S, U[j]);
+    for (int j = 0; j < kBatch; ++j) {
+      const int i = i0 + j;
+      if (i < nseg) {
+        const int seg = dir == 0 ? i : nseg - 1 - i;
+        uint16_t* spm = sp + slot(seg, dir) * kBwdStateElems;
+        float* tm = term + slot(seg, dir) * kBwdStateElems;
+#pragma unroll
+        for (int pk = 0; pk < 2; ++pk) {
+          const float rd = __builtin_sqrtf(D[j][pk]);
+          *reinterpret_cast<uint32_t*>(spm + (ch0 + pk) * 64 + v0) = pack_bf16x2(rd * S[pk][0], rd * S[pk][1]);
+#pragma unroll
+          for (int pv = 0; pv < 2; ++pv) {
+            tm[e[pk][pv]] = S[pk][pv] * Q[j][pk][pv];
+            S[pk][pv] = __builtin_fmaf(D[j][pk], S[pk][pv], U[j][pk][pv]);
+          }
         }
       }
     }
   }
-  __shared__ float red[kBatch][256];
-  float R = 0.f, later = 0.f;
+  float R[2][2] = {{0.f, 0.f}, {0.f, 0.f}}, later[2] = {0.f, 0.f};
   for (int i0 = nseg - 1; i0 >= 0; i0 -= kBatch) {  // segments i0, i0 - 1, ... in this batch
-    float U[kBatch], D[kBatch], Q[kBatch], T1[kBatch];
+    float U[kBatch][2][2], Q[kBatch][2][2], T1[kBatch][2][2], D[kBatch][2];
 #pragma unroll
     for (int j = 0; j < kBatch; ++j) {
       const int i = max(i0 - j, 0);
       const int seg = dir == 0 ? i : nseg - 1 - i;
-      U[j] = D[j] = Q[j] = T1[j] = 0.f;
-      if (live) {
-        const float* f = ws_fwd + slot(seg, dir) * kGlaStateFloats;
-        U[j] = f[e], D[j] = f[64 * 64 + ch];
-        Q[j] = ws_grad[slot(seg, gdir) * kGlaStateFloats + e];
-        T1[j] = term[slot(seg, dir) * kBwdStateElems + e];
+      const float* f = ws_fwd + slot(seg, dir) * kGlaStateFloats;
+      const float* g = ws_grad + slot(seg, gdir) * kGlaStateFloats;
+      const float* tm = term + slot(seg, dir) * kBwdStateElems;
+#pragma unroll
+      for (int pk = 0; pk < 2; ++pk) {
+        D[j][pk] = f[64 * 64 + ch0 + pk];
+#pragma unroll
+        for (int pv = 0; pv < 2; ++pv)
+          U[j][pk][pv] = f[e[pk][pv]], Q[j][pk][pv] = g[e[pk][pv]], T1[j][pk][pv] = tm[e[pk][pv]];
       }
     }
 #pragma unroll
     for (int j = 0; j < kBatch; ++j) {
       const int i = i0 - j;
-      red[j][tid] = later;
+      red[j][0][tid] = later[0];
+      red[j][1][tid] = later[1];
       if (i >= 0) {
-        if (live) {
-          const int seg = dir == 0 ? i : nseg - 1 - i;
-          const uint16_t x = f32_to_bf16(__builtin_sqrtf(D[j]) * R);
-          rp[slot(seg, dir) * kBwdStateElems + ch * 64 + vch] = x;
-          rpt[slot(seg, dir) * kBwdStateElems + vch * 64 + ch] = x;
+        const int seg = dir == 0 ? i : nseg - 1 - i;
+        uint16_t* rpm = rp + slot(seg, dir) * kBwdStateElems;
+        uint16_t* rtm = rpt + slot(seg, dir) * kBwdStateElems;
+        float x[2][2];
+#pragma unroll
+        for (int pk = 0; pk < 2; ++pk) {
+          const float rd = __builtin_sqrtf(D[j][pk]);
+          x[pk][0] = rd * R[pk][0], x[pk][1] = rd * R[pk][1];
+          *reinterpret_cast<uint32_t*>(rpm + (ch0 + pk) * 64 + v0) = pack_bf16x2(x[pk][0], x[pk][1]);
         }
-        later += T1[j] - R * U[j];
-        R = __builtin_fmaf(D[j], R, Q[j]);
+#pragma unroll
+        for (int pv = 0; pv < 2; ++pv)
+          *reinterpret_cast<uint32_t*>(rtm + (v0 + pv) * 64 + ch0) = pack_bf16x2(x[0][pv], x[1][pv]);
+#pragma unroll
+        for (int pk = 0; pk < 2; ++pk)
+#pragma unroll
+          for (int pv = 0; pv < 2; ++pv) {
+            later[pk] += T1[j][pk][pv] - R[pk][pv] * U[j][pk][pv];
+            R[pk][pv] = __builtin_fmaf(D[j][pk], R[pk][pv], Q[j][pk][pv]);
+          }
       }
     }
-    // the block holds 8 channels (lane half h, register m) x the 32 v columns of its half: summed in a fixed order
+    // the block holds 16 channels (lane half h, register m, pk) x all 64 v columns: summed in a fixed order
     __syncthreads();
-    if (tid < 8 * kBatch && live) {
-      const int j = tid >> 3, hh = (tid >> 2) & 1, mm = tid & 3;
+    if (tid < 16 * kBatch) {
+      const int j = tid >> 4, hh = (tid >> 3) & 1, mm = (tid >> 1) & 3, pk = tid & 1;
       const int i = i0 - j;
       if (i >= 0) {
         const int seg = dir == 0 ? i : nseg - 1 - i;
         float acc = 0.f;
-        for (int x = 0; x < 32; ++x) acc += red[j][(32 * hh + x) * 4 + mm];
-        carry[slot(seg, dir) * 128 + pv * 64 + 8 * ng * hh + 8 * cq + 2 * mm + pk] = acc;
+        for (int x = 0; x < 32; ++x) acc += red[j][pk][(32 * hh + x) * 4 + mm];
+        const int ch = 8 * ng * hh + 8 * cq + 2 * mm + pk;
+        carry[slot(seg, dir) * 128 + ch] = acc;
+        carry[slot(seg, dir) * 128 + 64 + ch] = 0.f;
       }
     }
     __syncthreads();
@@ -680,7 +717,7 @@ int launch_gla_backward_mfma(const void* q, const void* k, const void* v, const 
     rc = launch_gla_mfma(a);
     if (rc != 0) return rc;
     const int ndir = gb ? 2 : 1;
-    hipLaunchKernelGGL(gla_backward_segment_scan_kernel, dim3(64 * 64 / 256, B * H * ndir), dim3(256), 0, stream, ws_fwd,
+    hipLaunchKernelGGL(gla_backward_segment_scan_kernel, dim3(4, B * H * ndir), dim3(256), 0, stream, ws_fwd,
                        ws_grad, term, sp, rp, rpt, carry, flags, B * H, gla_segments(L), ndir, Dk / 16);
     sg = BwdSegments{sp, rp, rpt, carry, gla_segments(L), gla_segment_len(L)};
     nslabs = B * H * sg.nseg;
