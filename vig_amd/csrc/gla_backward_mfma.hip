@@ -701,20 +701,18 @@ int launch_gla_backward_mfma(const void* q, const void* k, const void* v, const 
     uint16_t* sp = (uint16_t*)(carry + n * 128);
     uint16_t* rp = sp + n * kBwdStateElems;
     uint16_t* rpt = rp + n * kBwdStateElems;
-    // the forward's state pass: contributions k~^T v and decays of every segment, both directions
+    // One launch for both state passes.  The forward's: contributions k~^T v and decays of every segment, both
+    // directions.  The gradient states: the same pass on (q for k, do for v) with each token's own gate included in
+    // its weight.  A state pass anchors a token at the END of its walk (the weight of token j is the decay from j to
+    // the last token walked); the gradient state needs the decay from the FIRST token walked to i, i.e. the walk of
+    // the other direction over the same gates: the forward gates go to the reverse waves and the reverse gates to the
+    // forward waves, and slot d of that pass belongs to direction 1 - d.  (The causal op runs both directions on its
+    // one gate tensor and uses the forward slot of the first pass and the reverse slot of the second.)
     GlaArgs a{};
-    a.q = q, a.k = k, a.v = v, a.g_fwd = gf, a.g_bwd = gb, a.o = nullptr, a.workspace = ws_fwd;
+    a.q = q, a.k = k, a.v = v, a.g_fwd = gf, a.g_bwd = gb ? gb : gf, a.o = const_cast<void*>(d_o), a.workspace = ws_fwd;
     a.B = B, a.H = H, a.L = L, a.Dk = Dk, a.Dv = 64, a.scale = 1.f, a.out_scale = 1.f, a.io_dtype = 1, a.gate_dtype = 1;
-    a.stream = stream, a.state_pass = 1;
-    int rc = launch_gla_mfma(a);
-    if (rc != 0) return rc;
-    // the gradient states: the same pass on (q for k, do for v) with each token's own gate included in its weight.
-    // A state pass anchors a token at the END of its walk (the weight of token j is the decay from j to the last
-    // token walked); the gradient state needs the decay from the FIRST token walked to i, i.e. the walk of the other
-    // direction over the same gates: the forward gates go to the reverse waves and the reverse gates to the forward
-    // waves, and slot d of this pass belongs to direction 1 - d.
-    a.k = q, a.v = d_o, a.g_fwd = gb ? gb : gf, a.g_bwd = gf, a.workspace = ws_grad, a.state_pass = 2;
-    rc = launch_gla_mfma(a);
+    a.stream = stream, a.state_pass = 2;
+    const int rc = launch_gla_mfma(a);
     if (rc != 0) return rc;
     const int ndir = gb ? 2 : 1;
     hipLaunchKernelGGL(gla_backward_segment_scan_kernel, dim3(4, B * H * ndir), dim3(256), 0, stream, ws_fwd,

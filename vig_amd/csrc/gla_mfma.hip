@@ -264,11 +264,13 @@ __device__ __forceinline__ void issue_first_phase(const ChunkSrc& src, int r, in
 //               contribution and total decay are written to the workspace (no outputs);
 //   kModeChain  pass 2 of a long sequence: the state entering the segment (from the left for the forward direction,
 //               from the right for the reverse one) is read from the workspace and outputs are produced.
-//   kModeStateStrict  kModeState with the cumulative gates taken exclusive of a token's own gate (so that the weight of
-//               a token reaches back to and includes it): the backward of a long sequence builds its per-segment
-//               gradient states with this pass, fed q for k and the output gradient for v.
-constexpr int kModeSlab = 0, kModeState = 1, kModeChain = 2, kModeStateStrict = 3;
-constexpr bool is_state_mode(int mode) { return mode == kModeState || mode == kModeStateStrict; }
+//   kModeStateDual  two state passes in one launch, for the backward of a long sequence: items below
+//               Geometry::dual_first are kModeState items; the others build the per-segment gradient states: the
+//               same pass fed the q tensor for k and the output gradient (the o argument) for v, with the other
+//               direction's gates and the cumulative gates taken exclusive of a token's own gate (so that the weight
+//               of a token reaches back to and includes it).
+constexpr int kModeSlab = 0, kModeState = 1, kModeChain = 2, kModeStateDual = 3;
+constexpr bool is_state_mode(int mode) { return mode == kModeState || mode == kModeStateDual; }
 constexpr int kStateFloats = kGlaStateFloats;  // per (sequence, segment, direction): state in unit order, then 64 decays
 
 // Intra-chunk part of one wave: scores of the three tile pairs of its chunk, applied to V; k~ (bf16) goes to the
@@ -417,7 +419,7 @@ struct GateLayout {
 template <bool FWD, int MODE, int NG, bool F16, bool GATE>
 __device__ __forceinline__ bool direction_wave(const ChunkSrc& cur, const ChunkSrc& nxt, rsrc_t o, int c, int lane,
                                                char* lds, float oscale, bool bidir, float* state, Prefetch<NG>& pf,
-                                               const GateCtx& gate) {
+                                               const GateCtx& gate, bool strict = false) {
   constexpr bool OUT = !is_state_mode(MODE);  // produces outputs (needs q)
   int r = lane & 31, h = lane >> 5;
   const int wi = (FWD ? 0 : 4) + c;
@@ -439,8 +441,8 @@ __device__ __forceinline__ bool direction_wave(const ChunkSrc& cur, const ChunkS
     u32x4_t gfrag[4][2];
     finish_tfrags<4>(pf.gD, gfrag);
     const u32x4_t ones = {0x3F803F80u, 0x3F803F80u, 0x3F803F80u, 0x3F803F80u};
-    constexpr bool STRICT = MODE == kModeStateStrict;
-    const u32x4_t tri0 = tri_frag<FWD, STRICT>(0, 0, r, h), tri1 = tri_frag<FWD, STRICT>(1, 0, r, h);
+    u32x4_t tri0 = tri_frag<FWD>(0, 0, r, h), tri1 = tri_frag<FWD>(1, 0, r, h);
+    if (MODE == kModeStateDual && strict) tri0 = tri_frag<FWD, true>(0, 0, r, h), tri1 = tri_frag<FWD, true>(1, 0, r, h);
     // k-steps of the tile walked first / second (the triangular operand depends on (k-step, tile) only through
     // their offset, so two fragments serve both tiles)
     constexpr int A0 = FWD ? 0 : 2, B0 = FWD ? 2 : 0;
@@ -754,28 +756,33 @@ struct Geometry {
   int L, nseg, seg_len, cw, nitems;
   int gw, gh, heads;  // fused locality gate only: token grid and heads per batch element
   int wide_gates;     // nonzero: skip the fp16 score variant from the start
+  int dual_first;     // kModeStateDual: first item of the gradient-state set (= items of the plain set)
 };
 
 template <bool FWD, int MODE, int NG, bool F16, bool GATE>
 __device__ __forceinline__ int wave_loop(const uint16_t* q, const uint16_t* k, const uint16_t* v, const uint16_t* g,
-                                         uint16_t* o, const Geometry& geo, int item, int c, int lane, char* lds,
-                                         float oscale, bool bidir, float* state_ws, const float* gate_w) {
+                                         const uint16_t* g_other, uint16_t* o, const Geometry& geo, int item, int c,
+                                         int lane, char* lds, float oscale, bool bidir, float* state_ws,
+                                         const float* gate_w) {
   constexpr bool OUT = !is_state_mode(MODE);
   constexpr int DK = 16 * NG;
   // descriptors of this wave's chunk of an item; past the last item (or for a chunk with no tokens) they are empty
   auto locate = [&](int it, ChunkSrc& src, rsrc_t& dst) {
     int nvalid = 0;
     size_t off = 0;
+    const uint16_t *kk = k, *vv = v, *gg = g;
     if (it < geo.nitems) {
-      const int seq = it / geo.nseg, seg = it - seq * geo.nseg;
+      int it2 = it;
+      if (MODE == kModeStateDual && it >= geo.dual_first) it2 = it - geo.dual_first, kk = q, vv = o, gg = g_other;
+      const int seq = it2 / geo.nseg, seg = it2 - seq * geo.nseg;
       const int seg_tokens = min(geo.seg_len, geo.L - seg * geo.seg_len);
       nvalid = min(max(seg_tokens - c * geo.cw, 0), geo.cw);
       off = (size_t)seq * geo.L + (size_t)seg * geo.seg_len + (size_t)(nvalid > 0 ? c * geo.cw : 0);  // in tokens
     }
     src.q = chunk_rsrc(q + off * DK, nvalid, 2 * DK);
-    src.k = chunk_rsrc(k + off * DK, nvalid, 2 * DK);
-    src.g = chunk_rsrc(g + off * DK, nvalid, 2 * DK);
-    src.v = chunk_rsrc(v + off * 64, nvalid, 128);
+    src.k = chunk_rsrc(kk + off * DK, nvalid, 2 * DK);
+    src.g = chunk_rsrc(gg + off * DK, nvalid, 2 * DK);
+    src.v = chunk_rsrc(vv + off * 64, nvalid, 128);
     dst = chunk_rsrc(o + off * 64, nvalid, 128);
   };
   Prefetch<NG> pf;
@@ -797,8 +804,9 @@ __device__ __forceinline__ int wave_loop(const uint16_t* q, const uint16_t* k, c
       const int nvalid = min(max(geo.L - c * geo.cw, 0), geo.cw);
       gate = GateCtx{gate_w + (size_t)(item % geo.heads) * (64 * 9), geo.gw, geo.gh, c * geo.cw, nvalid};
     }
+    const bool strict = MODE == kModeStateDual && item >= geo.dual_first;
     const bool ok =
-        direction_wave<FWD, MODE, NG, F16, GATE>(cur, nxt, dst, c, lane, lds, oscale, bidir, state, pf, gate);
+        direction_wave<FWD, MODE, NG, F16, GATE>(cur, nxt, dst, c, lane, lds, oscale, bidir, state, pf, gate, strict);
     lds_barrier();  // (D) the next item reuses the LDS regions
     if (F16 && !ok) break;  // this item again, and all that follow, with split-bf16 scores
     cur = nxt;
@@ -810,13 +818,15 @@ __device__ __forceinline__ int wave_loop(const uint16_t* q, const uint16_t* k, c
 // The items of one wave: fp16 score operands until a segment refuses them, split bf16 from there on.
 template <bool FWD, int MODE, int NG, bool GATE>
 __device__ __forceinline__ void wave_items(const uint16_t* q, const uint16_t* k, const uint16_t* v, const uint16_t* g,
-                                           uint16_t* o, const Geometry& geo, int c, int lane, char* lds, float oscale,
-                                           bool bidir, float* state_ws, const float* gate_w) {
+                                           const uint16_t* g_other, uint16_t* o, const Geometry& geo, int c, int lane,
+                                           char* lds, float oscale, bool bidir, float* state_ws, const float* gate_w) {
   int item = (int)blockIdx.x;
   // (a caller that knows its gates to be strong starts with the split-bf16 variant: no segment is walked in vain)
   if (!geo.wide_gates)
-    item = wave_loop<FWD, MODE, NG, true, GATE>(q, k, v, g, o, geo, item, c, lane, lds, oscale, bidir, state_ws, gate_w);
-  wave_loop<FWD, MODE, NG, false, GATE>(q, k, v, g, o, geo, item, c, lane, lds, oscale, bidir, state_ws, gate_w);
+    item = wave_loop<FWD, MODE, NG, true, GATE>(q, k, v, g, g_other, o, geo, item, c, lane, lds, oscale, bidir,
+                                                state_ws, gate_w);
+  wave_loop<FWD, MODE, NG, false, GATE>(q, k, v, g, g_other, o, geo, item, c, lane, lds, oscale, bidir, state_ws,
+                                        gate_w);
 }
 
 }  // namespace
@@ -836,9 +846,9 @@ __global__ __launch_bounds__(512) void gla_mfma_kernel(const uint16_t* __restric
   if (tid == 0) *reinterpret_cast<int*>(lds + kLdsVeto) = 0;
   lds_barrier();
   if (wi < 4) {
-    wave_items<true, MODE, NG, GATE>(q, k, v, gf, o, geo, c, lane, lds, oscale, bidir, state_ws, gate_w);
+    wave_items<true, MODE, NG, GATE>(q, k, v, gf, gb, o, geo, c, lane, lds, oscale, bidir, state_ws, gate_w);
   } else if (bidir) {
-    wave_items<false, MODE, NG, GATE>(q, k, v, gb, o, geo, c, lane, lds, oscale, bidir, state_ws, gate_w);
+    wave_items<false, MODE, NG, GATE>(q, k, v, gb, gf, o, geo, c, lane, lds, oscale, bidir, state_ws, gate_w);
   } else {
     // idle half of a one-direction launch: keeps the barrier count of the working waves, including the segment
     // that is walked twice when the fp16 variant is refused
@@ -954,7 +964,7 @@ static int launch_gla_mfma_t(const GlaArgs& a, int num_cu, int dev) {
                               reinterpret_cast<const void*>(gla_mfma_kernel<kModeState, NG>),
                               reinterpret_cast<const void*>(gla_mfma_kernel<kModeChain, NG>),
                               reinterpret_cast<const void*>(gla_mfma_kernel<kModeSlab, NG, true>),
-                              reinterpret_cast<const void*>(gla_mfma_kernel<kModeStateStrict, NG>)};
+                              reinterpret_cast<const void*>(gla_mfma_kernel<kModeStateDual, NG>)};
     for (const void* kf : kernels)
       if (hipFuncSetAttribute(kf, hipFuncAttributeMaxDynamicSharedMemorySize, kLdsTotal) != hipSuccess) return -5;
     attr_done = true;
@@ -972,10 +982,15 @@ static int launch_gla_mfma_t(const GlaArgs& a, int num_cu, int dev) {
   const float* no_gate = nullptr;
   if (a.state_pass) {
     // one state pass alone: contributions and decays of every (sequence, segment, direction), no scan, no outputs
-    if (a.state_pass == 2)
-      hipLaunchKernelGGL((gla_mfma_kernel<kModeStateStrict, NG>), dim3(grid), dim3(512), kLdsTotal, a.stream, q, k, v,
+    if (a.state_pass == 2) {
+      // plain set on (k, v, gates) and gradient-state set on (q for k, o for v, gates exchanged) in one launch
+      if (!gb) return -22;
+      geo.dual_first = geo.nitems;
+      geo.nitems *= 2;
+      grid = geo.nitems < num_cu ? geo.nitems : num_cu;
+      hipLaunchKernelGGL((gla_mfma_kernel<kModeStateDual, NG>), dim3(grid), dim3(512), kLdsTotal, a.stream, q, k, v,
                          gf, gb, o, geo, oscale, (float*)a.workspace, no_gate);
-    else
+    } else
       hipLaunchKernelGGL((gla_mfma_kernel<kModeState, NG>), dim3(grid), dim3(512), kLdsTotal, a.stream, q, k, v, gf, gb,
                          o, geo, oscale, (float*)a.workspace, no_gate);
   } else if (a.gate_w) {

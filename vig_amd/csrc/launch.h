@@ -28,8 +28,10 @@ struct GlaArgs {
   // causal op only (g_bwd null): fp32 [B, H, Dk, Dv] state before the first token / after the last one; null: zero / not wanted
   const float* init_state = nullptr;
   float* final_state = nullptr;
-  // bf16 MFMA path, any L: run one state pass alone into `workspace` (1: plain, 2: with the cumulative gates exclusive
-  // of each token's own gate): per (sequence, segment, direction) kGlaStateFloats floats, no scan, no outputs
+  // bf16 MFMA path, any L: run state passes alone into `workspace`, per (sequence, segment, direction)
+  // kGlaStateFloats floats, no scan, no outputs.  1: the forward's pass on (k, v, gates).  2 (both directions only):
+  // that pass and, behind its slots, the gradient-state pass of the backward on (q for k, `o` read as the output
+  // gradient for v, the two directions' gates exchanged, cumulative gates exclusive of each token's own gate).
   int state_pass = 0;
 };
 
