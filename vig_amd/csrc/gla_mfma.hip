@@ -572,24 +572,32 @@ __device__ __forceinline__ bool direction_wave(const ChunkSrc& cur, const ChunkS
           for (int m = 0; m < 4; ++m) S[pk][j][m] *= dw[2 * m + pk];
         }
       }
+    // every decay vector and contribution a slice needs is fetched before its serial chain starts: one LDS round
+    // trip per slice instead of one per chunk (3 % on the Dk = 32 slab shape, neutral on the others)
+    constexpr int I0 = MODE == kModeChain ? 0 : 1;
 #pragma unroll
-    for (int i = (MODE == kModeChain ? 0 : 1); i < 4; ++i) {
-      const int wc = W0 + STEP * i;  // consumer chunk: needs exp(G_end(wc)/2) * S as fragments
-      char* creg = dirbase + wc * kRegionBytes;
-      const bool add_u = is_state_mode(MODE) || i < 3;
+    for (int j = 0; j < NQ; ++j) {
+      const int cq = cqa + j;
+      f32x4_t d0[4], d1[4], u0[4], u1[4];
 #pragma unroll
-      for (int j = 0; j < NQ; ++j) {
-        const int cq = cqa + j;
-        const f32x4_t d0 = *reinterpret_cast<const f32x4_t*>(ddir + wc * 64 + HC * h + 8 * cq);
-        const f32x4_t d1 = *reinterpret_cast<const f32x4_t*>(ddir + wc * 64 + HC * h + 8 * cq + 4);
-        // half decay of row (m, pk): element 2*m + pk of the eight
-        const float dk0[4] = {d0[0], d0[2], d1[0], d1[2]};
-        const float dk1[4] = {d0[1], d0[3], d1[1], d1[3]};
-        f32x4_t u0 = {0.f, 0.f, 0.f, 0.f}, u1 = {0.f, 0.f, 0.f, 0.f};
-        if (add_u) {
-          u0 = *reinterpret_cast<const f32x4_t*>(unit_ptr(creg, (0 * 2 + pv) * 4 + cq, lane));
-          u1 = *reinterpret_cast<const f32x4_t*>(unit_ptr(creg, (1 * 2 + pv) * 4 + cq, lane));
+      for (int i = I0; i < 4; ++i) {
+        const int wc = W0 + STEP * i;  // consumer chunk: needs exp(G_end(wc)/2) * S as fragments
+        char* creg = dirbase + wc * kRegionBytes;
+        d0[i] = *reinterpret_cast<const f32x4_t*>(ddir + wc * 64 + HC * h + 8 * cq);
+        d1[i] = *reinterpret_cast<const f32x4_t*>(ddir + wc * 64 + HC * h + 8 * cq + 4);
+        u0[i] = u1[i] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+        if (is_state_mode(MODE) || i < 3) {
+          u0[i] = *reinterpret_cast<const f32x4_t*>(unit_ptr(creg, (0 * 2 + pv) * 4 + cq, lane));
+          u1[i] = *reinterpret_cast<const f32x4_t*>(unit_ptr(creg, (1 * 2 + pv) * 4 + cq, lane));
         }
+      }
+#pragma unroll
+      for (int i = I0; i < 4; ++i) {
+        const int wc = W0 + STEP * i;
+        char* creg = dirbase + wc * kRegionBytes;
+        // half decay of row (m, pk): element 2*m + pk of the eight
+        const float dk0[4] = {d0[i][0], d0[i][2], d1[i][0], d1[i][2]};
+        const float dk1[4] = {d0[i][1], d0[i][3], d1[i][1], d1[i][3]};
         u32x4_t fr;
 #pragma unroll
         for (int m = 0; m < 4; ++m) {
@@ -597,8 +605,8 @@ __device__ __forceinline__ bool direction_wave(const ChunkSrc& cur, const ChunkS
           const float t0 = S[0][j][m] * dk0[m];
           const float t1 = S[1][j][m] * dk1[m];
           fr[m] = pack_bf16x2(t0, t1);
-          S[0][j][m] = (t0 + u0[m]) * dk0[m];
-          S[1][j][m] = (t1 + u1[m]) * dk1[m];
+          S[0][j][m] = (t0 + u0[i][m]) * dk0[m];
+          S[1][j][m] = (t1 + u1[i][m]) * dk1[m];
         }
         if (OUT) *reinterpret_cast<u32x4_t*>(unit_ptr(creg, pv * 4 + cq, lane)) = fr;
       }
