@@ -294,6 +294,8 @@ __device__ __forceinline__ bool tile_phase(const ChunkSrc& cur, const Prefetch<N
   u32x4_t rawk[NG], rawq[NG];
   uint32_t vDb[2][8];
   f32x4acc_t gram = {0.f, 0.f, 0.f, 0.f};  // (fp16 variant) magnitude guard over the chunk's q, k and V
+  // a reverse wave only runs beside the forward wave of the same chunk, which sees the same q, k and V rows
+  constexpr bool GUARD = F16 && FWD;
   auto set_vfrag = [&](const uint32_t (&D)[2][8], int t0) {
     u32x4_t vf[2][2];
     finish_tfrags<2>(D, vf);
@@ -302,7 +304,7 @@ __device__ __forceinline__ bool tile_phase(const ChunkSrc& cur, const Prefetch<N
 #pragma unroll
       for (int p = 0; p < 2; ++p) {
         if (F16) {  // bf16 pairs -> fp16 pairs (exact for magnitudes the variant admits: the guard sees them first)
-          gram_acc(vf[tl][p], gram);
+          if (GUARD) gram_acc(vf[tl][p], gram);
 #pragma unroll
           for (int x = 0; x < 4; ++x) vf[tl][p][x] = pack_f16x2(bf16lo_to_f32(vf[tl][p][x]), bf16hi_to_f32(vf[tl][p][x]));
         }
@@ -318,8 +320,8 @@ __device__ __forceinline__ bool tile_phase(const ChunkSrc& cur, const Prefetch<N
   if (F16) {
 #pragma unroll
     for (int g = 0; g < NG; ++g) {
-      gram_acc(pf.rawk[g], gram);
-      if (OUT) gram_acc(pf.rawq[g], gram);
+      if (GUARD) gram_acc(pf.rawk[g], gram);
+      if (GUARD && OUT) gram_acc(pf.rawq[g], gram);
     }
     u32x4_t ka[NG], qb[NG];
     // the second tile's loads go out before the first tile's operands are built where registers allow it (measured:
@@ -339,8 +341,8 @@ __device__ __forceinline__ bool tile_phase(const ChunkSrc& cur, const Prefetch<N
     VIG_PHASE();
 #pragma unroll
     for (int g = 0; g < NG; ++g) {
-      gram_acc(rawk[g], gram);
-      if (OUT) gram_acc(rawq[g], gram);
+      if (GUARD) gram_acc(rawk[g], gram);
+      if (GUARD && OUT) gram_acc(rawq[g], gram);
     }
     u32x4_t kb[NG];
     make_pair16<OUT, NG>(rawq, rawk, G[TB], gend2, qb, kb, qkeep[TB]);
@@ -349,7 +351,7 @@ __device__ __forceinline__ bool tile_phase(const ChunkSrc& cur, const Prefetch<N
     VIG_PHASE();
     set_vfrag(vDb, 2 * TB);
     if (OUT) apply_scores<MASK, true>(score_tile16<NG>(kb, qb), TB, r, h, vfrag, O[0][TB], O[1][TB]);
-    too_large = gram_too_large(gram);
+    too_large = GUARD && gram_too_large(gram);
   } else {
     HalfOps<NG> ka, qb;
     {
