@@ -280,6 +280,44 @@ def test_backward_hiervig_head_shape_on_the_matrix_cores(B, H, L):
         assert torch.equal(a, b)
 
 
+def test_long_sequence_forward_and_backward_replay_as_a_graph():
+    """The multi-launch paths of a long sequence (forward: state pass, segment scan, output pass; backward: dual
+    state pass, segment scan, quadratic forms, flag pass) are plain kernel sequences on the caller's stream: captured
+    as one HIP graph they reproduce the eager results bit for bit on every replay, with eager work and
+    synchronisations between the replays and after the inputs change in place."""
+    announce("L = 700 forward + backward captured as a HIP graph, 4 replays")
+    q, k, v, gf, gb = (t.cuda() for t in make_gla_inputs(2, 3, 700, 64, 64, seed=91, dtype=torch.bfloat16))
+    do = _do(v.shape, 18, torch.bfloat16).cuda()
+    q2, k2, v2, gf2, gb2 = (t.cuda() for t in make_gla_inputs(2, 3, 700, 64, 64, seed=92, dtype=torch.bfloat16))
+    static = [t.clone() for t in (q, k, v, gf, gb, do)]
+
+    def run(ts):
+        o = vig_amd.gla_bidir_forward(*ts[:5])
+        return (o,) + tuple(vig_amd.gla_bidir_backward(*ts))
+
+    want_a = [t.clone() for t in run([q, k, v, gf, gb, do])]
+    want_b = [t.clone() for t in run([q2, k2, v2, gf2, gb2, do])]
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        run(static)
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        outs = run(static)
+    for i in range(4):
+        src, want = (([q, k, v, gf, gb], want_a), ([q2, k2, v2, gf2, gb2], want_b))[i % 2]
+        for dst, s_ in zip(static[:5], src):
+            dst.copy_(s_)
+        graph.replay()
+        torch.cuda.synchronize()
+        for name, g_, w_ in zip(("o", "dq", "dk", "dv", "dg_fwd", "dg_bwd"), outs, want):
+            assert torch.equal(g_, w_), (i, name)
+        run([q2, k2, v2, gf2, gb2, do])  # eager work between the replays
+        torch.cuda.synchronize()
+
+
 def test_autograd_keeps_the_exact_path():
     """gla_bidir_forward(exact=True) under autograd: the backward runs the fp32-arithmetic kernel too, bit-equal to
     gla_bidir_backward(exact=True) (and different from the matrix-core gradients of the default path)."""
