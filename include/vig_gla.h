@@ -63,9 +63,10 @@ const char* vig_gla_strerror(int code);
  * stay below about 80 (beyond it results may be inf / NaN, never silently wrong
  * finite numbers).  q, k and v may hold any finite bf16 values: the kernel
  * checks their magnitudes and the gate totals per chunk and takes its fp16
- * operands (scaled q and k, scores, v) only where they are exact enough (rows
- * with sums of squares below 2^15, i.e. elements below about 180; gate total of
- * a chunk within about 8), bf16 hi + lo pairs otherwise.  HierViG's head shape
+ * operands (scaled q and k, scores, v, and for L <= 256 each chunk's 64 x 64
+ * sum of k^T v) only where they are exact enough (rows with sums of squares
+ * below 2^15, i.e. elements below about 180; gate total of a chunk within about
+ * 8; chunk sums below 60000), bf16 hi + lo pairs otherwise.  HierViG's head shape
  * (bf16, Dk = 16, Dv = 32, both directions) takes the same path from L = 128 on,
  * zero-padded to Dk 32 / Dv 64 in the workspace (classification/models/vig_h.py:
  * 377-385 with EXPAND_K 0.5, EXPAND_V 1.0).  Other combinations run on the

@@ -8,10 +8,13 @@ so state update and inter-chunk product carry exp(G_end/2) each.
 
 splits:  qk = score operands: "f16" (one fp16 rounding each), 1 (bf16 hi*hi) or 3 (+ lo*hi + hi*lo),
          p = P terms in P V: "f16" (P rounded once to fp16; V is exact in fp16), 1 or 2 (bf16 hi, hi + lo),
-         iq = q~ terms in the inter-chunk product, st = state terms,
+         iq = q~ terms in the inter-chunk product, st = state terms, or st = "direct": no chained state, every earlier
+         chunk j of the direction adds f16(q~) @ f16(E * f16(U_j)) with U_j = k~^T V of that chunk and the per-channel
+         factor E = h_c h_j prod(h_i^2, i between), h = exp(G_end/2) in fp16, every product rounded to fp16,
          u = k~ in the state update: "f16" (the score operand again), 1 or 2 bf16 terms.
-The shipped kernel is qk="f16", p="f16", iq=1, st=1, u="f16"; for chunks whose gate total or operand magnitudes leave
-the fp16 range it falls back to qk=3, p=2, u=1 (FALLBACK).
+The shipped kernel is qk="f16", p="f16", st="direct", u="f16" for whole slabs (SHIPPED) and qk="f16", p="f16", iq=1,
+st=1, u="f16" for the chained segments of long sequences (SHIPPED_SEGMENTS); for chunks whose gate total or operand
+magnitudes leave the fp16 range it falls back to qk=3, p=2, iq=1, st=1, u=1 (FALLBACK).
 """
 from __future__ import annotations
 
@@ -40,7 +43,8 @@ def f16_round(x):
     return np.asarray(x, dtype=np.float32).astype(np.float16).astype(np.float32)
 
 
-SHIPPED = dict(qk="f16", p="f16", iq=1, st=1, u="f16")
+SHIPPED = dict(qk="f16", p="f16", iq=1, st="direct", u="f16")
+SHIPPED_SEGMENTS = dict(qk="f16", p="f16", iq=1, st=1, u="f16")
 FALLBACK = dict(qk=3, p=2, iq=1, st=1, u=1)
 PLAIN = dict(qk=1, p=1, iq=1, st=1, u=1)
 
@@ -57,6 +61,7 @@ def emulate(q, k, v, gf, gb, chunk, splits=SHIPPED):
     for direction in (0, 1):
         g = gf if direction == 0 else gb
         S = np.zeros((N, Dk, Dv), np.float32)
+        earlier = []  # (st == "direct") fp16 contribution and fp16 half decay of every chunk walked so far, nearest first
         order = range(nchunk) if direction == 0 else range(nchunk - 1, -1, -1)
         for c in order:
             sl = slice(c * chunk, min(L, (c + 1) * chunk))
@@ -91,12 +96,20 @@ def emulate(q, k, v, gf, gb, chunk, splits=SHIPPED):
                     oc += _mm(Pl, vc)
             sd = T(np.exp(half).astype(np.float32))  # half decay per key channel
             Sd = S * sd
-            Sh, Sl = _split(Sd)
-            oc += _mm(qh, Sh)
-            if splits["iq"] >= 2:
-                oc += _mm(ql, Sh)
-            if splits["st"] >= 2:
-                oc += _mm(qh, Sl)
+            if splits["st"] == "direct":
+                h16 = f16_round(np.exp(half).astype(np.float32))  # [N, 1, Dk]
+                base = h16
+                for Uj16, hj16 in earlier:
+                    e = f16_round(base * hj16)
+                    oc += _mm(f16_round(qt), f16_round(Uj16 * T(e)))
+                    base = f16_round(e * hj16)
+            else:
+                Sh, Sl = _split(Sd)
+                oc += _mm(qh, Sh)
+                if splits["iq"] >= 2:
+                    oc += _mm(ql, Sh)
+                if splits["st"] >= 2:
+                    oc += _mm(qh, Sl)
             o[:, sl] += s * oc
             if splits["u"] == "f16":
                 U = _mm(T(f16_round(kt)), vc)
@@ -104,5 +117,7 @@ def emulate(q, k, v, gf, gb, chunk, splits=SHIPPED):
                 U = _mm(T(kh), vc)
                 if splits["u"] >= 2:
                     U += _mm(T(kl), vc)
+            if splits["st"] == "direct":
+                earlier.insert(0, (f16_round(U), f16_round(np.exp(half).astype(np.float32))))
             S = (Sd + U) * sd
     return o

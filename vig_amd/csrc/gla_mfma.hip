@@ -56,7 +56,8 @@ constexpr int kLdsDvec = 8 * kRegionBytes;   // per wave: 64 chunk decays exp(G_
 constexpr int kLdsGend = kLdsDvec + 8 * 64 * 4;  // per wave: 64 anchors G_end * log2(e), laid out [h][p][16]
 constexpr int kLdsVeto = kLdsGend + 8 * 64 * 4;  // one word: some chunk refused the fp16 variant
 constexpr int kLdsGateW = kLdsVeto + 16;          // fused locality gate: the 64 x 9 stencil weights of the slab's head
-constexpr int kLdsTotal = kLdsGateW + 64 * 9 * 4;
+constexpr int kLdsHalf16 = kLdsGateW + 64 * 9 * 4;  // per wave: 64 half decays exp(G_end/2) as fp16, channel order
+constexpr int kLdsTotal = kLdsHalf16 + 8 * 64 * 2;
 
 typedef _Float16 f16x2_t __attribute__((ext_vector_type(2)));
 typedef _Float16 f16x8_t __attribute__((ext_vector_type(8)));
@@ -68,6 +69,11 @@ __device__ __forceinline__ uint32_t pack_f16x2(float lo, float hi) {
   f32x2_t x = {lo, hi};
   f16x2_t y = __builtin_convertvector(x, f16x2_t);  // round to nearest even
   return __builtin_bit_cast(uint32_t, y);
+}
+// elementwise product of two fp16 pairs (operands by value: a bit cast straight from a vector element reads the
+// vector's first word)
+__device__ __forceinline__ uint32_t mul_f16x2(uint32_t a, uint32_t b) {
+  return __builtin_bit_cast(uint32_t, __builtin_bit_cast(f16x2_t, a) * __builtin_bit_cast(f16x2_t, b));
 }
 
 // Magnitude guard of the fp16 score variant.  Raw bf16 rows go through a 16x16x32 matrix instruction as both
@@ -125,8 +131,9 @@ __device__ __forceinline__ void make_half(const u32x4_t (&raw)[NG], const f32x16
 // q~ and k~ of one 32-token tile for the fp16 score path: one exponent per element serves both (the factors are
 // reciprocal), each product is rounded once to fp16 (11-bit significand): k~ serves the scores and, through LDS, the
 // state update (against V converted to fp16, which holds every bf16 value of ordinary magnitude exactly); q~ is
-// rounded a second time to bf16 for the inter-chunk product with the bf16 state fragments.
-template <bool WITH_Q, int NG>
+// rounded a second time to bf16 for the inter-chunk product with the bf16 state fragments, or (KEEP16: whole slabs)
+// kept as it is for the products with the earlier chunks' fp16 contributions.
+template <bool WITH_Q, int NG, bool KEEP16 = false>
 __device__ __forceinline__ void make_pair16(const u32x4_t (&rawq)[NG], const u32x4_t (&rawk)[NG],
                                             const f32x16_t (&G)[2], const float* gend2, u32x4_t (&q16)[NG],
                                             u32x4_t (&k16)[NG], u32x4_t (&qb)[NG]) {
@@ -148,8 +155,12 @@ __device__ __forceinline__ void make_pair16(const u32x4_t (&rawq)[NG], const u32
         const float q0 = bf16lo_to_f32(wq) * exp2_fast(x0);
         const float q1 = bf16hi_to_f32(wq) * exp2_fast(x1);
         q16[g][m] = pack_f16x2(q0, q1);
-        qb[g][m] = pack_bf16x2(q0, q1);
-        asm volatile("" : "+v"(qb[g][m]));  // packed here: the two floats must not stay alive until the pair is used
+        if (KEEP16) {
+          qb[g][m] = q16[g][m];
+        } else {
+          qb[g][m] = pack_bf16x2(q0, q1);
+          asm volatile("" : "+v"(qb[g][m]));  // packed here: the two floats must not stay alive until the pair is used
+        }
       }
     }
   }
@@ -331,7 +342,7 @@ __device__ __forceinline__ bool tile_phase(const ChunkSrc& cur, const Prefetch<N
     VIG_PHASE();
     {
       u32x4_t qa[NG];
-      make_pair16<OUT, NG>(pf.rawq, pf.rawk, G[TA], gend2, qa, ka, qkeep[TA]);
+      make_pair16<OUT, NG, MODE == kModeSlab>(pf.rawq, pf.rawk, G[TA], gend2, qa, ka, qkeep[TA]);
       store_kt<NG>(kt, 32 * TA + r, h, ka);
       VIG_PHASE();
       if (!EARLY) fetch_second();
@@ -345,7 +356,7 @@ __device__ __forceinline__ bool tile_phase(const ChunkSrc& cur, const Prefetch<N
       if (GUARD && OUT) gram_acc(rawq[g], gram);
     }
     u32x4_t kb[NG];
-    make_pair16<OUT, NG>(rawq, rawk, G[TB], gend2, qb, kb, qkeep[TB]);
+    make_pair16<OUT, NG, MODE == kModeSlab>(rawq, rawk, G[TB], gend2, qb, kb, qkeep[TB]);
     store_kt<NG>(kt, 32 * TB + r, h, kb);
     if (OUT) apply_scores<0, true>(score_tile16<NG>(ka, qb), TA, r, h, vfrag, O[0][TB], O[1][TB]);
     VIG_PHASE();
@@ -495,7 +506,12 @@ __device__ __forceinline__ bool direction_wave(const ChunkSrc& cur, const ChunkS
     *mine = an;
     const int p = (lane >> 4) & 1, g = (lane >> 2) & 3, m = lane & 3;
     // half decay of channel 8*g + 2*m + p of this lane half (register quads >= NG carry no channel)
-    if (g < NG) dvec_all[wi * 64 + HC * h + 8 * g + 2 * m + p] = exp2_fast(an);
+    if (g < NG) {
+      if (MODE == kModeSlab && F16)
+        reinterpret_cast<_Float16*>(lds + kLdsHalf16)[wi * 64 + HC * h + 8 * g + 2 * m + p] = (_Float16)exp2_fast(an);
+      else
+        dvec_all[wi * 64 + HC * h + 8 * g + 2 * m + p] = exp2_fast(an);
+    }
   }
   wave_lds_sync();
   // ---- intra-chunk scores, tile by tile ----
@@ -521,6 +537,31 @@ __device__ __forceinline__ bool direction_wave(const ChunkSrc& cur, const ChunkS
         for (int pv = 0; pv < 2; ++pv)
           U[pk][pv] = F16 ? mfma_f16(ktf[pk], vfrag[t][pv], U[pk][pv]) : mfma(ktf[pk], vfrag[t][pv], U[pk][pv]);
     }
+    constexpr bool DIRECT = MODE == kModeSlab && F16;
+    if (DIRECT) {
+      // whole slab on fp16 operands: the later chunks of the direction take this contribution as it is (fp16, as
+      // ready fragments: dword m of unit pv*4 + cq holds rows (pk = 0, 1) of register 4*cq + m) instead of a state
+      // chained through it; its entries have to fit fp16
+      float umax = 0.f;
+#pragma unroll
+      for (int pk = 0; pk < 2; ++pk)
+#pragma unroll
+        for (int pv = 0; pv < 2; ++pv)
+#pragma unroll
+          for (int i = 0; i < 16; ++i) umax = fmaxf(umax, fabsf(U[pk][pv][i]));
+      if (__builtin_amdgcn_ballot_w64(!(umax < 60000.0f)) != 0) fast = false;
+      if (FWD ? (c < 3) : (c > 0)) {
+#pragma unroll
+        for (int pv = 0; pv < 2; ++pv)
+#pragma unroll
+          for (int cq = 0; cq < NG; ++cq) {
+            u32x4_t fr;
+#pragma unroll
+            for (int m = 0; m < 4; ++m) fr[m] = pack_f16x2(U[0][pv][4 * cq + m], U[1][pv][4 * cq + m]);
+            *reinterpret_cast<u32x4_t*>(unit_ptr(region, pv * 4 + cq, lane)) = fr;
+          }
+      }
+    } else
     // the chunk walked last is consumed by nobody inside the segment, unless the segment's own total is wanted
     if (is_state_mode(MODE) || (FWD ? (c < 3) : (c > 0))) {
 #pragma unroll
@@ -552,8 +593,51 @@ __device__ __forceinline__ bool direction_wave(const ChunkSrc& cur, const ChunkS
   // same answer in every wave: the word is only written before this barrier and the variant is left once it is set
   const bool ok = !F16 || __builtin_amdgcn_readfirstlane(*veto) == 0;
   if (F16 && !ok) return false;  // every wave alike: the segment is walked again, barriers B and C are skipped by all
-  // ---- state recurrence over the chunks of this direction, one slice (pv, NG/2 register quads) per wave ----
-  {
+  constexpr bool DIRECT = MODE == kModeSlab && F16;
+  if (DIRECT) {
+    // ---- whole slab on fp16 operands: O^T += (E (.) U_j)^T q~ for every chunk j walked earlier in this direction,
+    // E = h_c h_j prod(h_i^2, i between) per k channel with h = exp(G_end/2) <= 1 (the decay from the end of chunk j
+    // to the tokens of this chunk, given the half anchors inside q~ and U_j); fp16 x fp16 -> fp16, no factor exceeds
+    // one, tiny products may flush to zero.  No state, no serial chain: a wave with d earlier chunks does d products.
+    const int npairs = FWD ? c : 3 - c;
+    const _Float16* hdir = reinterpret_cast<const _Float16*>(lds + kLdsHalf16) + (FWD ? 0 : 4) * 64 + HC * h;
+    u32x4_t base16[NG];  // h_c times the squares of the chunks passed so far
+#pragma unroll
+    for (int g = 0; g < NG; ++g) base16[g] = *reinterpret_cast<const u32x4_t*>(hdir + 64 * c + 8 * g);
+#pragma unroll 1
+    for (int d = 1; d <= npairs; ++d) {
+      const int j = FWD ? c - d : c + d;
+      u32x4_t e16[NG];
+#pragma unroll
+      for (int g = 0; g < NG; ++g) {
+        const u32x4_t hj = *reinterpret_cast<const u32x4_t*>(hdir + 64 * j + 8 * g);
+#pragma unroll
+        for (int m = 0; m < 4; ++m) {
+          const uint32_t x = hj[m];
+          e16[g][m] = mul_f16x2(base16[g][m], x);
+          base16[g][m] = mul_f16x2(e16[g][m], x);
+        }
+      }
+      char* ureg = lds + ((FWD ? 0 : 4) + j) * kRegionBytes;
+      // (E goes onto the contribution's fragments, whose dwords hold the same k-channel pairs as q~'s: one scaling
+      // serves both query tiles)
+#pragma unroll
+      for (int pv = 0; pv < 2; ++pv) {
+        u32x4_t uf[NG];
+#pragma unroll
+        for (int ks = 0; ks < NG; ++ks) {
+          uf[ks] = *reinterpret_cast<const u32x4_t*>(unit_ptr(ureg, pv * 4 + ks, lane));
+#pragma unroll
+          for (int m = 0; m < 4; ++m) uf[ks][m] = mul_f16x2(uf[ks][m], e16[ks][m]);
+        }
+#pragma unroll
+        for (int ks = 0; ks < NG; ++ks)
+#pragma unroll
+          for (int it = 0; it < 2; ++it) O[pv][it] = mfma_f16(uf[ks], qkeep[it][ks], O[pv][it]);
+      }
+    }
+  } else {
+    // ---- state recurrence over the chunks of this direction, one slice (pv, NG/2 register quads) per wave ----
     constexpr int NQ = NG / 2;
     const int pv = c & 1, cqa = NQ * (c >> 1);
     char* dirbase = lds + (FWD ? 0 : 4) * kRegionBytes;
@@ -629,7 +713,7 @@ __device__ __forceinline__ bool direction_wave(const ChunkSrc& cur, const ChunkS
   lds_barrier();  // (B) incoming-state fragments of every chunk visible
   if (OUT) {
     // ---- O^T += (exp(G_end) * S_in) q~hi  for every chunk that has an incoming state ----
-    if (MODE == kModeChain || (FWD ? (c > 0) : (c < 3))) {
+    if (!DIRECT && (MODE == kModeChain || (FWD ? (c > 0) : (c < 3)))) {
 #pragma unroll
       for (int pv = 0; pv < 2; ++pv)
 #pragma unroll
