@@ -710,7 +710,10 @@ __device__ __forceinline__ bool direction_wave(const ChunkSrc& cur, const ChunkS
       }
     }
   }
-  lds_barrier();  // (B) incoming-state fragments of every chunk visible
+  // (whole slabs on fp16 operands without the fused gate send their output halves through the upper halves of the
+  // regions, which nothing else uses there: the published contributions stay readable and barrier B is not needed)
+  constexpr int kSendUnit = DIRECT && !GATE ? 8 : 0;
+  if (!(DIRECT && !GATE)) lds_barrier();  // (B) incoming-state fragments of every chunk visible
   if (OUT) {
     // ---- O^T += (exp(G_end) * S_in) q~hi  for every chunk that has an incoming state ----
     if (!DIRECT && (MODE == kModeChain || (FWD ? (c > 0) : (c < 3)))) {
@@ -733,7 +736,7 @@ __device__ __forceinline__ bool direction_wave(const ChunkSrc& cur, const ChunkS
         for (int cq = 0; cq < 4; ++cq) {
           const f32x4_t x = {O[pv][SEND][4 * cq], O[pv][SEND][4 * cq + 1], O[pv][SEND][4 * cq + 2],
                              O[pv][SEND][4 * cq + 3]};
-          *reinterpret_cast<f32x4_t*>(unit_ptr(region, pv * 4 + cq, lane)) = x;
+          *reinterpret_cast<f32x4_t*>(unit_ptr(region, kSendUnit + pv * 4 + cq, lane)) = x;
         }
     }
     lds_barrier();  // (C) swapped output halves visible
@@ -743,7 +746,7 @@ __device__ __forceinline__ bool direction_wave(const ChunkSrc& cur, const ChunkS
       for (int pv = 0; pv < 2; ++pv)
 #pragma unroll
         for (int cq = 0; cq < 4; ++cq) {
-          const f32x4_t x = *reinterpret_cast<const f32x4_t*>(unit_ptr(partner, pv * 4 + cq, lane));
+          const f32x4_t x = *reinterpret_cast<const f32x4_t*>(unit_ptr(partner, kSendUnit + pv * 4 + cq, lane));
 #pragma unroll
           for (int m = 0; m < 4; ++m) O[pv][KEEP][4 * cq + m] += x[m];
         }
@@ -953,7 +956,7 @@ __global__ __launch_bounds__(512) void gla_mfma_kernel(const uint16_t* __restric
       lds_barrier();  // (A)
       const bool refused = __builtin_amdgcn_readfirstlane(*veto) != 0;
       if (!refused) {  // a refused segment leaves after barrier A
-        lds_barrier();
+        if (MODE != kModeSlab) lds_barrier();  // (B: not in the fp16 variant of whole slabs)
         lds_barrier();
       }
       lds_barrier();  // (D)
