@@ -904,7 +904,12 @@ __device__ __forceinline__ int wave_loop(const uint16_t* q, const uint16_t* k, c
     const bool strict = MODE == kModeStateDual && item >= geo.dual_first;
     const bool ok =
         direction_wave<FWD, MODE, NG, F16, GATE>(cur, nxt, dst, c, lane, lds, oscale, bidir, state, pf, gate, strict);
-    lds_barrier();  // (D) the next item reuses the LDS regions
+    // (D) the next item reuses the LDS regions.  Not needed after an fp16 slab without the fused gate: what a wave
+    // writes before the next barrier A is its own (k~ scratch, anchors, contribution fragments: read by others only
+    // between A and C of the same slab), and the output half it sends after the next A was read by its partner
+    // before that wave could reach the next A.  (Measured: -2.0 us on the Dk = 32 slab shape, +0.7 us at Dk = 64,
+    // where the waves that run ahead take issue slots from the late ones' stores: dropped for Dk = 32 only.)
+    if (!(MODE == kModeSlab && F16 && !GATE && NG == 2 && ok)) lds_barrier();
     if (F16 && !ok) break;  // this item again, and all that follow, with split-bf16 scores
     cur = nxt;
     dst = dst_next;
@@ -959,7 +964,7 @@ __global__ __launch_bounds__(512) void gla_mfma_kernel(const uint16_t* __restric
         if (MODE != kModeSlab) lds_barrier();  // (B: not in the fp16 variant of whole slabs)
         lds_barrier();
       }
-      lds_barrier();  // (D)
+      if (MODE != kModeSlab || NG != 2 || refused) lds_barrier();  // (D: only behind a refused segment for Dk = 32 fp16 slabs)
       if (refused) break;
     }
     for (; item < geo.nitems; item += gridDim.x) {
