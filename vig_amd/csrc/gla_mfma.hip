@@ -51,6 +51,12 @@ namespace {
 // fp16 score operands are used while |G_end|/2 * log2(e) <= this for every channel of the chunk: the scaled
 // operands then stay within 2^6 of the inputs' magnitudes (fp16 holds |x| < 65504 and full precision above 6e-5).
 constexpr float kFastHalfRange = 6.0f;
+// bf16 / fp16 elements per row of a wave's k~ scratch.  Dk = 64: 128-byte rows padded to 144 (conflict-free 16-byte
+// writes), 9 KB, i.e. reaching into unit 8 of the region.  Dk = 32: 64-byte rows padded to 80 (eight lanes' writes
+// still cover all 32 banks once), 5 KB: inside the lower half, as the Dk = 32 slabs without barrier D need it (their
+// unit 8 carries an output half that the partner may still be reading when the next slab's scratch is written).
+template <int NG>
+constexpr int kFwdKtStride = NG == 4 ? kKtStride : 40;
 constexpr int kRegionBytes = 16 * 1024;      // per wave: k~ scratch, then published U / state fragments / output half
 constexpr int kLdsDvec = 8 * kRegionBytes;   // per wave: 64 chunk decays exp(G_end)
 constexpr int kLdsGend = kLdsDvec + 8 * 64 * 4;  // per wave: 64 anchors G_end * log2(e), laid out [h][p][16]
@@ -343,7 +349,7 @@ __device__ __forceinline__ bool tile_phase(const ChunkSrc& cur, const Prefetch<N
     {
       u32x4_t qa[NG];
       make_pair16<OUT, NG, MODE == kModeSlab>(pf.rawq, pf.rawk, G[TA], gend2, qa, ka, qkeep[TA]);
-      store_kt<NG>(kt, 32 * TA + r, h, ka);
+      store_kt<NG, kFwdKtStride<NG>>(kt, 32 * TA + r, h, ka);
       VIG_PHASE();
       if (!EARLY) fetch_second();
       set_vfrag(pf.vD, 2 * TA);
@@ -357,7 +363,7 @@ __device__ __forceinline__ bool tile_phase(const ChunkSrc& cur, const Prefetch<N
     }
     u32x4_t kb[NG];
     make_pair16<OUT, NG, MODE == kModeSlab>(rawq, rawk, G[TB], gend2, qb, kb, qkeep[TB]);
-    store_kt<NG>(kt, 32 * TB + r, h, kb);
+    store_kt<NG, kFwdKtStride<NG>>(kt, 32 * TB + r, h, kb);
     if (OUT) apply_scores<0, true>(score_tile16<NG>(ka, qb), TA, r, h, vfrag, O[0][TB], O[1][TB]);
     VIG_PHASE();
     set_vfrag(vDb, 2 * TB);
@@ -373,7 +379,7 @@ __device__ __forceinline__ bool tile_phase(const ChunkSrc& cur, const Prefetch<N
       fetch_second();
       set_vfrag(pf.vD, 2 * TA);
       if (OUT) apply_scores<MASK>(score_tile(ka, qa), TA, r, h, vfrag, O[0][TA], O[1][TA]);
-      store_kt<NG>(kt, 32 * TA + r, h, ka.h);
+      store_kt<NG, kFwdKtStride<NG>>(kt, 32 * TA + r, h, ka.h);
       if (OUT) {
 #pragma unroll
         for (int ks = 0; ks < NG; ++ks) qkeep[TA][ks] = qa.h[ks];
@@ -390,7 +396,7 @@ __device__ __forceinline__ bool tile_phase(const ChunkSrc& cur, const Prefetch<N
       make_half<false, NG>(rawk, G[TB], gend2, kb);
       set_vfrag(vDb, 2 * TB);
       if (OUT) apply_scores<MASK>(score_tile(kb, qb), TB, r, h, vfrag, O[0][TB], O[1][TB]);
-      store_kt<NG>(kt, 32 * TB + r, h, kb.h);
+      store_kt<NG, kFwdKtStride<NG>>(kt, 32 * TB + r, h, kb.h);
     }
     if (OUT) {
 #pragma unroll
@@ -530,7 +536,7 @@ __device__ __forceinline__ bool direction_wave(const ChunkSrc& cur, const ChunkS
 #pragma unroll
     for (int t = 0; t < 4; ++t) {
       u32x4_t ktf[2];
-      load_tfrag_lds<NG>(kt, t, r, h, ktf);
+      load_tfrag_lds<NG, kFwdKtStride<NG>>(kt, t, r, h, ktf);
 #pragma unroll
       for (int pk = 0; pk < 2; ++pk)
 #pragma unroll

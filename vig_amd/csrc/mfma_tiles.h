@@ -101,14 +101,14 @@ __device__ __forceinline__ void issue_raw_tile(rsrc_t rows, int it, int r, int h
 }
 
 // one k-step of transposed fragments from the wave's k~ scratch in LDS
-template <int NG>
+template <int NG, int STRIDE = kKtStride>
 __device__ __forceinline__ void load_tfrag_lds(const uint16_t* kt, int t, int r, int h, u32x4_t (&frag)[2]) {
   const bool row_ok = row_has_channel<NG>(r);
   const int c2 = row_ok ? 2 * cpair<NG>(r) : 0;
   uint32_t D[8];
 #pragma unroll
   for (int e = 0; e < 8; ++e) {
-    const uint32_t d = *reinterpret_cast<const uint32_t*>(kt + jmap(t, h, e) * kKtStride + c2);
+    const uint32_t d = *reinterpret_cast<const uint32_t*>(kt + jmap(t, h, e) * STRIDE + c2);
     D[e] = (NG == 4 || row_ok) ? d : 0u;
   }
 #pragma unroll
@@ -134,10 +134,10 @@ __device__ __forceinline__ u32x4_t tri_frag(int t, int it, int r, int h) {
   return f;
 }
 
-template <int NG>
+template <int NG, int STRIDE = kKtStride>
 __device__ __forceinline__ void store_kt(uint16_t* kt, int row, int h, const u32x4_t (&kh)[NG]) {
 #pragma unroll
-  for (int g = 0; g < NG; ++g) *reinterpret_cast<u32x4_t*>(kt + row * kKtStride + 8 * NG * h + 8 * g) = kh[g];
+  for (int g = 0; g < NG; ++g) *reinterpret_cast<u32x4_t*>(kt + row * STRIDE + 8 * NG * h + 8 * g) = kh[g];
 }
 
 
