@@ -414,20 +414,22 @@ struct GateCtx {
   int gw, gh;      // token grid: gw columns, gh rows, gw * gh = L
   int t0, nvalid;  // first token of this wave's chunk in the slab and its number of rows
 };
-// The rounded outputs of the slab are staged as a zero-padded (gh+2) x (gw+2) grid of 128-byte cells in the upper
-// halves of the LDS regions (free after barrier B).  A padded row never straddles two regions: each upper half takes
-// rph = 64 / (gw+2) whole rows, so the three taps of a stencil row are at constant offsets from the first.
+// The rounded outputs of the slab are staged as a zero-padded (gh+2) x (gw+2) grid of 128-byte cells in one half of
+// every LDS region (the half that is dead by then: the lower one, behind the fp16 variant's contributions, the upper
+// one otherwise).  A padded row never straddles two regions: each half takes rph = 64 / (gw+2) whole rows, so the
+// three taps of a stencil row are at constant offsets from the first.
 constexpr int kGateCellsPerRegion = 64;
 struct GateLayout {
-  int pw, rph;
+  int pw, rph, half;  // half: byte offset of the staging half inside a region
   float inv_rph;
-  __device__ __forceinline__ GateLayout(int gw) : pw(gw + 2), rph(kGateCellsPerRegion / (gw + 2)) {
+  __device__ __forceinline__ GateLayout(int gw, int half_offset)
+      : pw(gw + 2), rph(kGateCellsPerRegion / (gw + 2)), half(half_offset) {
     inv_rph = 1.0f / (float)rph;
   }
   // byte offset in LDS of padded cell (py, 0); exact for py < 2^20
   __device__ __forceinline__ int row(int py) const {
     const int reg = (int)(((float)py + 0.5f) * inv_rph);
-    return reg * kRegionBytes + kRegionBytes / 2 + __mul24(py - __mul24(reg, rph), pw * 128);  // (24-bit: full rate)
+    return reg * kRegionBytes + half + __mul24(py - __mul24(reg, rph), pw * 128);  // (24-bit: full rate)
   }
 };
 
@@ -716,10 +718,10 @@ __device__ __forceinline__ bool direction_wave(const ChunkSrc& cur, const ChunkS
       }
     }
   }
-  // (whole slabs on fp16 operands without the fused gate send their output halves through the upper halves of the
-  // regions, which nothing else uses there: the published contributions stay readable and barrier B is not needed)
-  constexpr int kSendUnit = DIRECT && !GATE ? 8 : 0;
-  if (!(DIRECT && !GATE)) lds_barrier();  // (B) incoming-state fragments of every chunk visible
+  // (whole slabs on fp16 operands send their output halves through the upper halves of the regions, which nothing
+  // else uses there: the published contributions stay readable and barrier B is not needed)
+  constexpr int kSendUnit = DIRECT ? 8 : 0;
+  if (!DIRECT) lds_barrier();  // (B) incoming-state fragments of every chunk visible
   if (OUT) {
     // ---- O^T += (exp(G_end) * S_in) q~hi  for every chunk that has an incoming state ----
     if (!DIRECT && (MODE == kModeChain || (FWD ? (c > 0) : (c < 3)))) {
@@ -759,7 +761,9 @@ __device__ __forceinline__ bool direction_wave(const ChunkSrc& cur, const ChunkS
     }
     if (GATE) {
       // (needs both directions: every wave owns the 32-row tile KEEP of its chunk)
-      const GateLayout lay(gate.gw);
+      // (fp16 variant: the output halves travelled through the upper region halves, the cells go to the lower ones,
+      // where the contributions are dead after barrier C; otherwise the other way round)
+      const GateLayout lay(gate.gw, DIRECT ? 0 : kRegionBytes / 2);
       const float inv_w = 1.0f / (float)gate.gw;
       {
         const int row = 32 * KEEP + r;
