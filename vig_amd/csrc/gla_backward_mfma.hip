@@ -17,8 +17,10 @@
 // cores in the register layout that feeds the next product directly (mfma_tiles.h), operands with tokens in the
 // contraction slots are read from the LDS rows as dwords.  The two directions take turns in LDS; a tile that is heavy
 // in one direction is light in the other, so over both every wave does the same amount of work.  dg needs a running
-// sum over tokens: the tile's q dq - k dk goes through LDS, lane = channel scans its 32 tokens, tile totals are
-// exchanged.  Loads of the next direction (or slab) are issued during that scan, the one phase with registers to spare.
+// sum over tokens: inside the tile the lanes (= tokens) add up q dq - k dk by lane shifts, the tile totals are
+// exchanged through LDS.  Loads of the next direction (or slab) are issued before that exchange, when the accumulators
+// are dead.  Three barriers per direction: gate totals, staged q~ / k~, totals of q dq - k dk; the last one also tells
+// that nobody reads this direction's staged rows any more.
 //
 // Slabs whose gate totals exceed the anchor's range (|G_total| / 2 * log2(e) > 60 in some channel) are not computed
 // here: the workgroup raises the slab's flag and the token-recurrent kernel, launched afterwards with that flag
@@ -41,8 +43,6 @@ constexpr int kBwdLdsTot = 4 * kBwdMatBytes;           // [8][64] f32: gate tota
 constexpr int kBwdLdsOff = kBwdLdsTot + 8 * 64 * 4;    // [8][64] f32: per wave, (prefix - anchor) of its tile
 constexpr int kBwdLdsDgTot = kBwdLdsOff + 8 * 64 * 4;  // [8][64] f32: totals of q dq - k dk of the tiles
 constexpr int kBwdLdsTotal = kBwdLdsDgTot + 8 * 64 * 4;
-constexpr int kXStride = 68;  // floats per token row of the dg scratch (272 B: conflict-free 16-byte writes)
-static_assert(8 * 32 * kXStride * 4 <= 2 * kBwdMatBytes, "dg scratch overlays the q~ and k~ matrices");
 constexpr float kBwdHalfRange = 60.0f;
 
 
@@ -72,6 +72,23 @@ __device__ __forceinline__ void mask_diag(f32x16_t& T, int r, int h, bool diag) 
     const bool keep = !diag || (FWD ? (j <= i) : (j >= i));
     T[c] = keep ? T[c] : 0.f;
   }
+}
+
+// Inclusive running sum over the 32 tokens of a lane half (lanes 32h .. 32h + 31, in lane order): four shifted adds
+// inside the rows of 16 lanes (lanes shifted in from outside a row read zero), then lane 15 of the lower row added to
+// every lane of the upper one.
+template <int CTRL>
+__device__ __forceinline__ float row_shifted(float v) {
+  return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xf, 0xf, true));
+}
+__device__ __forceinline__ float half_prefix_sum(float x) {
+  x += row_shifted<0x111>(x);  // row_shr:1
+  x += row_shifted<0x112>(x);  // row_shr:2
+  x += row_shifted<0x114>(x);  // row_shr:4
+  x += row_shifted<0x118>(x);  // row_shr:8
+  // row_bcast:15 into rows 1 and 3 (row mask 0b1010); rows 0 and 2 keep the zero
+  x += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), 0x142, 0xa, 0xf, false));
+  return x;
 }
 
 struct BwdSlab {
@@ -173,7 +190,7 @@ __device__ __forceinline__ bool bwd_direction(const BwdSlab& sl, int L, int ntil
       tot[w * 64 + ch + 1] = G[1][c];
     }
   }
-  lds_barrier();  // (1) tile totals (and v, do rows) visible; the previous direction's scratch is dead
+  lds_barrier();  // (1) tile totals (and v, do rows) visible
   // lane = channel: gates before this tile in walking order, minus the anchor (half the slab total)
   bool out_of_range;
   {
@@ -382,53 +399,58 @@ __device__ __forceinline__ bool bwd_direction(const BwdSlab& sl, int L, int ntil
       }
     }
   }
-  lds_barrier();  // (3) nobody reads q~, k~ any more: their space becomes the dg scratch
+  // ---- dg: the running sum of X over the tokens the gate acts on.  Inside the tile by lane shifts (lane = token),
+  // across tiles through the tile totals in LDS: walking forward a token takes everything from itself to the end,
+  // i.e. the totals of this and the later tiles minus what lies before it in the tile. ----
   {
-    float* xs = reinterpret_cast<float*>(lds + kBwdLdsQ) + w * 32 * kXStride;
+    float pfx[2][4 * NG];
 #pragma unroll
-    for (int gq = 0; gq < NG; ++gq) {
-      const f32x4_t a = {X[0][4 * gq], X[1][4 * gq], X[0][4 * gq + 1], X[1][4 * gq + 1]};
-      const f32x4_t b = {X[0][4 * gq + 2], X[1][4 * gq + 2], X[0][4 * gq + 3], X[1][4 * gq + 3]};
-      *reinterpret_cast<f32x4_t*>(xs + r * kXStride + HC * h + 8 * gq) = a;
-      *reinterpret_cast<f32x4_t*>(xs + r * kXStride + HC * h + 8 * gq + 4) = b;
+    for (int p = 0; p < 2; ++p)
+#pragma unroll
+      for (int c = 0; c < 4 * NG; ++c) pfx[p][c] = half_prefix_sum(X[p][c]);
+    if (r == 31) {
+#pragma unroll
+      for (int c = 0; c < 4 * NG; ++c) {
+        const int ch = HC * h + 8 * (c >> 2) + 2 * (c & 3);
+        dgtot[w * 64 + ch] = pfx[0][c];
+        dgtot[w * 64 + ch + 1] = pfx[1][c];
+      }
     }
-    wave_lds_sync();
-    // the next direction's loads travel while this one scans and stores
+    // the next direction's loads travel while this one finishes
     issue_bwd_loads<LAST, NG>(nxt, w, r, h, ld);
-    // lane = channel (lanes past Dk idle along): the tile's total, then (with the totals of the tiles behind it) the
-    // running sum over its tokens against the walking order, written back in place
-    const int cl = lane < DK ? lane : 0;
-    float acc = 0.f;
+    lds_barrier();  // (4) tile totals of X visible; nobody reads q~, k~, v, do of this direction any more
+    {
+      const int cl = lane < DK ? lane : 0;
+      float run = 0.f;
 #pragma unroll
-    for (int t = 0; t < 32; ++t) acc += xs[t * kXStride + cl];
-    if (lane < DK) dgtot[w * 64 + lane] = acc;
-    lds_barrier();  // (4) tile totals of X visible
-    float run = 0.f;
-#pragma unroll
-    for (int t = 0; t < kBwdTiles; ++t) {
-      const float y = dgtot[t * 64 + cl];
-      run += (FWD ? (t > w) : (t < w)) ? y : 0.f;
-    }
-    if (SEG) {
-      const float* cy = sl.carry + (FWD ? 0 : 128) + cl;
-      run += s * (cy[0] + cy[64]);
-    }
-#pragma unroll
-    for (int i = 0; i < 32; ++i) {
-      const int t = FWD ? 31 - i : i;
-      run += xs[t * kXStride + cl];
-      if (lane < DK) xs[t * kXStride + lane] = run;
+      for (int t = 0; t < kBwdTiles; ++t) {
+        const float y = dgtot[t * 64 + cl];
+        run += (FWD ? (t >= w) : (t < w)) ? y : 0.f;
+      }
+      if (SEG) {
+        const float* cy = sl.carry + (FWD ? 0 : 128) + cl;
+        run += s * (cy[0] + cy[64]);
+      }
+      offs[lane] = run;
     }
     wave_lds_sync();
-    // back to lane = token: 16-byte stores of the gate gradient
     uint16_t* dg = FWD ? sl.dgf : sl.dgb;
     const rsrc_t rdg = chunk_rsrc(dg + tk, rows, 2 * DK);
 #pragma unroll
     for (int gq = 0; gq < NG; ++gq) {
-      const f32x4_t a = *reinterpret_cast<const f32x4_t*>(xs + r * kXStride + HC * h + 8 * gq);
-      const f32x4_t b = *reinterpret_cast<const f32x4_t*>(xs + r * kXStride + HC * h + 8 * gq + 4);
-      const u32x4_t out = {pack_bf16x2(a[0], a[1]), pack_bf16x2(a[2], a[3]), pack_bf16x2(b[0], b[1]),
-                           pack_bf16x2(b[2], b[3])};
+      const f32x4_t o0 = *reinterpret_cast<const f32x4_t*>(offs + HC * h + 8 * gq);
+      const f32x4_t o1 = *reinterpret_cast<const f32x4_t*>(offs + HC * h + 8 * gq + 4);
+      const float o8[8] = {o0[0], o0[1], o0[2], o0[3], o1[0], o1[1], o1[2], o1[3]};
+      u32x4_t out;
+#pragma unroll
+      for (int m = 0; m < 4; ++m) {
+        const int c = 4 * gq + m;
+        float d[2];
+#pragma unroll
+        for (int p = 0; p < 2; ++p)
+          d[p] = FWD ? o8[2 * m + p] - (pfx[p][c] - X[p][c]) : o8[2 * m + p] + pfx[p][c];
+        out[m] = pack_bf16x2(d[0], d[1]);
+      }
       __builtin_amdgcn_raw_buffer_store_b128(out, rdg, (unsigned)r * (2u * DK) + (2u * HC) * h + 16u * gq, 0, 0);
     }
   }
@@ -493,7 +515,6 @@ __global__ __launch_bounds__(512) void gla_backward_mfma_kernel(
     if constexpr (BIDIR) {
       ok = bwd_direction<true, true, false, NG, SEG>(sl, sl.L, ntiles, w, lane, lds, s, dvacc, keepq, keepk, ld, second);
       if (ok) {
-        lds_barrier();  // (5) the dg scratch of direction 1 is dead before q~, k~ of direction 2 are staged
         ok = bwd_direction<false, false, true, NG, SEG>(sl, sl.L, ntiles, w, lane, lds, s, dvacc, keepq, keepk, ld,
                                                         next_first);
       }
@@ -502,13 +523,15 @@ __global__ __launch_bounds__(512) void gla_backward_mfma_kernel(
                                                     next_first);
     }
     // a direction that left early has not issued the loads of the slab that follows
-    if (!ok) issue_bwd_loads<true, NG>(next_first, w, r, h, ld);
+    if (!ok) {
+      issue_bwd_loads<true, NG>(next_first, w, r, h, ld);
+      lds_barrier();  // a wave that has left must not touch the gate totals the others still read
+    }
     if (SEG) {  // one flag per sequence, cleared by the segment scan: any segment out of range gives the sequence away
       if (tid == 0 && !ok) flags[slab / sg.nseg] = 1;
     } else if (tid == 0) {
       flags[slab] = ok ? 0 : 1;
     }
-    lds_barrier();  // the next slab restages everything
   }
 }
 
