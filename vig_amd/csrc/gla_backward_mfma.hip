@@ -19,8 +19,9 @@
 // in one direction is light in the other, so over both every wave does the same amount of work.  dg needs a running
 // sum over tokens: inside the tile the lanes (= tokens) add up q dq - k dk by lane shifts, the tile totals are
 // exchanged through LDS.  Loads of the next direction (or slab) are issued before that exchange, when the accumulators
-// are dead.  Three barriers per direction: gate totals, staged q~ / k~, totals of q dq - k dk; the last one also tells
-// that nobody reads this direction's staged rows any more.
+// are dead (its gates a phase earlier), and its cumulative gates and their tile totals are prepared there as well.
+// Two barriers per direction: staged q~ / k~, and the totals of q dq - k dk together with the next direction's gate
+// totals; the second also tells that nobody reads this direction's staged rows any more.
 //
 // Slabs whose gate totals exceed the anchor's range (|G_total| / 2 * log2(e) > 60 in some channel) are not computed
 // here: the workgroup raises the slab's flag and the token-recurrent kernel, launched afterwards with that flag
@@ -74,21 +75,30 @@ __device__ __forceinline__ void mask_diag(f32x16_t& T, int r, int h, bool diag) 
   }
 }
 
-// Inclusive running sum over the 32 tokens of a lane half (lanes 32h .. 32h + 31, in lane order): four shifted adds
-// inside the rows of 16 lanes (lanes shifted in from outside a row read zero), then lane 15 of the lower row added to
-// every lane of the upper one.
+// Inclusive running sums over the 32 tokens of a lane half (lanes 32h .. 32h + 31, in lane order) for N values at
+// once: four shifted adds inside the rows of 16 lanes (lanes shifted in from outside a row read zero), then lane 15 of
+// the lower row added to every lane of the upper one.  Step by step over all values, so that consecutive lane-shift
+// instructions never wait for each other's results.
 template <int CTRL>
 __device__ __forceinline__ float row_shifted(float v) {
   return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xf, 0xf, true));
 }
-__device__ __forceinline__ float half_prefix_sum(float x) {
-  x += row_shifted<0x111>(x);  // row_shr:1
-  x += row_shifted<0x112>(x);  // row_shr:2
-  x += row_shifted<0x114>(x);  // row_shr:4
-  x += row_shifted<0x118>(x);  // row_shr:8
-  // row_bcast:15 into rows 1 and 3 (row mask 0b1010); rows 0 and 2 keep the zero
-  x += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), 0x142, 0xa, 0xf, false));
-  return x;
+template <int CTRL, int N>
+__device__ __forceinline__ void add_row_shifted(float (&x)[N]) {
+#pragma unroll
+  for (int i = 0; i < N; ++i) x[i] += row_shifted<CTRL>(x[i]);
+  __builtin_amdgcn_sched_barrier(0);
+}
+template <int N>
+__device__ __forceinline__ void half_prefix_sums(float (&x)[N]) {
+  __builtin_amdgcn_sched_barrier(0);
+  add_row_shifted<0x111>(x);  // row_shr:1
+  add_row_shifted<0x112>(x);  // row_shr:2
+  add_row_shifted<0x114>(x);  // row_shr:4
+  add_row_shifted<0x118>(x);  // row_shr:8
+#pragma unroll
+  for (int i = 0; i < N; ++i)  // row_bcast:15 into rows 1 and 3 (row mask 0b1010); rows 0 and 2 keep the zero
+    x[i] += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x[i]), 0x142, 0xa, 0xf, false));
 }
 
 struct BwdSlab {
@@ -113,17 +123,48 @@ struct BwdNext {  // the direction whose loads are issued while this one finishe
   const uint16_t* g;
   int L;  // 0: nothing follows (empty descriptors, no memory traffic)
 };
-template <bool WITH_VDO, int NG>
-__device__ __forceinline__ void issue_bwd_loads(const BwdNext& n, int w, int r, int h, BwdLoads<NG>& ld) {
+template <int NG>
+__device__ __forceinline__ void issue_bwd_gate_loads(const BwdNext& n, int w, int r, int h, BwdLoads<NG>& ld) {
   constexpr int DK = 16 * NG;
   const int rows = __builtin_amdgcn_readfirstlane(min(max(n.L - 32 * w, 0), 32));  // (scalar: descriptors stay in SGPRs)
+  issue_tdwords<0, 2, NG>(chunk_rsrc(n.g + (size_t)32 * w * DK, rows, 2 * DK), r, h, ld.gD);
+}
+template <bool WITH_VDO, int NG>
+__device__ __forceinline__ void issue_bwd_row_loads(const BwdNext& n, int w, int r, int h, BwdLoads<NG>& ld) {
+  constexpr int DK = 16 * NG;
+  const int rows = __builtin_amdgcn_readfirstlane(min(max(n.L - 32 * w, 0), 32));
   const size_t tk = (size_t)32 * w * DK, tv = (size_t)32 * w * 64;
-  issue_tdwords<0, 2, NG>(chunk_rsrc(n.g + tk, rows, 2 * DK), r, h, ld.gD);
   issue_raw_tile<NG>(chunk_rsrc(n.sl.q + tk, rows, 2 * DK), 0, r, h, ld.rawq);
   issue_raw_tile<NG>(chunk_rsrc(n.sl.k + tk, rows, 2 * DK), 0, r, h, ld.rawk);
   if (WITH_VDO) {
     issue_raw_tile<4>(chunk_rsrc(n.sl.v + tv, rows, 128), 0, r, h, ld.rawv);
     issue_raw_tile<4>(chunk_rsrc(n.sl.d_o + tv, rows, 128), 0, r, h, ld.rawd);
+  }
+}
+
+// Tile-local cumulative gates of the direction whose gate dwords have arrived: G^T = g^T T, lane = token, registers =
+// channels HC*h + 8g + 2m + p; the tile total (at the tile's last token in walking order) goes to `tot`.
+template <bool FWD, int NG>
+__device__ __forceinline__ void bwd_cumulate_gates(const BwdLoads<NG>& ld, int w, int lane, char* lds, f32x16_t (&G)[2]) {
+  constexpr int HC = 8 * NG;
+  const int r = lane & 31, h = lane >> 5;
+  float* tot = reinterpret_cast<float*>(lds + kBwdLdsTot);
+  u32x4_t gfrag[2][2];
+  finish_tfrags<2>(ld.gD, gfrag);  // (rows that carry no channel, NG = 2, hold zeros)
+  const u32x4_t tri0 = tri_frag<FWD>(0, 0, r, h), tri1 = tri_frag<FWD>(1, 0, r, h);
+#pragma unroll
+  for (int p = 0; p < 2; ++p) {
+    f32x16_t z = {0.f};
+    z = mfma(gfrag[0][p], tri0, z);
+    G[p] = mfma(gfrag[1][p], tri1, z);
+  }
+  if (r == (FWD ? 31 : 0)) {
+#pragma unroll
+    for (int c = 0; c < 4 * NG; ++c) {
+      const int ch = HC * h + 8 * (c >> 2) + 2 * (c & 3);
+      tot[w * 64 + ch] = G[0][c];
+      tot[w * 64 + ch + 1] = G[1][c];
+    }
   }
 }
 
@@ -140,7 +181,7 @@ __device__ __forceinline__ void issue_bwd_loads(const BwdNext& n, int w, int r, 
 template <bool FWD, bool FIRST, bool LAST, int NG, bool SEG>
 __device__ __forceinline__ bool bwd_direction(const BwdSlab& sl, int L, int ntiles, int w, int lane, char* lds,
                                               float s, f32x16_t (&dv)[2], u32x4_t (&keepq)[NG], u32x4_t (&keepk)[NG],
-                                              BwdLoads<NG>& ld, const BwdNext& nxt) {
+                                              BwdLoads<NG>& ld, const BwdNext& nxt, f32x16_t (&G)[2]) {
   // where the first direction's dq, dk (bf16) wait for the second: in registers when the kernel has them to spare
   // (Dk = 32), else parked in the output tensors
   constexpr bool kKeepInRegs = NG == 2;
@@ -159,7 +200,8 @@ __device__ __forceinline__ bool bwd_direction(const BwdSlab& sl, int L, int ntil
   const int rows = __builtin_amdgcn_readfirstlane(min(max(L - 32 * w, 0), 32));  // valid tokens of this wave's tile
   const size_t tk = (size_t)32 * w * DK, tv = (size_t)32 * w * 64;
 
-  // ---- this tile's loads were issued a phase ago; v and do rows go to LDS once per slab ----
+  // ---- this tile's loads were issued a phase ago; v and do rows go to LDS once per slab (nobody reads the previous
+  // slab's any more; the next barrier makes them visible) ----
   if (stage_vdo) {
     store_kt<4>(V, 32 * w + r, h, ld.rawv);
     store_kt<4>(DO, 32 * w + r, h, ld.rawd);
@@ -168,29 +210,8 @@ __device__ __forceinline__ bool bwd_direction(const BwdSlab& sl, int L, int ntil
 #pragma unroll
   for (int i = 0; i < NG; ++i) rawq[i] = ld.rawq[i], rawk[i] = ld.rawk[i];
 
-  // ---- tile-local cumulative gates: G^T = g^T T, lane = token, registers = channels HC*h + 8g + 2m + p ----
-  f32x16_t G[2];
-  {
-    u32x4_t gfrag[2][2];
-    finish_tfrags<2>(ld.gD, gfrag);  // (rows that carry no channel, NG = 2, hold zeros)
-    const u32x4_t tri0 = tri_frag<FWD>(0, 0, r, h), tri1 = tri_frag<FWD>(1, 0, r, h);
-#pragma unroll
-    for (int p = 0; p < 2; ++p) {
-      f32x16_t z = {0.f};
-      z = mfma(gfrag[0][p], tri0, z);
-      G[p] = mfma(gfrag[1][p], tri1, z);
-    }
-  }
-  // the tile total sits at its last token in walking order
-  if (r == (FWD ? 31 : 0)) {
-#pragma unroll
-    for (int c = 0; c < 4 * NG; ++c) {
-      const int ch = HC * h + 8 * (c >> 2) + 2 * (c & 3);
-      tot[w * 64 + ch] = G[0][c];
-      tot[w * 64 + ch + 1] = G[1][c];
-    }
-  }
-  lds_barrier();  // (1) tile totals (and v, do rows) visible
+  // ---- the cumulative gates G of this tile and every tile's total were left by the previous direction's tail (or
+  // the kernel's head), one barrier ago ----
   // lane = channel: gates before this tile in walking order, minus the anchor (half the slab total)
   bool out_of_range;
   {
@@ -291,40 +312,73 @@ __device__ __forceinline__ bool bwd_direction(const BwdSlab& sl, int L, int ntil
       prevk[gq] = __builtin_amdgcn_raw_buffer_load_b128(okk, off, 0, 0);
     }
   }
-  // ---- dv, then dk of tile w: over the query tiles I the direction keeps (two loops: fewer live registers) ----
+  // ---- dv and dk of tile w: over the query tiles I the direction keeps.  Dk = 32 has the registers to do both in
+  // one loop: the two score tiles of a step are independent, so one's masks and packs run under the other's matrix
+  // instructions.  Dk = 64: two loops (fewer live registers). ----
   f32x16_t dkh[2] = {{0.f}, {0.f}};
   if (w < ntiles) {
     const int i0 = FWD ? w : 0, i1 = FWD ? ntiles - 1 : w;
+    if constexpr (NG == 2) {
 #pragma unroll 1
-    for (int I = i0; I <= i1; ++I) {
-      f32x16_t P = {0.f};  // rows i in I, columns j in tile w
+      for (int I = i0; I <= i1; ++I) {
+        f32x16_t P = {0.f}, A = {0.f};  // rows i in I, columns j in tile w
 #pragma unroll
-      for (int ks = 0; ks < NG; ++ks) P = mfma(row_frag(Q, 32 * I + r, ks, h), row_frag(K, 32 * w + r, ks, h), P);
-      mask_diag<FWD, true>(P, r, h, I == w);
-      u32x4_t pf[2];
-      tile_frags(P, pf);
+        for (int ks = 0; ks < NG; ++ks) P = mfma(row_frag(Q, 32 * I + r, ks, h), row_frag(K, 32 * w + r, ks, h), P);
 #pragma unroll
-      for (int t = 0; t < 2; ++t) {
-        u32x4_t df[2];
-        load_tfrag_lds<4>(DO + 32 * I * kKtStride, t, r, h, df);
-        dv[0] = mfma(df[0], pf[t], dv[0]);
-        dv[1] = mfma(df[1], pf[t], dv[1]);
+        for (int ks = 0; ks < 4; ++ks) A = mfma(row_frag(DO, 32 * I + r, ks, h), row_frag(V, 32 * w + r, ks, h), A);
+        mask_diag<FWD, true>(P, r, h, I == w);
+        u32x4_t pf[2];
+        tile_frags(P, pf);
+#pragma unroll
+        for (int t = 0; t < 2; ++t) {
+          u32x4_t df[2];
+          load_tfrag_lds<4>(DO + 32 * I * kKtStride, t, r, h, df);
+          dv[0] = mfma(df[0], pf[t], dv[0]);
+          dv[1] = mfma(df[1], pf[t], dv[1]);
+        }
+        mask_diag<FWD, true>(A, r, h, I == w);
+        u32x4_t af[2];
+        tile_frags(A, af);
+#pragma unroll
+        for (int t = 0; t < 2; ++t) {
+          u32x4_t qf[2];
+          load_tfrag_lds<NG>(Q + 32 * I * kKtStride, t, r, h, qf);
+          dkh[0] = mfma(qf[0], af[t], dkh[0]);
+          dkh[1] = mfma(qf[1], af[t], dkh[1]);
+        }
       }
-    }
+    } else {
 #pragma unroll 1
-    for (int I = i0; I <= i1; ++I) {
-      f32x16_t A = {0.f};
+      for (int I = i0; I <= i1; ++I) {
+        f32x16_t P = {0.f};  // rows i in I, columns j in tile w
 #pragma unroll
-      for (int ks = 0; ks < 4; ++ks) A = mfma(row_frag(DO, 32 * I + r, ks, h), row_frag(V, 32 * w + r, ks, h), A);
-      mask_diag<FWD, true>(A, r, h, I == w);
-      u32x4_t af[2];
-      tile_frags(A, af);
+        for (int ks = 0; ks < NG; ++ks) P = mfma(row_frag(Q, 32 * I + r, ks, h), row_frag(K, 32 * w + r, ks, h), P);
+        mask_diag<FWD, true>(P, r, h, I == w);
+        u32x4_t pf[2];
+        tile_frags(P, pf);
 #pragma unroll
-      for (int t = 0; t < 2; ++t) {
-        u32x4_t qf[2];
-        load_tfrag_lds<NG>(Q + 32 * I * kKtStride, t, r, h, qf);
-        dkh[0] = mfma(qf[0], af[t], dkh[0]);
-        dkh[1] = mfma(qf[1], af[t], dkh[1]);
+        for (int t = 0; t < 2; ++t) {
+          u32x4_t df[2];
+          load_tfrag_lds<4>(DO + 32 * I * kKtStride, t, r, h, df);
+          dv[0] = mfma(df[0], pf[t], dv[0]);
+          dv[1] = mfma(df[1], pf[t], dv[1]);
+        }
+      }
+#pragma unroll 1
+      for (int I = i0; I <= i1; ++I) {
+        f32x16_t A = {0.f};
+#pragma unroll
+        for (int ks = 0; ks < 4; ++ks) A = mfma(row_frag(DO, 32 * I + r, ks, h), row_frag(V, 32 * w + r, ks, h), A);
+        mask_diag<FWD, true>(A, r, h, I == w);
+        u32x4_t af[2];
+        tile_frags(A, af);
+#pragma unroll
+        for (int t = 0; t < 2; ++t) {
+          u32x4_t qf[2];
+          load_tfrag_lds<NG>(Q + 32 * I * kKtStride, t, r, h, qf);
+          dkh[0] = mfma(qf[0], af[t], dkh[0]);
+          dkh[1] = mfma(qf[1], af[t], dkh[1]);
+        }
       }
     }
     if (SEG) {  // the gradient of the state leaving the segment, against this tile's k~ rows (dv) and v rows (dk)
@@ -350,6 +404,7 @@ __device__ __forceinline__ bool bwd_direction(const BwdSlab& sl, int L, int ntil
         }
     }
   }
+  issue_bwd_gate_loads<NG>(nxt, w, r, h, ld);  // the next direction's gates travel under the rest of this one
   // ---- scale back; X = q dq - k dk = s (q~ dq^ - k~ dk^): the exponentials cancel, and the staged rows serve ----
   f32x16_t X[2];
   {
@@ -403,22 +458,25 @@ __device__ __forceinline__ bool bwd_direction(const BwdSlab& sl, int L, int ntil
   // across tiles through the tile totals in LDS: walking forward a token takes everything from itself to the end,
   // i.e. the totals of this and the later tiles minus what lies before it in the tile. ----
   {
-    float pfx[2][4 * NG];
+    float pfx[8 * NG];  // [p][c]
 #pragma unroll
     for (int p = 0; p < 2; ++p)
 #pragma unroll
-      for (int c = 0; c < 4 * NG; ++c) pfx[p][c] = half_prefix_sum(X[p][c]);
+      for (int c = 0; c < 4 * NG; ++c) pfx[4 * NG * p + c] = X[p][c];
+    half_prefix_sums(pfx);
     if (r == 31) {
 #pragma unroll
       for (int c = 0; c < 4 * NG; ++c) {
         const int ch = HC * h + 8 * (c >> 2) + 2 * (c & 3);
-        dgtot[w * 64 + ch] = pfx[0][c];
-        dgtot[w * 64 + ch + 1] = pfx[1][c];
+        dgtot[w * 64 + ch] = pfx[c];
+        dgtot[w * 64 + ch + 1] = pfx[4 * NG + c];
       }
     }
-    // the next direction's loads travel while this one finishes
-    issue_bwd_loads<LAST, NG>(nxt, w, r, h, ld);
-    lds_barrier();  // (4) tile totals of X visible; nobody reads q~, k~, v, do of this direction any more
+    // the next direction's rows travel while this one finishes; its cumulative gates and tile totals are prepared
+    // here, so that one barrier serves both exchanges
+    issue_bwd_row_loads<LAST, NG>(nxt, w, r, h, ld);
+    bwd_cumulate_gates<LAST, NG>(ld, w, lane, lds, G);
+    lds_barrier();  // (4) tile totals of X and of the next gates visible; nobody reads q~, k~, v, do of this direction
     {
       const int cl = lane < DK ? lane : 0;
       float run = 0.f;
@@ -448,7 +506,7 @@ __device__ __forceinline__ bool bwd_direction(const BwdSlab& sl, int L, int ntil
         float d[2];
 #pragma unroll
         for (int p = 0; p < 2; ++p)
-          d[p] = FWD ? o8[2 * m + p] - (pfx[p][c] - X[p][c]) : o8[2 * m + p] + pfx[p][c];
+          d[p] = FWD ? o8[2 * m + p] - (pfx[4 * NG * p + c] - X[p][c]) : o8[2 * m + p] + pfx[4 * NG * p + c];
         out[m] = pack_bf16x2(d[0], d[1]);
       }
       __builtin_amdgcn_raw_buffer_store_b128(out, rdg, (unsigned)r * (2u * DK) + (2u * HC) * h + 16u * gq, 0, 0);
@@ -499,9 +557,14 @@ __global__ __launch_bounds__(512) void gla_backward_mfma_kernel(
   };
   const int r = lane & 31, h = lane >> 5;
   BwdLoads<NG> ld;
+  f32x16_t G[2];  // cumulative gates of the direction about to run, prepared one barrier ahead of it
   if ((int)blockIdx.x < nslabs) {
     const BwdSlab s0 = slab_of(blockIdx.x);
-    issue_bwd_loads<true, NG>(BwdNext{s0, s0.gf, s0.L}, w, r, h, ld);
+    const BwdNext first{s0, s0.gf, s0.L};
+    issue_bwd_gate_loads<NG>(first, w, r, h, ld);
+    issue_bwd_row_loads<true, NG>(first, w, r, h, ld);
+    bwd_cumulate_gates<true, NG>(ld, w, lane, lds, G);
+    lds_barrier();
   }
   for (int slab = blockIdx.x; slab < nslabs; slab += gridDim.x) {
     const BwdSlab sl = slab_of(slab);
@@ -513,19 +576,22 @@ __global__ __launch_bounds__(512) void gla_backward_mfma_kernel(
     u32x4_t keepq[NG], keepk[NG];
     bool ok;
     if constexpr (BIDIR) {
-      ok = bwd_direction<true, true, false, NG, SEG>(sl, sl.L, ntiles, w, lane, lds, s, dvacc, keepq, keepk, ld, second);
+      ok = bwd_direction<true, true, false, NG, SEG>(sl, sl.L, ntiles, w, lane, lds, s, dvacc, keepq, keepk, ld, second, G);
       if (ok) {
         ok = bwd_direction<false, false, true, NG, SEG>(sl, sl.L, ntiles, w, lane, lds, s, dvacc, keepq, keepk, ld,
-                                                        next_first);
+                                                        next_first, G);
       }
     } else {  // the causal op: the forward direction alone, first and last at once
       ok = bwd_direction<true, true, true, NG, SEG>(sl, sl.L, ntiles, w, lane, lds, s, dvacc, keepq, keepk, ld,
-                                                    next_first);
+                                                    next_first, G);
     }
-    // a direction that left early has not issued the loads of the slab that follows
+    // a direction that left early has neither issued the loads of the slab that follows nor prepared its gates
     if (!ok) {
-      issue_bwd_loads<true, NG>(next_first, w, r, h, ld);
       lds_barrier();  // a wave that has left must not touch the gate totals the others still read
+      issue_bwd_gate_loads<NG>(next_first, w, r, h, ld);
+      issue_bwd_row_loads<true, NG>(next_first, w, r, h, ld);
+      bwd_cumulate_gates<true, NG>(ld, w, lane, lds, G);
+      lds_barrier();
     }
     if (SEG) {  // one flag per sequence, cleared by the segment scan: any segment out of range gives the sequence away
       if (tid == 0 && !ok) flags[slab / sg.nseg] = 1;
