@@ -263,21 +263,29 @@ __device__ __forceinline__ bool bwd_direction(const BwdSlab& sl, int L, int ntil
 #pragma unroll
     for (int ks = 0; ks < 4; ++ks) doB[ks] = row_frag(DO, 32 * w + r, ks, h);
     const int j0 = FWD ? 0 : w, j1 = FWD ? w : ntiles - 1;
+    // Two steps in flight: the score tile of the next key tile is on the matrix cores while this one is masked,
+    // packed and multiplied on (after the last tile the next one is that tile again, computed and dropped).
+    f32x16_t T = {0.f};  // A^T tile: rows j in J, columns i in tile w
+#pragma unroll
+    for (int ks = 0; ks < 4; ++ks) T = mfma(row_frag(V, 32 * j0 + r, ks, h), doB[ks], T);
 #pragma unroll 1
     for (int J = j0; J <= j1; ++J) {
-      f32x16_t T = {0.f};  // A^T tile: rows j in J, columns i in tile w
+      const int Jn = min(J + 1, j1);
+      u32x4_t kf[2][2];
 #pragma unroll
-      for (int ks = 0; ks < 4; ++ks) T = mfma(row_frag(V, 32 * J + r, ks, h), doB[ks], T);
+      for (int t = 0; t < 2; ++t) load_tfrag_lds<NG>(K + 32 * J * kKtStride, t, r, h, kf[t]);
+      f32x16_t Tn = {0.f};
+#pragma unroll
+      for (int ks = 0; ks < 4; ++ks) Tn = mfma(row_frag(V, 32 * Jn + r, ks, h), doB[ks], Tn);
       mask_diag<FWD, false>(T, r, h, J == w);
       u32x4_t f[2];
       tile_frags(T, f);
 #pragma unroll
       for (int t = 0; t < 2; ++t) {
-        u32x4_t kf[2];
-        load_tfrag_lds<NG>(K + 32 * J * kKtStride, t, r, h, kf);
-        dqh[0] = mfma(kf[0], f[t], dqh[0]);
-        dqh[1] = mfma(kf[1], f[t], dqh[1]);
+        dqh[0] = mfma(kf[t][0], f[t], dqh[0]);
+        dqh[1] = mfma(kf[t][1], f[t], dqh[1]);
       }
+      T = Tn;
     }
     if (SEG) {  // the state entering the segment: rows = the k channels of this lane's accumulator rows, over v
       const uint16_t* sp = sl.sp + (FWD ? 0 : kBwdStateElems);
