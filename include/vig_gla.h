@@ -79,6 +79,26 @@ int vig_gla_bidir_fwd(const void* q, const void* k, const void* v,
                       float scale, float out_scale,
                       int io_dtype, int gate_dtype, void* stream);
 
+/*
+ * vig_gla_bidir_fwd on q, k, v that are not plain [B, H, L, D] tensors: element (b, h, l, d) of q lies at
+ * q + b*q_strides[0] + h*q_strides[1] + l*q_strides[2] + d (likewise k, v; the channels of one (token, head) are
+ * contiguous).  For the column blocks of a projection output [B, L, H*(2*Dk + Dv)] read in place that is
+ * {L*row, Dk (or Dv), row} with row = H*(2*Dk + Dv), so no head-major copies of q, k, v are made.  g_fwd, g_bwd and o
+ * stay plain [B, H, L, D].  Strides are positive multiples of 8 elements (16-byte rows), the token stride at most 2^20.
+ * Built for the matrix-core slab kernel only: bf16 tensors and gates, Dk in {32, 64}, Dv = 64, L <= 256 (no workspace);
+ * VIG_ENOTSUP otherwise.  Same arithmetic and results as vig_gla_bidir_fwd on contiguous copies.
+ *
+ * Replaces: the stride arguments of the reference's kernels (s_qk_h, s_qk_t, s_qk_d, s_vo_h, s_vo_t, s_vo_d,
+ * flash-linear-attention/fla/ops/gla/chunk_fuse.py:23-38), which its wrapper feeds with contiguous copies
+ * (@contiguous, chunk_fuse.py:315) of the head-split views made at classification/models/vig.py:402-406 and :436-438.
+ */
+int vig_gla_bidir_fwd_strided(const void* q, const void* k, const void* v,
+                              const void* g_fwd, const void* g_bwd, void* o,
+                              int B, int H, int L, int Dk, int Dv,
+                              const long long* q_strides, const long long* k_strides, const long long* v_strides,
+                              float scale, float out_scale,
+                              int io_dtype, int gate_dtype, void* stream);
+
 /* Workspace that is enough for every gate dtype and for one or two directions (the largest over the kernels the
  * call may dispatch to for this shape and io_dtype). */
 size_t vig_gla_bidir_fwd_workspace(int B, int H, int L, int Dk, int Dv, int io_dtype);

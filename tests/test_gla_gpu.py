@@ -260,6 +260,56 @@ def test_bf16_hiervig_head_shape_on_the_matrix_cores(B, H, L):
     assert not torch.equal(got, exact)  # (the two kernels round differently: proves the padded path ran)
 
 
+@pytest.mark.parametrize("B,H,L,Dk,both", [(3, 6, 196, 32, True), (2, 3, 196, 64, True), (2, 2, 37, 64, True),
+                                           (1, 4, 256, 32, False), (130, 2, 100, 64, True)])
+def test_q_k_v_read_in_place_from_projection_rows(B, H, L, Dk, both):
+    """vig_gla_bidir_fwd_strided: q, k, v as head-split views of one [B, L, H*(2*Dk + Dv) + extra] matrix (the stacked
+    input projection's output, classification/models/vig.py:436-438) give bit for bit the result of the op on
+    contiguous copies, and the op is checked against the oracle on the same inputs; views the kernel cannot read in
+    place (rows off a 16-byte boundary, long sequences) are copied by the Python op."""
+    announce(f"strided q/k/v B={B} H={H} L={L} Dk={Dk} both={both}")
+    from vig_amd import _lib, ops
+    Dv = 64
+    q, k, v, gf, gb = (t.bfloat16() for t in dev(*make_gla_inputs(B, H, L, Dk, Dv, seed=31 + L)))
+    if not both:
+        gb = None
+    row = H * (2 * Dk + Dv) + 24  # (other column blocks follow in the same rows)
+    z = torch.randn(B, L, row, device="cuda").bfloat16()
+    z[..., :H * Dk] = q.transpose(1, 2).reshape(B, L, H * Dk)
+    z[..., H * Dk:2 * H * Dk] = k.transpose(1, 2).reshape(B, L, H * Dk)
+    z[..., 2 * H * Dk:2 * H * Dk + H * Dv] = v.transpose(1, 2).reshape(B, L, H * Dv)
+    qs, ks, vs = (t.unflatten(-1, (H, d)).transpose(1, 2)
+                  for t, d in zip(z[..., :H * (2 * Dk + Dv)].split((H * Dk, H * Dk, H * Dv), -1), (Dk, Dk, Dv)))
+    assert not qs.is_contiguous() and torch.equal(qs, q) and torch.equal(vs, v)
+    want = vig_amd.gla_bidir_forward(q, k, v, gf, gb)
+    assert ops._head_view_strides(ks) == (L * row, Dk, row)
+    got = vig_amd.gla_bidir_forward(qs, ks, vs, gf, gb)
+    assert torch.equal(got, want)
+    # one strided operand among contiguous ones
+    assert torch.equal(vig_amd.gla_bidir_forward(q, ks, v, gf, gb), want)
+    if B * H * L <= 4000:
+        ref = oracle_bidir(q, k, v, gf, gb)
+        assert max_abs(f64(got), ref) <= BF16_TOL
+    # the C ABI refuses what the slab kernel does not take
+    lib = _lib.load()
+    import ctypes
+    st = (ctypes.c_longlong * 3)(L * row, Dk, row)
+    sv = (ctypes.c_longlong * 3)(L * row, Dv, row)
+    bad = (ctypes.c_longlong * 3)(L * row, Dk, row + 4)
+    out = torch.empty_like(v)
+
+    def call(sq, L_arg=L):
+        return lib.vig_gla_bidir_fwd_strided(qs.data_ptr(), ks.data_ptr(), vs.data_ptr(), gf.data_ptr(),
+                                             gb.data_ptr() if both else None, out.data_ptr(), B, H, L_arg, Dk, Dv,
+                                             ctypes.addressof(sq), ctypes.addressof(st), ctypes.addressof(sv), Dk ** -0.5,
+                                             1.0, _lib.VIG_BF16, _lib.VIG_BF16, ops._stream_ptr(q))
+    assert call(st) == _lib.VIG_OK
+    torch.cuda.synchronize()
+    assert torch.equal(out, want)
+    assert call(bad) == _lib.VIG_EINVAL
+    assert call(st, 300) == _lib.VIG_ENOTSUP
+
+
 def test_pointers_off_a_16_byte_boundary():
     """The library refuses a tensor that does not start on a 16-byte boundary (nothing is enqueued); the Python op
     copies such a view first and gives the result of the aligned call."""

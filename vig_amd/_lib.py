@@ -28,6 +28,7 @@ SIGNATURES = {
     "vig_gla_bidir_fwd": (_c_int, _GLA_SIG),
     "vig_gla_bidir_fwd_exact": (_c_int, _GLA_SIG),
     "vig_gla_bidir_fwd_wide": (_c_int, _GLA_SIG),
+    "vig_gla_bidir_fwd_strided": (_c_int, [_c_void_p] * 6 + [_c_int] * 5 + [_c_void_p] * 3 + [_c_float, _c_float, _c_int, _c_int, _c_void_p]),
     "vig_gla_bidir_fwd_workspace": (_c_size_t, [_c_int] * 6),
     "vig_gla_bidir_fwd_noalloc": (_c_int, [_c_void_p] * 6 + [_c_int] * 5 + [_c_float, _c_float, _c_int, _c_int, _c_void_p]),
     "vig_gla_bidir_fwd_noalloc_max_workspace": (_c_size_t, []),

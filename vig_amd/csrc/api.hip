@@ -194,6 +194,22 @@ int vig_gla_bidir_fwd(const void* q, const void* k, const void* v, const void* g
                        io_dtype, gate_dtype, stream, 0);
 }
 
+// q, k, v read in place from wider rows (e.g. the column blocks of a stacked projection's output): the matrix-core slab
+// kernel with the rows' pitches in scalar registers; no workspace.
+int vig_gla_bidir_fwd_strided(const void* q, const void* k, const void* v, const void* g_fwd, const void* g_bwd, void* o,
+                              int B, int H, int L, int Dk, int Dv, const long long* q_strides,
+                              const long long* k_strides, const long long* v_strides, float scale, float out_scale,
+                              int io_dtype, int gate_dtype, void* stream) {
+  if (!q_strides || !k_strides || !v_strides) return VIG_EINVAL;
+  vig::GlaArgs a;
+  const int rc = fill_args(a, q, k, v, g_fwd, g_bwd, o, nullptr, 0, B, H, L, Dk, Dv, scale, out_scale, io_dtype,
+                           gate_dtype, stream);
+  if (rc != VIG_OK) return rc;
+  if (!vig::gla_mfma_supported(a) || L > 256) return VIG_ENOTSUP;
+  a.q_strides = q_strides, a.k_strides = k_strides, a.v_strides = v_strides;
+  return vig::launch_gla_mfma(a);
+}
+
 // The causal op with a state carried in and / or out.
 static size_t causal_state_workspace(int B, int H, int L, int Dk, int Dv, int io_dtype, int gate_dtype) {
   if (io_dtype == VIG_BF16 && gate_dtype == VIG_BF16 && (Dk == 64 || Dk == 32) && Dv == 64)

@@ -252,26 +252,36 @@ struct Prefetch {
   u32x4_t rawk[NG], rawq[NG];  // raw rows of the tile walked first
 };
 
-// The four tensors of one chunk (q, k, g: 32*NG bytes per row; v: 128).
+// The four tensors of one chunk: gate rows are contiguous (32*NG bytes); q, k and v rows lie a pitch apart, which is
+// the row itself for plain [B, H, L, D] tensors and more when a head's channels sit inside wider token rows.
 struct ChunkSrc {
   rsrc_t q, k, v, g;
+  unsigned q_pitch, k_pitch, v_pitch;  // bytes
 };
 
 template <int NG>
 __device__ __forceinline__ void issue_gates(const ChunkSrc& src, int r, int h, Prefetch<NG>& pf) {
   issue_tdwords<0, 4, NG>(src.g, r, h, pf.gD);
 }
-template <bool FWD, bool WITH_Q, int NG>
+// (PITCHED: q, k, v rows lie the descriptors' pitches apart; else they are contiguous and every token offset is an
+// instruction immediate)
+template <bool FWD, bool WITH_Q, int NG, bool PITCHED = false>
 __device__ __forceinline__ void issue_rows(const ChunkSrc& src, int r, int h, Prefetch<NG>& pf) {
   constexpr int TA = FWD ? 0 : 1;
-  issue_raw_tile<NG>(src.k, TA, r, h, pf.rawk);
-  if (WITH_Q) issue_raw_tile<NG>(src.q, TA, r, h, pf.rawq);
-  issue_tdwords<2 * TA, 2, 4>(src.v, r, h, pf.vD);
+  if (PITCHED) {
+    issue_raw_tile_pitched<NG>(src.k, TA, r, h, src.k_pitch, pf.rawk);
+    if (WITH_Q) issue_raw_tile_pitched<NG>(src.q, TA, r, h, src.q_pitch, pf.rawq);
+    issue_tdwords_pitched<2 * TA, 2, 4>(src.v, r, h, src.v_pitch, pf.vD);
+  } else {
+    issue_raw_tile<NG>(src.k, TA, r, h, pf.rawk);
+    if (WITH_Q) issue_raw_tile<NG>(src.q, TA, r, h, pf.rawq);
+    issue_tdwords<2 * TA, 2, 4>(src.v, r, h, pf.vD);
+  }
 }
-template <bool FWD, bool WITH_Q, int NG>
+template <bool FWD, bool WITH_Q, int NG, bool PITCHED = false>
 __device__ __forceinline__ void issue_first_phase(const ChunkSrc& src, int r, int h, Prefetch<NG>& pf) {
   issue_gates<NG>(src, r, h, pf);
-  issue_rows<FWD, WITH_Q, NG>(src, r, h, pf);
+  issue_rows<FWD, WITH_Q, NG, PITCHED>(src, r, h, pf);
 }
 
 // Segment modes of the kernel.  A sequence longer than 256 tokens is cut into segments of <= 256 tokens that are
@@ -286,8 +296,12 @@ __device__ __forceinline__ void issue_first_phase(const ChunkSrc& src, int r, in
 //               same pass fed the q tensor for k and the output gradient (the o argument) for v, with the other
 //               direction's gates and the cumulative gates taken exclusive of a token's own gate (so that the weight
 //               of a token reaches back to and includes it).
-constexpr int kModeSlab = 0, kModeState = 1, kModeChain = 2, kModeStateDual = 3;
+//   kModeSlabPitched  kModeSlab on q, k, v whose token rows lie a pitch apart (column blocks of a wider matrix read in
+//               place): the same arithmetic, token offsets in scalar registers instead of instruction immediates.
+constexpr int kModeSlab = 0, kModeState = 1, kModeChain = 2, kModeStateDual = 3, kModeSlabPitched = 4;
 constexpr bool is_state_mode(int mode) { return mode == kModeState || mode == kModeStateDual; }
+constexpr bool is_slab(int mode) { return mode == kModeSlab || mode == kModeSlabPitched; }
+constexpr bool is_pitched(int mode) { return mode == kModeSlabPitched; }
 constexpr int kStateFloats = kGlaStateFloats;  // per (sequence, segment, direction): state in unit order, then 64 decays
 
 // Intra-chunk part of one wave: scores of the three tile pairs of its chunk, applied to V; k~ (bf16) goes to the
@@ -329,9 +343,15 @@ __device__ __forceinline__ bool tile_phase(const ChunkSrc& cur, const Prefetch<N
       }
   };
   auto fetch_second = [&]() {
-    if (OUT) issue_raw_tile<NG>(cur.q, TB, r, h, rawq);
-    issue_raw_tile<NG>(cur.k, TB, r, h, rawk);
-    issue_tdwords<2 * TB, 2, 4>(cur.v, r, h, vDb);
+    if (is_pitched(MODE)) {
+      if (OUT) issue_raw_tile_pitched<NG>(cur.q, TB, r, h, cur.q_pitch, rawq);
+      issue_raw_tile_pitched<NG>(cur.k, TB, r, h, cur.k_pitch, rawk);
+      issue_tdwords_pitched<2 * TB, 2, 4>(cur.v, r, h, cur.v_pitch, vDb);
+    } else {
+      if (OUT) issue_raw_tile<NG>(cur.q, TB, r, h, rawq);
+      issue_raw_tile<NG>(cur.k, TB, r, h, rawk);
+      issue_tdwords<2 * TB, 2, 4>(cur.v, r, h, vDb);
+    }
   };
   bool too_large = false;
   if (F16) {
@@ -343,12 +363,12 @@ __device__ __forceinline__ bool tile_phase(const ChunkSrc& cur, const Prefetch<N
     u32x4_t ka[NG], qb[NG];
     // the second tile's loads go out before the first tile's operands are built where registers allow it (measured:
     // earlier is better for whole slabs, later for the chained segments of long sequences)
-    constexpr bool EARLY = MODE == kModeSlab;
+    constexpr bool EARLY = is_slab(MODE);
     if (EARLY) fetch_second();
     VIG_PHASE();
     {
       u32x4_t qa[NG];
-      make_pair16<OUT, NG, MODE == kModeSlab>(pf.rawq, pf.rawk, G[TA], gend2, qa, ka, qkeep[TA]);
+      make_pair16<OUT, NG, is_slab(MODE)>(pf.rawq, pf.rawk, G[TA], gend2, qa, ka, qkeep[TA]);
       store_kt<NG, kFwdKtStride<NG>>(kt, 32 * TA + r, h, ka);
       VIG_PHASE();
       if (!EARLY) fetch_second();
@@ -362,7 +382,7 @@ __device__ __forceinline__ bool tile_phase(const ChunkSrc& cur, const Prefetch<N
       if (GUARD && OUT) gram_acc(rawq[g], gram);
     }
     u32x4_t kb[NG];
-    make_pair16<OUT, NG, MODE == kModeSlab>(rawq, rawk, G[TB], gend2, qb, kb, qkeep[TB]);
+    make_pair16<OUT, NG, is_slab(MODE)>(rawq, rawk, G[TB], gend2, qb, kb, qkeep[TB]);
     store_kt<NG, kFwdKtStride<NG>>(kt, 32 * TB + r, h, kb);
     if (OUT) apply_scores<0, true>(score_tile16<NG>(ka, qb), TA, r, h, vfrag, O[0][TB], O[1][TB]);
     VIG_PHASE();
@@ -449,7 +469,7 @@ __device__ __forceinline__ bool direction_wave(const ChunkSrc& cur, const ChunkS
   char* region = lds + wi * kRegionBytes;
   uint16_t* kt = reinterpret_cast<uint16_t*>(region);
   float* dvec_all = reinterpret_cast<float*>(lds + kLdsDvec);
-  if (!FWD) issue_rows<FWD, OUT, NG>(cur, r, h, pf);
+  if (!FWD) issue_rows<FWD, OUT, NG, is_pitched(MODE)>(cur, r, h, pf);
   // fused gate: the first 144 threads fetch the head's stencil weights now and park them in LDS before barrier A
   f32x4_t gate_w4 = {0.f, 0.f, 0.f, 0.f};
   const bool gate_w_mine = GATE && wi * 64 + lane < 64 * 9 / 4;
@@ -515,7 +535,7 @@ __device__ __forceinline__ bool direction_wave(const ChunkSrc& cur, const ChunkS
     const int p = (lane >> 4) & 1, g = (lane >> 2) & 3, m = lane & 3;
     // half decay of channel 8*g + 2*m + p of this lane half (register quads >= NG carry no channel)
     if (g < NG) {
-      if (MODE == kModeSlab && F16)
+      if (is_slab(MODE) && F16)
         reinterpret_cast<_Float16*>(lds + kLdsHalf16)[wi * 64 + HC * h + 8 * g + 2 * m + p] = (_Float16)exp2_fast(an);
       else
         dvec_all[wi * 64 + HC * h + 8 * g + 2 * m + p] = exp2_fast(an);
@@ -545,7 +565,7 @@ __device__ __forceinline__ bool direction_wave(const ChunkSrc& cur, const ChunkS
         for (int pv = 0; pv < 2; ++pv)
           U[pk][pv] = F16 ? mfma_f16(ktf[pk], vfrag[t][pv], U[pk][pv]) : mfma(ktf[pk], vfrag[t][pv], U[pk][pv]);
     }
-    constexpr bool DIRECT = MODE == kModeSlab && F16;
+    constexpr bool DIRECT = is_slab(MODE) && F16;
     if (DIRECT) {
       // whole slab on fp16 operands: the later chunks of the direction take this contribution as it is (fp16, as
       // ready fragments: dword m of unit pv*4 + cq holds rows (pk = 0, 1) of register 4*cq + m) instead of a state
@@ -587,7 +607,7 @@ __device__ __forceinline__ bool direction_wave(const ChunkSrc& cur, const ChunkS
   // dwords (needed first) here and the rows at the top of the segment: a wave stalls while the memory pipe accepts
   // its loads, and this way the other wave of the SIMD has math to do.  (Always issued: after the last segment the
   // descriptors are empty, which keeps branches off the loads.) ----
-  if (FWD) issue_first_phase<FWD, OUT, NG>(nxt, r, h, pf);
+  if (FWD) issue_first_phase<FWD, OUT, NG, is_pitched(MODE)>(nxt, r, h, pf);
   else issue_gates<NG>(nxt, r, h, pf);
   // lane-derived addresses of the exchange phases are rebuilt here instead of being carried (and spilled) across
   // the register-heavy tile phase
@@ -601,7 +621,7 @@ __device__ __forceinline__ bool direction_wave(const ChunkSrc& cur, const ChunkS
   // same answer in every wave: the word is only written before this barrier and the variant is left once it is set
   const bool ok = !F16 || __builtin_amdgcn_readfirstlane(*veto) == 0;
   if (F16 && !ok) return false;  // every wave alike: the segment is walked again, barriers B and C are skipped by all
-  constexpr bool DIRECT = MODE == kModeSlab && F16;
+  constexpr bool DIRECT = is_slab(MODE) && F16;
   if (DIRECT) {
     // ---- whole slab on fp16 operands: O^T += (E (.) U_j)^T q~ for every chunk j walked earlier in this direction,
     // E = h_c h_j prod(h_i^2, i between) per k channel with h = exp(G_end/2) <= 1 (the decay from the end of chunk j
@@ -859,8 +879,15 @@ __device__ __forceinline__ bool direction_wave(const ChunkSrc& cur, const ChunkS
 
 // Geometry of the work items: item = sequence * nseg + segment; a segment holds seg_len tokens (the last one of a
 // sequence possibly fewer) cut into 4 chunks of cw tokens.
+// where sequence (b, h) of a tensor starts and how far its token rows lie apart, in elements
+struct Strides {
+  long long batch, head;
+  int token;
+};
 struct Geometry {
   int L, nseg, seg_len, cw, nitems;
+  int H;               // heads per batch element: sequence = b * H + h
+  Strides sq, sk, sv;  // q, k, v (gates and outputs are contiguous [B, H, L, D])
   int gw, gh, heads;  // fused locality gate only: token grid and heads per batch element
   int wide_gates;     // nonzero: skip the fp16 score variant from the start
   int dual_first;     // kModeStateDual: first item of the gradient-state set (= items of the plain set)
@@ -876,7 +903,8 @@ __device__ __forceinline__ int wave_loop(const uint16_t* q, const uint16_t* k, c
   // descriptors of this wave's chunk of an item; past the last item (or for a chunk with no tokens) they are empty
   auto locate = [&](int it, ChunkSrc& src, rsrc_t& dst) {
     int nvalid = 0;
-    size_t off = 0;
+    size_t off = 0, tok = 0;
+    int b = 0, hd = 0;
     const uint16_t *kk = k, *vv = v, *gg = g;
     if (it < geo.nitems) {
       int it2 = it;
@@ -884,12 +912,22 @@ __device__ __forceinline__ int wave_loop(const uint16_t* q, const uint16_t* k, c
       const int seq = it2 / geo.nseg, seg = it2 - seq * geo.nseg;
       const int seg_tokens = min(geo.seg_len, geo.L - seg * geo.seg_len);
       nvalid = min(max(seg_tokens - c * geo.cw, 0), geo.cw);
-      off = (size_t)seq * geo.L + (size_t)seg * geo.seg_len + (size_t)(nvalid > 0 ? c * geo.cw : 0);  // in tokens
+      tok = (size_t)seg * geo.seg_len + (size_t)(nvalid > 0 ? c * geo.cw : 0);
+      off = (size_t)seq * geo.L + tok;  // in tokens
+      b = seq / geo.H, hd = seq - b * geo.H;
     }
-    src.q = chunk_rsrc(q + off * DK, nvalid, 2 * DK);
-    src.k = chunk_rsrc(kk + off * DK, nvalid, 2 * DK);
+    if (is_pitched(MODE)) {
+      src.q_pitch = 2u * geo.sq.token, src.k_pitch = 2u * geo.sk.token, src.v_pitch = 2u * geo.sv.token;
+      src.q = chunk_rsrc(q + b * geo.sq.batch + hd * geo.sq.head + tok * geo.sq.token, nvalid, src.q_pitch);
+      src.k = chunk_rsrc(kk + b * geo.sk.batch + hd * geo.sk.head + tok * geo.sk.token, nvalid, src.k_pitch);
+      src.v = chunk_rsrc(vv + b * geo.sv.batch + hd * geo.sv.head + tok * geo.sv.token, nvalid, src.v_pitch);
+    } else {
+      src.q_pitch = src.k_pitch = 2 * DK, src.v_pitch = 128;
+      src.q = chunk_rsrc(q + off * DK, nvalid, 2 * DK);
+      src.k = chunk_rsrc(kk + off * DK, nvalid, 2 * DK);
+      src.v = chunk_rsrc(vv + off * 64, nvalid, 128);
+    }
     src.g = chunk_rsrc(gg + off * DK, nvalid, 2 * DK);
-    src.v = chunk_rsrc(vv + off * 64, nvalid, 128);
     dst = chunk_rsrc(o + off * 64, nvalid, 128);
   };
   Prefetch<NG> pf;
@@ -897,7 +935,7 @@ __device__ __forceinline__ int wave_loop(const uint16_t* q, const uint16_t* k, c
   rsrc_t dst;
   locate(item, cur, dst);
   if (item < geo.nitems) {
-    if (FWD) issue_first_phase<FWD, OUT, NG>(cur, lane & 31, lane >> 5, pf);
+    if (FWD) issue_first_phase<FWD, OUT, NG, is_pitched(MODE)>(cur, lane & 31, lane >> 5, pf);
     else issue_gates<NG>(cur, lane & 31, lane >> 5, pf);
   }
   for (; item < geo.nitems; item += gridDim.x) {
@@ -919,7 +957,7 @@ __device__ __forceinline__ int wave_loop(const uint16_t* q, const uint16_t* k, c
     // between A and C of the same slab), and the output half it sends after the next A was read by its partner
     // before that wave could reach the next A.  (Measured: -2.0 us on the Dk = 32 slab shape, +0.7 us at Dk = 64,
     // where the waves that run ahead take issue slots from the late ones' stores: dropped for Dk = 32 only.)
-    if (!(MODE == kModeSlab && F16 && !GATE && NG == 2 && ok)) lds_barrier();
+    if (!(is_slab(MODE) && F16 && !GATE && NG == 2 && ok)) lds_barrier();
     if (F16 && !ok) break;  // this item again, and all that follow, with split-bf16 scores
     cur = nxt;
     dst = dst_next;
@@ -971,10 +1009,10 @@ __global__ __launch_bounds__(512) void gla_mfma_kernel(const uint16_t* __restric
       lds_barrier();  // (A)
       const bool refused = __builtin_amdgcn_readfirstlane(*veto) != 0;
       if (!refused) {  // a refused segment leaves after barrier A
-        if (MODE != kModeSlab) lds_barrier();  // (B: not in the fp16 variant of whole slabs)
+        if (!is_slab(MODE)) lds_barrier();  // (B: not in the fp16 variant of whole slabs)
         lds_barrier();
       }
-      if (MODE != kModeSlab || NG != 2 || refused) lds_barrier();  // (D: only behind a refused segment for Dk = 32 fp16 slabs)
+      if (!is_slab(MODE) || NG != 2 || refused) lds_barrier();  // (D: only behind a refused segment for Dk = 32 fp16 slabs)
       if (refused) break;
     }
     for (; item < geo.nitems; item += gridDim.x) {
@@ -1040,6 +1078,11 @@ static Geometry make_geometry(int nseq, int L) {
   g.nitems = nseq * g.nseg;
   return g;
 }
+// plain [B, H, L, D] layout of a tensor, or the caller's strides (batch, head, token; channels contiguous)
+static Strides make_strides(const long long* given, int H, int L, int D) {
+  if (given && given[2] != 0) return Strides{given[0], given[1], (int)given[2]};
+  return Strides{(long long)H * L * D, (long long)L * D, D};
+}
 
 // the padded grid must fit the staging cells: whole padded rows per region half, eight halves
 bool gla_mfma_gate_grid_ok(int rows, int cols) {
@@ -1072,7 +1115,8 @@ static int launch_gla_mfma_t(const GlaArgs& a, int num_cu, int dev) {
   static bool attr_done_dev[kMaxDevices] = {};
   bool& attr_done = attr_done_dev[dev];
   if (!attr_done) {
-    const void* kernels[5] = {reinterpret_cast<const void*>(gla_mfma_kernel<kModeSlab, NG>),
+    const void* kernels[6] = {reinterpret_cast<const void*>(gla_mfma_kernel<kModeSlab, NG>),
+                              reinterpret_cast<const void*>(gla_mfma_kernel<kModeSlabPitched, NG>),
                               reinterpret_cast<const void*>(gla_mfma_kernel<kModeState, NG>),
                               reinterpret_cast<const void*>(gla_mfma_kernel<kModeChain, NG>),
                               reinterpret_cast<const void*>(gla_mfma_kernel<kModeSlab, NG, true>),
@@ -1083,6 +1127,19 @@ static int launch_gla_mfma_t(const GlaArgs& a, int num_cu, int dev) {
   }
   Geometry geo = make_geometry(a.B * a.H, a.L);
   geo.wide_gates = a.wide_gates;
+  geo.H = a.H;
+  geo.sq = make_strides(a.q_strides, a.H, a.L, a.Dk);
+  geo.sk = make_strides(a.k_strides, a.H, a.L, a.Dk);
+  geo.sv = make_strides(a.v_strides, a.H, a.L, a.Dv);
+  // q, k, v read in place from wider rows: whole-sequence slabs only; rows 16-byte aligned, pitches within the
+  // descriptors' 32-bit extents
+  const bool pitched = a.q_strides || a.k_strides || a.v_strides;
+  if (pitched) {
+    if (geo.nseg != 1 || a.state_pass || a.init_state || a.final_state) return -95;
+    for (const Strides* st : {&geo.sq, &geo.sk, &geo.sv})
+      if (st->token <= 0 || st->token % 8 != 0 || st->batch % 8 != 0 || st->head % 8 != 0 || st->token > (1 << 20))
+        return -22;
+  }
   int grid = geo.nitems < num_cu ? geo.nitems : num_cu;
   const uint16_t* q = (const uint16_t*)a.q;
   const uint16_t* k = (const uint16_t*)a.k;
@@ -1113,11 +1170,16 @@ static int launch_gla_mfma_t(const GlaArgs& a, int num_cu, int dev) {
     geo.gw = a.gate_cols;
     geo.gh = a.gate_rows;
     geo.heads = a.H;
+    if (pitched) return -95;
     hipLaunchKernelGGL((gla_mfma_kernel<kModeSlab, NG, true>), dim3(grid), dim3(512), kLdsTotal, a.stream, q, k, v, gf,
                        gb, o, geo, oscale, (float*)nullptr, a.gate_w);
   } else if (geo.nseg == 1 && !a.init_state && !a.final_state) {
-    hipLaunchKernelGGL((gla_mfma_kernel<kModeSlab, NG>), dim3(grid), dim3(512), kLdsTotal, a.stream, q, k, v, gf, gb, o,
-                       geo, oscale, (float*)nullptr, no_gate);
+    if (pitched)
+      hipLaunchKernelGGL((gla_mfma_kernel<kModeSlabPitched, NG>), dim3(grid), dim3(512), kLdsTotal, a.stream, q, k, v,
+                         gf, gb, o, geo, oscale, (float*)nullptr, no_gate);
+    else
+      hipLaunchKernelGGL((gla_mfma_kernel<kModeSlab, NG>), dim3(grid), dim3(512), kLdsTotal, a.stream, q, k, v, gf, gb,
+                         o, geo, oscale, (float*)nullptr, no_gate);
   } else {
     if ((a.init_state || a.final_state) && gb) return -22;  // a state in or out belongs to the causal op
     float* ws = (float*)a.workspace;

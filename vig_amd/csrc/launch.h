@@ -33,6 +33,12 @@ struct GlaArgs {
   // that pass and, behind its slots, the gradient-state pass of the backward on (q for k, `o` read as the output
   // gradient for v, the two directions' gates exchanged, cumulative gates exclusive of each token's own gate).
   int state_pass = 0;
+  // bf16 MFMA path: q, k, v that are not plain [B, H, L, D] tensors: element strides (batch, head, token) with the
+  // channels of a (token, head) contiguous, e.g. column blocks of a projection output [B, L, H*(2*Dk + Dv)] read in
+  // place.  Null (or token stride 0): plain layout.  Strides are multiples of 8 elements.
+  const long long* q_strides = nullptr;
+  const long long* k_strides = nullptr;
+  const long long* v_strides = nullptr;
 };
 
 // Per (sequence, segment, direction) slot of a state pass: the 64 x 64 state contribution in the matrix cores' register

@@ -78,6 +78,18 @@ __device__ __forceinline__ void issue_tdwords(rsrc_t rows, int r, int h, uint32_
       D[t][e] = __builtin_amdgcn_raw_buffer_load_b32(rows, base + (unsigned)jmap(T0 + t, 0, e) * RB, 0, 0);
 }
 
+// the same for rows that lie `pitch` bytes apart (a head's channels inside wider token rows): the token offsets travel
+// in the scalar offset operand instead of the immediate
+template <int T0, int NT, int NG>
+__device__ __forceinline__ void issue_tdwords_pitched(rsrc_t rows, int r, int h, unsigned pitch, uint32_t (&D)[NT][8]) {
+  const unsigned base = row_has_channel<NG>(r) ? (4u * h) * pitch + 4u * cpair<NG>(r) : kOutOfRange;
+#pragma unroll
+  for (int t = 0; t < NT; ++t)
+#pragma unroll
+    for (int e = 0; e < 8; ++e)
+      D[t][e] = __builtin_amdgcn_raw_buffer_load_b32(rows, base, (unsigned)jmap(T0 + t, 0, e) * pitch, 0);
+}
+
 // fragments from raw dwords: frag[t][p] has lane index = channel 2*cpair(r)+p, slots = tokens jmap(t,h,.)
 template <int NT>
 __device__ __forceinline__ void finish_tfrags(const uint32_t (&D)[NT][8], u32x4_t (&frag)[NT][2]) {
@@ -98,6 +110,15 @@ __device__ __forceinline__ void issue_raw_tile(rsrc_t rows, int it, int r, int h
 #pragma unroll
   for (int gq = 0; gq < NG; ++gq)
     raw[gq] = __builtin_amdgcn_raw_buffer_load_b128(rows, base + (unsigned)it * 32u * RB + 16u * gq, 0, 0);
+}
+
+template <int NG>
+__device__ __forceinline__ void issue_raw_tile_pitched(rsrc_t rows, int it, int r, int h, unsigned pitch,
+                                                       u32x4_t (&raw)[NG]) {
+  const unsigned base = (unsigned)r * pitch + (16u * NG) * h;
+#pragma unroll
+  for (int gq = 0; gq < NG; ++gq)
+    raw[gq] = __builtin_amdgcn_raw_buffer_load_b128(rows, base + 16u * gq, (unsigned)it * 32u * pitch, 0);
 }
 
 // one k-step of transposed fragments from the wave's k~ scratch in LDS

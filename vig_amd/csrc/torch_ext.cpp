@@ -380,10 +380,27 @@ Tensor gla_block_mix(const Tensor& x, int64_t grid_h, int64_t grid_w, const Tens
   Tensor z = at::linear(xs, w_in, b_in);
   const int64_t n0 = H * (2 * Dk + Dv), n1 = n0 + H * Dv, rank = w_up.size(1);
   TORCH_CHECK(z.size(-1) >= n1 + rank, "vig_amd: stacked projection is narrower than qkv | g | gate rows");
-  auto qkv = split_heads_fwd(z.narrow(-1, 0, n0), H, Dk, Dv);
   Tensor gates = dirgate_lowrank_fwd(z.narrow(-1, n1, rank), w_up, b_up, H, normalizer, clamp_min);
-  Tensor o = gla_bidir_fwd(std::get<0>(qkv), std::get<1>(qkv), std::get<2>(qkv), gates.select(0, 0), gates.select(0, 1), -1.0,
-                           out_scale, 0);
+  Tensor o;
+  const int64_t B = z.size(0), L = z.size(1), ld = z.size(-1);
+  if (z.scalar_type() == at::kBFloat16 && gates.scalar_type() == at::kBFloat16 && L <= 256 && (Dk == 32 || Dk == 64) &&
+      Dv == 64 && ld % 8 == 0 && z.is_contiguous() && reinterpret_cast<uintptr_t>(z.data_ptr()) % 16 == 0) {
+    // the matrix-core slab kernel reads q, k, v in place from the projection's rows: no head-major copies
+    const c10::DeviceGuard guard(z.device());
+    o = at::empty({B, H, L, Dv}, z.options());
+    const long long sqk[3] = {(long long)(L * ld), (long long)Dk, (long long)ld};
+    const long long sv[3] = {(long long)(L * ld), (long long)Dv, (long long)ld};
+    const auto* base = static_cast<const at::BFloat16*>(z.data_ptr());
+    Tensor gf = gates.select(0, 0), gb = gates.select(0, 1);
+    check_rc(vig_gla_bidir_fwd_strided(base, base + H * Dk, base + 2 * H * Dk, gf.data_ptr(), gb.data_ptr(), o.data_ptr(),
+                                       (int)B, (int)H, (int)L, (int)Dk, (int)Dv, sqk, sqk, sv,
+                                       resolve_scale(-1.0, (int)Dk), (float)out_scale, VIG_BF16, VIG_BF16, stream_of(z)),
+             "vig_gla_bidir_fwd_strided");
+  } else {
+    auto qkv = split_heads_fwd(z.narrow(-1, 0, n0), H, Dk, Dv);
+    o = gla_bidir_fwd(std::get<0>(qkv), std::get<1>(qkv), std::get<2>(qkv), gates.select(0, 0), gates.select(0, 1), -1.0,
+                      out_scale, 0);
+  }
   Tensor y = locality_blend_fwd(o, xs, z.narrow(-1, n0, H * Dv), w_gnorm, w_lnorm, eps, out_act);
   return at::linear(y, w_o);
 }

@@ -221,7 +221,13 @@ class GatedLinearAttention(_CacheMixin, nn.Module):
         xs = ops.dwconv3x3(x, _f32(self, "conv_w", conv.weight, (-1, 3, 3)), hw, bias=_f32(self, "conv_b", conv.bias),
                            silu=self.use_act_in_conv)
         qkv, g_lin, gk_low = self._input_projections(xs)
-        q, k, v = ops.split_heads(qkv, H, self.head_qk_dim, self.head_v_dim)
+        dk, dv = self.head_qk_dim, self.head_v_dim
+        if qkv.dtype == torch.bfloat16 and qkv.shape[1] <= 256 and dk in (32, 64) and dv == 64 and qkv.stride(1) % 8 == 0:
+            # head-split views of the projection's rows: the matrix-core slab kernel reads them in place
+            q, k, v = (t.unflatten(-1, (H, d)).transpose(1, 2)
+                       for t, d in zip(qkv.split((H * dk, H * dk, H * dv), -1), (dk, dk, dv)))
+        else:
+            q, k, v = ops.split_heads(qkv, H, dk, dv)
         up = self.gk_proj[1]
         if gk_low.shape[-1] == ops.GATE_RANK:  # the rank-16 up-projection runs inside the gate kernel
             gates = ops.dirgate_lowrank(gk_low, up.weight, up.bias, H, self.gate_logit_normalizer, self.clamp_min)

@@ -11,6 +11,7 @@ merged bidirectional op has no working backward, recurrent_fuse.py:443,456).
 """
 from __future__ import annotations
 
+import ctypes
 import math
 from typing import Optional, Tuple
 
@@ -128,9 +129,58 @@ class _GLABidirFunction(torch.autograd.Function):
         return dq, dk, dv, dgf, dgb, None, None, None
 
 
+def _head_view_strides(t):
+    """(batch, head, token) element strides of a [B,H,L,D] view whose channels are contiguous and whose rows start on
+    16-byte boundaries, or None: what vig_gla_bidir_fwd_strided reads in place."""
+    sb, sh, st, sd = t.stride()
+    if t.is_contiguous() or sd != 1 or min(sb, sh, st) <= 0 or sb % 8 or sh % 8 or st % 8 or st > (1 << 20):
+        return None
+    return (sb, sh, st) if t.data_ptr() % 16 == 0 else None
+
+
+def _gla_bidir_forward_strided(q, k, v, g_fwd, g_bwd, scale, out_scale, out):
+    """The op on head-split views of wider token rows (e.g. column blocks of a projection output), read in place by
+    the matrix-core slab kernel; None when the call is not of that kind."""
+    if not (q.dtype == torch.bfloat16 and g_fwd.dtype == torch.bfloat16 and q.dim() == 4 and q.shape[2] <= 256
+            and q.shape[3] in (32, 64) and v.shape[-1] == 64):
+        return None
+    if k.shape != q.shape or g_fwd.shape != q.shape or v.shape[:3] != q.shape[:3] or k.dtype != q.dtype or v.dtype != q.dtype:
+        return None
+    B, H, L, Dk = q.shape
+    strides = []
+    for t, D in ((q, Dk), (k, Dk), (v, 64)):
+        st = _head_view_strides(t)
+        if st is None:
+            if not t.is_contiguous() or t.data_ptr() % 16:
+                return None
+            st = (H * L * D, L * D, D)
+        strides.append((ctypes.c_longlong * 3)(*st))
+    if all(t.is_contiguous() for t in (q, k, v)):
+        return None
+    lib = _lib.load()
+    g_fwd = _dense(g_fwd)
+    g_bwd = _dense(g_bwd) if g_bwd is not None else None
+    if out is None:
+        out = torch.empty(B, H, L, 64, dtype=q.dtype, device=q.device)
+    if scale == -1 or scale is None:
+        scale = Dk ** -0.5
+    with torch.cuda.device(q.device):
+        rc = lib.vig_gla_bidir_fwd_strided(q.data_ptr(), k.data_ptr(), v.data_ptr(), g_fwd.data_ptr(),
+                                           g_bwd.data_ptr() if g_bwd is not None else None, out.data_ptr(),
+                                           B, H, L, Dk, 64, ctypes.addressof(strides[0]), ctypes.addressof(strides[1]),
+                                           ctypes.addressof(strides[2]), float(scale), float(out_scale),
+                                           _lib.VIG_BF16, _lib.VIG_BF16, _stream_ptr(q))
+    _lib.check(rc, "vig_gla_bidir_fwd_strided")
+    return out
+
+
 def _gla_bidir_forward_raw(q, k, v, g_fwd, g_bwd, scale, out_scale, exact, out, strong_gates=False):
     lib = _lib.load()
     _check_cuda(q, k, v, g_fwd, g_bwd)
+    if not exact and not strong_gates and (out is None or (out.is_contiguous() and out.data_ptr() % 16 == 0)):
+        o = _gla_bidir_forward_strided(q, k, v, g_fwd, g_bwd, scale, out_scale, out)
+        if o is not None:
+            return o
     q, k, v, g_fwd = (_dense(t) for t in (q, k, v, g_fwd))
     if g_bwd is not None:
         g_bwd = _dense(g_bwd)
