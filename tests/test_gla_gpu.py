@@ -210,7 +210,7 @@ def test_bf16_strong_gates_one_direction(B, L):
     assert max_abs(got, want) <= BF16_TOL
 
 
-@pytest.mark.parametrize("idx,batch", [(1, None), (2, None), (3, None), (4, 64)])
+@pytest.mark.parametrize("idx,batch", [(1, None), (2, None), (3, None), (4, None)])
 def test_bf16_named_configs_full_size(idx, batch):
     """Full-size named workloads against the oracle (the oracle finishes these in seconds)."""
     s = CONFIGS[idx]
