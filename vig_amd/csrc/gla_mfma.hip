@@ -877,13 +877,13 @@ __device__ __forceinline__ bool direction_wave(const ChunkSrc& cur, const ChunkS
   return ok;
 }
 
-// Geometry of the work items: item = sequence * nseg + segment; a segment holds seg_len tokens (the last one of a
-// sequence possibly fewer) cut into 4 chunks of cw tokens.
 // where sequence (b, h) of a tensor starts and how far its token rows lie apart, in elements
 struct Strides {
   long long batch, head;
   int token;
 };
+// Geometry of the work items: item = sequence * nseg + segment; a segment holds seg_len tokens (the last one of a
+// sequence possibly fewer) cut into 4 chunks of cw tokens.
 struct Geometry {
   int L, nseg, seg_len, cw, nitems;
   int H;               // heads per batch element: sequence = b * H + h

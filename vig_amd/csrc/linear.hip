@@ -7,9 +7,11 @@
 //
 // With K this short a wave's whole slice of W fits in registers: a wave keeps the 32 gate rows and the 32 matching
 // up rows of one channel tile as matrix-instruction A operands for the life of the workgroup, eight waves cover 256
-// channels, and the workgroup streams 32-token tiles of A through LDS (double-buffered, the next tile's global loads
-// in flight during the matrix instructions): every 16-byte LDS read feeds two v_mfma_f32_32x32x16_bf16.  Matrix rows
-// are assigned channels so that a lane ends with 16 consecutive channels of one token (32 contiguous bytes).
+// channels, and the workgroup streams 32-token tiles of A through LDS, double-buffered: the next tile travels from
+// memory straight into its buffer (direct-to-LDS loads, whole token rows per wave, no registers) during the matrix
+// instructions of the current one, and every 16-byte LDS read, issued three k-steps ahead of its use, feeds two
+// v_mfma_f32_32x32x16_bf16.  The two waves of a SIMD take turns on its matrix and vector pipes (see the loop).  Matrix
+// rows are assigned channels so that a lane ends with 16 consecutive channels of one token (32 contiguous bytes).
 // Workgroups of the same column group are spread over the token tiles; the column groups of one token tile run on the
 // same XCD (workers are a multiple of the XCD count apart in block index), so a tile of A leaves HBM once.
 #include "common.h"
@@ -45,9 +47,10 @@ __global__ __launch_bounds__(64 * kLinWaves) void linear_swiglu_kernel(const uin
                                                                        int nworkers) {
   constexpr int K = 16 * KS;
   constexpr int kThreads = 64 * kLinWaves;
-  constexpr int kRow = K + 8;                                // LDS row stride in elements (conflict-free 16-byte reads)
-  constexpr int kChunks = 32 * K / 8;                        // 16-byte chunks of a 32-token tile
-  constexpr int kPer = (kChunks + kThreads - 1) / kThreads;  // chunks per thread
+  constexpr int kCols = K / 8;                 // 16-byte chunks per token row
+  constexpr int kRow = K + 8;                  // LDS row stride in elements (conflict-free 16-byte reads)
+  constexpr int kPer = 32 / kLinWaves;         // token rows per wave
+  static_assert(kCols <= 64 && 32 % kLinWaves == 0, "a wave loads whole token rows");
   extern __shared__ __align__(16) char smem[];
   uint16_t* buf = reinterpret_cast<uint16_t*>(smem);  // [2][32][kRow]
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -68,53 +71,27 @@ __global__ __launch_bounds__(64 * kLinWaves) void linear_swiglu_kernel(const uin
     }
   }
   const int ntiles_t = (T + 31) / 32;
-  // a 32-token tile of A is one contiguous run of 32*K elements: chunk c of it goes to row c / (K/8) of the buffer
-  int lds_off[kPer];
-#pragma unroll
-  for (int i = 0; i < kPer; ++i) {
-    const int c = tid + kThreads * i;
-    lds_off[i] = (c / (K / 8)) * kRow + (c % (K / 8)) * 8;
-  }
-  auto fetch = [&](int tile, u32x4_t (&v)[kPer]) {
+  // A tile travels from memory straight into its LDS buffer (no registers): lane i of a wave lands 16 i bytes behind
+  // the wave's base, so a wave loads whole token rows (the first K/8 lanes, one 16-byte chunk each) to the rows' padded
+  // places.  Token rows past the end are not requested: their rows of the buffer keep old data, and their products
+  // are never stored.
+  typedef __attribute__((address_space(3))) void* lds_ptr_t;
+  auto fetch = [&](int tile, int which) {
+    if (tile >= ntiles_t) return;
+    char* base = reinterpret_cast<char*>(buf + which * (32 * kRow));
 #pragma unroll
     for (int i = 0; i < kPer; ++i) {
-      const int c = tid + kThreads * i;
-      v[i] = u32x4_t{0u, 0u, 0u, 0u};
-      if (tile < ntiles_t && c < kChunks && tile * 32 + c / (K / 8) < T)
-        v[i] = *reinterpret_cast<const u32x4_t*>(A + (size_t)tile * (32 * K) + (size_t)c * 8);
+      const int row = i * kLinWaves + wave;
+      if (lane < kCols && tile * 32 + row < T)
+        __builtin_amdgcn_global_load_lds(A + (size_t)tile * (32 * K) + (size_t)row * K + lane * 8,
+                                         (lds_ptr_t)(base + row * (kRow * 2)), 16, 0, 0);
     }
   };
-  u32x4_t v[kPer];
-  fetch(worker, v);
-  int cur = 0;
-#ifdef VIG_TIMING
-  unsigned long long ph[6] = {0, 0, 0, 0, 0, 0}, last_ = __builtin_readcyclecounter();
-  const unsigned long long t_begin = last_;
-#endif
-  for (int tile = worker; tile < ntiles_t; tile += nworkers, cur ^= 1) {
-    uint16_t* mine = buf + cur * (32 * kRow);
+  f32x16_t g, u;
 #pragma unroll
-    for (int i = 0; i < kPer; ++i)
-      if (tid + kThreads * i < kChunks) *reinterpret_cast<u32x4_t*>(mine + lds_off[i]) = v[i];
-    VIG_LIN_T(0);
-    __syncthreads();  // the tile is staged; the other buffer was last read before the previous barrier
-    VIG_LIN_T(1);
-    fetch(tile + nworkers, v);
-    VIG_LIN_T(2);
-    f32x16_t g, u;
-#pragma unroll
-    for (int j = 0; j < 16; ++j) g[j] = 0.f, u[j] = 0.f;
-    const uint16_t* xrow = mine + r * kRow + 8 * h;
-#pragma unroll
-    for (int t = 0; t < KS; ++t) {
-      const u32x4_t x = *reinterpret_cast<const u32x4_t*>(xrow + 16 * t);
-      g = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, wg[t]), __builtin_bit_cast(bf16x8_t, x),
-                                                  g, 0, 0, 0);
-      u = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, wu[t]), __builtin_bit_cast(bf16x8_t, x),
-                                                  u, 0, 0, 0);
-    }
-    VIG_LIN_T(3);
-    // (no run-time branch between the matrix instructions and the first read of their results)
+  for (int j = 0; j < 16; ++j) g[j] = 0.f, u[j] = 0.f;
+  // SwiGLU on the rounded gate and up values of one finished tile, 16 consecutive channels of one token per lane
+  auto epilogue = [&](int etile) {
     u32x4_t lo, hi;
 #pragma unroll
     for (int j = 0; j < 8; ++j) {
@@ -128,14 +105,64 @@ __global__ __launch_bounds__(64 * kLinWaves) void linear_swiglu_kernel(const uin
       if (j < 4) lo[j] = pk;
       else hi[j - 4] = pk;
     }
-    const int token = tile * 32 + r;
+    const int token = etile * 32 + r;
     if (have && token < T) {
       uint16_t* dst = out + (size_t)token * I + 32 * ct + 16 * h;
       *reinterpret_cast<u32x4_t*>(dst) = lo;
       *reinterpret_cast<u32x4_t*>(dst + 8) = hi;
     }
+  };
+  // this tile's products: operand reads run kAhead k-steps ahead of the matrix instructions that use them
+  auto products = [&](const uint16_t* mine) {
+#pragma unroll
+    for (int j = 0; j < 16; ++j) g[j] = 0.f, u[j] = 0.f;
+    const uint16_t* xrow = mine + r * kRow + 8 * h;
+    constexpr int kAhead = 3;
+    u32x4_t x[kAhead];
+#pragma unroll
+    for (int t = 0; t < kAhead; ++t) x[t] = *reinterpret_cast<const u32x4_t*>(xrow + 16 * t);
+#pragma unroll
+    for (int t = 0; t < KS; ++t) {
+      const u32x4_t xt = x[t % kAhead];
+      g = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, wg[t]), __builtin_bit_cast(bf16x8_t, xt),
+                                                  g, 0, 0, 0);
+      u = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, wu[t]), __builtin_bit_cast(bf16x8_t, xt),
+                                                  u, 0, 0, 0);
+      if (t + kAhead < KS) x[t % kAhead] = *reinterpret_cast<const u32x4_t*>(xrow + 16 * (t + kAhead));
+      __builtin_amdgcn_sched_barrier(0);
+    }
+  };
+  fetch(worker, 0);
+  int cur = 0;
+#ifdef VIG_TIMING
+  unsigned long long ph[6] = {0, 0, 0, 0, 0, 0}, last_ = __builtin_readcyclecounter();
+  const unsigned long long t_begin = last_;
+#endif
+  for (int tile = worker; tile < ntiles_t; tile += nworkers, cur ^= 1) {
+    const uint16_t* mine = buf + cur * (32 * kRow);
+    __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): this thread's chunks of the tile have landed
+    VIG_LIN_T(0);
+    __syncthreads();  // the tile is complete; the other buffer was last read before the previous barrier
+    VIG_LIN_T(1);
+    fetch(tile + nworkers, cur ^ 1);
+    VIG_LIN_T(2);
+    // The two waves of a SIMD (w and w + 4) take turns on its two pipes: the lower wave runs this tile's matrix
+    // instructions first and its SwiGLU epilogue after; the upper wave first runs the epilogue of its PREVIOUS tile
+    // (its accumulators waited in registers) and then this tile's matrix instructions.  So one wave's vector work
+    // runs under the other's matrix work in both halves of a tile's time, with one barrier per tile as before.
+    if (wave < kLinWaves / 2) {
+      products(mine);
+      VIG_LIN_T(3);
+      epilogue(tile);  // (straight-line after the matrix instructions: no run-time branch in between)
+    } else {
+      if (tile > worker) epilogue(tile - nworkers);
+      VIG_LIN_T(3);
+      products(mine);
+    }
     VIG_LIN_T(4);
   }
+  if (wave >= kLinWaves / 2 && worker < ntiles_t)  // the upper waves' last tile
+    epilogue(worker + ((ntiles_t - 1 - worker) / nworkers) * nworkers);
 #ifdef VIG_TIMING
   if (blockIdx.x == 0 && lane == 0) {
     for (int i = 0; i < 5; ++i) g_lin_stamp[wave][i] = ph[i];
