@@ -453,6 +453,21 @@ int vig_linear_swiglu_fwd(const void* x, const void* weight, void* y, long long 
                           void* stream);
 
 /*
+ * vig_locality_blend_fwd and o_proj in one kernel, for square blocks with 64-channel heads at the widths whose weight
+ * tiles fit the registers (C = H*Dv = 384 or 192, the hidden sizes of ViG-S / ViG-T), bf16, fp32 accumulation:
+ *   out [B*L, C] = y . weight [C, H*Dv]^T with y the blend above, rounded to bf16 as vig_locality_blend_fwd stores
+ *   it; y itself is never written.  Arguments as in vig_locality_blend_fwd (Dv = 64, g_row_stride likewise);
+ *   weight and out packed row-major.  Other shapes or dtypes return VIG_ENOTSUP (make the two calls).
+ *
+ * Replaces: classification/models/vig.py:444-463 (head norms, sigmoid blend, out_act, o_proj) without the
+ * [B, L, H*Dv] intermediate.
+ */
+int vig_locality_blend_linear_fwd(const void* o, const void* local, const void* g_lin,
+                                  const float* w_g, const float* w_l, const void* weight, void* out,
+                                  int B, int H, int L, int Dv, int C, long long g_row_stride, float eps, int silu_out,
+                                  int io_dtype, void* stream);
+
+/*
  * First convolution of the v2 patch embedding, without its bias (vig_layernorm_fwd's pre_bias takes that):
  *   x [B, Cin, H, W] (bf16, the layout images arrive in)  ->  y [B, OH, OW, Cout] (bf16, channels-last rows),
  *   OH = (H + 2*padding - KH) / stride + 1, OW likewise.

@@ -138,6 +138,42 @@ def test_locality_blend(dtype, tol, H, Dv, L):
         assert torch.equal(got, got2)
 
 
+@pytest.mark.parametrize("B,H,L", [(2, 6, 196), (1, 3, 49), (3, 6, 37), (256, 6, 196), (1, 6, 1)])
+def test_locality_blend_linear(B, H, L):
+    """The blend and o_proj in one kernel against (a) an fp64 product of the stored (bf16-rounded) blend with the
+    weight -- the fused kernel feeds the matrix instructions exactly those values, so what remains is fp32 accumulation
+    and one rounding of the output -- and (b) the two library steps it replaces (vig_locality_blend_fwd, torch GEMM);
+    g_lin as a column block of a wider tensor gives the same bits."""
+    announce(f"blend + o_proj in one kernel B{B} H{H} L{L}")
+    Dv, C = 64, H * 64
+    dt = torch.bfloat16
+    o = _randn((B, H, L, Dv), 20, dt).cuda()
+    loc = _randn((B, L, C), 21, dt).cuda()
+    gl = _randn((B, L, C), 22, dt).cuda()
+    wg = (_randn((Dv,), 23) * 0.1 + 1).cuda()
+    wl = (_randn((Dv,), 24) * 0.1 + 1).cuda()
+    w = (_randn((C, C), 25, dt) * (C ** -0.5)).cuda()
+    assert vig_amd.ops.locality_blend_linear_supported(o, w)
+    for silu in (False, True):
+        got = vig_amd.ops.locality_blend_linear(o, loc, gl, wg, wl, w, 1e-6, silu)
+        assert tuple(got.shape) == (B, L, C)
+        y = vig_amd.locality_blend(o, loc, gl, wg, wl, 1e-6, silu)
+        two = torch.nn.functional.linear(y, w)
+        err2 = (got.double() - two.double()).abs() / two.double().abs().clamp_min(1.0)
+        assert err2.max().item() <= 2 * 2.0 ** -8, err2.max().item()
+        if B * L <= 1200:
+            want = f64(y) @ f64(w).T
+            err = np.abs(f64(got).reshape(-1, C) - want.reshape(-1, C)) / np.maximum(1.0, np.abs(want.reshape(-1, C)))
+            assert err.max() <= 2.0 ** -8, err.max()
+            ref = O.locality_blend_reference(f64(o), f64(loc), f64(gl), f64(wg), f64(wl), 1e-6, silu) @ f64(w).T
+            assert max_abs(f64(got), ref) <= 3e-2
+        wide = torch.zeros(B, L, C + 24, dtype=dt).cuda()
+        wide[..., 16:16 + C] = gl
+        assert torch.equal(vig_amd.ops.locality_blend_linear(o, loc, wide[..., 16:16 + C], wg, wl, w, 1e-6, silu), got)
+    assert not vig_amd.ops.locality_blend_linear_supported(o.float(), w.float())
+    assert not vig_amd.ops.locality_blend_linear_supported(o, w[:, :C - 64])
+
+
 # ---- the locality gate fused into the GLA kernel (vig_gla_bidir_locgate_fwd) ----
 def _gla_inputs(B, H, L, Dk, seed, gate_scale=None):
     from vig_amd.synthetic import make_gla_inputs

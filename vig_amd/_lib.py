@@ -49,6 +49,7 @@ SIGNATURES = {
     "vig_layernorm_fwd": (_c_int, [_c_void_p] * 4 + [_c_longlong, _c_int, _c_float, _c_int, _c_void_p, _c_void_p, _c_int, _c_int, _c_void_p]),
     "vig_rmsnorm_fwd": (_c_int, [_c_void_p] * 5 + [ctypes.c_longlong, _c_int, _c_float, _c_int, _c_int, _c_void_p]),
     "vig_split_heads_fwd": (_c_int, [_c_void_p] * 4 + [_c_int] * 5 + [_c_longlong, _c_int, _c_void_p]),
+    "vig_locality_blend_linear_fwd": (_c_int, [_c_void_p] * 7 + [_c_int] * 5 + [_c_longlong, _c_float, _c_int, _c_int, _c_void_p]),
     "vig_linear_swiglu_fwd": (_c_int, [_c_void_p] * 3 + [_c_longlong, _c_int, _c_int, _c_int, _c_void_p]),
     "vig_patch_conv_fwd": (_c_int, [_c_void_p] * 3 + [_c_int] * 10 + [_c_void_p]),
     "vig_locality_blend_bwd_workspace": (_c_size_t, [_c_int] * 3),

@@ -42,6 +42,10 @@ int launch_swiglu_bwd(const void* in, const void* dy, void* din, long long rows,
 size_t rmsnorm_bwd_workspace(long long rows, int C);
 int launch_rmsnorm_bwd(const void* s, const float* weight, const void* dy, const void* d_sum, void* ds, float* dweight,
                        void* workspace, long long rows, int C, float eps, int io_dtype, hipStream_t stream);
+bool blend_linear_supported(int H, int Dv, int C);
+int launch_blend_linear(const void* o, const void* loc, const void* glin, const float* w_g, const float* w_l,
+                        const void* W, void* out, int B, int H, int L, int Dv, int C, long long ldg, float eps,
+                        int silu_out, hipStream_t stream);
 bool linear_swiglu_supported(int K, int I);
 int launch_linear_swiglu(const void* A, const void* W, void* out, long long T, int K, int I, hipStream_t stream);
 bool patch_conv_supported(int Cin, int H, int W, int KH, int KW, int stride, int padding, int Cout);
@@ -484,6 +488,18 @@ int vig_patch_conv_fwd(const void* x, const void* w_packed, void* y, int B, int 
   if (!strided_rows_ok(x, W, io_dtype) || !strided_rows_ok(w_packed, 16, io_dtype) || !strided_rows_ok(y, Cout, io_dtype))
     return VIG_EINVAL;
   return vig::launch_patch_conv(x, w_packed, y, B, Cin, H, W, KH, KW, Cout, (hipStream_t)stream);
+}
+
+int vig_locality_blend_linear_fwd(const void* o, const void* local, const void* g_lin, const float* w_g,
+                                  const float* w_l, const void* weight, void* out, int B, int H, int L, int Dv, int C,
+                                  long long g_row_stride, float eps, int silu_out, int io_dtype, void* stream) {
+  if (!o || !local || !g_lin || !w_g || !w_l || !weight || !out || B <= 0 || H <= 0 || L <= 0) return VIG_EINVAL;
+  if (!aligned16(o, local, w_g, w_l, weight, out)) return VIG_EINVAL;
+  if (io_dtype != VIG_BF16 || !vig::blend_linear_supported(H, Dv, C)) return VIG_ENOTSUP;
+  const long long ldg = g_row_stride > 0 ? g_row_stride : (long long)H * Dv;
+  if (ldg < (long long)H * Dv || !strided_rows_ok(g_lin, ldg, io_dtype)) return VIG_EINVAL;
+  return vig::launch_blend_linear(o, local, g_lin, w_g, w_l, weight, out, B, H, L, Dv, C, ldg, eps, silu_out,
+                                  (hipStream_t)stream);
 }
 
 int vig_linear_swiglu_fwd(const void* x, const void* weight, void* y, long long rows, int K, int I, int io_dtype,

@@ -186,7 +186,205 @@ int launch_linear_swiglu_t(const void* A, const void* W, void* out, long long T,
   return hipGetLastError() == hipSuccess ? 0 : -5;
 }
 
+// ---------------------------------------------------------------------------
+// The mixer's epilogue and o_proj in one kernel:
+//   y[t, h, :] = rms(o[b, h, l, :]) w_g sigmoid(g) + rms(loc[t, h, :]) w_l (1 - sigmoid(g))   (optionally y <- y sigmoid(y)),
+//   out[t, :]  = y[t, :] . W[c, :]                                   (W = o_proj.weight [C, H*Dv], K = H*Dv = 16 * KS)
+// with t = b*L + l, the head norms over the Dv = 64 channels of a (token, head), g = g_lin rows of pitch ldg
+// (classification/models/vig.py:444-463).  y is rounded to bf16 as the separate blend kernel would store it and never
+// leaves the chip: the workgroup computes a 32-token tile of it straight into the LDS buffer the matrix instructions
+// read (double-buffered).  The o / loc / g octets of the next tile travel from memory straight into thread-private
+// LDS slots (no registers: lane i of a wave lands at the wave's slot base + 16 i) while the matrix instructions of the
+// current tile run.  NW waves hold TPW 32-channel tiles of W each as matrix-instruction operands for the life of the
+// workgroup, so one workgroup makes whole output rows (C = 32 * TPW * NW) and every tile of y is computed once.
+// ---------------------------------------------------------------------------
+template <int KS, int NW, int TPW>
+__global__ __launch_bounds__(64 * NW) void blend_linear_kernel(const uint16_t* __restrict__ o,
+                                                              const uint16_t* __restrict__ loc,
+                                                              const uint16_t* __restrict__ glin,
+                                                              const float* __restrict__ w_g,
+                                                              const float* __restrict__ w_l,
+                                                              const uint16_t* __restrict__ W,
+                                                              uint16_t* __restrict__ out, int T, int L, int H,
+                                                              long long ldg, float eps, int silu_out) {
+  constexpr int K = 16 * KS;
+  constexpr int C = 32 * TPW * NW;             // TPW 32-channel tiles of W per wave
+  constexpr int kThreads = 64 * NW;
+  constexpr int kCols = K / 8;                 // channel octets per token row
+  constexpr int kRow = K + 8;                  // LDS row stride in elements (conflict-free 16-byte reads)
+  constexpr int kChunks = 32 * kCols;          // channel octets of a 32-token tile
+  constexpr int kPer = kChunks / kThreads;     // octets per thread
+  static_assert(kChunks % kThreads == 0, "whole octets per thread");
+  static_assert(kThreads % kCols == 0, "a thread's octets share their column");
+  extern __shared__ __align__(16) char smem[];
+  uint16_t* buf = reinterpret_cast<uint16_t*>(smem);  // [2][32][kRow]
+  float* wnorm = reinterpret_cast<float*>(smem + (size_t)2 * 32 * kRow * sizeof(uint16_t));  // w_g | w_l, 64 floats each
+  // thread-private slots for the fetched octets of the tile that comes next: [octet i][o, loc, g][thread]
+  u32x4_t* park = reinterpret_cast<u32x4_t*>(smem + (size_t)2 * 32 * kRow * sizeof(uint16_t) + 128 * sizeof(float));
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int r = lane & 31, h = lane >> 5;
+  if (tid < 128) wnorm[tid] = tid < 64 ? w_g[tid] : w_l[tid - 64];
+  // matrix row i holds channel 16*((i>>2)&1) + 4*(i>>3) + (i&3) of the tile: lane (r, h) ends with channels 16h..16h+15
+  const int chan_of_row = 16 * ((r >> 2) & 1) + 4 * (r >> 3) + (r & 3);
+  u32x4_t wt[TPW][KS];  // channel tiles TPW * wave ..
+#pragma unroll
+  for (int j = 0; j < TPW; ++j) {
+    const uint16_t* pw = W + (size_t)(32 * (TPW * wave + j) + chan_of_row) * K + 8 * h;
+#pragma unroll
+    for (int t = 0; t < KS; ++t) wt[j][t] = *reinterpret_cast<const u32x4_t*>(pw + 16 * t);
+  }
+  const int ntiles_t = (T + 31) / 32;
+  const float* wg8 = wnorm + ((tid % kCols) & 7) * 8;  // (all octets of a thread lie in the same column)
+  const float* wl8 = wg8 + 64;
+  typedef __attribute__((address_space(3))) void* lds_ptr_t;
+  // requests this thread's octets of a tile into its slots; tokens past the end are not requested (their rows of y
+  // hold whatever the slots held: their products are never stored)
+  auto fetch = [&](int tile) {
+#pragma unroll 1
+    for (int i = 0; i < kPer; ++i) {  // (one octet's addresses at a time: the weight tiles leave few registers)
+      const int c = tid + kThreads * i;
+      const int row = c / kCols, col = c % kCols;
+      const long long t = (long long)tile * 32 + row;
+      if (tile < ntiles_t && t < T) {
+        const int b = (int)(t / L), l = (int)(t - (long long)b * L);
+        const int hd = col >> 3, d8 = col & 7;
+        char* slot = reinterpret_cast<char*>(park + (i * 3) * kThreads + wave * 64);  // (wave-uniform; lanes 16 B apart)
+        __builtin_amdgcn_global_load_lds(o + (((size_t)b * H + hd) * L + l) * 64 + d8 * 8, (lds_ptr_t)slot, 16, 0, 0);
+        __builtin_amdgcn_global_load_lds(loc + (size_t)t * K + col * 8, (lds_ptr_t)(slot + kThreads * 16), 16, 0, 0);
+        __builtin_amdgcn_global_load_lds(glin + (size_t)t * ldg + col * 8, (lds_ptr_t)(slot + 2 * kThreads * 16), 16, 0, 0);
+      }
+    }
+  };
+  const int nworkers = gridDim.x;
+  fetch(blockIdx.x);
+  __syncthreads();  // the norm weights are in place
+  int cur = 0;
+  for (int tile = blockIdx.x; tile < ntiles_t; tile += nworkers, cur ^= 1) {
+    uint16_t* mine = buf + cur * (32 * kRow);
+    __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): this tile's octets are in their slots
+    // ---- the blend of this tile, straight into the operand buffer ----
+#pragma unroll 1
+    for (int i = 0; i < kPer; ++i) {
+      const u32x4_t po = park[(i * 3 + 0) * kThreads + tid], pl = park[(i * 3 + 1) * kThreads + tid],
+                    pg = park[(i * 3 + 2) * kThreads + tid];
+      float fo[8], fl[8], fg[8];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        fo[2 * j] = bf16_to_f32((uint16_t)(po[j] & 0xffffu)), fo[2 * j + 1] = bf16_to_f32((uint16_t)(po[j] >> 16));
+        fl[2 * j] = bf16_to_f32((uint16_t)(pl[j] & 0xffffu)), fl[2 * j + 1] = bf16_to_f32((uint16_t)(pl[j] >> 16));
+        fg[2 * j] = bf16_to_f32((uint16_t)(pg[j] & 0xffffu)), fg[2 * j + 1] = bf16_to_f32((uint16_t)(pg[j] >> 16));
+      }
+      float so = 0.f, sl = 0.f;
+#pragma unroll
+      for (int j = 0; j < 8; ++j) so += fo[j] * fo[j], sl += fl[j] * fl[j];
+#pragma unroll
+      for (int m = 1; m < 8; m <<= 1) {
+        so += __shfl_xor(so, m, 64);
+        sl += __shfl_xor(sl, m, 64);
+      }
+      const float ro = rsqrtf(so * (1.0f / 64.0f) + eps);
+      const float rl = rsqrtf(sl * (1.0f / 64.0f) + eps);
+      u32x4_t y;
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        float e[2];
+#pragma unroll
+        for (int q = 0; q < 2; ++q) {
+          const int jj = 2 * j + q;
+          const float sg = sigmoidf_(fg[jj]);
+          float v = fo[jj] * ro * wg8[jj] * sg + fl[jj] * rl * wl8[jj] * (1.f - sg);
+          if (silu_out) v = v * sigmoidf_(v);
+          e[q] = v;
+        }
+        y[j] = pack_bf16x2(e[0], e[1]);
+      }
+      const int c = tid + kThreads * i;
+      *reinterpret_cast<u32x4_t*>(mine + (c / kCols) * kRow + (c % kCols) * 8) = y;
+    }
+    fetch(tile + nworkers);  // (this thread has read its slots)
+    __syncthreads();         // the tile is staged; the other buffer was last read before the previous barrier
+    f32x16_t acc[TPW];
+#pragma unroll
+    for (int j = 0; j < TPW; ++j)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) acc[j][e] = 0.f;
+    const uint16_t* xrow = mine + r * kRow + 8 * h;
+    constexpr int kAhead = TPW == 2 ? 3 : 1;  // operand reads this many k-steps ahead of the matrix instructions that
+                                              // use them, where the registers allow
+    u32x4_t x[kAhead];
+#pragma unroll
+    for (int t = 0; t < kAhead; ++t) x[t] = *reinterpret_cast<const u32x4_t*>(xrow + 16 * t);
+#pragma unroll
+    for (int t = 0; t < KS; ++t) {
+      const u32x4_t xt = x[t % kAhead];
+#pragma unroll
+      for (int j = 0; j < TPW; ++j)
+        acc[j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, wt[j][t]),
+                                                         __builtin_bit_cast(bf16x8_t, xt), acc[j], 0, 0, 0);
+      if (t + kAhead < KS) x[t % kAhead] = *reinterpret_cast<const u32x4_t*>(xrow + 16 * (t + kAhead));
+      if (TPW == 2) __builtin_amdgcn_sched_barrier(0);
+    }
+    // (no run-time branch between the matrix instructions and the first read of their results)
+    const int token = tile * 32 + r;
+#pragma unroll
+    for (int j = 0; j < TPW; ++j) {
+      u32x4_t lo, hi;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        lo[e] = pack_bf16x2(acc[j][2 * e], acc[j][2 * e + 1]);
+        hi[e] = pack_bf16x2(acc[j][8 + 2 * e], acc[j][8 + 2 * e + 1]);
+      }
+      if (token < T) {
+        uint16_t* dst = out + (size_t)token * C + 32 * (TPW * wave + j) + 16 * h;
+        *reinterpret_cast<u32x4_t*>(dst) = lo;
+        *reinterpret_cast<u32x4_t*>(dst + 8) = hi;
+      }
+    }
+  }
+}
+
+template <int KS, int NW, int TPW>
+int launch_blend_linear_t(const void* o, const void* loc, const void* glin, const float* w_g, const float* w_l,
+                          const void* W, void* out, long long T, int L, int H, long long ldg, float eps, int silu_out,
+                          int num_cu, int dev, hipStream_t stream) {
+  constexpr int K = 16 * KS;
+  const size_t lds = (size_t)2 * 32 * (K + 8) * sizeof(uint16_t) + 128 * sizeof(float) +
+                     (size_t)(32 * K / 8) * 3 * sizeof(u32x4_t);
+  const long long ntiles_t = (T + 31) / 32;
+  const int grid = ntiles_t < num_cu ? (int)ntiles_t : num_cu;
+  static bool attr_done[64] = {};
+  if (!attr_done[dev]) {  // (per device; concurrent first calls only repeat an idempotent setting)
+    if (hipFuncSetAttribute(reinterpret_cast<const void*>(blend_linear_kernel<KS, NW, TPW>),
+                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds) != hipSuccess)
+      return -5;
+    attr_done[dev] = true;
+  }
+  hipLaunchKernelGGL((blend_linear_kernel<KS, NW, TPW>), dim3(grid), dim3(64 * NW), lds, stream, (const uint16_t*)o,
+                     (const uint16_t*)loc, (const uint16_t*)glin, w_g, w_l, (const uint16_t*)W, (uint16_t*)out, (int)T, L,
+                     H, ldg, eps, silu_out);
+  return hipGetLastError() == hipSuccess ? 0 : -5;
+}
+
 }  // namespace
+
+// o_proj of a square block (d_model = H * Dv) with 64-channel heads, at the widths the weights fit the registers
+bool blend_linear_supported(int H, int Dv, int C) { return Dv == 64 && C == H * Dv && (C == 384 || C == 192); }
+
+int launch_blend_linear(const void* o, const void* loc, const void* glin, const float* w_g, const float* w_l,
+                        const void* W, void* out, int B, int H, int L, int Dv, int C, long long ldg, float eps,
+                        int silu_out, hipStream_t stream) {
+  if (!blend_linear_supported(H, Dv, C) || B <= 0 || L <= 0 || (long long)B * L > 0x7fffffffLL - 64 || ldg % 8 != 0 ||
+      ldg < C)
+    return -95;
+  int dev = 0, n = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return -5;
+  if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess) return -5;
+  const int num_cu = n > 0 ? n : 256;
+  const long long T = (long long)B * L;
+  // twelve waves with one weight tile each (three per SIMD at 168 registers) at the wider size, six at the narrower
+  return C == 384 ? launch_blend_linear_t<24, 12, 1>(o, loc, glin, w_g, w_l, W, out, T, L, H, ldg, eps, silu_out, num_cu, dev, stream)
+                  : launch_blend_linear_t<12, 6, 1>(o, loc, glin, w_g, w_l, W, out, T, L, H, ldg, eps, silu_out, num_cu, dev, stream);
+}
 
 bool linear_swiglu_supported(int K, int I) { return (K == 384 || K == 192) && I % 32 == 0 && I >= 32; }
 

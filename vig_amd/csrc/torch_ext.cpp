@@ -243,6 +243,37 @@ Tensor locality_gate_fwd(const Tensor& o, const Tensor& weight, int64_t h, int64
   return y;
 }
 
+// o_proj(locality_blend(...)) in one kernel where the library builds it (bf16, 64-channel heads, square o_proj of
+// width 384 or 192); the two steps otherwise.
+Tensor locality_blend_fwd(const Tensor& o, const Tensor& local, const Tensor& g_lin, const Tensor& w_g, const Tensor& w_l,
+                          double eps, bool silu_out);
+Tensor locality_blend_linear_fwd(const Tensor& o, const Tensor& local, const Tensor& g_lin, const Tensor& w_g,
+                                 const Tensor& w_l, const Tensor& weight, double eps, bool silu_out) {
+  TORCH_CHECK(o.dim() == 4 && weight.dim() == 2, "vig_amd: o must be [B, H, L, Dv], weight [C, H*Dv]");
+  const int64_t B = o.size(0), H = o.size(1), L = o.size(2), Dv = o.size(3), C = weight.size(0);
+  const bool fused = o.scalar_type() == at::kBFloat16 && weight.scalar_type() == at::kBFloat16 && Dv == 64 &&
+                     weight.size(1) == H * Dv && C == H * Dv && (C == 384 || C == 192) && weight.is_contiguous() &&
+                     reinterpret_cast<uintptr_t>(weight.data_ptr()) % 16 == 0;
+  if (!fused) return at::linear(locality_blend_fwd(o, local, g_lin, w_g, w_l, eps, silu_out), weight);
+  check_dense(o, o, "o");
+  check_dense(local, o, "local");
+  const int64_t ldg = token_row_stride(g_lin, o, "g_lin");
+  TORCH_CHECK(local.dim() == 3 && local.size(0) == B && local.size(1) == L && local.size(2) == H * Dv &&
+                  g_lin.size(0) == B && g_lin.size(1) == L && g_lin.size(2) == H * Dv,
+              "vig_amd: local and g_lin must be [B, L, H*Dv]");
+  TORCH_CHECK(local.scalar_type() == o.scalar_type() && g_lin.scalar_type() == o.scalar_type(),
+              "vig_amd: o, local, g_lin must share a dtype");
+  check_f32_vec(w_g, o, Dv, "w_g");
+  check_f32_vec(w_l, o, Dv, "w_l");
+  const c10::DeviceGuard guard(o.device());
+  Tensor out = at::empty({B, L, C}, o.options());
+  check_rc(vig_locality_blend_linear_fwd(o.data_ptr(), local.data_ptr(), g_lin.data_ptr(), w_g.data_ptr<float>(),
+                                         w_l.data_ptr<float>(), weight.data_ptr(), out.data_ptr(), (int)B, (int)H, (int)L,
+                                         (int)Dv, (int)C, ldg, (float)eps, silu_out ? 1 : 0, dt(o), stream_of(o)),
+           "vig_locality_blend_linear_fwd");
+  return out;
+}
+
 Tensor locality_blend_fwd(const Tensor& o, const Tensor& local, const Tensor& g_lin, const Tensor& w_g, const Tensor& w_l,
                           double eps, bool silu_out) {
   TORCH_CHECK(o.dim() == 4, "vig_amd: o must be [B, H, L, Dv]");
@@ -401,8 +432,7 @@ Tensor gla_block_mix(const Tensor& x, int64_t grid_h, int64_t grid_w, const Tens
     o = gla_bidir_fwd(std::get<0>(qkv), std::get<1>(qkv), std::get<2>(qkv), gates.select(0, 0), gates.select(0, 1), -1.0,
                       out_scale, 0);
   }
-  Tensor y = locality_blend_fwd(o, xs, z.narrow(-1, n0, H * Dv), w_gnorm, w_lnorm, eps, out_act);
-  return at::linear(y, w_o);
+  return locality_blend_linear_fwd(o, xs, z.narrow(-1, n0, H * Dv), w_gnorm, w_lnorm, w_o, eps, out_act);
 }
 
 // One eval-mode GLA block in the carried form (classification/models/vig.py:582-608 with the closing residual add of
@@ -458,6 +488,9 @@ TORCH_LIBRARY(vig_amd, m) {
         &split_heads_fwd);
   m.def("swiglu_fwd(Tensor gate_up) -> Tensor", &swiglu_fwd);
   m.def("linear_swiglu_fwd(Tensor x, Tensor weight) -> Tensor", &linear_swiglu_fwd);
+  m.def("locality_blend_linear_fwd(Tensor o, Tensor local, Tensor g_lin, Tensor w_g, Tensor w_l, Tensor weight, float eps, "
+        "bool silu_out) -> Tensor",
+        &locality_blend_linear_fwd);
   m.def("patch_conv_fwd(Tensor x, Tensor w_packed, int kh, int kw, int stride, int padding) -> Tensor", &patch_conv_fwd);
   m.def("gla_block_mix(Tensor x, int grid_h, int grid_w, Tensor conv_w, Tensor? conv_b, bool act_in_conv, Tensor w_in, Tensor b_in, int num_heads, int head_qk_dim, int head_v_dim, Tensor w_up, Tensor b_up, float normalizer, float? clamp_min, Tensor w_gnorm, Tensor w_lnorm, float eps, bool out_act, Tensor w_o, float out_scale) -> Tensor",
         &gla_block_mix);

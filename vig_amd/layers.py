@@ -234,6 +234,9 @@ class GatedLinearAttention(_CacheMixin, nn.Module):
         else:
             gates = ops.dirgate(up(gk_low), H, self.gate_logit_normalizer, self.clamp_min)
         o = ops.gla_bidir_forward(q, k, v, gates[0], gates[1], scale=-1, out_scale=out_scale)
+        if ops.locality_blend_linear_supported(o, self.o_proj.weight):  # ViG-S / ViG-T widths: no blended intermediate
+            return ops.locality_blend_linear(o, xs, g_lin, self.g_norm._w32(), self.l_norm._w32(), self.o_proj.weight,
+                                             eps=self.layernorm_eps, silu_out=self.use_out_act)
         y = ops.locality_blend(o, xs, g_lin, self.g_norm._w32(), self.l_norm._w32(),
                                eps=self.layernorm_eps, silu_out=self.use_out_act)
         return self.o_proj(y)

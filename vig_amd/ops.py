@@ -594,6 +594,41 @@ def _locality_blend_raw(o, local, g_lin, w_g, w_l, eps, silu_out):
     return y
 
 
+def locality_blend_linear_supported(o: torch.Tensor, weight: torch.Tensor) -> bool:
+    """Whether locality_blend_linear takes this block (bf16 on the GPU, 64-channel heads, square o_proj of width 384 or
+    192)."""
+    return (o.is_cuda and o.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16 and o.dim() == 4
+            and o.shape[-1] == 64 and weight.dim() == 2 and weight.shape[0] == weight.shape[1] == o.shape[1] * 64
+            and weight.shape[0] in (384, 192))
+
+
+def locality_blend_linear(o: torch.Tensor, local: torch.Tensor, g_lin: torch.Tensor, w_g: torch.Tensor,
+                          w_l: torch.Tensor, weight: torch.Tensor, eps: float = 1e-6,
+                          silu_out: bool = False) -> torch.Tensor:
+    """o_proj(locality_blend(...)) in one kernel (vig.py:444-463): the blended [B, L, H*Dv] tensor, rounded to bf16
+    as locality_blend stores it, feeds the matrix instructions from on-chip memory and is never written.
+    Inference only (no autograd node)."""
+    lib = _lib.load()
+    _check_cuda(o, local, g_lin, w_g, w_l, weight)
+    o, local, w = _dense(o), _dense(local), _dense(weight.detach())
+    g_lin, ldg = _token_rows(g_lin)
+    B, H, L, Dv = o.shape
+    if local.shape != (B, L, H * Dv) or g_lin.shape != (B, L, H * Dv):
+        raise ValueError("local and g_lin must be [B, L, H*Dv]")
+    if not (local.dtype == g_lin.dtype == w.dtype == o.dtype):
+        raise TypeError("o, local, g_lin and weight must share a dtype")
+    C = w.shape[0]
+    out = torch.empty(B, L, C, dtype=o.dtype, device=o.device)
+    wg = _dense(w_g.detach().float())
+    wl = _dense(w_l.detach().float())
+    with torch.cuda.device(o.device):
+        rc = lib.vig_locality_blend_linear_fwd(o.data_ptr(), local.data_ptr(), g_lin.data_ptr(), wg.data_ptr(),
+                                               wl.data_ptr(), w.data_ptr(), out.data_ptr(), B, H, L, Dv, C, ldg,
+                                               float(eps), int(silu_out), _dt(o), _stream_ptr(o))
+    _lib.check(rc, "vig_locality_blend_linear_fwd")
+    return out
+
+
 def rmsnorm(x: torch.Tensor, weight: torch.Tensor, eps: float = 1e-6, residual: Optional[torch.Tensor] = None,
             prenorm: bool = False, round_sum: bool = False):
     """Residual-add + RMS norm over the last dimension (fla/modules/rmsnorm.py:69-125 semantics).
