@@ -198,6 +198,17 @@ int launch_linear_swiglu_t(const void* A, const void* W, void* out, long long T,
 // current tile run.  NW waves hold TPW 32-channel tiles of W each as matrix-instruction operands for the life of the
 // workgroup, so one workgroup makes whole output rows (C = 32 * TPW * NW) and every tile of y is computed once.
 // ---------------------------------------------------------------------------
+// value of the lane a DPP control names (inside a row of 16 lanes)
+template <int CTRL>
+__device__ __forceinline__ float lane_permuted(float v) {
+  return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xf, 0xf, true));
+}
+
+// This wave's LDS writes done, then the barrier, and nothing else: global requests and stores issued before it stay in
+// flight.  (A fence would drain them: the compiler counts loads that land in LDS as LDS writes.  Whoever reads what
+// such a load brings waits for it by itself.)
+__device__ __forceinline__ void tile_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
+
 template <int KS, int NW, int TPW>
 __global__ __launch_bounds__(64 * NW) void blend_linear_kernel(const uint16_t* __restrict__ o,
                                                               const uint16_t* __restrict__ loc,
@@ -234,22 +245,23 @@ __global__ __launch_bounds__(64 * NW) void blend_linear_kernel(const uint16_t* _
     for (int t = 0; t < KS; ++t) wt[j][t] = *reinterpret_cast<const u32x4_t*>(pw + 16 * t);
   }
   const int ntiles_t = (T + 31) / 32;
-  const float* wg8 = wnorm + ((tid % kCols) & 7) * 8;  // (all octets of a thread lie in the same column)
+  const float* wg8 = wnorm + ((tid % kCols) & 7) * 8;  // (kThreads % kCols == 0: a thread's octets share their column)
   const float* wl8 = wg8 + 64;
   typedef __attribute__((address_space(3))) void* lds_ptr_t;
   // requests this thread's octets of a tile into its slots; tokens past the end are not requested (their rows of y
   // hold whatever the slots held: their products are never stored)
+  const int col = tid % kCols, row0 = tid / kCols;  // this thread's octets: column col of rows row0 + kRowStep * i
+  constexpr int kRowStep = kThreads / kCols;
+  const size_t o_col = ((size_t)(col >> 3) * L) * 64 + (col & 7) * 8;  // head col / 8, channels 8 (col % 8) ..
+  const size_t o_batch = (size_t)H * L * 64;
   auto fetch = [&](int tile) {
 #pragma unroll 1
     for (int i = 0; i < kPer; ++i) {  // (one octet's addresses at a time: the weight tiles leave few registers)
-      const int c = tid + kThreads * i;
-      const int row = c / kCols, col = c % kCols;
-      const long long t = (long long)tile * 32 + row;
+      const int t = tile * 32 + row0 + kRowStep * i;
       if (tile < ntiles_t && t < T) {
-        const int b = (int)(t / L), l = (int)(t - (long long)b * L);
-        const int hd = col >> 3, d8 = col & 7;
+        const unsigned b = (unsigned)t / (unsigned)L, l = (unsigned)t - b * (unsigned)L;
         char* slot = reinterpret_cast<char*>(park + (i * 3) * kThreads + wave * 64);  // (wave-uniform; lanes 16 B apart)
-        __builtin_amdgcn_global_load_lds(o + (((size_t)b * H + hd) * L + l) * 64 + d8 * 8, (lds_ptr_t)slot, 16, 0, 0);
+        __builtin_amdgcn_global_load_lds(o + b * o_batch + (size_t)l * 64 + o_col, (lds_ptr_t)slot, 16, 0, 0);
         __builtin_amdgcn_global_load_lds(loc + (size_t)t * K + col * 8, (lds_ptr_t)(slot + kThreads * 16), 16, 0, 0);
         __builtin_amdgcn_global_load_lds(glin + (size_t)t * ldg + col * 8, (lds_ptr_t)(slot + 2 * kThreads * 16), 16, 0, 0);
       }
@@ -273,29 +285,27 @@ __global__ __launch_bounds__(64 * NW) void blend_linear_kernel(const uint16_t* _
       float so = 0.f, sl = 0.f;
 #pragma unroll
       for (int j = 0; j < 8; ++j) so += fo[j] * fo[j], sl += fl[j] * fl[j];
-#pragma unroll
-      for (int m = 1; m < 8; m <<= 1) {
-        so += __shfl_xor(so, m, 64);
-        sl += __shfl_xor(sl, m, 64);
-      }
+      // the eight lanes of a (token, head): lane ^ 1, lane ^ 2 inside the quad, then the other quad of the eight
+      so += lane_permuted<0xB1>(so), sl += lane_permuted<0xB1>(sl);    // quad_perm:[1,0,3,2]
+      so += lane_permuted<0x4E>(so), sl += lane_permuted<0x4E>(sl);    // quad_perm:[2,3,0,1]
+      so += lane_permuted<0x141>(so), sl += lane_permuted<0x141>(sl);  // row_half_mirror
       const float ro = rsqrtf(so * (1.0f / 64.0f) + eps);
       const float rl = rsqrtf(sl * (1.0f / 64.0f) + eps);
+      float e[8];
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        const float sg = sigmoidf_(fg[j]);
+        e[j] = fo[j] * ro * wg8[j] * sg + fl[j] * rl * wl8[j] * (1.f - sg);
+      }
+      if (silu_out) {
+        asm volatile("");  // (a real branch: as a select, the second sigmoid is computed for every caller)
+#pragma unroll
+        for (int j = 0; j < 8; ++j) e[j] = e[j] * sigmoidf_(e[j]);
+      }
       u32x4_t y;
 #pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        float e[2];
-#pragma unroll
-        for (int q = 0; q < 2; ++q) {
-          const int jj = 2 * j + q;
-          const float sg = sigmoidf_(fg[jj]);
-          float v = fo[jj] * ro * wg8[jj] * sg + fl[jj] * rl * wl8[jj] * (1.f - sg);
-          if (silu_out) v = v * sigmoidf_(v);
-          e[q] = v;
-        }
-        y[j] = pack_bf16x2(e[0], e[1]);
-      }
-      const int c = tid + kThreads * i;
-      *reinterpret_cast<u32x4_t*>(mine + (c / kCols) * kRow + (c % kCols) * 8) = y;
+      for (int j = 0; j < 4; ++j) y[j] = pack_bf16x2(e[2 * j], e[2 * j + 1]);
+      *reinterpret_cast<u32x4_t*>(mine + (row0 + kRowStep * i) * kRow + col * 8) = y;
     }
   };
   // this wave's products of a staged tile, and its rows of the result
@@ -346,7 +356,7 @@ __global__ __launch_bounds__(64 * NW) void blend_linear_kernel(const uint16_t* _
   fetch(blockIdx.x);
   blend(buf);
   fetch(blockIdx.x + nworkers);
-  __syncthreads();
+  tile_barrier();
   int cur = 0;
   for (int tile = blockIdx.x; tile < ntiles_t; tile += nworkers, cur ^= 1) {
     const uint16_t* mine = buf + cur * (32 * kRow);
@@ -365,7 +375,7 @@ __global__ __launch_bounds__(64 * NW) void blend_linear_kernel(const uint16_t* _
       }
       products(mine, tile);
     }
-    __syncthreads();
+    tile_barrier();  // (the requests for the tile after the next and this tile's stores stay in flight)
   }
 }
 
