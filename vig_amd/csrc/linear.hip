@@ -19,23 +19,6 @@
 
 namespace vig {
 
-// Optional phase timing (development builds only: -DVIG_TIMING): cycles per phase, summed over the tiles of workgroup 0.
-#ifdef VIG_TIMING
-__device__ unsigned long long g_lin_stamp[8][8];
-#define VIG_LIN_T(i)                                             \
-  do {                                                           \
-    __builtin_amdgcn_sched_barrier(0);                           \
-    const unsigned long long now_ = __builtin_readcyclecounter(); \
-    ph[i] += now_ - last_;                                       \
-    last_ = now_;                                                \
-    __builtin_amdgcn_sched_barrier(0);                           \
-  } while (0)
-#else
-#define VIG_LIN_T(i) \
-  do {               \
-  } while (0)
-#endif
-
 namespace {
 
 constexpr int kLinWaves = 8;
@@ -134,41 +117,25 @@ __global__ __launch_bounds__(64 * kLinWaves) void linear_swiglu_kernel(const uin
   };
   fetch(worker, 0);
   int cur = 0;
-#ifdef VIG_TIMING
-  unsigned long long ph[6] = {0, 0, 0, 0, 0, 0}, last_ = __builtin_readcyclecounter();
-  const unsigned long long t_begin = last_;
-#endif
   for (int tile = worker; tile < ntiles_t; tile += nworkers, cur ^= 1) {
     const uint16_t* mine = buf + cur * (32 * kRow);
     __builtin_amdgcn_s_waitcnt(0x0F70);  // vmcnt(0): this thread's chunks of the tile have landed
-    VIG_LIN_T(0);
     __syncthreads();  // the tile is complete; the other buffer was last read before the previous barrier
-    VIG_LIN_T(1);
     fetch(tile + nworkers, cur ^ 1);
-    VIG_LIN_T(2);
     // The two waves of a SIMD (w and w + 4) take turns on its two pipes: the lower wave runs this tile's matrix
     // instructions first and its SwiGLU epilogue after; the upper wave first runs the epilogue of its PREVIOUS tile
     // (its accumulators waited in registers) and then this tile's matrix instructions.  So one wave's vector work
     // runs under the other's matrix work in both halves of a tile's time, with one barrier per tile as before.
     if (wave < kLinWaves / 2) {
       products(mine);
-      VIG_LIN_T(3);
       epilogue(tile);  // (straight-line after the matrix instructions: no run-time branch in between)
     } else {
       if (tile > worker) epilogue(tile - nworkers);
-      VIG_LIN_T(3);
       products(mine);
     }
-    VIG_LIN_T(4);
   }
   if (wave >= kLinWaves / 2 && worker < ntiles_t)  // the upper waves' last tile
     epilogue(worker + ((ntiles_t - 1 - worker) / nworkers) * nworkers);
-#ifdef VIG_TIMING
-  if (blockIdx.x == 0 && lane == 0) {
-    for (int i = 0; i < 5; ++i) g_lin_stamp[wave][i] = ph[i];
-    g_lin_stamp[wave][5] = __builtin_readcyclecounter() - t_begin;
-  }
-#endif
 }
 
 template <int KS>
@@ -441,8 +408,3 @@ int launch_linear_swiglu(const void* A, const void* W, void* out, long long T, i
 
 }  // namespace vig
 
-#ifdef VIG_TIMING
-extern "C" int vig_debug_read_lin_stamps(unsigned long long* host_out) {
-  return hipMemcpyFromSymbol(host_out, HIP_SYMBOL(vig::g_lin_stamp), sizeof(vig::g_lin_stamp)) == hipSuccess ? 0 : -5;
-}
-#endif
