@@ -223,7 +223,7 @@ __global__ __launch_bounds__(256) void dirgate_lowrank_kernel(const TI* __restri
         const float x = Stored<TI>::of(acc[j] + bias[j]);
         float yv = logsigmoidf_(x);
         yv *= inv_norm;
-        if (use_clamp) yv = fmaxf(yv, clamp_min);
+        yv = fmaxf(yv, clamp_min);  // (no clamp: clamp_min is NaN and fmaxf returns the other operand)
         acc[j] = yv;
       }
       Vec8<TO>::store(dst + (size_t)l * Dk, acc);
@@ -246,6 +246,7 @@ __global__ __launch_bounds__(256) void dirgate_lowrank_mfma_kernel(const uint16_
                                                                     int H, int Dk, float inv_norm, float clamp_min,
                                                                     int use_clamp) {
   constexpr int R = kGateRank;
+  (void)use_clamp;  // (a NaN clamp_min already means "no clamp" to fmaxf)
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int r = lane & 31, h = lane >> 5;
   // NTG groups of 32 tokens per workgroup: their low-rank rows are fetched first, a weight tile serves all of them
@@ -264,21 +265,30 @@ __global__ __launch_bounds__(256) void dirgate_lowrank_mfma_kernel(const uint16_
   const int chan_of_row = 16 * ((r >> 2) & 1) + 4 * (r >> 3) + (r & 3);
   const int ntiles = 2 * H * Dk / 32;
   const size_t dir_stride = (size_t)B * H * L * Dk;
+  // a tile's weights and biases are requested one tile ahead (a wave walks tiles wave, wave + 4, ...)
+  auto request = [&](int tile, u32x4_t& wa, u32x4_t& blo, u32x4_t& bhi) {
+    const int c0 = min(tile, ntiles - 1) * 32;
+    wa = *reinterpret_cast<const u32x4_t*>(w1 + (size_t)(c0 + chan_of_row) * R + 8 * h);
+    blo = *reinterpret_cast<const u32x4_t*>(b1 + c0 + 16 * h);
+    bhi = *reinterpret_cast<const u32x4_t*>(b1 + c0 + 16 * h + 8);
+  };
+  u32x4_t wa_next, blo_next, bhi_next;
+  request(wave, wa_next, blo_next, bhi_next);
+  const float inv_dk = 1.0f / (float)Dk, inv_h = 1.0f / (float)H;
   for (int tile = wave; tile < ntiles; tile += 4) {
     const int c0 = tile * 32;
-    const u32x4_t wa = *reinterpret_cast<const u32x4_t*>(w1 + (size_t)(c0 + chan_of_row) * R + 8 * h);
+    const u32x4_t wa = wa_next, blo = blo_next, bhi = bhi_next;
+    request(tile + 4, wa_next, blo_next, bhi_next);
     float bias[16];
-    {
-      float x[8];
-      Vec8<uint16_t>::load(b1 + c0 + 16 * h, x);
 #pragma unroll
-      for (int j = 0; j < 8; ++j) bias[j] = x[j];
-      Vec8<uint16_t>::load(b1 + c0 + 16 * h + 8, x);
-#pragma unroll
-      for (int j = 0; j < 8; ++j) bias[8 + j] = x[j];
+    for (int j = 0; j < 4; ++j) {
+      bias[2 * j] = bf16lo_to_f32(blo[j]), bias[2 * j + 1] = bf16hi_to_f32(blo[j]);
+      bias[8 + 2 * j] = bf16lo_to_f32(bhi[j]), bias[8 + 2 * j + 1] = bf16hi_to_f32(bhi[j]);
     }
     const int c = c0 + 16 * h;  // first of this lane's 16 channels
-    const int d = c % Dk, hh = (c / Dk) % H, dir = c / (Dk * H);
+    // (quotients by float reciprocals: exact for channel numbers below 2^20, a fraction of the integer division's cost)
+    const int cd = (int)(((float)c + 0.5f) * inv_dk), d = c - cd * Dk;
+    const int dir = (int)(((float)cd + 0.5f) * inv_h), hh = cd - dir * H;
     TO* const dst0 = out + (size_t)dir * dir_stride + (size_t)hh * L * Dk + d;
 #pragma unroll
     for (int g = 0; g < NTG; ++g) {
@@ -293,7 +303,7 @@ __global__ __launch_bounds__(256) void dirgate_lowrank_mfma_kernel(const uint16_
         const float x = Stored<uint16_t>::of(acc[j] + bias[j]);
         float yv = logsigmoidf_(x);
         yv *= inv_norm;
-        if (use_clamp) yv = fmaxf(yv, clamp_min);
+        yv = fmaxf(yv, clamp_min);  // (no clamp: clamp_min is NaN and fmaxf returns the other operand)
         if (j < 8) lo[j] = yv;
         else hi[j - 8] = yv;
       }
@@ -320,7 +330,7 @@ int launch_dirgate_lowrank(const void* low, long long ld, const void* w1, const 
                            int H, int Dk, int rank, float inv_norm, float clamp_min, int in_dtype, int out_dtype,
                            hipStream_t stream) {
   if (rank != kGateRank) return -95;
-  if (in_dtype == 1 && Dk % 16 == 0 && (long long)B * L < 0x7fffffffLL - 64) {
+  if (in_dtype == 1 && Dk % 16 == 0 && (long long)B * L < 0x7fffffffLL - 64 && 2LL * H * Dk <= (1 << 20)) {
     const int use_clamp = clamp_min == clamp_min;  // NaN disables
     const long long ntok = (long long)B * L;
     constexpr int kGroups = 1;  // token groups of 32 per workgroup (two measured no faster)
