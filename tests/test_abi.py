@@ -53,8 +53,10 @@ def test_argument_validation_without_gpu():
     # more (sequence, direction) pairs than the long-sequence scan's grid takes
     assert lib.vig_gla_bidir_fwd(one, one, one, one, one, one, one, 1 << 40, 40000, 2, 300, 64, 64, 1.0, 1.0, 1, 1,
                                  None) == -95
-    assert lib.vig_gla_bidir_fwd(one, one, one, one, None, one, one, 1 << 40, 40000, 1, 300, 64, 64, 1.0, 1.0, 1, 1,
-                                 None) != -95  # one direction: 40000 pairs fit (a workspace error or success path)
+    # one direction: 40000 pairs fit the grid, so the call gets as far as the workspace check, which refuses it (no
+    # workspace is offered: a call on dummy addresses must never reach a launch)
+    assert lib.vig_gla_bidir_fwd(one, one, one, one, None, one, None, 0, 40000, 1, 300, 64, 64, 1.0, 1.0, 1, 1,
+                                 None) == -28
     big = 1 << 40
     assert lib.vig_gla_bidir_bwd(one, one, one, one, one, one, one, one, one, one, one, one, big, 70000, 70000, 8, 64,
                                  64, 1.0, 1.0, 1, 1, None) == -22
