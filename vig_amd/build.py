@@ -15,7 +15,7 @@ OBJ = os.path.join(CSRC, "build")
 LIBDIR = os.path.join(HERE, "lib")
 LIB = os.path.join(LIBDIR, "libvig_gla.so")
 
-SOURCES = ["api.hip", "gla_recurrent.hip", "gla_mfma.hip", "gates.hip", "block.hip", "gla_backward.hip", "gla_backward_mfma.hip", "patch_conv.hip", "linear.hip"]
+SOURCES = ["api.hip", "gla_recurrent.hip", "gla_mfma.hip", "gla_tiles.hip", "gates.hip", "block.hip", "gla_backward.hip", "gla_backward_mfma.hip", "patch_conv.hip", "linear.hip"]
 
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 # -packed-fp32-ops is switched off: the compiler must not form packed fp32 VALU ops.

@@ -39,6 +39,7 @@
 #include "common.h"
 #include "launch.h"
 #include "mfma_tiles.h"
+#include <stdlib.h>
 
 namespace vig {
 
@@ -65,32 +66,6 @@ constexpr int kLdsGateW = kLdsVeto + 16;          // fused locality gate: the 64
 constexpr int kLdsHalf16 = kLdsGateW + 64 * 9 * 4;  // per wave: 64 half decays exp(G_end/2) as fp16, channel order
 constexpr int kLdsTotal = kLdsHalf16 + 8 * 64 * 2;
 
-typedef _Float16 f16x2_t __attribute__((ext_vector_type(2)));
-typedef _Float16 f16x8_t __attribute__((ext_vector_type(8)));
-__device__ __forceinline__ f32x16_t mfma_f16(const u32x4_t& a, const u32x4_t& b, const f32x16_t& c) {
-  return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8_t, a), __builtin_bit_cast(f16x8_t, b), c, 0,
-                                                0, 0);
-}
-__device__ __forceinline__ uint32_t pack_f16x2(float lo, float hi) {
-  f32x2_t x = {lo, hi};
-  f16x2_t y = __builtin_convertvector(x, f16x2_t);  // round to nearest even
-  return __builtin_bit_cast(uint32_t, y);
-}
-// elementwise product of two fp16 pairs (operands by value: a bit cast straight from a vector element reads the
-// vector's first word)
-__device__ __forceinline__ uint32_t mul_f16x2(uint32_t a, uint32_t b) {
-  return __builtin_bit_cast(uint32_t, __builtin_bit_cast(f16x2_t, a) * __builtin_bit_cast(f16x2_t, b));
-}
-
-// Magnitude guard of the fp16 score variant.  Raw bf16 rows go through a 16x16x32 matrix instruction as both
-// operands: whatever the slot assignment, the result is a Gram matrix whose diagonal entries are sums of squares that
-// cover every value fed in and whose other entries are no larger than the largest diagonal one.  Eight passes and four
-// accumulator registers per step, no vector work until the one comparison at the end.
-typedef float f32x4acc_t __attribute__((ext_vector_type(4)));
-__device__ __forceinline__ void gram_acc(const u32x4_t& raw, f32x4acc_t& acc) {
-  acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, raw), __builtin_bit_cast(bf16x8_t, raw), acc,
-                                                0, 0, 0);
-}
 // The fp16 variant rounds q~ = q 2^x and k~ = k 2^-x (|x| <= kFastHalfRange = 6), the scores P = q~ . k~ and V to fp16.
 // With every row's sum of squares below 2^15 (the guard sums the rows of two tokens of q, k and V, which only makes it
 // stricter), elements stay below 182, the scaled operands below 182 * 64, and |P| <= |q_i| |k_j| below 2^15: all
@@ -99,39 +74,6 @@ constexpr float kFastMaxSquares = 32768.0f;
 __device__ __forceinline__ bool gram_too_large(const f32x4acc_t& acc) {
   const float m = fmaxf(fmaxf(fabsf(acc[0]), fabsf(acc[1])), fmaxf(fabsf(acc[2]), fabsf(acc[3])));
   return __builtin_amdgcn_ballot_w64(!(m < kFastMaxSquares)) != 0;
-}
-
-template <int NG>
-struct HalfOps {
-  u32x4_t h[NG], l[NG];  // bf16 hi / lo fragments of one 32-token tile, per k-step (16 channels)
-};
-
-// q~ (ISQ) or k~ of one 32-token tile: raw * exp(+-(G - G_end)), split into bf16 hi (round to nearest) and
-// lo (the fp32 remainder, rounded).  Padding rows arrive as zeros and stay zero (their exponents are finite).
-template <bool ISQ, int NG>
-__device__ __forceinline__ void make_half(const u32x4_t (&raw)[NG], const f32x16_t (&G)[2],
-                                          const float* gend2 /* LDS, this lane half: [p][16] */, HalfOps<NG>& op) {
-#pragma unroll
-  for (int g = 0; g < NG; ++g) {
-    const f32x4_t a0 = *reinterpret_cast<const f32x4_t*>(gend2 + 4 * g);
-    const f32x4_t a1 = *reinterpret_cast<const f32x4_t*>(gend2 + 16 + 4 * g);
-#pragma unroll
-    for (int m = 0; m < 4; ++m) {
-      const int c = 4 * g + m;
-      const uint32_t w = raw[g][m];
-      float t[2];
-#pragma unroll
-      for (int p = 0; p < 2; ++p) {
-        const float an = p ? a1[m] : a0[m];
-        const float x = ISQ ? __builtin_fmaf(G[p][c], kLog2e, -an) : __builtin_fmaf(G[p][c], -kLog2e, an);
-        const float f = p ? bf16hi_to_f32(w) : bf16lo_to_f32(w);
-        t[p] = f * exp2_fast(x);
-      }
-      const uint32_t hi = pack_bf16x2(t[0], t[1]);
-      op.h[g][m] = hi;
-      op.l[g][m] = pack_bf16x2(t[0] - bf16lo_to_f32(hi), t[1] - bf16hi_to_f32(hi));
-    }
-  }
 }
 
 // q~ and k~ of one 32-token tile for the fp16 score path: one exponent per element serves both (the factors are
@@ -170,28 +112,6 @@ __device__ __forceinline__ void make_pair16(const u32x4_t (&rawq)[NG], const u32
       }
     }
   }
-}
-
-// P^T tile = k~ (rows j) x q~ (columns i) on fp16 operands.
-template <int NG>
-__device__ __forceinline__ f32x16_t score_tile16(const u32x4_t (&k16)[NG], const u32x4_t (&q16)[NG]) {
-  f32x16_t acc = {0.f};
-#pragma unroll
-  for (int ks = 0; ks < NG; ++ks) acc = mfma_f16(k16[ks], q16[ks], acc);
-  return acc;
-}
-
-// P^T tile = k~ (rows j) x q~ (columns i), three-term split product.
-template <int NG>
-__device__ __forceinline__ f32x16_t score_tile(const HalfOps<NG>& kop, const HalfOps<NG>& qop) {
-  f32x16_t acc = {0.f};
-#pragma unroll
-  for (int ks = 0; ks < NG; ++ks) {
-    acc = mfma(kop.h[ks], qop.h[ks], acc);
-    acc = mfma(kop.l[ks], qop.h[ks], acc);
-    acc = mfma(kop.h[ks], qop.l[ks], acc);
-  }
-  return acc;
 }
 
 // O^T[p] += V^T (k-steps 2*jt, 2*jt+1 of vfrag) x P^T tile, with P split into bf16 hi + lo against bf16 V, or (F16)
@@ -240,9 +160,6 @@ __device__ __forceinline__ void apply_scores(f32x16_t P, int jt, int r, int h, c
     O1 = mfma(vfrag[t][1], pl, O1);
   }
 }
-
-// LDS "unit" u of a region = 64 lanes x 16 B, register-native: lane l owns bytes [(u*64 + l)*16, +16).
-__device__ __forceinline__ char* unit_ptr(char* region, int u, int lane) { return region + (u * 64 + lane) * 16; }
 
 // What a wave carries from the end of one slab to the start of the next: the loads of its first phase.
 template <int NG>
@@ -1195,6 +1112,12 @@ static int launch_gla_mfma_t(const GlaArgs& a, int num_cu, int dev) {
 }
 
 int launch_gla_mfma(const GlaArgs& a) {
+  // whole-sequence slabs go to the tile-pair kernel (VIG_GLA_CHUNKED_SLABS=1 keeps them here: comparisons only)
+  static const bool chunked_slabs = [] {
+    const char* e = getenv("VIG_GLA_CHUNKED_SLABS");
+    return e && e[0] == '1';
+  }();
+  if (!chunked_slabs && gla_tiles_supported(a)) return launch_gla_tiles(a);
   static int num_cu_dev[kMaxDevices] = {};
   int dev = 0;
   if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return -5;

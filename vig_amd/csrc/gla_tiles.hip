@@ -1,0 +1,544 @@
+// Bidirectional GLA forward for whole-sequence slabs (L <= 256) on MFMA tiles (gfx950), Dk in {32, 64}, Dv = 64,
+// bf16 in and out: one workgroup per (batch, head) slab, one wave per 32-token query tile, both directions in the
+// same wave.
+//
+// Wave i owns the queries of tile i.  Along the forward direction they see the keys of tiles j <= i, along the
+// reverse direction those of tiles j >= i, so every wave multiplies against NT + 1 key tiles whatever its position, the
+// two directions add up in the wave's own accumulators (no exchange of outputs), and the only thing waves hand each
+// other is what a key tile contributes: its decayed keys, its values and its total decay, published once in LDS.
+// A wave
+//   1. loads its 32 rows of q, k, v and of both gate tensors,
+//   2. forms the tile-local cumulative log-gates G with a triangular-ones MFMA (bf16 gates are exact MFMA inputs,
+//      the sums accumulate in fp32); the tile total T is G at the tile's last token walked,
+//   3. builds q^ = q exp(G) (decay from the tile's first token walked: what an earlier tile's keys still see),
+//      k^ = k exp(T - G) (decay up to the end of the tile: what a later tile's queries see) and, for its own diagonal
+//      tile only, k' = k exp(-G); all as fp16 (11-bit significands, one MFMA term per k-step),
+//   4. publishes k^ (both directions), V as fp16 transposed fragments and D = exp(T) per channel,
+//   5. computes its diagonal tile from registers: P = mask_fwd(k'_f q^_f) + mask_rev(k'_r q^_r), O = V^T P,
+//   6. after the one workgroup barrier walks outwards over the other tiles, P = k^_j (q^ (.) decays of the tiles in
+//      between), O += V_j^T P, and stores its 32 output rows once.
+// Every published factor is at most one in magnitude relative to its input, so distant tiles underflow gracefully; only
+// k' grows (by exp(|T|)), which is why the fp16 form asks for |T| log2(e) <= 10 per 32-token tile and channel (ViG's
+// logsigmoid(.)/16 gates reach about 2.5) and for rows of q, k, v of ordinary magnitude (sums of squares checked
+// through a Gram-matrix MFMA).  A slab outside that range is redone by the same workgroup in the general form: inputs
+// rescaled by slab-wide powers of two, the diagonal tile on half-anchored bf16 hi + lo operands with three MFMA terms
+// per k-step (any tile total down to about -160, i.e. gates of -5 per token).
+//
+// Chunk algebra follows flash-linear-attention/fla/ops/gla/chunk_util.py:9-78 and chunk_fuse.py:76-97,245-254 (there
+// with 16-token chunks and a carried state; here 32-token tiles and direct tile-pair products, which for L <= 256 cost
+// fewer matrix instructions than carrying the Dk x Dv state); both directions in one launch as in
+// recurrent_fuse.py:19-148.
+//
+// Register layouts as in mfma_tiles.h.  LDS: k^ tiles of the forward direction (tiles 0..NT-2) and of the reverse
+// direction (tiles 1..NT-1) as ready A-operand units, V tiles as ready A-operand units, decays as fp16 in channel
+// order; a wave's V region doubles as its private scratch until the values are published.
+#include "common.h"
+#include "launch.h"
+#include "mfma_tiles.h"
+
+namespace vig {
+
+namespace {
+
+#define VIG_PHASE() __builtin_amdgcn_sched_barrier(0)
+
+constexpr float kTileRange = 10.0f;     // fp16 form: |tile total| * log2(e) per channel
+constexpr float kMaxSquaresQ = 32768.0f;  // rows of q: |q| < 182
+constexpr float kMaxSquaresK = 1024.0f;   // rows of k: |k| < 32, so k' = k 2^10 stays inside fp16, and |P| <= |q||k| < 5800
+constexpr float kMaxSquaresV = 1.0e8f;    // |v| < 10^4
+constexpr float kExpFloor = -240.0f;      // general form: exponents are clamped here (what lies beyond is zero)
+
+struct TileGeo {
+  int L, NT, H;             // tokens per sequence, 32-token tiles per sequence, heads per batch element
+  long long sq[3], sk[3], sv[3];  // (batch, head, token) strides in elements of q, k, v
+  int wide;                 // nonzero: go straight to the general form
+};
+
+// byte offsets of the workgroup's LDS areas
+template <int NG>
+struct TileLds {
+  static constexpr int KB = NG * 1024;  // one k^ tile: NG units
+  static constexpr int VB = 4096;       // one V tile: 4 units
+  int kf, kb, v, d, scratch, guard, total;
+  __host__ __device__ explicit TileLds(int NT) {
+    kf = 0;
+    kb = (NT - 1) * KB;
+    v = 2 * (NT - 1) * KB;
+    d = v + NT * VB;
+    scratch = d + 2 * NT * 128;  // per wave: 64 floats (tile totals on their way from one lane pair to a lane per channel)
+    guard = scratch + NT * 256;
+    total = guard + NT * 16;
+  }
+};
+
+struct TileCtx {
+  rsrc_t q, k, v, gf, gb, o;
+  unsigned q_pitch, k_pitch, v_pitch;
+  char* lds;
+  int ti, NT, lane;
+  float oscale;
+};
+
+__device__ __forceinline__ float wave_max(float x) {
+#pragma unroll
+  for (int s = 32; s >= 1; s >>= 1) x = fmaxf(x, __shfl_xor(x, s, 64));
+  return x;
+}
+// power of two e such that m * 4^-e <= 2^target (m >= 0; inf or nan: the largest exponent)
+__device__ __forceinline__ int scale_exponent(float m, int target) {
+  const int ex = (int)((__float_as_uint(m) >> 23) & 0xffu) - 127;  // m < 2^(ex+1)
+  const int e = (ex + 1 - target + 1) >> 1;
+  return e > 0 ? e : 0;
+}
+
+// tile-local cumulative gates of one direction: G[p][4g+m] = channel 8*NG*h + 8g + 2m + p of token r
+template <bool FWD>
+__device__ __forceinline__ void cumulative_gates(const uint32_t (&gD)[2][8], int r, int h, f32x16_t (&G)[2]) {
+  u32x4_t gfrag[2][2];
+  finish_tfrags<2>(gD, gfrag);
+  const u32x4_t tri0 = tri_frag<FWD>(0, 0, r, h), tri1 = tri_frag<FWD>(1, 0, r, h);
+#pragma unroll
+  for (int p = 0; p < 2; ++p) {
+    f32x16_t g = {0.f};
+    g = mfma(gfrag[0][p], tri0, g);
+    g = mfma(gfrag[1][p], tri1, g);
+    G[p] = g;
+  }
+}
+
+// the tile totals (G at the last token walked) travel from the one lane pair that holds them to a lane per channel:
+// sc[32h + 16p + 4g + m] = total of channel 8*NG*h + 8g + 2m + p
+template <bool FWD>
+__device__ __forceinline__ void park_totals(const f32x16_t (&G)[2], float* sc, int r, int h) {
+  if (r == (FWD ? 31 : 0)) {
+#pragma unroll
+    for (int p = 0; p < 2; ++p)
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        const f32x4_t x = {G[p][4 * g], G[p][4 * g + 1], G[p][4 * g + 2], G[p][4 * g + 3]};
+        *reinterpret_cast<f32x4_t*>(sc + 32 * h + 16 * p + 4 * g) = x;
+      }
+  }
+  wave_lds_sync();
+}
+
+// Operands of one direction for this wave's tile, the publication of what other tiles need from it, and the diagonal
+// score tile (masked to the pairs the direction sees and rounded to fp16 pairs: the B operand of the value product).
+//   qh: q^ = q exp(G)      (B operand of every score product of this wave; kept)
+//   k^ = k exp(T - G)      (published to kreg unless null, piece by piece)
+//   D  = exp(T)            (published to dtab, fp16, channel order)
+// fp16 form (GENERAL false): the diagonal tile uses k' = k exp(-G) against q^; returns (wave-uniform) whether some
+// channel's tile total is outside the form's range.
+// General form: inputs carry the power-of-two scales 2^-eq, 2^-ek; the diagonal tile uses the half-anchored pair
+// q~ = q exp(G - T/2), k~ = k exp(T/2 - G) as bf16 hi + lo, three MFMA terms per k-step.
+template <int NG, bool FWD, bool GENERAL>
+__device__ __forceinline__ bool prepare_direction(const uint32_t (&gD)[2][8], const u32x4_t (&rawq)[NG],
+                                                  const u32x4_t (&rawk)[NG], float* sc, _Float16* dtab, char* kreg,
+                                                  int lane, int eq, int ek, u32x4_t (&qh)[NG], u32x4_t (&p16)[2]) {
+  const int r = lane & 31, h = lane >> 5;
+  constexpr int HC = 8 * NG;
+  f32x16_t G[2];
+  cumulative_gates<FWD>(gD, r, h, G);
+  park_totals<FWD>(G, sc, r, h);
+  float tl = sc[lane] * kLog2e;
+  bool wide = false;
+  if (!GENERAL) wide = __builtin_amdgcn_ballot_w64(!(fabsf(tl) <= kTileRange)) != 0;
+  else tl = fmaxf(tl, kExpFloor);
+  const float dT = exp2_fast(tl);
+  sc[lane] = GENERAL ? tl : dT;
+  {
+    const int p = (lane >> 4) & 1, g = (lane >> 2) & 3, m = lane & 3;
+    if (g < NG) dtab[HC * h + 8 * g + 2 * m + p] = (_Float16)dT;
+  }
+  wave_lds_sync();
+  const float* mine = sc + 32 * h;
+  const float fq = -(float)eq, fk = -(float)ek;
+  f32x16_t P = {0.f};
+#pragma unroll
+  for (int g = 0; g < NG; ++g) {
+    const f32x4_t d0 = *reinterpret_cast<const f32x4_t*>(mine + 4 * g);
+    const f32x4_t d1 = *reinterpret_cast<const f32x4_t*>(mine + 16 + 4 * g);
+    u32x4_t kh;
+    if (!GENERAL) {
+      u32x4_t kc;
+#pragma unroll
+      for (int m = 0; m < 4; ++m) {
+        const int c = 4 * g + m;
+        const float x0 = G[0][c] * kLog2e, x1 = G[1][c] * kLog2e;
+        const float a0 = exp2_fast(x0), a1 = exp2_fast(x1);
+        const float b0 = exp2_fast(-x0), b1 = exp2_fast(-x1);
+        const uint32_t wq = rawq[g][m], wk = rawk[g][m];
+        qh[g][m] = pack_f16x2(bf16lo_to_f32(wq) * a0, bf16hi_to_f32(wq) * a1);
+        const float k0 = bf16lo_to_f32(wk) * b0, k1 = bf16hi_to_f32(wk) * b1;
+        kc[m] = pack_f16x2(k0, k1);
+        kh[m] = pack_f16x2(k0 * d0[m], k1 * d1[m]);
+      }
+      P = mfma_f16(kc, qh[g], P);
+    } else {
+      u32x4_t qhi, qlo, khi, klo;
+#pragma unroll
+      for (int m = 0; m < 4; ++m) {
+        const int c = 4 * g + m;
+        const uint32_t wq = rawq[g][m], wk = rawk[g][m];
+        const float qv[2] = {bf16lo_to_f32(wq), bf16hi_to_f32(wq)}, kv[2] = {bf16lo_to_f32(wk), bf16hi_to_f32(wk)};
+        float qhat[2], khat[2], qt[2], kt[2];
+#pragma unroll
+        for (int p = 0; p < 2; ++p) {
+          const float tl_c = p ? d1[m] : d0[m];
+          const float x = fmaxf(G[p][c] * kLog2e, kExpFloor);
+          const float an = 0.5f * tl_c;
+          qhat[p] = qv[p] * exp2_fast(x + fq);
+          khat[p] = kv[p] * exp2_fast(tl_c - x + fk);
+          qt[p] = qv[p] * exp2_fast(x - an + fq);
+          kt[p] = kv[p] * exp2_fast(an - x + fk);
+        }
+        qh[g][m] = pack_f16x2(qhat[0], qhat[1]);
+        kh[m] = pack_f16x2(khat[0], khat[1]);
+        qhi[m] = pack_bf16x2(qt[0], qt[1]);
+        khi[m] = pack_bf16x2(kt[0], kt[1]);
+        qlo[m] = pack_bf16x2(qt[0] - bf16lo_to_f32(qhi[m]), qt[1] - bf16hi_to_f32(qhi[m]));
+        klo[m] = pack_bf16x2(kt[0] - bf16lo_to_f32(khi[m]), kt[1] - bf16hi_to_f32(khi[m]));
+      }
+      P = mfma(khi, qhi, P);
+      P = mfma(klo, qhi, P);
+      P = mfma(khi, qlo, P);
+    }
+    if (kreg) *reinterpret_cast<u32x4_t*>(unit_ptr(kreg, g, lane)) = kh;
+  }
+  // keep the pairs the direction sees (P^T[j, i]: lane = column i, register 4g+m = row 8g + 4h + m), round to fp16
+#pragma unroll
+  for (int t = 0; t < 2; ++t)
+#pragma unroll
+    for (int x = 0; x < 4; ++x) {
+      const int c = 4 * (2 * t + (x >> 1)) + 2 * (x & 1);
+      const int j = 8 * (c >> 2) + 4 * h + (c & 3);
+      const float lo = (FWD ? (j <= r) : (j >= r)) ? P[c] : 0.f;
+      const float hi = (FWD ? (j + 1 <= r) : (j + 1 >= r)) ? P[c + 1] : 0.f;
+      p16[t][x] = pack_f16x2(lo, hi);
+    }
+  return wide;
+}
+
+// O^T[pv] += V^T (fragments vf[t][pv] of one key tile) x P^T given as fp16 pairs
+__device__ __forceinline__ void apply_values16(const u32x4_t (&p16)[2], const u32x4_t (&vf)[2][2], f32x16_t (&O)[2]) {
+#pragma unroll
+  for (int t = 0; t < 2; ++t) {
+    O[0] = mfma_f16(vf[t][0], p16[t], O[0]);
+    O[1] = mfma_f16(vf[t][1], p16[t], O[1]);
+  }
+}
+
+// O^T[pv] += V^T x P^T, P rounded once to fp16
+__device__ __forceinline__ void apply_values(const f32x16_t& P, const u32x4_t (&vf)[2][2], f32x16_t (&O)[2]) {
+  u32x4_t p16[2];
+#pragma unroll
+  for (int t = 0; t < 2; ++t)
+#pragma unroll
+    for (int x = 0; x < 4; ++x) {
+      const int c = 4 * (2 * t + (x >> 1)) + 2 * (x & 1);
+      p16[t][x] = pack_f16x2(P[c], P[c + 1]);
+    }
+  apply_values16(p16, vf, O);
+}
+
+// One outward walk of a wave over the key tiles of one direction: tiles ti-1 .. 0 (FWD) or ti+1 .. NT-1.  q^ picks up
+// the total decay of every tile it passes (fp16 x fp16, every factor at most one).
+template <int NG, bool FWD>
+__device__ __forceinline__ void walk_tiles(char* lds, const TileLds<NG>& lay, int ti, int NT, int lane,
+                                           u32x4_t (&qh)[NG], f32x16_t (&O)[2]) {
+  const int h = lane >> 5;
+  constexpr int HC = 8 * NG;
+  const int kbase = FWD ? lay.kf : lay.kb - TileLds<NG>::KB;  // reverse regions start at tile 1
+  const char* dbase = lds + lay.d + (FWD ? 0 : NT * 128) + 2 * HC * h;
+  const int n = FWD ? ti : NT - 1 - ti;
+#pragma unroll 1
+  for (int s = 1; s <= n; ++s) {
+    const int j = FWD ? ti - s : ti + s;
+    if (s > 1) {  // the tile passed last: j + 1 forward, j - 1 reverse
+      const char* dp = dbase + (FWD ? j + 1 : j - 1) * 128;
+#pragma unroll
+      for (int g = 0; g < NG; ++g) {
+        const u32x4_t d = *reinterpret_cast<const u32x4_t*>(dp + 16 * g);
+#pragma unroll
+        for (int m = 0; m < 4; ++m) qh[g][m] = mul_f16x2(qh[g][m], d[m]);
+      }
+    }
+    char* kreg = lds + kbase + j * TileLds<NG>::KB;
+    char* vreg = lds + lay.v + j * TileLds<NG>::VB;
+    u32x4_t kf[NG];
+#pragma unroll
+    for (int g = 0; g < NG; ++g) kf[g] = *reinterpret_cast<const u32x4_t*>(unit_ptr(kreg, g, lane));
+    u32x4_t vf[2][2];
+#pragma unroll
+    for (int t = 0; t < 2; ++t)
+#pragma unroll
+      for (int pv = 0; pv < 2; ++pv) vf[t][pv] = *reinterpret_cast<const u32x4_t*>(unit_ptr(vreg, 2 * t + pv, lane));
+    const f32x16_t P = score_tile16<NG>(kf, qh);
+    apply_values(P, vf, O);
+  }
+}
+
+// Everything one wave does for its slab.  The fp16 form (GENERAL false) returns true, for every wave of the workgroup
+// alike and before anything is stored, when some tile of the slab is outside its range.
+template <int NG, bool BIDIR, bool PITCHED, bool GENERAL>
+__device__ __forceinline__ bool tile_pass(const TileCtx& cx) {
+  const int lane = cx.lane, r = lane & 31, h = lane >> 5;
+  const int ti = cx.ti, NT = cx.NT;
+  const TileLds<NG> lay(NT);
+  char* lds = cx.lds;
+  char* vregion = lds + lay.v + ti * TileLds<NG>::VB;
+  float* sc = reinterpret_cast<float*>(lds + lay.scratch + ti * 256);
+  float* guard = reinterpret_cast<float*>(lds + lay.guard);
+  _Float16* dtab_f = reinterpret_cast<_Float16*>(lds + lay.d + ti * 128);
+  _Float16* dtab_b = reinterpret_cast<_Float16*>(lds + lay.d + (NT + ti) * 128);
+
+  // ---- loads: v and gates as transposed dwords, q / k rows ----
+  uint32_t gDf[2][8], gDb[2][8], vD[2][8];
+  u32x4_t rawq[NG], rawk[NG];
+  if (PITCHED) issue_tdwords_pitched<0, 2, 4>(cx.v, r, h, cx.v_pitch, vD);
+  else issue_tdwords<0, 2, 4>(cx.v, r, h, vD);
+  issue_tdwords<0, 2, NG>(cx.gf, r, h, gDf);
+  if (PITCHED) {
+    issue_raw_tile_pitched<NG>(cx.q, 0, r, h, cx.q_pitch, rawq);
+    issue_raw_tile_pitched<NG>(cx.k, 0, r, h, cx.k_pitch, rawk);
+  } else {
+    issue_raw_tile<NG>(cx.q, 0, r, h, rawq);
+    issue_raw_tile<NG>(cx.k, 0, r, h, rawk);
+  }
+#ifndef VIG_LATE_GB
+  if (BIDIR) issue_tdwords<0, 2, NG>(cx.gb, r, h, gDb);
+#endif
+
+  // ---- magnitudes (Gram matrices of the raw rows); values: bf16 pairs -> fp16 pairs, published ----
+  int eq = 0, ek = 0, ev = 0;
+  bool veto = false;
+  {
+    u32x4_t vraw[2][2];
+    finish_tfrags<2>(vD, vraw);
+    f32x4acc_t gq = {0.f, 0.f, 0.f, 0.f}, gk = gq, gv = gq;
+#pragma unroll
+    for (int t = 0; t < 2; ++t)
+#pragma unroll
+      for (int p = 0; p < 2; ++p) gram_acc(vraw[t][p], gv);
+#pragma unroll
+    for (int g = 0; g < NG; ++g) {
+      gram_acc(rawq[g], gq);
+      gram_acc(rawk[g], gk);
+    }
+    const float mq = fmaxf(fmaxf(fabsf(gq[0]), fabsf(gq[1])), fmaxf(fabsf(gq[2]), fabsf(gq[3])));
+    const float mk = fmaxf(fmaxf(fabsf(gk[0]), fabsf(gk[1])), fmaxf(fabsf(gk[2]), fabsf(gk[3])));
+    const float mv = fmaxf(fmaxf(fabsf(gv[0]), fabsf(gv[1])), fmaxf(fabsf(gv[2]), fabsf(gv[3])));
+    if (!GENERAL) {
+      veto = __builtin_amdgcn_ballot_w64(!(mq < kMaxSquaresQ) || !(mk < kMaxSquaresK) || !(mv < kMaxSquaresV)) != 0;
+    } else {
+      // slab-wide scales for k and v (their tiles meet every wave's queries), a scale of its own for this wave's q
+      const float wq = wave_max(mq), wk = wave_max(mk), wv = wave_max(mv);
+      if (lane == 0) {
+        guard[4 * ti + 1] = wk;
+        guard[4 * ti + 2] = wv;
+      }
+      lds_barrier();
+      float sk = 0.f, sv = 0.f;
+      for (int t = 0; t < NT; ++t) {
+        sk = fmaxf(sk, guard[4 * t + 1]);
+        sv = fmaxf(sv, guard[4 * t + 2]);
+      }
+      eq = scale_exponent(wq, 10);
+      ek = scale_exponent(sk, 10);
+      ev = scale_exponent(sv, 20);
+    }
+    const float vs = GENERAL ? __builtin_amdgcn_exp2f(-(float)ev) : 1.0f;
+#pragma unroll
+    for (int t = 0; t < 2; ++t)
+#pragma unroll
+      for (int p = 0; p < 2; ++p) {
+        u32x4_t f;
+#pragma unroll
+        for (int x = 0; x < 4; ++x) {
+          const uint32_t w = vraw[t][p][x];
+          f[x] = GENERAL ? pack_f16x2(bf16lo_to_f32(w) * vs, bf16hi_to_f32(w) * vs)
+                         : pack_f16x2(bf16lo_to_f32(w), bf16hi_to_f32(w));
+        }
+        *reinterpret_cast<u32x4_t*>(unit_ptr(vregion, 2 * t + p, lane)) = f;
+      }
+  }
+  VIG_PHASE();
+  // ---- both directions: operands, publication, diagonal scores ----
+  u32x4_t qhf[NG], qhb[NG];
+  u32x4_t p16[2];
+  {
+    char* kreg = ti < NT - 1 ? lds + lay.kf + ti * TileLds<NG>::KB : nullptr;
+    if (prepare_direction<NG, true, GENERAL>(gDf, rawq, rawk, sc, dtab_f, kreg, lane, eq, ek, qhf, p16)) veto = true;
+  }
+  VIG_PHASE();
+#ifdef VIG_LATE_GB
+  if (BIDIR) issue_tdwords<0, 2, NG>(cx.gb, r, h, gDb);
+#endif
+  if (BIDIR) {
+    char* kreg = ti > 0 ? lds + lay.kb + (ti - 1) * TileLds<NG>::KB : nullptr;
+    u32x4_t pb[2];
+    // (opaque copies: the unpacked halves of the raw rows are rebuilt here instead of being carried, 64 registers wide,
+    // from the forward direction's loop)
+#pragma unroll
+    for (int g = 0; g < NG; ++g)
+#pragma unroll
+      for (int m = 0; m < 4; ++m) {
+        asm volatile("" : "+v"(rawq[g][m]));
+        asm volatile("" : "+v"(rawk[g][m]));
+      }
+    if (prepare_direction<NG, false, GENERAL>(gDb, rawq, rawk, sc, dtab_b, kreg, lane, eq, ek, qhb, pb)) veto = true;
+    // (the two directions meet on the pairs j = i only: one more fp16 rounding there)
+#pragma unroll
+    for (int t = 0; t < 2; ++t)
+#pragma unroll
+      for (int x = 0; x < 4; ++x) p16[t][x] = add_f16x2(p16[t][x], pb[t][x]);
+  }
+  VIG_PHASE();
+  // ---- diagonal tile ----
+  f32x16_t O[2] = {f32x16_t{0.f}, f32x16_t{0.f}};
+  {
+    wave_lds_sync();
+    u32x4_t vf[2][2];
+#pragma unroll
+    for (int t = 0; t < 2; ++t)
+#pragma unroll
+      for (int pv = 0; pv < 2; ++pv) vf[t][pv] = *reinterpret_cast<const u32x4_t*>(unit_ptr(vregion, 2 * t + pv, lane));
+    apply_values16(p16, vf, O);
+  }
+  if (!GENERAL && lane == 0) guard[4 * ti] = veto ? 1.0f : 0.0f;
+  lds_barrier();  // every tile's k^, V and decays are visible
+  if (!GENERAL) {
+    const float mine = lane < NT ? guard[4 * lane] : 0.0f;
+    if (__builtin_amdgcn_ballot_w64(mine != 0.0f) != 0) return true;
+  }
+  // ---- the other tiles, outwards ----
+  walk_tiles<NG, true>(lds, lay, ti, NT, lane, qhf, O);
+  if (BIDIR) walk_tiles<NG, false>(lds, lay, ti, NT, lane, qhb, O);
+  // ---- store: lane (r, h) holds channels [32h, 32h + 32) of token r; rows beyond the sequence are dropped ----
+  float os = cx.oscale;
+  if (GENERAL) os *= __builtin_amdgcn_exp2f((float)(eq + ek + ev));
+#pragma unroll
+  for (int gq = 0; gq < 4; ++gq) {
+    u32x4_t x;
+#pragma unroll
+    for (int m = 0; m < 4; ++m) x[m] = pack_bf16x2(O[0][4 * gq + m] * os, O[1][4 * gq + m] * os);
+    __builtin_amdgcn_raw_buffer_store_b128(x, cx.o, (unsigned)r * 128u + 64u * h + 16u * gq, 0, 0);
+  }
+  return false;
+}
+
+template <int NG, bool BIDIR, bool PITCHED>
+__device__ __forceinline__ TileCtx make_tile_ctx(const uint16_t* q, const uint16_t* k, const uint16_t* v,
+                                                 const uint16_t* gf, const uint16_t* gb, uint16_t* o,
+                                                 const TileGeo& geo, float oscale, char* lds) {
+  constexpr int DK = 16 * NG;
+  TileCtx cx;
+  cx.lds = lds;
+  cx.ti = __builtin_amdgcn_readfirstlane((int)threadIdx.x >> 6);
+  cx.lane = threadIdx.x & 63;
+  cx.NT = geo.NT;
+  cx.oscale = oscale;
+  const int seq = blockIdx.x;
+  const int tok = 32 * cx.ti;
+  const int nvalid = min(32, geo.L - tok);
+  const size_t off = (size_t)seq * geo.L + tok;  // in tokens
+  if (PITCHED) {
+    const int b = seq / geo.H, hd = seq - b * geo.H;
+    cx.q_pitch = 2u * (unsigned)geo.sq[2], cx.k_pitch = 2u * (unsigned)geo.sk[2], cx.v_pitch = 2u * (unsigned)geo.sv[2];
+    cx.q = chunk_rsrc(q + b * geo.sq[0] + hd * geo.sq[1] + (long long)tok * geo.sq[2], nvalid, cx.q_pitch);
+    cx.k = chunk_rsrc(k + b * geo.sk[0] + hd * geo.sk[1] + (long long)tok * geo.sk[2], nvalid, cx.k_pitch);
+    cx.v = chunk_rsrc(v + b * geo.sv[0] + hd * geo.sv[1] + (long long)tok * geo.sv[2], nvalid, cx.v_pitch);
+  } else {
+    cx.q_pitch = cx.k_pitch = 2 * DK, cx.v_pitch = 128;
+    cx.q = chunk_rsrc(q + off * DK, nvalid, 2 * DK);
+    cx.k = chunk_rsrc(k + off * DK, nvalid, 2 * DK);
+    cx.v = chunk_rsrc(v + off * 64, nvalid, 128);
+  }
+  cx.gf = chunk_rsrc(gf + off * DK, nvalid, 2 * DK);
+  cx.gb = chunk_rsrc(BIDIR ? gb + off * DK : gf, BIDIR ? nvalid : 0, 2 * DK);
+  cx.o = chunk_rsrc(o + off * 64, nvalid, 128);
+  return cx;
+}
+
+// the general form as a function of its own: its register needs stay out of the fp16 form's allocation
+template <int NG, bool BIDIR, bool PITCHED>
+__device__ __noinline__ void tile_pass_general(const uint16_t* q, const uint16_t* k, const uint16_t* v,
+                                               const uint16_t* gf, const uint16_t* gb, uint16_t* o, const TileGeo* geo,
+                                               float oscale, char* lds) {
+  const TileCtx cx = make_tile_ctx<NG, BIDIR, PITCHED>(q, k, v, gf, gb, o, *geo, oscale, lds);
+  tile_pass<NG, BIDIR, PITCHED, true>(cx);
+}
+
+}  // namespace
+
+template <int NG, bool BIDIR, bool PITCHED>
+__global__ __launch_bounds__(512, 4) void gla_tile_kernel(const uint16_t* __restrict__ q, const uint16_t* __restrict__ k,
+                                                          const uint16_t* __restrict__ v,
+                                                          const uint16_t* __restrict__ gf,
+                                                          const uint16_t* __restrict__ gb, uint16_t* __restrict__ o,
+                                                          TileGeo geo, float oscale) {
+  extern __shared__ __align__(16) char lds[];
+  bool redo = true;
+  if (!geo.wide) {
+    const TileCtx cx = make_tile_ctx<NG, BIDIR, PITCHED>(q, k, v, gf, gb, o, geo, oscale, lds);
+    redo = tile_pass<NG, BIDIR, PITCHED, false>(cx);
+  }
+  if (redo) tile_pass_general<NG, BIDIR, PITCHED>(q, k, v, gf, gb, o, &geo, oscale, lds);
+}
+
+bool gla_tiles_supported(const GlaArgs& a) {
+  return a.io_dtype == 1 && a.gate_dtype == 1 && (a.Dk == 64 || a.Dk == 32) && a.Dv == 64 && a.L <= 256 &&
+         !a.init_state && !a.final_state && !a.state_pass && !a.gate_w;
+}
+
+template <int NG, bool BIDIR, bool PITCHED>
+static int launch_tiles_t(const GlaArgs& a, const TileGeo& geo, int dev) {
+  constexpr int kMaxDevices = 64;
+  static bool attr_done_dev[kMaxDevices] = {};
+  const void* kf = reinterpret_cast<const void*>(gla_tile_kernel<NG, BIDIR, PITCHED>);
+  if (!attr_done_dev[dev]) {
+    if (hipFuncSetAttribute(kf, hipFuncAttributeMaxDynamicSharedMemorySize, TileLds<NG>(8).total) != hipSuccess) return -5;
+    attr_done_dev[dev] = true;
+  }
+  const TileLds<NG> lay(geo.NT);
+  hipLaunchKernelGGL((gla_tile_kernel<NG, BIDIR, PITCHED>), dim3(a.B * a.H), dim3(64 * geo.NT), lay.total, a.stream,
+                     (const uint16_t*)a.q, (const uint16_t*)a.k, (const uint16_t*)a.v, (const uint16_t*)a.g_fwd,
+                     (const uint16_t*)a.g_bwd, (uint16_t*)a.o, geo, a.scale * a.out_scale);
+  return hipGetLastError() == hipSuccess ? 0 : -5;
+}
+
+int launch_gla_tiles(const GlaArgs& a) {
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return -5;
+  TileGeo geo{};
+  geo.L = a.L;
+  geo.NT = (a.L + 31) / 32;
+  geo.H = a.H;
+  geo.wide = a.wide_gates;
+  const bool pitched = a.q_strides || a.k_strides || a.v_strides;
+  if (pitched) {
+    const long long* given[3] = {a.q_strides, a.k_strides, a.v_strides};
+    long long* dst[3] = {geo.sq, geo.sk, geo.sv};
+    const int D[3] = {a.Dk, a.Dk, a.Dv};
+    for (int i = 0; i < 3; ++i) {
+      if (given[i] && given[i][2] != 0) {
+        // rows 16-byte aligned, pitches within the descriptors' 32-bit extents
+        for (int j = 0; j < 3; ++j)
+          if (given[i][j] <= 0 || given[i][j] % 8 != 0) return -22;
+        if (given[i][2] > (1 << 20)) return -22;
+        dst[i][0] = given[i][0], dst[i][1] = given[i][1], dst[i][2] = given[i][2];
+      } else {
+        dst[i][0] = (long long)a.H * a.L * D[i], dst[i][1] = (long long)a.L * D[i], dst[i][2] = D[i];
+      }
+    }
+  }
+  const bool bidir = a.g_bwd != nullptr;
+  if (a.Dk == 64) {
+    if (pitched) return bidir ? launch_tiles_t<4, true, true>(a, geo, dev) : launch_tiles_t<4, false, true>(a, geo, dev);
+    return bidir ? launch_tiles_t<4, true, false>(a, geo, dev) : launch_tiles_t<4, false, false>(a, geo, dev);
+  }
+  if (pitched) return bidir ? launch_tiles_t<2, true, true>(a, geo, dev) : launch_tiles_t<2, false, true>(a, geo, dev);
+  return bidir ? launch_tiles_t<2, true, false>(a, geo, dev) : launch_tiles_t<2, false, false>(a, geo, dev);
+}
+
+}  // namespace vig

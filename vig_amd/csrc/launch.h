@@ -55,6 +55,9 @@ size_t gla_recurrent_workspace(int B, int H, int L, int Dv, int io_dtype);
 // bf16 MFMA chunked path (bf16 io and gates).
 bool gla_mfma_supported(const GlaArgs& a);
 int launch_gla_mfma(const GlaArgs& a);
+// bf16 tile-pair path for whole-sequence slabs (L <= 256): one wave per 32-token tile, both directions per wave.
+bool gla_tiles_supported(const GlaArgs& a);
+int launch_gla_tiles(const GlaArgs& a);
 bool gla_mfma_gate_grid_ok(int rows, int cols);  // token grids the fused locality gate takes
 size_t gla_mfma_workspace(int B, int H, int L, int Dk, int Dv);
 size_t gla_mfma_state_workspace(int B, int H, int L, int Dk, int Dv);  // causal op with an initial / final state

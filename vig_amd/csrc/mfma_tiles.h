@@ -161,6 +161,96 @@ __device__ __forceinline__ void store_kt(uint16_t* kt, int row, int h, const u32
   for (int g = 0; g < NG; ++g) *reinterpret_cast<u32x4_t*>(kt + row * STRIDE + 8 * NG * h + 8 * g) = kh[g];
 }
 
+// ---- fp16 operands, magnitude guard, split-bf16 operands, LDS units (shared by the forward kernels) ----
+typedef _Float16 f16x2_t __attribute__((ext_vector_type(2)));
+typedef _Float16 f16x8_t __attribute__((ext_vector_type(8)));
+__device__ __forceinline__ f32x16_t mfma_f16(const u32x4_t& a, const u32x4_t& b, const f32x16_t& c) {
+  return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8_t, a), __builtin_bit_cast(f16x8_t, b), c, 0,
+                                                0, 0);
+}
+__device__ __forceinline__ uint32_t pack_f16x2(float lo, float hi) {
+  f32x2_t x = {lo, hi};
+  f16x2_t y = __builtin_convertvector(x, f16x2_t);  // round to nearest even
+  return __builtin_bit_cast(uint32_t, y);
+}
+// elementwise product of two fp16 pairs (operands by value: a bit cast straight from a vector element reads the
+// vector's first word)
+__device__ __forceinline__ uint32_t mul_f16x2(uint32_t a, uint32_t b) {
+  return __builtin_bit_cast(uint32_t, __builtin_bit_cast(f16x2_t, a) * __builtin_bit_cast(f16x2_t, b));
+}
+
+__device__ __forceinline__ uint32_t add_f16x2(uint32_t a, uint32_t b) {
+  return __builtin_bit_cast(uint32_t, __builtin_bit_cast(f16x2_t, a) + __builtin_bit_cast(f16x2_t, b));
+}
+
+// Magnitude guard of the fp16 score variant.  Raw bf16 rows go through a 16x16x32 matrix instruction as both
+// operands: whatever the slot assignment, the result is a Gram matrix whose diagonal entries are sums of squares that
+// cover every value fed in and whose other entries are no larger than the largest diagonal one.  Eight passes and four
+// accumulator registers per step, no vector work until the one comparison at the end.
+typedef float f32x4acc_t __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ void gram_acc(const u32x4_t& raw, f32x4acc_t& acc) {
+  acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, raw), __builtin_bit_cast(bf16x8_t, raw), acc,
+                                                0, 0, 0);
+}
+template <int NG>
+struct HalfOps {
+  u32x4_t h[NG], l[NG];  // bf16 hi / lo fragments of one 32-token tile, per k-step (16 channels)
+};
+
+// q~ (ISQ) or k~ of one 32-token tile: raw * exp(+-(G - G_end)), split into bf16 hi (round to nearest) and
+// lo (the fp32 remainder, rounded).  Padding rows arrive as zeros and stay zero (their exponents are finite).
+template <bool ISQ, int NG>
+__device__ __forceinline__ void make_half(const u32x4_t (&raw)[NG], const f32x16_t (&G)[2],
+                                          const float* gend2 /* LDS, this lane half: [p][16] */, HalfOps<NG>& op) {
+#pragma unroll
+  for (int g = 0; g < NG; ++g) {
+    const f32x4_t a0 = *reinterpret_cast<const f32x4_t*>(gend2 + 4 * g);
+    const f32x4_t a1 = *reinterpret_cast<const f32x4_t*>(gend2 + 16 + 4 * g);
+#pragma unroll
+    for (int m = 0; m < 4; ++m) {
+      const int c = 4 * g + m;
+      const uint32_t w = raw[g][m];
+      float t[2];
+#pragma unroll
+      for (int p = 0; p < 2; ++p) {
+        const float an = p ? a1[m] : a0[m];
+        const float x = ISQ ? __builtin_fmaf(G[p][c], kLog2e, -an) : __builtin_fmaf(G[p][c], -kLog2e, an);
+        const float f = p ? bf16hi_to_f32(w) : bf16lo_to_f32(w);
+        t[p] = f * exp2_fast(x);
+      }
+      const uint32_t hi = pack_bf16x2(t[0], t[1]);
+      op.h[g][m] = hi;
+      op.l[g][m] = pack_bf16x2(t[0] - bf16lo_to_f32(hi), t[1] - bf16hi_to_f32(hi));
+    }
+  }
+}
+
+// P^T tile = k~ (rows j) x q~ (columns i) on fp16 operands.
+template <int NG>
+__device__ __forceinline__ f32x16_t score_tile16(const u32x4_t (&k16)[NG], const u32x4_t (&q16)[NG]) {
+  f32x16_t acc = {0.f};
+#pragma unroll
+  for (int ks = 0; ks < NG; ++ks) acc = mfma_f16(k16[ks], q16[ks], acc);
+  return acc;
+}
+
+// P^T tile = k~ (rows j) x q~ (columns i), three-term split product.
+template <int NG>
+__device__ __forceinline__ f32x16_t score_tile(const HalfOps<NG>& kop, const HalfOps<NG>& qop) {
+  f32x16_t acc = {0.f};
+#pragma unroll
+  for (int ks = 0; ks < NG; ++ks) {
+    acc = mfma(kop.h[ks], qop.h[ks], acc);
+    acc = mfma(kop.l[ks], qop.h[ks], acc);
+    acc = mfma(kop.h[ks], qop.l[ks], acc);
+  }
+  return acc;
+}
+
+// LDS "unit" u of a region = 64 lanes x 16 B, register-native: lane l owns bytes [(u*64 + l)*16, +16).
+__device__ __forceinline__ char* unit_ptr(char* region, int u, int lane) { return region + (u * 64 + lane) * 16; }
+
+
 
 }  // namespace
 }  // namespace vig
