@@ -35,12 +35,16 @@
 #include "common.h"
 #include "launch.h"
 #include "mfma_tiles.h"
+#include <stdlib.h>
 
 namespace vig {
 
 namespace {
 
 #define VIG_PHASE() __builtin_amdgcn_sched_barrier(0)
+#ifndef VIG_GENERAL_INLINE
+#define VIG_GENERAL_INLINE __noinline__
+#endif
 
 constexpr float kTileRange = 10.0f;     // fp16 form: |tile total| * log2(e) per channel
 constexpr float kMaxSquaresQ = 32768.0f;  // rows of q: |q| < 182
@@ -52,6 +56,7 @@ struct TileGeo {
   int L, NT, H;             // tokens per sequence, 32-token tiles per sequence, heads per batch element
   long long sq[3], sk[3], sv[3];  // (batch, head, token) strides in elements of q, k, v
   int wide;                 // nonzero: go straight to the general form
+  int gw, gh, heads;        // fused locality gate: token grid (gw columns, gh rows, gw * gh = L), heads per batch element
 };
 
 // byte offsets of the workgroup's LDS areas
@@ -60,18 +65,27 @@ struct TileLds {
   static constexpr int KB = NG * 1024;  // one k^ tile: NG units
   static constexpr int VB = 4096;       // one V tile: 4 units
   int kf, kb, v, d, scratch, guard, total;
-  __host__ __device__ explicit TileLds(int NT) {
+  // gate_bytes: what the fused locality gate stages in the tile regions once they are dead (0: no gate)
+  __host__ __device__ explicit TileLds(int NT, int gate_bytes = 0) {
     kf = 0;
     kb = (NT - 1) * KB;
     v = 2 * (NT - 1) * KB;
     d = v + NT * VB;
+    if (d < gate_bytes) d = gate_bytes;
     scratch = d + 2 * NT * 128;  // per wave: 64 floats (tile totals on their way from one lane pair to a lane per channel)
     guard = scratch + NT * 256;
     total = guard + NT * 16;
   }
 };
 
+// Fused locality gate: the slab's rounded outputs as a zero-padded (gh + 2) x (gw + 2) grid of 128-byte cells, then
+// the 64 x 9 stencil weights of the slab's head.
+constexpr int kGateWeightBytes = 64 * 9 * 4;
+__host__ __device__ inline int gate_stage_bytes(int gw, int gh) { return (gw + 2) * (gh + 2) * 128 + kGateWeightBytes; }
+
 struct TileCtx {
+  const float* gate_w;  // fused locality gate: [64][9] stencil weights of this slab's head
+  int gw, gh;
   rsrc_t q, k, v, gf, gb, o;
   unsigned q_pitch, k_pitch, v_pitch;
   char* lds;
@@ -91,12 +105,33 @@ __device__ __forceinline__ int scale_exponent(float m, int target) {
   return e > 0 ? e : 0;
 }
 
+// Which of the tile's tokens a direction keeps for column token r (j <= r forward, j >= r reverse), as a bit per token,
+// shifted so that both lane halves read their tokens (4h + ...) at the same bit positions.
+template <bool FWD>
+__device__ __forceinline__ uint32_t keep_bits(int r, int h) {
+  const uint32_t K = FWD ? (2u << r) - 1u : 0xFFFFFFFFu << r;
+  return K >> (4 * h);
+}
+// 0xFFFF for each of the two token slots of dword X of k-step T (tokens jmap(T, h, 2X) and the next one) that is kept
+template <int T, int X>
+__device__ __forceinline__ uint32_t keep_mask(uint32_t kh) {
+  constexpr unsigned j0 = 16 * T + 8 * (X >> 1) + 2 * (X & 1);
+  const uint32_t lo = (uint32_t)__builtin_amdgcn_sbfe((int)kh, j0, 1), hi = (uint32_t)__builtin_amdgcn_sbfe((int)kh, j0 + 1, 1);
+  return __builtin_amdgcn_perm(hi, lo, 0x07060100u);
+}
+template <int T>
+__device__ __forceinline__ u32x4_t keep_masks(uint32_t kh) {
+  return u32x4_t{keep_mask<T, 0>(kh), keep_mask<T, 1>(kh), keep_mask<T, 2>(kh), keep_mask<T, 3>(kh)};
+}
+
 // tile-local cumulative gates of one direction: G[p][4g+m] = channel 8*NG*h + 8g + 2m + p of token r
 template <bool FWD>
 __device__ __forceinline__ void cumulative_gates(const uint32_t (&gD)[2][8], int r, int h, f32x16_t (&G)[2]) {
   u32x4_t gfrag[2][2];
   finish_tfrags<2>(gD, gfrag);
-  const u32x4_t tri0 = tri_frag<FWD>(0, 0, r, h), tri1 = tri_frag<FWD>(1, 0, r, h);
+  // B operand: bf16 ones where token slot j is on the kept side of column token r
+  const uint32_t kh = keep_bits<FWD>(r, h);
+  const u32x4_t tri0 = keep_masks<0>(kh) & 0x3F803F80u, tri1 = keep_masks<1>(kh) & 0x3F803F80u;
 #pragma unroll
   for (int p = 0; p < 2; ++p) {
     f32x16_t g = {0.f};
@@ -135,43 +170,49 @@ template <int NG, bool FWD, bool GENERAL>
 __device__ __forceinline__ bool prepare_direction(const uint32_t (&gD)[2][8], const u32x4_t (&rawq)[NG],
                                                   const u32x4_t (&rawk)[NG], float* sc, _Float16* dtab, char* kreg,
                                                   int lane, int eq, int ek, u32x4_t (&qh)[NG], u32x4_t (&p16)[2]) {
-  const int r = lane & 31, h = lane >> 5;
   constexpr int HC = 8 * NG;
   f32x16_t G[2];
-  cumulative_gates<FWD>(gD, r, h, G);
-  park_totals<FWD>(G, sc, r, h);
+  cumulative_gates<FWD>(gD, lane & 31, lane >> 5, G);
+  park_totals<FWD>(G, sc, lane & 31, lane >> 5);
   float tl = sc[lane] * kLog2e;
   bool wide = false;
   if (!GENERAL) wide = __builtin_amdgcn_ballot_w64(!(fabsf(tl) <= kTileRange)) != 0;
   else tl = fmaxf(tl, kExpFloor);
   const float dT = exp2_fast(tl);
-  sc[lane] = GENERAL ? tl : dT;
+  if (GENERAL) sc[lane] = tl;
   {
     const int p = (lane >> 4) & 1, g = (lane >> 2) & 3, m = lane & 3;
-    if (g < NG) dtab[HC * h + 8 * g + 2 * m + p] = (_Float16)dT;
+    if (g < NG) dtab[HC * (lane >> 5) + 8 * g + 2 * m + p] = (_Float16)dT;
   }
   wave_lds_sync();
-  const float* mine = sc + 32 * h;
+  const float* mine = sc + 32 * (lane >> 5);
+  const u32x4_t* dmine = reinterpret_cast<const u32x4_t*>(dtab + HC * (lane >> 5));  // this lane half's decays as fp16 pairs
   const float fq = -(float)eq, fk = -(float)ek;
   f32x16_t P = {0.f};
 #pragma unroll
   for (int g = 0; g < NG; ++g) {
-    const f32x4_t d0 = *reinterpret_cast<const f32x4_t*>(mine + 4 * g);
-    const f32x4_t d1 = *reinterpret_cast<const f32x4_t*>(mine + 16 + 4 * g);
     u32x4_t kh;
+    f32x4_t d0, d1;
+    if (GENERAL) {
+      d0 = *reinterpret_cast<const f32x4_t*>(mine + 4 * g);
+      d1 = *reinterpret_cast<const f32x4_t*>(mine + 16 + 4 * g);
+    }
     if (!GENERAL) {
+      // rawq / rawk hold fp16 pairs here; the decay factors are rounded to fp16 and applied as packed products
+      const u32x4_t d16 = dmine[g];
       u32x4_t kc;
 #pragma unroll
       for (int m = 0; m < 4; ++m) {
         const int c = 4 * g + m;
         const float x0 = G[0][c] * kLog2e, x1 = G[1][c] * kLog2e;
-        const float a0 = exp2_fast(x0), a1 = exp2_fast(x1);
-        const float b0 = exp2_fast(-x0), b1 = exp2_fast(-x1);
-        const uint32_t wq = rawq[g][m], wk = rawk[g][m];
-        qh[g][m] = pack_f16x2(bf16lo_to_f32(wq) * a0, bf16hi_to_f32(wq) * a1);
-        const float k0 = bf16lo_to_f32(wk) * b0, k1 = bf16hi_to_f32(wk) * b1;
-        kc[m] = pack_f16x2(k0, k1);
-        kh[m] = pack_f16x2(k0 * d0[m], k1 * d1[m]);
+        const uint32_t a16 = pack_f16x2(exp2_fast(x0), exp2_fast(x1));
+        const uint32_t b16 = pack_f16x2(exp2_fast(-x0), exp2_fast(-x1));
+        qh[g][m] = mul_f16x2(rawq[g][m], a16);
+        kc[m] = mul_f16x2(rawk[g][m], b16);
+        kh[m] = mul_f16x2(kc[m], d16[m]);
+#ifdef VIG_PREP_FENCE
+        if (m & 1) VIG_PHASE();
+#endif
       }
       P = mfma_f16(kc, qh[g], P);
     } else {
@@ -205,17 +246,20 @@ __device__ __forceinline__ bool prepare_direction(const uint32_t (&gD)[2][8], co
     }
     if (kreg) *reinterpret_cast<u32x4_t*>(unit_ptr(kreg, g, lane)) = kh;
   }
-  // keep the pairs the direction sees (P^T[j, i]: lane = column i, register 4g+m = row 8g + 4h + m), round to fp16
+  // keep the pairs the direction sees (P^T[j, i]: lane = column i, register 4g+m = row 8g + 4h + m: the token of slot
+  // pair x of k-step t, as in the triangular operand), round to fp16
+  // (token masks rebuilt from an opaque lane: shared with the triangular operands above they would be carried, and
+  // spilled, across the whole loop)
+  int lane_m = lane;
+  asm volatile("" : "+v"(lane_m));
+  const uint32_t kh = keep_bits<FWD>(lane_m & 31, lane_m >> 5);
+  const u32x4_t m0 = keep_masks<0>(kh), m1 = keep_masks<1>(kh);
 #pragma unroll
-  for (int t = 0; t < 2; ++t)
-#pragma unroll
-    for (int x = 0; x < 4; ++x) {
-      const int c = 4 * (2 * t + (x >> 1)) + 2 * (x & 1);
-      const int j = 8 * (c >> 2) + 4 * h + (c & 3);
-      const float lo = (FWD ? (j <= r) : (j >= r)) ? P[c] : 0.f;
-      const float hi = (FWD ? (j + 1 <= r) : (j + 1 >= r)) ? P[c + 1] : 0.f;
-      p16[t][x] = pack_f16x2(lo, hi);
-    }
+  for (int x = 0; x < 4; ++x) {
+    const int c = 4 * (x >> 1) + 2 * (x & 1);
+    p16[0][x] = pack_f16x2(P[c], P[c + 1]) & m0[x];
+    p16[1][x] = pack_f16x2(P[8 + c], P[8 + c + 1]) & m1[x];
+  }
   return wide;
 }
 
@@ -280,11 +324,11 @@ __device__ __forceinline__ void walk_tiles(char* lds, const TileLds<NG>& lay, in
 
 // Everything one wave does for its slab.  The fp16 form (GENERAL false) returns true, for every wave of the workgroup
 // alike and before anything is stored, when some tile of the slab is outside its range.
-template <int NG, bool BIDIR, bool PITCHED, bool GENERAL>
+template <int NG, bool BIDIR, bool PITCHED, bool GENERAL, bool GATE>
 __device__ __forceinline__ bool tile_pass(const TileCtx& cx) {
   const int lane = cx.lane, r = lane & 31, h = lane >> 5;
   const int ti = cx.ti, NT = cx.NT;
-  const TileLds<NG> lay(NT);
+  const TileLds<NG> lay(NT, GATE ? gate_stage_bytes(cx.gw, cx.gh) : 0);
   char* lds = cx.lds;
   char* vregion = lds + lay.v + ti * TileLds<NG>::VB;
   float* sc = reinterpret_cast<float*>(lds + lay.scratch + ti * 256);
@@ -305,10 +349,7 @@ __device__ __forceinline__ bool tile_pass(const TileCtx& cx) {
     issue_raw_tile<NG>(cx.q, 0, r, h, rawq);
     issue_raw_tile<NG>(cx.k, 0, r, h, rawk);
   }
-#ifndef VIG_LATE_GB
   if (BIDIR) issue_tdwords<0, 2, NG>(cx.gb, r, h, gDb);
-#endif
-
   // ---- magnitudes (Gram matrices of the raw rows); values: bf16 pairs -> fp16 pairs, published ----
   int eq = 0, ek = 0, ev = 0;
   bool veto = false;
@@ -347,6 +388,15 @@ __device__ __forceinline__ bool tile_pass(const TileCtx& cx) {
       ek = scale_exponent(sk, 10);
       ev = scale_exponent(sv, 20);
     }
+    if (!GENERAL) {  // bf16 pairs -> fp16 pairs (exact for the magnitudes the guard admits)
+#pragma unroll
+      for (int g = 0; g < NG; ++g)
+#pragma unroll
+        for (int m = 0; m < 4; ++m) {
+          rawq[g][m] = pack_f16x2(bf16lo_to_f32(rawq[g][m]), bf16hi_to_f32(rawq[g][m]));
+          rawk[g][m] = pack_f16x2(bf16lo_to_f32(rawk[g][m]), bf16hi_to_f32(rawk[g][m]));
+        }
+    }
     const float vs = GENERAL ? __builtin_amdgcn_exp2f(-(float)ev) : 1.0f;
 #pragma unroll
     for (int t = 0; t < 2; ++t)
@@ -371,22 +421,24 @@ __device__ __forceinline__ bool tile_pass(const TileCtx& cx) {
     if (prepare_direction<NG, true, GENERAL>(gDf, rawq, rawk, sc, dtab_f, kreg, lane, eq, ek, qhf, p16)) veto = true;
   }
   VIG_PHASE();
-#ifdef VIG_LATE_GB
-  if (BIDIR) issue_tdwords<0, 2, NG>(cx.gb, r, h, gDb);
-#endif
   if (BIDIR) {
     char* kreg = ti > 0 ? lds + lay.kb + (ti - 1) * TileLds<NG>::KB : nullptr;
     u32x4_t pb[2];
-    // (opaque copies: the unpacked halves of the raw rows are rebuilt here instead of being carried, 64 registers wide,
-    // from the forward direction's loop)
+    if (GENERAL) {
+      // (opaque copies: the unpacked halves of the raw rows are rebuilt here instead of being carried, 64 registers
+      // wide, from the forward direction's loop)
 #pragma unroll
-    for (int g = 0; g < NG; ++g)
+      for (int g = 0; g < NG; ++g)
 #pragma unroll
-      for (int m = 0; m < 4; ++m) {
-        asm volatile("" : "+v"(rawq[g][m]));
-        asm volatile("" : "+v"(rawk[g][m]));
-      }
-    if (prepare_direction<NG, false, GENERAL>(gDb, rawq, rawk, sc, dtab_b, kreg, lane, eq, ek, qhb, pb)) veto = true;
+        for (int m = 0; m < 4; ++m) {
+          asm volatile("" : "+v"(rawq[g][m]));
+          asm volatile("" : "+v"(rawk[g][m]));
+        }
+    }
+    // (lane-derived constants of this direction are built here, not carried from the top of the kernel)
+    int lane_b = lane;
+    asm volatile("" : "+v"(lane_b));
+    if (prepare_direction<NG, false, GENERAL>(gDb, rawq, rawk, sc, dtab_b, kreg, lane_b, eq, ek, qhb, pb)) veto = true;
     // (the two directions meet on the pairs j = i only: one more fp16 rounding there)
 #pragma unroll
     for (int t = 0; t < 2; ++t)
@@ -412,28 +464,122 @@ __device__ __forceinline__ bool tile_pass(const TileCtx& cx) {
     if (__builtin_amdgcn_ballot_w64(mine != 0.0f) != 0) return true;
   }
   // ---- the other tiles, outwards ----
-  walk_tiles<NG, true>(lds, lay, ti, NT, lane, qhf, O);
-  if (BIDIR) walk_tiles<NG, false>(lds, lay, ti, NT, lane, qhb, O);
-  // ---- store: lane (r, h) holds channels [32h, 32h + 32) of token r; rows beyond the sequence are dropped ----
+  int lane_w = lane;
+  asm volatile("" : "+v"(lane_w));
+  walk_tiles<NG, true>(lds, lay, ti, NT, lane_w, qhf, O);
+  if (BIDIR) walk_tiles<NG, false>(lds, lay, ti, NT, lane_w, qhb, O);
   float os = cx.oscale;
   if (GENERAL) os *= __builtin_amdgcn_exp2f((float)(eq + ek + ev));
+  if (GATE) {
+    // ---- fused locality gate: y = o * sigmoid(conv3x3(o)) per channel on the gw x gh token grid (zero padding), o
+    // being the bf16-rounded output.  The whole slab's outputs are staged in LDS where the tiles lay. ----
+    const int pw = cx.gw + 2;
+    char* cells = lds;
+    float* wlds = reinterpret_cast<float*>(lds + pw * (cx.gh + 2) * 128);
+    const float inv_w = 1.0f / (float)cx.gw;
+    // the head's stencil weights, fetched by the first 144 threads while the other waves finish their walks
+    f32x4_t w4 = {0.f, 0.f, 0.f, 0.f};
+    const bool w_mine = ti * 64 + lane_w < 64 * 9 / 4;
+    if (w_mine) w4 = reinterpret_cast<const f32x4_t*>(cx.gate_w)[ti * 64 + lane_w];
+    lds_barrier();  // every wave is done with the tiles
+    if (w_mine) reinterpret_cast<f32x4_t*>(wlds)[ti * 64 + lane_w] = w4;
+    // (workgroups of fewer than three waves: the rest of the 144 pieces)
+    for (int idx = ti * 64 + lane_w + 64 * NT; idx < 64 * 9 / 4; idx += 64 * NT)
+      reinterpret_cast<f32x4_t*>(wlds)[idx] = reinterpret_cast<const f32x4_t*>(cx.gate_w)[idx];
+    {
+      const int T = 32 * ti + (lane_w & 31);
+      if (T < cx.gw * cx.gh) {
+        const int y = (int)(((float)T + 0.5f) * inv_w), x = T - __mul24(y, cx.gw);
+        char* cell = cells + ((y + 1) * pw + x + 1) * 128 + 64 * (lane_w >> 5);
+#pragma unroll
+        for (int gq = 0; gq < 4; ++gq) {
+          u32x4_t w;
+#pragma unroll
+          for (int m = 0; m < 4; ++m) w[m] = pack_bf16x2(O[0][4 * gq + m] * os, O[1][4 * gq + m] * os);
+          *reinterpret_cast<u32x4_t*>(cell + 16 * gq) = w;
+        }
+      }
+    }
+    const int oct = lane_w & 7, tl = lane_w >> 3;
+    {  // the border cells, by the whole workgroup: top row, bottom row, then the two ends of every other row
+      const int nborder = 2 * pw + 2 * cx.gh;
+      const u32x4_t zero = {0u, 0u, 0u, 0u};
+      for (int bc = ti * 8 + tl; bc < nborder; bc += 8 * NT) {
+        int py, px;
+        if (bc < 2 * pw) {
+          py = bc < pw ? 0 : cx.gh + 1;
+          px = bc < pw ? bc : bc - pw;
+        } else {
+          const int j = bc - 2 * pw;
+          py = 1 + (j >> 1);
+          px = (j & 1) ? pw - 1 : 0;
+        }
+        *reinterpret_cast<u32x4_t*>(cells + (py * pw + px) * 128 + 16 * oct) = zero;
+      }
+    }
+    lds_barrier();  // the slab's outputs, the zero border and the weights are staged
+    float wreg[8][9];
+    {
+      const f32x4_t* wp = reinterpret_cast<const f32x4_t*>(wlds + oct * 72);
+#pragma unroll
+      for (int i = 0; i < 18; ++i) {
+        const f32x4_t x = wp[i];
+#pragma unroll
+        for (int m = 0; m < 4; ++m) wreg[(4 * i + m) / 9][(4 * i + m) % 9] = x[m];
+      }
+    }
+#pragma unroll 1
+    for (int i = 0; i < 4; ++i) {
+      const int row = tl + 8 * i;
+      const int T = 32 * ti + row;
+      if (T < cx.gw * cx.gh) {
+        const int y = (int)(((float)T + 0.5f) * inv_w), x = T - __mul24(y, cx.gw);
+        float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f}, ctr[8];
+#pragma unroll
+        for (int di = 0; di < 3; ++di) {
+          const char* tap = cells + ((y + di) * pw + x) * 128 + 16 * oct;  // padded cell of tap (di - 1, -1)
+#pragma unroll
+          for (int dj = 0; dj < 3; ++dj) {
+            const u32x4_t w = *reinterpret_cast<const u32x4_t*>(tap + dj * 128);
+#pragma unroll
+            for (int m = 0; m < 4; ++m) {
+              const float lo = bf16lo_to_f32(w[m]), hi = bf16hi_to_f32(w[m]);
+              acc[2 * m] = __builtin_fmaf(lo, wreg[2 * m][di * 3 + dj], acc[2 * m]);
+              acc[2 * m + 1] = __builtin_fmaf(hi, wreg[2 * m + 1][di * 3 + dj], acc[2 * m + 1]);
+              if (di == 1 && dj == 1) ctr[2 * m] = lo, ctr[2 * m + 1] = hi;
+            }
+          }
+        }
+        u32x4_t out;
+#pragma unroll
+        for (int m = 0; m < 4; ++m)
+          out[m] = pack_bf16x2(ctr[2 * m] * sigmoidf_(acc[2 * m]), ctr[2 * m + 1] * sigmoidf_(acc[2 * m + 1]));
+        __builtin_amdgcn_raw_buffer_store_b128(out, cx.o, (unsigned)row * 128u + 16u * oct, 0, 0);
+      }
+    }
+    return false;
+  }
+  // ---- store: lane (r, h) holds channels [32h, 32h + 32) of token r; rows beyond the sequence are dropped ----
 #pragma unroll
   for (int gq = 0; gq < 4; ++gq) {
     u32x4_t x;
 #pragma unroll
     for (int m = 0; m < 4; ++m) x[m] = pack_bf16x2(O[0][4 * gq + m] * os, O[1][4 * gq + m] * os);
-    __builtin_amdgcn_raw_buffer_store_b128(x, cx.o, (unsigned)r * 128u + 64u * h + 16u * gq, 0, 0);
+    __builtin_amdgcn_raw_buffer_store_b128(x, cx.o, (unsigned)(lane_w & 31) * 128u + 64u * (lane_w >> 5) + 16u * gq, 0, 0);
   }
   return false;
 }
 
-template <int NG, bool BIDIR, bool PITCHED>
+template <int NG, bool BIDIR, bool PITCHED, bool GATE>
 __device__ __forceinline__ TileCtx make_tile_ctx(const uint16_t* q, const uint16_t* k, const uint16_t* v,
                                                  const uint16_t* gf, const uint16_t* gb, uint16_t* o,
-                                                 const TileGeo& geo, float oscale, char* lds) {
+                                                 const TileGeo& geo, float oscale, const float* gate_w, char* lds) {
   constexpr int DK = 16 * NG;
   TileCtx cx;
   cx.lds = lds;
+  cx.gw = GATE ? geo.gw : 0, cx.gh = GATE ? geo.gh : 0;
+  // (slab = batch element * heads + head)
+  cx.gate_w = GATE ? gate_w + (size_t)((int)blockIdx.x % geo.heads) * (64 * 9) : nullptr;
   cx.ti = __builtin_amdgcn_readfirstlane((int)threadIdx.x >> 6);
   cx.lane = threadIdx.x & 63;
   cx.NT = geo.NT;
@@ -461,49 +607,66 @@ __device__ __forceinline__ TileCtx make_tile_ctx(const uint16_t* q, const uint16
 }
 
 // the general form as a function of its own: its register needs stay out of the fp16 form's allocation
-template <int NG, bool BIDIR, bool PITCHED>
-__device__ __noinline__ void tile_pass_general(const uint16_t* q, const uint16_t* k, const uint16_t* v,
+template <int NG, bool BIDIR, bool PITCHED, bool GATE>
+__device__ VIG_GENERAL_INLINE void tile_pass_general(const uint16_t* q, const uint16_t* k, const uint16_t* v,
                                                const uint16_t* gf, const uint16_t* gb, uint16_t* o, const TileGeo* geo,
-                                               float oscale, char* lds) {
-  const TileCtx cx = make_tile_ctx<NG, BIDIR, PITCHED>(q, k, v, gf, gb, o, *geo, oscale, lds);
-  tile_pass<NG, BIDIR, PITCHED, true>(cx);
+                                               float oscale, const float* gate_w, char* lds) {
+  const TileCtx cx = make_tile_ctx<NG, BIDIR, PITCHED, GATE>(q, k, v, gf, gb, o, *geo, oscale, gate_w, lds);
+  tile_pass<NG, BIDIR, PITCHED, true, GATE>(cx);
 }
 
 }  // namespace
 
-template <int NG, bool BIDIR, bool PITCHED>
+template <int NG, bool BIDIR, bool PITCHED, bool GATE>
 __global__ __launch_bounds__(512, 4) void gla_tile_kernel(const uint16_t* __restrict__ q, const uint16_t* __restrict__ k,
                                                           const uint16_t* __restrict__ v,
                                                           const uint16_t* __restrict__ gf,
                                                           const uint16_t* __restrict__ gb, uint16_t* __restrict__ o,
-                                                          TileGeo geo, float oscale) {
+                                                          TileGeo geo, float oscale,
+                                                          const float* __restrict__ gate_w) {
   extern __shared__ __align__(16) char lds[];
   bool redo = true;
   if (!geo.wide) {
-    const TileCtx cx = make_tile_ctx<NG, BIDIR, PITCHED>(q, k, v, gf, gb, o, geo, oscale, lds);
-    redo = tile_pass<NG, BIDIR, PITCHED, false>(cx);
+    const TileCtx cx = make_tile_ctx<NG, BIDIR, PITCHED, GATE>(q, k, v, gf, gb, o, geo, oscale, gate_w, lds);
+    redo = tile_pass<NG, BIDIR, PITCHED, false, GATE>(cx);
   }
-  if (redo) tile_pass_general<NG, BIDIR, PITCHED>(q, k, v, gf, gb, o, &geo, oscale, lds);
+  if (redo) {
+    // (a copy made here: taking the address of the kernel argument itself would move it, and with it every
+    // descriptor built from it, into per-lane memory for the whole kernel)
+    TileGeo geo_copy = geo;
+    tile_pass_general<NG, BIDIR, PITCHED, GATE>(q, k, v, gf, gb, o, &geo_copy, oscale, gate_w, lds);
+  }
 }
+
+constexpr int kTileMaxLds = 160 * 1024;
 
 bool gla_tiles_supported(const GlaArgs& a) {
-  return a.io_dtype == 1 && a.gate_dtype == 1 && (a.Dk == 64 || a.Dk == 32) && a.Dv == 64 && a.L <= 256 &&
-         !a.init_state && !a.final_state && !a.state_pass && !a.gate_w;
+  if (!(a.io_dtype == 1 && a.gate_dtype == 1 && (a.Dk == 64 || a.Dk == 32) && a.Dv == 64 && a.L <= 256 &&
+        !a.init_state && !a.final_state && !a.state_pass))
+    return false;
+  if (a.gate_w) {  // fused locality gate: both directions, plain tensors, the padded grid has to fit in LDS
+    if (!a.g_bwd || a.q_strides || a.k_strides || a.v_strides || a.gate_cols <= 0 || a.gate_rows <= 0 ||
+        (long long)a.gate_cols * a.gate_rows != a.L)
+      return false;
+    if (TileLds<4>((a.L + 31) / 32, gate_stage_bytes(a.gate_cols, a.gate_rows)).total > kTileMaxLds) return false;
+  }
+  return true;
 }
 
-template <int NG, bool BIDIR, bool PITCHED>
+template <int NG, bool BIDIR, bool PITCHED, bool GATE>
 static int launch_tiles_t(const GlaArgs& a, const TileGeo& geo, int dev) {
   constexpr int kMaxDevices = 64;
   static bool attr_done_dev[kMaxDevices] = {};
-  const void* kf = reinterpret_cast<const void*>(gla_tile_kernel<NG, BIDIR, PITCHED>);
+  const void* kf = reinterpret_cast<const void*>(gla_tile_kernel<NG, BIDIR, PITCHED, GATE>);
   if (!attr_done_dev[dev]) {
-    if (hipFuncSetAttribute(kf, hipFuncAttributeMaxDynamicSharedMemorySize, TileLds<NG>(8).total) != hipSuccess) return -5;
+    if (hipFuncSetAttribute(kf, hipFuncAttributeMaxDynamicSharedMemorySize, kTileMaxLds) != hipSuccess) return -5;
     attr_done_dev[dev] = true;
   }
-  const TileLds<NG> lay(geo.NT);
-  hipLaunchKernelGGL((gla_tile_kernel<NG, BIDIR, PITCHED>), dim3(a.B * a.H), dim3(64 * geo.NT), lay.total, a.stream,
+  const TileLds<NG> lay(geo.NT, GATE ? gate_stage_bytes(geo.gw, geo.gh) : 0);
+  if (lay.total > kTileMaxLds) return -95;
+  hipLaunchKernelGGL((gla_tile_kernel<NG, BIDIR, PITCHED, GATE>), dim3(a.B * a.H), dim3(64 * geo.NT), lay.total, a.stream,
                      (const uint16_t*)a.q, (const uint16_t*)a.k, (const uint16_t*)a.v, (const uint16_t*)a.g_fwd,
-                     (const uint16_t*)a.g_bwd, (uint16_t*)a.o, geo, a.scale * a.out_scale);
+                     (const uint16_t*)a.g_bwd, (uint16_t*)a.o, geo, a.scale * a.out_scale, a.gate_w);
   return hipGetLastError() == hipSuccess ? 0 : -5;
 }
 
@@ -533,12 +696,19 @@ int launch_gla_tiles(const GlaArgs& a) {
     }
   }
   const bool bidir = a.g_bwd != nullptr;
-  if (a.Dk == 64) {
-    if (pitched) return bidir ? launch_tiles_t<4, true, true>(a, geo, dev) : launch_tiles_t<4, false, true>(a, geo, dev);
-    return bidir ? launch_tiles_t<4, true, false>(a, geo, dev) : launch_tiles_t<4, false, false>(a, geo, dev);
+  if (a.gate_w) {
+    geo.gw = a.gate_cols, geo.gh = a.gate_rows, geo.heads = a.H;
+    return a.Dk == 64 ? launch_tiles_t<4, true, false, true>(a, geo, dev) : launch_tiles_t<2, true, false, true>(a, geo, dev);
   }
-  if (pitched) return bidir ? launch_tiles_t<2, true, true>(a, geo, dev) : launch_tiles_t<2, false, true>(a, geo, dev);
-  return bidir ? launch_tiles_t<2, true, false>(a, geo, dev) : launch_tiles_t<2, false, false>(a, geo, dev);
+  geo.heads = 1;
+  if (a.Dk == 64) {
+    if (pitched)
+      return bidir ? launch_tiles_t<4, true, true, false>(a, geo, dev) : launch_tiles_t<4, false, true, false>(a, geo, dev);
+    return bidir ? launch_tiles_t<4, true, false, false>(a, geo, dev) : launch_tiles_t<4, false, false, false>(a, geo, dev);
+  }
+  if (pitched)
+    return bidir ? launch_tiles_t<2, true, true, false>(a, geo, dev) : launch_tiles_t<2, false, true, false>(a, geo, dev);
+  return bidir ? launch_tiles_t<2, true, false, false>(a, geo, dev) : launch_tiles_t<2, false, false, false>(a, geo, dev);
 }
 
 }  // namespace vig
