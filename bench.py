@@ -202,6 +202,85 @@ def backward_time(lib, sets, s, io_dt, scale, sp, stream, dev, iters=60):
                        "matrix cores (segments of <= 256 tokens linked by states), bf16 operands")}
 
 
+
+def other_workload_time(lib, idx, dev, stream, steps=20, warmup=5):
+    """Event-bracketed time of one more named workload (op only): inputs of the workload's shape and distributions drawn
+    on the device (timing only: the parity tests use the seeded CPU draws), >= 3 sets and > 256 MB rotated."""
+    import torch
+    import torch.nn.functional as F
+
+    from vig_amd import _lib
+    from vig_amd.synthetic import CONFIGS, make_locality_weight
+
+    s = CONFIGS[idx]
+    g = torch.Generator(device=dev)
+    g.manual_seed(1000 + idx)
+    nsets = max(3, int(300e6 // s.alg_bytes()) + 1)
+    sets = []
+    for _ in range(nsets):
+        q = torch.randn(s.B, s.H, s.L, s.Dk, device=dev, generator=g)
+        k = torch.randn(s.B, s.H, s.L, s.Dk, device=dev, generator=g) * s.Dk ** -0.5
+        v = torch.randn(s.B, s.H, s.L, s.Dv, device=dev, generator=g)
+        gf = F.logsigmoid(torch.randn(s.B, s.H, s.L, s.Dk, device=dev, generator=g)) / 16
+        gb = F.logsigmoid(torch.randn(s.B, s.H, s.L, s.Dk, device=dev, generator=g)) / 16
+        sets.append(tuple(t.bfloat16() for t in (q, k, v, gf, gb)) + (torch.empty(s.B, s.H, s.L, s.Dv, dtype=torch.bfloat16, device=dev),))
+    ws_bytes = lib.vig_gla_bidir_fwd_workspace(s.B, s.H, s.L, s.Dk, s.Dv, _lib.VIG_BF16)
+    ws = torch.empty(max(ws_bytes, 1), dtype=torch.uint8, device=dev)
+    sp = stream.cuda_stream
+    scale = s.Dk ** -0.5
+    gate_w = None
+    if idx == 2:
+        gate_w = make_locality_weight(s.H * s.Dv, 2002).reshape(s.H * s.Dv, 9).float().contiguous().to(dev)
+
+    def step(i):
+        q, k, v, gf, gb, o = sets[i % nsets]
+        if gate_w is not None:
+            rc = lib.vig_gla_bidir_locgate_fwd(q.data_ptr(), k.data_ptr(), v.data_ptr(), gf.data_ptr(), gb.data_ptr(),
+                                               gate_w.data_ptr(), o.data_ptr(), s.B, s.H, s.L, s.Dk, s.Dv, s.grid[0],
+                                               s.grid[1], scale, 1.0, _lib.VIG_BF16, _lib.VIG_BF16, sp)
+        else:
+            rc = lib.vig_gla_bidir_fwd(q.data_ptr(), k.data_ptr(), v.data_ptr(), gf.data_ptr(), gb.data_ptr(), o.data_ptr(),
+                                       ws.data_ptr(), ws_bytes, s.B, s.H, s.L, s.Dk, s.Dv, scale, 1.0, _lib.VIG_BF16,
+                                       _lib.VIG_BF16, sp)
+        if rc != 0:
+            raise RuntimeError(f"workload {idx}: rc={rc}")
+
+    for i in range(warmup):
+        step(i)
+    evs = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(steps)]
+    for i, (a, b) in enumerate(evs):
+        a.record(stream)
+        step(i)
+        b.record(stream)
+    torch.cuda.synchronize()
+    durs = sorted(a.elapsed_time(b) * 1e3 for a, b in evs)
+    us = sum(durs) / len(durs)
+    gbps = s.alg_bytes() / (us * 1e-6) / 1e9
+    out = {"workload": s.name, "steps": steps, "us": us, "us_min": durs[0], "algorithmic_bytes": s.alg_bytes(),
+           "achieved_GBps": gbps, "frac": gbps / HBM_PEAK_GBPS, "tflops_algorithmic": s.alg_flops() / (us * 1e-6) / 1e12,
+           "inputs": "the workload's shape and distributions, drawn on the device", "traffic": None}
+    out.update(_measured_traffic(s.name, "traffic"))
+    if idx == 2:
+        out["locality_gate"] = "inside the GLA kernel"
+    del sets
+    return out
+
+
+def _measured_traffic(key, field="traffic"):
+    """HBM bytes per launch from the rocprofv3 counter runs kept under profiles/ (FETCH_SIZE / WRITE_SIZE scaled by a
+    copy kernel of known size), with the source commit and date of that counter run."""
+    try:
+        with open(os.path.join(ROOT, "profiles", "hbm_traffic.json")) as f:
+            t = json.load(f)
+        e = t.get(key)
+        if not e:
+            return {field: None}
+        return {field: e.get("bytes_per_launch"),
+                field + "_measured": {"commit": e.get("commit", t.get("_commit")), "date": e.get("date", t.get("_date")),
+                                      "kernels": e.get("kernels")}}
+    except (OSError, ValueError):
+        return {field: None}
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -342,13 +421,8 @@ def main():
     log(f"wall {ms_per_step*1e3:.1f} us/step; event-bracketed launch avg {k_avg*1e3:.1f} us, median {k_med*1e3:.1f}, min {k_min*1e3:.1f}")
 
     # HBM bytes per launch measured with rocprofv3 --pmc (FETCH_SIZE / WRITE_SIZE, scaled by a copy kernel of known
-    # size); the figures live with the profile summaries and are keyed by workload
-    traffic = None
-    try:
-        with open(os.path.join(ROOT, "profiles", "hbm_traffic.json")) as f:
-            traffic = json.load(f).get(s.name, {}).get("bytes_per_launch")
-    except (OSError, ValueError):
-        pass
+    # size); the figures live with the profile summaries, keyed by workload, with the commit and date they were taken at
+    traffic = _measured_traffic(s.name)
 
     tflops = alg_flops / (ms_per_step * 1e-3) / 1e12
     achieved_gbps = alg_bytes / (k_avg * 1e-3) / 1e9
@@ -376,7 +450,7 @@ def main():
         "executed_tflops_chunk64": s.tokens * exec_flops_tok / (ms_per_step * 1e-3) / 1e12,
         "kernel_us": {"avg": k_avg * 1e3, "median": k_med * 1e3, "min": k_min * 1e3},
         "roofline": {"bound": "hbm", "achieved": achieved_gbps, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-                     "frac": achieved_gbps / HBM_PEAK_GBPS, "traffic": traffic},
+                     "frac": achieved_gbps / HBM_PEAK_GBPS, **traffic},
     }
     # the headline run (config 1) also reports the other half of the metric (ViG-S images/s) and the backward
     want_backward = (args.backward or args.config == 1) and not args.op_only and not args.exact
@@ -384,11 +458,15 @@ def main():
     if want_backward:
         out["backward"] = backward_time(lib, sets, s, io_dt, scale, sp, stream, dev)
         if out["backward"] is not None:
-            try:  # measured HBM bytes of the backward launch, where the profile summaries hold them
-                with open(os.path.join(ROOT, "profiles", "hbm_traffic.json")) as f:
-                    out["backward"]["traffic"] = json.load(f).get(s.name + ":backward", {}).get("bytes_per_launch")
-            except (OSError, ValueError):
-                out["backward"]["traffic"] = None
+            out["backward"].update(_measured_traffic(s.name + ":backward"))
+    if args.config == 1 and not args.op_only and not args.exact:
+        # the other named workloads, op only, 20 steps each: every roofline figure of the report is timed by this run
+        others = {}
+        for idx in (2, 3, 4):
+            others[f"cfg{idx}"] = other_workload_time(lib, idx, dev, stream)
+            log(f"workload {idx}: {others[f'cfg{idx}']['us']:.1f} us, {100 * others[f'cfg{idx}']['frac']:.1f} % of HBM peak")
+        out["other_workloads"] = others
+        out["long_sequence"] = others["cfg3"]  # the 4096-token workload: the second named target
     if want_model:
         if args.train:
             out["vig_s_train_step"] = train_step_throughput(dev, tune_gemm=not args.no_gemm_tuning)

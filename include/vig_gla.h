@@ -58,18 +58,23 @@ const char* vig_gla_strerror(int code);
  *
  * Built shapes: Dk in {16, 32, 64, 128}, Dv in {32, 64, 128}, any L >= 1.
  *
- * Numeric range of the matrix-core path (bf16 tensors and gates, Dk in {32, 64},
- * Dv = 64): the sum of |g| over any 64 consecutive tokens of one channel must
- * stay below about 80 (beyond it results may be inf / NaN, never silently wrong
- * finite numbers).  q, k and v may hold any finite bf16 values: the kernel
- * checks their magnitudes and the gate totals per chunk and takes its fp16
- * operands (scaled q and k, scores, v, and for L <= 256 each chunk's 64 x 64
- * sum of k^T v) only where they are exact enough (rows with sums of squares
- * below 2^15, i.e. elements below about 180; gate total of a chunk within about
- * 8; chunk sums below 60000), bf16 hi + lo pairs otherwise.  HierViG's head shape
- * (bf16, Dk = 16, Dv = 32, both directions) takes the same path from L = 128 on,
- * zero-padded to Dk 32 / Dv 64 in the workspace (classification/models/vig_h.py:
- * 377-385 with EXPAND_K 0.5, EXPAND_V 1.0).  Other combinations run on the
+ * Numeric range of the matrix-core paths (bf16 tensors and gates, Dk in {32, 64},
+ * Dv = 64).  q, k and v may hold any finite bf16 values; the kernels check
+ * magnitudes and gate totals themselves and switch arithmetic where needed:
+ *   L <= 256 (one workgroup per sequence, one wave per 32-token tile): fp16
+ *   operands while every tile's gate total stays within about 7 (natural log
+ *   units) per channel and rows of q / k / v have sums of squares below 2^15 /
+ *   2^10 / 10^8; a sequence outside that is redone by the same workgroup with
+ *   power-of-two input scales and split-bf16 diagonal tiles, good for gates down
+ *   to about -5 per token (beyond: exponents are clamped, far tokens count as 0).
+ *   L > 256 (segments of <= 256 tokens chained through states in the workspace;
+ *   refused with VIG_ENOTSUP when B*H*directions > 65535): the sum of |g| over
+ *   any 64 consecutive tokens of one channel must stay below about 80 (beyond it
+ *   results may be inf / NaN, never silently wrong finite numbers).
+ * HierViG's head shape (bf16, Dk = 16, Dv = 32, both directions) takes the same
+ * paths from L = 128 on, zero-padded to Dk 32 / Dv 64 in the workspace
+ * (classification/models/vig_h.py:377-385 with EXPAND_K 0.5, EXPAND_V 1.0).
+ * Other combinations run on the
  * fp32-arithmetic kernel, which has no such limit.
  */
 int vig_gla_bidir_fwd(const void* q, const void* k, const void* v,
@@ -160,8 +165,11 @@ int vig_gla_bidir_fwd_wide(const void* q, const void* k, const void* v,
  * vig_gla_bidir_fwd_workspace_for(...) exceeds that size returns VIG_ENOSPC and launches nothing (then use
  * vig_gla_bidir_fwd with a workspace of the caller's).  Calls no hipMalloc / hipFree and nothing else that allocates.
  * All calls on one GPU share the one array: calls that overlap in time on the same GPU (two streams, two threads)
- * race on it; serialise them.  It has no counterpart in the reference, whose ops allocate their temporaries through
- * torch (flash-linear-attention/fla/ops/gla/chunk_fuse.py:325-345).
+ * race on it; serialise them.  The tensors must live on the current device (another device's pointers: VIG_EINVAL).
+ * Under HIP graph capture: make one call per device and shape class outside the capture first.  The first call on a
+ * device looks up the array's address and sets the kernels' shared-memory attribute (no stream work, but not capturable
+ * either); every later call is kernel launches on `stream` only.  It has no counterpart in the reference, whose ops
+ * allocate their temporaries through torch (flash-linear-attention/fla/ops/gla/chunk_fuse.py:325-345).
  */
 #define VIG_GLA_NOALLOC_SCRATCH_BYTES (16u << 20)
 int vig_gla_bidir_fwd_noalloc(const void* q, const void* k, const void* v,

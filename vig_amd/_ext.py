@@ -36,6 +36,11 @@ def load():
     except Exception as e:  # an operator library built against another torch: the ctypes binding still works
         _error = f"{type(e).__name__}: {e}"
         _ops = None
+        import warnings
+
+        warnings.warn(f"vig_amd: {EXT_PATH} exists but did not load ({_error}); falling back to the ctypes binding, "
+                      "which costs about twice the host time per call. Rebuild it with `python -m vig_amd.build`.",
+                      RuntimeWarning, stacklevel=2)
     return _ops
 
 

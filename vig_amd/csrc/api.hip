@@ -280,9 +280,18 @@ constexpr int kScratchMaxDevices = 64;
 static void* scratch_ptr[kScratchMaxDevices] = {};
 static std::mutex scratch_mutex;
 
-static int scratch_for_current_device(void** out) {
+// `owned`: a device pointer of the call (q).  The array that serves a call is the one of the GPU that holds the
+// call's tensors, which has to be the current device (the kernels are launched there, and the symbol lookup answers
+// for the current device only): a caller on another device is refused instead of being handed the wrong GPU's array.
+static int scratch_for_current_device(void** out, const void* owned) {
   int dev = 0;
   if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kScratchMaxDevices) return VIG_ELAUNCH;
+  hipPointerAttribute_t attr;
+  if (hipPointerGetAttributes(&attr, owned) == hipSuccess) {
+    if (attr.type == hipMemoryTypeDevice && attr.device != dev) return VIG_EINVAL;
+  } else {
+    (void)hipGetLastError();  // (an unregistered pointer: the launch itself will report it)
+  }
   std::lock_guard<std::mutex> lock(scratch_mutex);
   if (!scratch_ptr[dev]) {
     void* p = nullptr;
@@ -305,7 +314,7 @@ int vig_gla_bidir_fwd_noalloc(const void* q, const void* k, const void* v, const
   if (need > kScratchBytes) return VIG_ENOSPC;
   void* ws = nullptr;
   if (need > 0) {
-    const int rc = scratch_for_current_device(&ws);
+    const int rc = scratch_for_current_device(&ws, q);
     if (rc != VIG_OK) return rc;
   }
   // Every kernel behind vig_gla_bidir_fwd writes the part of the workspace it later reads (segment states, padded

@@ -385,7 +385,9 @@ class GLABlock(nn.Module):
         if (ext is not None and not _recording(self) and not self.training and branch.is_cuda and branch.is_contiguous()
                 and type(at) is GatedLinearAttention and at.gk_proj[0].weight.shape[0] == ops.GATE_RANK
                 and branch.dtype == at.qkv_proj.weight.dtype and kwargs.get("token_position", None) is None
-                and (residual is None or (residual.is_contiguous() and residual.dtype == branch.dtype))):
+                and (residual is None or (residual.is_contiguous() and residual.dtype == branch.dtype))
+                # (the operator takes one eps for both norms and the eval-mode output scale)
+                and self.mlp_norm.eps == self.attn_norm.eps and not at.training):
             # the whole block as one operator of the library (csrc/torch_ext.cpp: the same kernel sequence as below)
             hw = tuple(kwargs["patch_resolution"])
             conv, up = at.in_proj[0], at.gk_proj[1]

@@ -147,6 +147,12 @@ def _gla_bidir_forward_strided(q, k, v, g_fwd, g_bwd, scale, out_scale, out):
     if k.shape != q.shape or g_fwd.shape != q.shape or v.shape[:3] != q.shape[:3] or k.dtype != q.dtype or v.dtype != q.dtype:
         return None
     B, H, L, Dk = q.shape
+    # the same refusals as the dense path, before anything is handed to a kernel that trusts its arguments
+    if g_bwd is not None and (g_bwd.dtype != g_fwd.dtype or g_bwd.shape != g_fwd.shape):
+        raise ValueError("g_bwd must match g_fwd in dtype and shape")
+    if out is not None and not (out.is_contiguous() and out.data_ptr() % 16 == 0 and out.shape == (B, H, L, 64)
+                                and out.dtype == q.dtype and out.device == q.device):
+        raise ValueError("bad `out` tensor")
     strides = []
     for t, D in ((q, Dk), (k, Dk), (v, 64)):
         st = _head_view_strides(t)
