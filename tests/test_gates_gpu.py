@@ -184,6 +184,16 @@ def _gla_inputs(B, H, L, Dk, seed, gate_scale=None):
     return q, k, v, gf, gb
 
 
+def _assert_fused_equals_two_calls(got, two, plain):
+    """The one-kernel gate against GLA kernel + stencil kernel: bit for bit, except under outputs of the GLA (`plain`)
+    below 2^-14: the fused kernel stages them as fp16, whose grid there (steps of 2^-24) is coarser than bf16's, so
+    such an output, and the gate's product with it, may move by that step."""
+    differs = got != two
+    assert not (differs & (plain.abs() >= 2.0 ** -14)).any()
+    assert ((got.float() - two.float()).abs() <= 2.0 ** -24).all()
+    assert differs.float().mean().item() <= 1e-4
+
+
 @pytest.mark.parametrize("B,H,hw,Dk", [(2, 12, (14, 14), 64), (3, 2, (16, 16), 64), (5, 3, (7, 7), 32),
                                         (2, 2, (3, 5), 64), (1, 3, (1, 9), 64), (2, 1, (12, 1), 32),
                                         (1, 2, (6, 40), 64), (1, 1, (1, 1), 64)])
@@ -197,8 +207,9 @@ def test_fused_locality_gate_matches_two_calls_and_oracle(B, H, hw, Dk):
     wt = make_locality_weight(H * 64, 31)
     dq, dk, dv, dgf, dgb = (t.cuda() for t in (q, k, v, gf, gb))
     got = vig_amd.gla_bidir_locality_gate(dq, dk, dv, dgf, dgb, wt.cuda(), hw)
-    two = vig_amd.locality_gate(vig_amd.gla_bidir_forward(dq, dk, dv, dgf, dgb), wt.cuda(), hw)
-    assert torch.equal(got, two)
+    plain = vig_amd.gla_bidir_forward(dq, dk, dv, dgf, dgb)
+    two = vig_amd.locality_gate(plain, wt.cuda(), hw)
+    _assert_fused_equals_two_calls(got, two, plain)
     o = oracle_bidir(q, k, v, gf, gb)
     want = O.locality_sigmoid_gate_reference(o, f64(wt), hw)
     assert max_abs(f64(got), want) <= 2e-2
@@ -216,9 +227,10 @@ def test_fused_locality_gate_many_slabs_mixed_gate_strength():
     wt = make_locality_weight(H * 64, 33)
     dq, dk, dv, dgf, dgb = (t.cuda() for t in (q, k, v, gf, gb))
     got = vig_amd.gla_bidir_locality_gate(dq, dk, dv, dgf, dgb, wt.cuda(), hw)
-    two = vig_amd.locality_gate(vig_amd.gla_bidir_forward(dq, dk, dv, dgf, dgb), wt.cuda(), hw)
+    plain = vig_amd.gla_bidir_forward(dq, dk, dv, dgf, dgb)
+    two = vig_amd.locality_gate(plain, wt.cuda(), hw)
     assert torch.isfinite(got.float()).all()
-    assert torch.equal(got, two)
+    _assert_fused_equals_two_calls(got, two, plain)
 
 
 def test_fused_locality_gate_other_shapes_take_two_calls():

@@ -78,10 +78,12 @@ struct TileLds {
   }
 };
 
-// Fused locality gate: the slab's rounded outputs as a zero-padded (gh + 2) x (gw + 2) grid of 128-byte cells, then
-// the 64 x 9 stencil weights of the slab's head.
+// Fused locality gate: the slab's rounded outputs as a zero-padded (gh + 2) x (gw + 2) grid of cells (64 channels as
+// fp16: 128 bytes, 144 bytes apart, so that eight lanes on neighbouring tokens cover every LDS bank once), then the
+// 64 x 9 stencil weights of the slab's head.
 constexpr int kGateWeightBytes = 64 * 9 * 4;
-__host__ __device__ inline int gate_stage_bytes(int gw, int gh) { return (gw + 2) * (gh + 2) * 128 + kGateWeightBytes; }
+constexpr int kGateCell = 144;
+__host__ __device__ inline int gate_stage_bytes(int gw, int gh) { return (gw + 2) * (gh + 2) * kGateCell + kGateWeightBytes; }
 
 struct TileCtx {
   const float* gate_w;  // fused locality gate: [64][9] stencil weights of this slab's head
@@ -189,6 +191,7 @@ __device__ __forceinline__ bool prepare_direction(const uint32_t (&gD)[2][8], co
   const u32x4_t* dmine = reinterpret_cast<const u32x4_t*>(dtab + HC * (lane >> 5));  // this lane half's decays as fp16 pairs
   const float fq = -(float)eq, fk = -(float)ek;
   f32x16_t P = {0.f};
+  u32x4_t kc[NG];  // fp16 form: k' = k exp(-G), the diagonal tile's A operand
 #pragma unroll
   for (int g = 0; g < NG; ++g) {
     u32x4_t kh;
@@ -199,8 +202,9 @@ __device__ __forceinline__ bool prepare_direction(const uint32_t (&gD)[2][8], co
     }
     if (!GENERAL) {
       // rawq / rawk hold fp16 pairs here; the decay factors are rounded to fp16 and applied as packed products
+      // (the diagonal tile's products wait until the loop is through: their 16 accumulators would otherwise sit
+      // beside the cumulative gates and the raw rows, which are at their fullest in the first pieces)
       const u32x4_t d16 = dmine[g];
-      u32x4_t kc;
 #pragma unroll
       for (int m = 0; m < 4; ++m) {
         const int c = 4 * g + m;
@@ -208,13 +212,9 @@ __device__ __forceinline__ bool prepare_direction(const uint32_t (&gD)[2][8], co
         const uint32_t a16 = pack_f16x2(exp2_fast(x0), exp2_fast(x1));
         const uint32_t b16 = pack_f16x2(exp2_fast(-x0), exp2_fast(-x1));
         qh[g][m] = mul_f16x2(rawq[g][m], a16);
-        kc[m] = mul_f16x2(rawk[g][m], b16);
-        kh[m] = mul_f16x2(kc[m], d16[m]);
-#ifdef VIG_PREP_FENCE
-        if (m & 1) VIG_PHASE();
-#endif
+        kc[g][m] = mul_f16x2(rawk[g][m], b16);
+        kh[m] = mul_f16x2(kc[g][m], d16[m]);
       }
-      P = mfma_f16(kc, qh[g], P);
     } else {
       u32x4_t qhi, qlo, khi, klo;
 #pragma unroll
@@ -245,6 +245,11 @@ __device__ __forceinline__ bool prepare_direction(const uint32_t (&gD)[2][8], co
       P = mfma(khi, qlo, P);
     }
     if (kreg) *reinterpret_cast<u32x4_t*>(unit_ptr(kreg, g, lane)) = kh;
+  }
+  if (!GENERAL) {
+    VIG_PHASE();
+#pragma unroll
+    for (int g = 0; g < NG; ++g) P = mfma_f16(kc[g], qh[g], P);
   }
   // keep the pairs the direction sees (P^T[j, i]: lane = column i, register 4g+m = row 8g + 4h + m: the token of slot
   // pair x of k-step t, as in the triangular operand), round to fp16
@@ -320,6 +325,117 @@ __device__ __forceinline__ void walk_tiles(char* lds, const TileLds<NG>& lay, in
     const f32x16_t P = score_tile16<NG>(kf, qh);
     apply_values(P, vf, O);
   }
+}
+
+// Fused locality gate: y = o * sigmoid(conv3x3(o)) per channel on the gw x gh token grid (zero padding), o being the
+// bf16-rounded output.  The whole slab's outputs are staged in LDS where the tiles lay.  (A function of its own: its
+// 72 weight registers stay out of the main path's allocation.)
+__device__ __forceinline__ void locality_gate_epilogue(f32x16_t O0, f32x16_t O1, float os, char* lds, const float* gate_w,
+                                                    rsrc_t o_rsrc, int gw, int gh, int ti, int NT, int lane_w) {
+  struct { int gw, gh; const float* gate_w; rsrc_t o; } cx{gw, gh, gate_w, o_rsrc};
+  const f32x16_t O[2] = {O0, O1};
+    // ---- fused locality gate: y = o * sigmoid(conv3x3(o)) per channel on the gw x gh token grid (zero padding), o
+    // being the bf16-rounded output.  The whole slab's outputs are staged in LDS where the tiles lay. ----
+    const int pw = cx.gw + 2;
+    char* cells = lds;
+    float* wlds = reinterpret_cast<float*>(lds + pw * (cx.gh + 2) * kGateCell);
+    const float inv_w = 1.0f / (float)cx.gw;
+    // the head's stencil weights, fetched by the first 144 threads while the other waves finish their walks
+    f32x4_t w4 = {0.f, 0.f, 0.f, 0.f};
+    const bool w_mine = ti * 64 + lane_w < 64 * 9 / 4;
+    if (w_mine) w4 = reinterpret_cast<const f32x4_t*>(cx.gate_w)[ti * 64 + lane_w];
+    lds_barrier();  // every wave is done with the tiles
+    if (w_mine) reinterpret_cast<f32x4_t*>(wlds)[ti * 64 + lane_w] = w4;
+    // (workgroups of fewer than three waves: the rest of the 144 pieces)
+    for (int idx = ti * 64 + lane_w + 64 * NT; idx < 64 * 9 / 4; idx += 64 * NT)
+      reinterpret_cast<f32x4_t*>(wlds)[idx] = reinterpret_cast<const f32x4_t*>(cx.gate_w)[idx];
+    // The rounded outputs are staged as fp16 pairs (every bf16 value down to 2^-17 is an fp16 value), so that the
+    // stencil's multiply-adds read them in place (v_fma_mix_f32: fp16 x fp32 + fp32, the same fp32 arithmetic as on
+    // unpacked values, without the unpacking).
+    {
+      const int T = 32 * ti + (lane_w & 31);
+      if (T < cx.gw * cx.gh) {
+        const int y = (int)(((float)T + 0.5f) * inv_w), x = T - __mul24(y, cx.gw);
+        const int cell_i = (y + 1) * pw + x + 1;
+        char* cell = cells + cell_i * kGateCell;
+        const int hb = 4 * (lane_w >> 5);
+#pragma unroll
+        for (int gq = 0; gq < 4; ++gq) {
+          u32x4_t w;
+#pragma unroll
+          for (int m = 0; m < 4; ++m) {
+            const uint32_t b = pack_bf16x2(O[0][4 * gq + m] * os, O[1][4 * gq + m] * os);
+            w[m] = pack_f16x2(bf16lo_to_f32(b), bf16hi_to_f32(b));
+          }
+          *reinterpret_cast<u32x4_t*>(cell + 16 * (hb + gq)) = w;
+        }
+      }
+    }
+    const int oct = lane_w & 7, tl = lane_w >> 3;
+    {  // the border cells, by the whole workgroup: top row, bottom row, then the two ends of every other row
+      const int nborder = 2 * pw + 2 * cx.gh;
+      const u32x4_t zero = {0u, 0u, 0u, 0u};
+      for (int bc = ti * 8 + tl; bc < nborder; bc += 8 * NT) {
+        int py, px;
+        if (bc < 2 * pw) {
+          py = bc < pw ? 0 : cx.gh + 1;
+          px = bc < pw ? bc : bc - pw;
+        } else {
+          const int j = bc - 2 * pw;
+          py = 1 + (j >> 1);
+          px = (j & 1) ? pw - 1 : 0;
+        }
+        *reinterpret_cast<u32x4_t*>(cells + (py * pw + px) * kGateCell + 16 * oct) = zero;
+      }
+    }
+    lds_barrier();  // the slab's outputs, the zero border and the weights are staged
+    float wreg[8][9];
+    {
+      const f32x4_t* wp = reinterpret_cast<const f32x4_t*>(wlds + oct * 72);
+#pragma unroll
+      for (int i = 0; i < 18; ++i) {
+        const f32x4_t x = wp[i];
+#pragma unroll
+        for (int m = 0; m < 4; ++m) wreg[(4 * i + m) / 9][(4 * i + m) % 9] = x[m];
+      }
+    }
+#pragma unroll 1
+    for (int i = 0; i < 4; ++i) {
+      const int row = tl + 8 * i;
+      const int T = 32 * ti + row;
+      if (T < cx.gw * cx.gh) {
+        const int y = (int)(((float)T + 0.5f) * inv_w), x = T - __mul24(y, cx.gw);
+        float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+        u32x4_t ctr = {0u, 0u, 0u, 0u};
+#pragma unroll
+        for (int di = 0; di < 3; ++di) {
+          const char* rowp = cells + ((y + di) * pw + x) * kGateCell + 16 * oct;  // padded cell of tap (di - 1, -1)
+#pragma unroll
+          for (int dj = 0; dj < 3; ++dj) {
+            const u32x4_t w = *reinterpret_cast<const u32x4_t*>(rowp + dj * kGateCell);
+#pragma unroll
+            for (int m = 0; m < 4; ++m) {
+              asm("v_fma_mix_f32 %0, %1, %2, %0 op_sel:[0,0,0] op_sel_hi:[1,0,0]"
+                  : "+v"(acc[2 * m]) : "v"(w[m]), "v"(wreg[2 * m][di * 3 + dj]));
+              asm("v_fma_mix_f32 %0, %1, %2, %0 op_sel:[1,0,0] op_sel_hi:[1,0,0]"
+                  : "+v"(acc[2 * m + 1]) : "v"(w[m]), "v"(wreg[2 * m + 1][di * 3 + dj]));
+            }
+            if (di == 1 && dj == 1) ctr = w;
+          }
+        }
+        u32x4_t out;
+#pragma unroll
+        for (int m = 0; m < 4; ++m) {
+          const uint32_t cw = ctr[m];
+          const float s0 = sigmoidf_(acc[2 * m]), s1 = sigmoidf_(acc[2 * m + 1]);
+          float y0, y1;  // the centre values, read as fp16 halves in place
+          asm("v_fma_mix_f32 %0, %1, %2, 0 op_sel:[0,0,0] op_sel_hi:[1,0,0]" : "=v"(y0) : "v"(cw), "v"(s0));
+          asm("v_fma_mix_f32 %0, %1, %2, 0 op_sel:[1,0,0] op_sel_hi:[1,0,0]" : "=v"(y1) : "v"(cw), "v"(s1));
+          out[m] = pack_bf16x2(y0, y1);
+        }
+        __builtin_amdgcn_raw_buffer_store_b128(out, cx.o, (unsigned)row * 128u + 16u * oct, 0, 0);
+      }
+    }
 }
 
 // Everything one wave does for its slab.  The fp16 form (GENERAL false) returns true, for every wave of the workgroup
@@ -471,92 +587,7 @@ __device__ __forceinline__ bool tile_pass(const TileCtx& cx) {
   float os = cx.oscale;
   if (GENERAL) os *= __builtin_amdgcn_exp2f((float)(eq + ek + ev));
   if (GATE) {
-    // ---- fused locality gate: y = o * sigmoid(conv3x3(o)) per channel on the gw x gh token grid (zero padding), o
-    // being the bf16-rounded output.  The whole slab's outputs are staged in LDS where the tiles lay. ----
-    const int pw = cx.gw + 2;
-    char* cells = lds;
-    float* wlds = reinterpret_cast<float*>(lds + pw * (cx.gh + 2) * 128);
-    const float inv_w = 1.0f / (float)cx.gw;
-    // the head's stencil weights, fetched by the first 144 threads while the other waves finish their walks
-    f32x4_t w4 = {0.f, 0.f, 0.f, 0.f};
-    const bool w_mine = ti * 64 + lane_w < 64 * 9 / 4;
-    if (w_mine) w4 = reinterpret_cast<const f32x4_t*>(cx.gate_w)[ti * 64 + lane_w];
-    lds_barrier();  // every wave is done with the tiles
-    if (w_mine) reinterpret_cast<f32x4_t*>(wlds)[ti * 64 + lane_w] = w4;
-    // (workgroups of fewer than three waves: the rest of the 144 pieces)
-    for (int idx = ti * 64 + lane_w + 64 * NT; idx < 64 * 9 / 4; idx += 64 * NT)
-      reinterpret_cast<f32x4_t*>(wlds)[idx] = reinterpret_cast<const f32x4_t*>(cx.gate_w)[idx];
-    {
-      const int T = 32 * ti + (lane_w & 31);
-      if (T < cx.gw * cx.gh) {
-        const int y = (int)(((float)T + 0.5f) * inv_w), x = T - __mul24(y, cx.gw);
-        char* cell = cells + ((y + 1) * pw + x + 1) * 128 + 64 * (lane_w >> 5);
-#pragma unroll
-        for (int gq = 0; gq < 4; ++gq) {
-          u32x4_t w;
-#pragma unroll
-          for (int m = 0; m < 4; ++m) w[m] = pack_bf16x2(O[0][4 * gq + m] * os, O[1][4 * gq + m] * os);
-          *reinterpret_cast<u32x4_t*>(cell + 16 * gq) = w;
-        }
-      }
-    }
-    const int oct = lane_w & 7, tl = lane_w >> 3;
-    {  // the border cells, by the whole workgroup: top row, bottom row, then the two ends of every other row
-      const int nborder = 2 * pw + 2 * cx.gh;
-      const u32x4_t zero = {0u, 0u, 0u, 0u};
-      for (int bc = ti * 8 + tl; bc < nborder; bc += 8 * NT) {
-        int py, px;
-        if (bc < 2 * pw) {
-          py = bc < pw ? 0 : cx.gh + 1;
-          px = bc < pw ? bc : bc - pw;
-        } else {
-          const int j = bc - 2 * pw;
-          py = 1 + (j >> 1);
-          px = (j & 1) ? pw - 1 : 0;
-        }
-        *reinterpret_cast<u32x4_t*>(cells + (py * pw + px) * 128 + 16 * oct) = zero;
-      }
-    }
-    lds_barrier();  // the slab's outputs, the zero border and the weights are staged
-    float wreg[8][9];
-    {
-      const f32x4_t* wp = reinterpret_cast<const f32x4_t*>(wlds + oct * 72);
-#pragma unroll
-      for (int i = 0; i < 18; ++i) {
-        const f32x4_t x = wp[i];
-#pragma unroll
-        for (int m = 0; m < 4; ++m) wreg[(4 * i + m) / 9][(4 * i + m) % 9] = x[m];
-      }
-    }
-#pragma unroll 1
-    for (int i = 0; i < 4; ++i) {
-      const int row = tl + 8 * i;
-      const int T = 32 * ti + row;
-      if (T < cx.gw * cx.gh) {
-        const int y = (int)(((float)T + 0.5f) * inv_w), x = T - __mul24(y, cx.gw);
-        float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f}, ctr[8];
-#pragma unroll
-        for (int di = 0; di < 3; ++di) {
-          const char* tap = cells + ((y + di) * pw + x) * 128 + 16 * oct;  // padded cell of tap (di - 1, -1)
-#pragma unroll
-          for (int dj = 0; dj < 3; ++dj) {
-            const u32x4_t w = *reinterpret_cast<const u32x4_t*>(tap + dj * 128);
-#pragma unroll
-            for (int m = 0; m < 4; ++m) {
-              const float lo = bf16lo_to_f32(w[m]), hi = bf16hi_to_f32(w[m]);
-              acc[2 * m] = __builtin_fmaf(lo, wreg[2 * m][di * 3 + dj], acc[2 * m]);
-              acc[2 * m + 1] = __builtin_fmaf(hi, wreg[2 * m + 1][di * 3 + dj], acc[2 * m + 1]);
-              if (di == 1 && dj == 1) ctr[2 * m] = lo, ctr[2 * m + 1] = hi;
-            }
-          }
-        }
-        u32x4_t out;
-#pragma unroll
-        for (int m = 0; m < 4; ++m)
-          out[m] = pack_bf16x2(ctr[2 * m] * sigmoidf_(acc[2 * m]), ctr[2 * m + 1] * sigmoidf_(acc[2 * m + 1]));
-        __builtin_amdgcn_raw_buffer_store_b128(out, cx.o, (unsigned)row * 128u + 16u * oct, 0, 0);
-      }
-    }
+    locality_gate_epilogue(O[0], O[1], os, lds, cx.gate_w, cx.o, cx.gw, cx.gh, ti, NT, lane_w);
     return false;
   }
   // ---- store: lane (r, h) holds channels [32h, 32h + 32) of token r; rows beyond the sequence are dropped ----
