@@ -637,12 +637,23 @@ __device__ __forceinline__ TileCtx make_tile_ctx(const uint16_t* q, const uint16
   return cx;
 }
 
-// the general form as a function of its own: its register needs stay out of the fp16 form's allocation
+// The kernel's argument block as the hardware lays it out (every argument at its natural alignment).
+struct TileKernArgs {
+  const uint16_t *q, *k, *v, *gf, *gb;
+  uint16_t* o;
+  TileGeo geo;
+  float oscale;
+  const float* gate_w;
+};
+
+// The general form as a function of its own: its register needs stay out of the fp16 form's allocation.  It reads
+// the kernel's arguments from the argument block itself (ka: the kernel's own kernarg segment pointer; the builtin
+// yields null inside a called function): handed over as parameters, the geometry would need a copy in per-lane
+// memory, and the compiler writes that copy at the top of the kernel, for every wave, redo or not.
 template <int NG, bool BIDIR, bool PITCHED, bool GATE>
-__device__ VIG_GENERAL_INLINE void tile_pass_general(const uint16_t* q, const uint16_t* k, const uint16_t* v,
-                                               const uint16_t* gf, const uint16_t* gb, uint16_t* o, const TileGeo* geo,
-                                               float oscale, const float* gate_w, char* lds) {
-  const TileCtx cx = make_tile_ctx<NG, BIDIR, PITCHED, GATE>(q, k, v, gf, gb, o, *geo, oscale, gate_w, lds);
+__device__ VIG_GENERAL_INLINE void tile_pass_general(const TileKernArgs* ka, char* lds) {
+  const TileCtx cx =
+      make_tile_ctx<NG, BIDIR, PITCHED, GATE>(ka->q, ka->k, ka->v, ka->gf, ka->gb, ka->o, ka->geo, ka->oscale, ka->gate_w, lds);
   tile_pass<NG, BIDIR, PITCHED, true, GATE>(cx);
 }
 
@@ -661,12 +672,8 @@ __global__ __launch_bounds__(512, 4) void gla_tile_kernel(const uint16_t* __rest
     const TileCtx cx = make_tile_ctx<NG, BIDIR, PITCHED, GATE>(q, k, v, gf, gb, o, geo, oscale, gate_w, lds);
     redo = tile_pass<NG, BIDIR, PITCHED, false, GATE>(cx);
   }
-  if (redo) {
-    // (a copy made here: taking the address of the kernel argument itself would move it, and with it every
-    // descriptor built from it, into per-lane memory for the whole kernel)
-    TileGeo geo_copy = geo;
-    tile_pass_general<NG, BIDIR, PITCHED, GATE>(q, k, v, gf, gb, o, &geo_copy, oscale, gate_w, lds);
-  }
+  if (redo)
+    tile_pass_general<NG, BIDIR, PITCHED, GATE>((const TileKernArgs*)__builtin_amdgcn_kernarg_segment_ptr(), lds);
 }
 
 constexpr int kTileMaxLds = 160 * 1024;
