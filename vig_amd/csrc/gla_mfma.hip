@@ -948,17 +948,24 @@ __global__ __launch_bounds__(512) void gla_mfma_kernel(const uint16_t* __restric
 // The causal op may start from a caller's state and hand the last one back (init / final: fp32 [nseq, Dk, Dv] row-major,
 // null: zero / not wanted; one direction only): the thread of state element e is also the one that knows its row
 // (k channel) and column (v channel).
+// maxima (null: not wanted): [nseq][2 directions][kGlaScanMaxima], the largest |state entering a segment| each block saw.
 __global__ __launch_bounds__(256) void gla_segment_scan_kernel(float* state_ws, int nseq, int nseg, int ndir, int ng,
-                                                               const float* __restrict__ init, float* __restrict__ final) {
+                                                               const float* __restrict__ init, float* __restrict__ final,
+                                                               float* __restrict__ maxima) {
+  static_assert(64 * 64 / 256 == kGlaScanMaxima, "one partial maximum per block of the scan");
+  __shared__ float wave_top[4];
   const int e = blockIdx.x * 256 + threadIdx.x;  // element in unit order: ((u*64 + lane)*4 + m)
   const int seq = blockIdx.y / ndir, dir = blockIdx.y % ndir;
   if (seq >= nseq) return;
   const int m = e & 3, lane = (e >> 2) & 63, u = e >> 8;
   const int pk = u >> 3, cq = u & 3, h = lane >> 5;
-  if (cq >= ng) return;  // register quads beyond Dk/16 carry no channel
+  if (cq >= ng) {  // register quads beyond Dk/16 carry no channel (a whole block at a time: u is block-uniform)
+    if (maxima && threadIdx.x == 0) maxima[((size_t)seq * 2 + dir) * kGlaScanMaxima + blockIdx.x] = 0.f;
+    return;
+  }
   const int ch = 8 * ng * h + 8 * cq + 2 * m + pk;
-  constexpr int kBatch = 8;
-  float S = 0.f;
+  constexpr int kBatch = 24;  // (a 4096-token sequence: 16 to 19 segments, fetched in one round)
+  float S = 0.f, top = 0.f;
   // column of the state held by (lane, unit): the v channel the accumulator column r of output tile pv belongs to
   const int vch = 2 * cpair<4>(lane & 31) + ((u >> 2) & 1);
   const size_t rc = ((size_t)seq * (16 * ng) + ch) * 64 + vch;
@@ -979,18 +986,29 @@ __global__ __launch_bounds__(256) void gla_segment_scan_kernel(float* state_ws, 
       if (i < nseg) {
         const int seg = dir == 0 ? i : nseg - 1 - i;
         state_ws[(((size_t)seq * nseg + seg) * 2 + dir) * kStateFloats + e] = S;
+        top = fmaxf(top, fabsf(S));
         S = __builtin_fmaf(ds[j], S, us[j]);
       }
     }
   }
   if (final) final[rc] = S;
+  if (maxima) {  // (uniform: every thread of the block is still here)
+#pragma unroll
+    for (int s = 32; s >= 1; s >>= 1) top = fmaxf(top, __shfl_xor(top, s, 64));
+    if ((threadIdx.x & 63) == 0) wave_top[threadIdx.x >> 6] = top;
+    __syncthreads();
+    if (threadIdx.x == 0)
+      maxima[((size_t)seq * 2 + dir) * kGlaScanMaxima + blockIdx.x] =
+          fmaxf(fmaxf(wave_top[0], wave_top[1]), fmaxf(wave_top[2], wave_top[3]));
+  }
 }
 
-static Geometry make_geometry(int nseq, int L) {
+// tiles: the segments of the tile-pair output pass (whole 32-token tiles) instead of this kernel's own
+static Geometry make_geometry(int nseq, int L, bool tiles = false) {
   Geometry g{};
   g.L = L;
-  g.nseg = gla_segments(L);
-  g.seg_len = gla_segment_len(L);
+  g.nseg = tiles ? gla_tile_segments(L) : gla_segments(L);
+  g.seg_len = tiles ? 32 * gla_tile_segment_tiles(L) : gla_segment_len(L);
   g.cw = (g.seg_len + 3) / 4;
   g.nitems = nseq * g.nseg;
   return g;
@@ -1011,10 +1029,12 @@ bool gla_mfma_supported(const GlaArgs& a) {
   return a.io_dtype == 1 && a.gate_dtype == 1 && (a.Dk == 64 || a.Dk == 32) && a.Dv == 64;
 }
 
+// (sized for either segmentation: the tile-pair output pass cuts finer, and wants the scan's maxima behind the slots)
 size_t gla_mfma_workspace(int B, int H, int L, int Dk, int Dv) {
   if ((Dk != 64 && Dk != 32) || Dv != 64 || L <= 256) return 0;
-  const Geometry g = make_geometry(B * H, L);
-  return (size_t)g.nitems * 2 * kStateFloats * sizeof(float);
+  const Geometry g = make_geometry(B * H, L), gt = make_geometry(B * H, L, true);
+  const size_t items = g.nitems > gt.nitems ? g.nitems : gt.nitems;
+  return (items * 2 * kStateFloats + (size_t)B * H * 2 * kGlaScanMaxima) * sizeof(float);
 }
 
 // with an initial or final state every sequence goes through the segment passes, also a single-segment one
@@ -1042,7 +1062,13 @@ static int launch_gla_mfma_t(const GlaArgs& a, int num_cu, int dev) {
       if (hipFuncSetAttribute(kf, hipFuncAttributeMaxDynamicSharedMemorySize, kLdsTotal) != hipSuccess) return -5;
     attr_done = true;
   }
-  Geometry geo = make_geometry(a.B * a.H, a.L);
+  // long sequences whose output pass the tile-pair kernel can do are cut its way
+  static const bool chunked_only = [] {
+    const char* e = getenv("VIG_GLA_CHUNKED_SLABS");
+    return e && e[0] == '1';
+  }();
+  const bool tile_chain = !chunked_only && !a.state_pass && gla_tiles_chain_supported(a);
+  Geometry geo = make_geometry(a.B * a.H, a.L, tile_chain);
   geo.wide_gates = a.wide_gates;
   geo.H = a.H;
   geo.sq = make_strides(a.q_strides, a.H, a.L, a.Dk);
@@ -1103,8 +1129,13 @@ static int launch_gla_mfma_t(const GlaArgs& a, int num_cu, int dev) {
     hipLaunchKernelGGL((gla_mfma_kernel<kModeState, NG>), dim3(grid), dim3(512), kLdsTotal, a.stream, q, k, v, gf, gb, o,
                        geo, oscale, ws, no_gate);
     const int ndir = gb ? 2 : 1;
+    float* maxima = tile_chain ? ws + (size_t)geo.nitems * 2 * kStateFloats : nullptr;
     hipLaunchKernelGGL(gla_segment_scan_kernel, dim3(64 * 64 / 256, a.B * a.H * ndir), dim3(256), 0, a.stream, ws,
-                       a.B * a.H, geo.nseg, ndir, NG, a.init_state, a.final_state);
+                       a.B * a.H, geo.nseg, ndir, NG, a.init_state, a.final_state, maxima);
+    if (tile_chain) {
+      if (hipGetLastError() != hipSuccess) return -5;
+      return launch_gla_tiles_chain(a, ws, maxima);
+    }
     hipLaunchKernelGGL((gla_mfma_kernel<kModeChain, NG>), dim3(grid), dim3(512), kLdsTotal, a.stream, q, k, v, gf, gb, o,
                        geo, oscale, ws, no_gate);
   }

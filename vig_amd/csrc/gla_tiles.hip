@@ -57,6 +57,11 @@ struct TileGeo {
   long long sq[3], sk[3], sv[3];  // (batch, head, token) strides in elements of q, k, v
   int wide;                 // nonzero: go straight to the general form
   int gw, gh, heads;        // fused locality gate: token grid (gw columns, gh rows, gw * gh = L), heads per batch element
+  // output pass of a long sequence: workgroup = sequence * nseg + segment, NT tiles per segment; the states entering
+  // the segments and their maxima as the segment scan leaves them
+  int nseg;
+  const float* states;
+  const float* maxima;
 };
 
 // byte offsets of the workgroup's LDS areas
@@ -93,6 +98,8 @@ struct TileCtx {
   char* lds;
   int ti, NT, lane;
   float oscale;
+  const float* state_in;  // long sequences: this segment's slots (forward, then reverse direction)
+  const float* state_top;  // ... and the sequence's maxima (kGlaScanMaxima floats per direction)
 };
 
 __device__ __forceinline__ float wave_max(float x) {
@@ -327,6 +334,69 @@ __device__ __forceinline__ void walk_tiles(char* lds, const TileLds<NG>& lay, in
   }
 }
 
+// Long sequences: what the state entering the segment (from the left for the forward direction, from the right for
+// the reverse one) adds to this wave's tile,  O^T[pv] += S_in^T q^,  q^ anchored at the segment's edge.  The slot holds
+// S_in in the matrix cores' register order: unit (pk, pv, g), lane, m is S_in[k channel 32h + 8g + 2m + pk][v column of
+// accumulator lane r, half pv], so two units make the A operand of k-step g as they are.  The state goes in as fp16:
+// directly while the scan saw nothing above 2^14, scaled by a power of two otherwise (`shift`, wave-uniform), the
+// product then passing through an accumulator of its own.  extra: power of two the result still needs (general form).
+template <int NG, bool FWD>
+__device__ __forceinline__ void apply_state(const float* slot, const float* top16, const char* dtab_edge, bool cross,
+                                            int lane, int extra, u32x4_t (&qh)[NG], f32x16_t (&O)[2]) {
+  if (cross) {  // q^ over the segment's edge tile (tile 0 forward, the last one reverse)
+#pragma unroll
+    for (int g = 0; g < NG; ++g) {
+      const u32x4_t d = *reinterpret_cast<const u32x4_t*>(dtab_edge + 16 * g);
+#pragma unroll
+      for (int m = 0; m < 4; ++m) qh[g][m] = mul_f16x2(qh[g][m], d[m]);
+    }
+  }
+  float top = lane < kGlaScanMaxima ? top16[lane] : 0.f;
+  top = wave_max(top);
+  const int ex = (int)((__float_as_uint(top) >> 23) & 0xffu) - 127;  // (inf / nan: 128, the result is not finite anyway)
+  const int shift = __builtin_amdgcn_readfirstlane(max(ex - 13, -30));
+  // (directly down to a top of 2^-4: smaller entries keep their weight relative to it in fp16's subnormal range)
+  if (shift <= 0 && shift >= -17 && extra == 0) {
+#pragma unroll
+    for (int pv = 0; pv < 2; ++pv) {
+      f32x4_t a[NG], b[NG];
+#pragma unroll
+      for (int g = 0; g < NG; ++g) {
+        a[g] = *reinterpret_cast<const f32x4_t*>(slot + (((0 * 2 + pv) * 4 + g) * 64 + lane) * 4);
+        b[g] = *reinterpret_cast<const f32x4_t*>(slot + (((1 * 2 + pv) * 4 + g) * 64 + lane) * 4);
+      }
+#pragma unroll
+      for (int g = 0; g < NG; ++g) {
+        u32x4_t f;
+#pragma unroll
+        for (int m = 0; m < 4; ++m) f[m] = pack_f16x2(a[g][m], b[g][m]);
+        O[pv] = mfma_f16(f, qh[g], O[pv]);
+      }
+    }
+    return;
+  }
+  const float pre = __builtin_amdgcn_exp2f(-(float)shift), post = __builtin_amdgcn_exp2f((float)(shift + extra));
+#pragma unroll
+  for (int pv = 0; pv < 2; ++pv) {
+    f32x16_t acc = {0.f};
+    f32x4_t a[NG], b[NG];
+#pragma unroll
+    for (int g = 0; g < NG; ++g) {
+      a[g] = *reinterpret_cast<const f32x4_t*>(slot + (((0 * 2 + pv) * 4 + g) * 64 + lane) * 4);
+      b[g] = *reinterpret_cast<const f32x4_t*>(slot + (((1 * 2 + pv) * 4 + g) * 64 + lane) * 4);
+    }
+#pragma unroll
+    for (int g = 0; g < NG; ++g) {
+      u32x4_t f;
+#pragma unroll
+      for (int m = 0; m < 4; ++m) f[m] = pack_f16x2(a[g][m] * pre, b[g][m] * pre);
+      acc = mfma_f16(f, qh[g], acc);
+    }
+#pragma unroll
+    for (int i = 0; i < 16; ++i) O[pv][i] = __builtin_fmaf(acc[i], post, O[pv][i]);
+  }
+}
+
 // Fused locality gate: y = o * sigmoid(conv3x3(o)) per channel on the gw x gh token grid (zero padding), o being the
 // bf16-rounded output.  The whole slab's outputs are staged in LDS where the tiles lay.  (A function of its own: its
 // 72 weight registers stay out of the main path's allocation.)
@@ -440,7 +510,7 @@ __device__ __forceinline__ void locality_gate_epilogue(f32x16_t O0, f32x16_t O1,
 
 // Everything one wave does for its slab.  The fp16 form (GENERAL false) returns true, for every wave of the workgroup
 // alike and before anything is stored, when some tile of the slab is outside its range.
-template <int NG, bool BIDIR, bool PITCHED, bool GENERAL, bool GATE>
+template <int NG, bool BIDIR, bool PITCHED, bool GENERAL, bool GATE, bool CHAIN>
 __device__ __forceinline__ bool tile_pass(const TileCtx& cx) {
   const int lane = cx.lane, r = lane & 31, h = lane >> 5;
   const int ti = cx.ti, NT = cx.NT;
@@ -583,7 +653,15 @@ __device__ __forceinline__ bool tile_pass(const TileCtx& cx) {
   int lane_w = lane;
   asm volatile("" : "+v"(lane_w));
   walk_tiles<NG, true>(lds, lay, ti, NT, lane_w, qhf, O);
+  // (general form: the state's term joins accumulators that carry 2^-(eq + ek + ev); q^ carries 2^-eq itself)
+  if (CHAIN)
+    apply_state<NG, true>(cx.state_in, cx.state_top, lds + lay.d + 16 * NG * (lane_w >> 5), ti > 0, lane_w,
+                          GENERAL ? -(ek + ev) : 0, qhf, O);
   if (BIDIR) walk_tiles<NG, false>(lds, lay, ti, NT, lane_w, qhb, O);
+  if (CHAIN && BIDIR)
+    apply_state<NG, false>(cx.state_in + kGlaStateFloats, cx.state_top + kGlaScanMaxima,
+                           lds + lay.d + (NT + NT - 1) * 128 + 16 * NG * (lane_w >> 5), ti < NT - 1, lane_w,
+                           GENERAL ? -(ek + ev) : 0, qhb, O);
   float os = cx.oscale;
   if (GENERAL) os *= __builtin_amdgcn_exp2f((float)(eq + ek + ev));
   if (GATE) {
@@ -601,7 +679,7 @@ __device__ __forceinline__ bool tile_pass(const TileCtx& cx) {
   return false;
 }
 
-template <int NG, bool BIDIR, bool PITCHED, bool GATE>
+template <int NG, bool BIDIR, bool PITCHED, bool GATE, bool CHAIN>
 __device__ __forceinline__ TileCtx make_tile_ctx(const uint16_t* q, const uint16_t* k, const uint16_t* v,
                                                  const uint16_t* gf, const uint16_t* gb, uint16_t* o,
                                                  const TileGeo& geo, float oscale, const float* gate_w, char* lds) {
@@ -615,10 +693,14 @@ __device__ __forceinline__ TileCtx make_tile_ctx(const uint16_t* q, const uint16
   cx.lane = threadIdx.x & 63;
   cx.NT = geo.NT;
   cx.oscale = oscale;
-  const int seq = blockIdx.x;
-  const int tok = 32 * cx.ti;
-  const int nvalid = min(32, geo.L - tok);
+  // (long sequences: workgroup = sequence * nseg + segment, a segment = NT tiles; tiles past the end hold no token)
+  const int seq = CHAIN ? (int)blockIdx.x / geo.nseg : (int)blockIdx.x;
+  const int seg = CHAIN ? (int)blockIdx.x - seq * geo.nseg : 0;
+  const int tok = 32 * (seg * geo.NT + cx.ti);
+  const int nvalid = CHAIN ? max(0, min(32, geo.L - tok)) : min(32, geo.L - tok);
   const size_t off = (size_t)seq * geo.L + tok;  // in tokens
+  cx.state_in = CHAIN ? geo.states + (size_t)blockIdx.x * 2 * kGlaStateFloats : nullptr;
+  cx.state_top = CHAIN ? geo.maxima + (size_t)seq * 2 * kGlaScanMaxima : nullptr;
   if (PITCHED) {
     const int b = seq / geo.H, hd = seq - b * geo.H;
     cx.q_pitch = 2u * (unsigned)geo.sq[2], cx.k_pitch = 2u * (unsigned)geo.sk[2], cx.v_pitch = 2u * (unsigned)geo.sv[2];
@@ -650,16 +732,16 @@ struct TileKernArgs {
 // the kernel's arguments from the argument block itself (ka: the kernel's own kernarg segment pointer; the builtin
 // yields null inside a called function): handed over as parameters, the geometry would need a copy in per-lane
 // memory, and the compiler writes that copy at the top of the kernel, for every wave, redo or not.
-template <int NG, bool BIDIR, bool PITCHED, bool GATE>
+template <int NG, bool BIDIR, bool PITCHED, bool GATE, bool CHAIN>
 __device__ VIG_GENERAL_INLINE void tile_pass_general(const TileKernArgs* ka, char* lds) {
-  const TileCtx cx =
-      make_tile_ctx<NG, BIDIR, PITCHED, GATE>(ka->q, ka->k, ka->v, ka->gf, ka->gb, ka->o, ka->geo, ka->oscale, ka->gate_w, lds);
-  tile_pass<NG, BIDIR, PITCHED, true, GATE>(cx);
+  const TileCtx cx = make_tile_ctx<NG, BIDIR, PITCHED, GATE, CHAIN>(ka->q, ka->k, ka->v, ka->gf, ka->gb, ka->o, ka->geo,
+                                                                     ka->oscale, ka->gate_w, lds);
+  tile_pass<NG, BIDIR, PITCHED, true, GATE, CHAIN>(cx);
 }
 
 }  // namespace
 
-template <int NG, bool BIDIR, bool PITCHED, bool GATE>
+template <int NG, bool BIDIR, bool PITCHED, bool GATE, bool CHAIN = false>
 __global__ __launch_bounds__(512, 4) void gla_tile_kernel(const uint16_t* __restrict__ q, const uint16_t* __restrict__ k,
                                                           const uint16_t* __restrict__ v,
                                                           const uint16_t* __restrict__ gf,
@@ -669,11 +751,11 @@ __global__ __launch_bounds__(512, 4) void gla_tile_kernel(const uint16_t* __rest
   extern __shared__ __align__(16) char lds[];
   bool redo = true;
   if (!geo.wide) {
-    const TileCtx cx = make_tile_ctx<NG, BIDIR, PITCHED, GATE>(q, k, v, gf, gb, o, geo, oscale, gate_w, lds);
-    redo = tile_pass<NG, BIDIR, PITCHED, false, GATE>(cx);
+    const TileCtx cx = make_tile_ctx<NG, BIDIR, PITCHED, GATE, CHAIN>(q, k, v, gf, gb, o, geo, oscale, gate_w, lds);
+    redo = tile_pass<NG, BIDIR, PITCHED, false, GATE, CHAIN>(cx);
   }
   if (redo)
-    tile_pass_general<NG, BIDIR, PITCHED, GATE>((const TileKernArgs*)__builtin_amdgcn_kernarg_segment_ptr(), lds);
+    tile_pass_general<NG, BIDIR, PITCHED, GATE, CHAIN>((const TileKernArgs*)__builtin_amdgcn_kernarg_segment_ptr(), lds);
 }
 
 constexpr int kTileMaxLds = 160 * 1024;
@@ -691,18 +773,19 @@ bool gla_tiles_supported(const GlaArgs& a) {
   return true;
 }
 
-template <int NG, bool BIDIR, bool PITCHED, bool GATE>
+template <int NG, bool BIDIR, bool PITCHED, bool GATE, bool CHAIN = false>
 static int launch_tiles_t(const GlaArgs& a, const TileGeo& geo, int dev) {
   constexpr int kMaxDevices = 64;
   static bool attr_done_dev[kMaxDevices] = {};
-  const void* kf = reinterpret_cast<const void*>(gla_tile_kernel<NG, BIDIR, PITCHED, GATE>);
+  const void* kf = reinterpret_cast<const void*>(gla_tile_kernel<NG, BIDIR, PITCHED, GATE, CHAIN>);
   if (!attr_done_dev[dev]) {
     if (hipFuncSetAttribute(kf, hipFuncAttributeMaxDynamicSharedMemorySize, kTileMaxLds) != hipSuccess) return -5;
     attr_done_dev[dev] = true;
   }
   const TileLds<NG> lay(geo.NT, GATE ? gate_stage_bytes(geo.gw, geo.gh) : 0);
   if (lay.total > kTileMaxLds) return -95;
-  hipLaunchKernelGGL((gla_tile_kernel<NG, BIDIR, PITCHED, GATE>), dim3(a.B * a.H), dim3(64 * geo.NT), lay.total, a.stream,
+  hipLaunchKernelGGL((gla_tile_kernel<NG, BIDIR, PITCHED, GATE, CHAIN>), dim3(a.B * a.H * (CHAIN ? geo.nseg : 1)),
+                     dim3(64 * geo.NT), lay.total, a.stream,
                      (const uint16_t*)a.q, (const uint16_t*)a.k, (const uint16_t*)a.v, (const uint16_t*)a.g_fwd,
                      (const uint16_t*)a.g_bwd, (uint16_t*)a.o, geo, a.scale * a.out_scale, a.gate_w);
   return hipGetLastError() == hipSuccess ? 0 : -5;
@@ -747,6 +830,31 @@ int launch_gla_tiles(const GlaArgs& a) {
   if (pitched)
     return bidir ? launch_tiles_t<2, true, true, false>(a, geo, dev) : launch_tiles_t<2, false, true, false>(a, geo, dev);
   return bidir ? launch_tiles_t<2, true, false, false>(a, geo, dev) : launch_tiles_t<2, false, false, false>(a, geo, dev);
+}
+
+bool gla_tiles_chain_supported(const GlaArgs& a) {
+  return a.io_dtype == 1 && a.gate_dtype == 1 && (a.Dk == 64 || a.Dk == 32) && a.Dv == 64 && a.L > 256 && !a.init_state &&
+         !a.final_state && !a.state_pass && !a.gate_w && !a.q_strides && !a.k_strides && !a.v_strides &&
+         (long long)a.B * a.H * gla_tile_segments(a.L) <= 0x7fffffffLL;
+}
+
+int launch_gla_tiles_chain(const GlaArgs& a, const float* states, const float* maxima) {
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return -5;
+  if (!gla_tiles_chain_supported(a) || !states || !maxima) return -22;
+  TileGeo geo{};
+  geo.L = a.L;
+  geo.NT = gla_tile_segment_tiles(a.L);
+  geo.H = a.H;
+  geo.wide = a.wide_gates;
+  geo.heads = 1;
+  geo.nseg = gla_tile_segments(a.L);
+  geo.states = states;
+  geo.maxima = maxima;
+  const bool bidir = a.g_bwd != nullptr;
+  if (a.Dk == 64)
+    return bidir ? launch_tiles_t<4, true, false, false, true>(a, geo, dev) : launch_tiles_t<4, false, false, false, true>(a, geo, dev);
+  return bidir ? launch_tiles_t<2, true, false, false, true>(a, geo, dev) : launch_tiles_t<2, false, false, false, true>(a, geo, dev);
 }
 
 }  // namespace vig

@@ -47,6 +47,14 @@ constexpr int kGlaStateFloats = 64 * 64 + 64;
 // Segments of a long sequence: ceil(L / 256) of them, ceil(L / nseg) tokens each (the last one possibly fewer).
 inline int gla_segments(int L) { return (L + 255) / 256; }
 inline int gla_segment_len(int L) { return (L + gla_segments(L) - 1) / gla_segments(L); }
+// The forward of a long sequence, when its output pass is the tile-pair kernel: segments of whole 32-token tiles, at
+// most 7 of them (one wave each, two workgroups per CU); the last segment of a sequence may hold fewer tokens, down to
+// none in its trailing tiles.
+inline int gla_tile_segments(int L) { return (L + 223) / 224; }
+inline int gla_tile_segment_tiles(int L) { return ((L + gla_tile_segments(L) - 1) / gla_tile_segments(L) + 31) / 32; }
+// Behind the state slots of a scanned workspace: per (sequence, direction) 16 partial maxima of |state entering a
+// segment| (one per block of the scan), for consumers that read the states as fp16.
+constexpr int kGlaScanMaxima = 16;
 
 // fp32-arithmetic token-recurrent path (any supported dtype combination).
 int launch_gla_recurrent(const GlaArgs& a);
@@ -58,6 +66,11 @@ int launch_gla_mfma(const GlaArgs& a);
 // bf16 tile-pair path for whole-sequence slabs (L <= 256): one wave per 32-token tile, both directions per wave.
 bool gla_tiles_supported(const GlaArgs& a);
 int launch_gla_tiles(const GlaArgs& a);
+// the same kernel as the output pass of a long sequence (L > 256): one workgroup per (sequence, segment), the states
+// entering the segments (scanned slots, kGlaStateFloats floats per (sequence, segment, direction)) and their maxima
+// (kGlaScanMaxima floats per (sequence, direction)) in `states` / `maxima`
+bool gla_tiles_chain_supported(const GlaArgs& a);
+int launch_gla_tiles_chain(const GlaArgs& a, const float* states, const float* maxima);
 bool gla_mfma_gate_grid_ok(int rows, int cols);  // token grids the fused locality gate takes
 size_t gla_mfma_workspace(int B, int H, int L, int Dk, int Dv);
 size_t gla_mfma_state_workspace(int B, int H, int L, int Dk, int Dv);  // causal op with an initial / final state
