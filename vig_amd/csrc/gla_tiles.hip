@@ -57,7 +57,7 @@ struct TileGeo {
   long long sq[3], sk[3], sv[3];  // (batch, head, token) strides in elements of q, k, v
   int wide;                 // nonzero: go straight to the general form
   int gw, gh, heads;        // fused locality gate: token grid (gw columns, gh rows, gw * gh = L), heads per batch element
-  // output pass of a long sequence: workgroup = sequence * nseg + segment, NT tiles per segment; the states entering
+  // output pass of a long sequence: grid (sequence, segment), NT tiles per segment; the states entering
   // the segments and their maxima as the segment scan leaves them
   int nseg;
   const float* states;
@@ -693,13 +693,15 @@ __device__ __forceinline__ TileCtx make_tile_ctx(const uint16_t* q, const uint16
   cx.lane = threadIdx.x & 63;
   cx.NT = geo.NT;
   cx.oscale = oscale;
-  // (long sequences: workgroup = sequence * nseg + segment, a segment = NT tiles; tiles past the end hold no token)
-  const int seq = CHAIN ? (int)blockIdx.x / geo.nseg : (int)blockIdx.x;
-  const int seg = CHAIN ? (int)blockIdx.x - seq * geo.nseg : 0;
+  // (long sequences: grid (sequence, segment), a segment = NT tiles; tiles past the end hold no token)
+  const int seq = blockIdx.x;
+  const int seg = CHAIN ? (int)blockIdx.y : 0;
   const int tok = 32 * (seg * geo.NT + cx.ti);
-  const int nvalid = CHAIN ? max(0, min(32, geo.L - tok)) : min(32, geo.L - tok);
+  // (the clamp from both sides compiles to a vector instruction: back to a scalar, or every descriptor built from it
+  // counts as divergent and every load gets a loop around it)
+  const int nvalid = CHAIN ? __builtin_amdgcn_readfirstlane(max(0, min(32, geo.L - tok))) : min(32, geo.L - tok);
   const size_t off = (size_t)seq * geo.L + tok;  // in tokens
-  cx.state_in = CHAIN ? geo.states + (size_t)blockIdx.x * 2 * kGlaStateFloats : nullptr;
+  cx.state_in = CHAIN ? geo.states + ((size_t)seq * geo.nseg + seg) * 2 * kGlaStateFloats : nullptr;
   cx.state_top = CHAIN ? geo.maxima + (size_t)seq * 2 * kGlaScanMaxima : nullptr;
   if (PITCHED) {
     const int b = seq / geo.H, hd = seq - b * geo.H;
@@ -784,7 +786,7 @@ static int launch_tiles_t(const GlaArgs& a, const TileGeo& geo, int dev) {
   }
   const TileLds<NG> lay(geo.NT, GATE ? gate_stage_bytes(geo.gw, geo.gh) : 0);
   if (lay.total > kTileMaxLds) return -95;
-  hipLaunchKernelGGL((gla_tile_kernel<NG, BIDIR, PITCHED, GATE, CHAIN>), dim3(a.B * a.H * (CHAIN ? geo.nseg : 1)),
+  hipLaunchKernelGGL((gla_tile_kernel<NG, BIDIR, PITCHED, GATE, CHAIN>), dim3(a.B * a.H, CHAIN ? geo.nseg : 1),
                      dim3(64 * geo.NT), lay.total, a.stream,
                      (const uint16_t*)a.q, (const uint16_t*)a.k, (const uint16_t*)a.v, (const uint16_t*)a.g_fwd,
                      (const uint16_t*)a.g_bwd, (uint16_t*)a.o, geo, a.scale * a.out_scale, a.gate_w);
@@ -835,7 +837,7 @@ int launch_gla_tiles(const GlaArgs& a) {
 bool gla_tiles_chain_supported(const GlaArgs& a) {
   return a.io_dtype == 1 && a.gate_dtype == 1 && (a.Dk == 64 || a.Dk == 32) && a.Dv == 64 && a.L > 256 && !a.init_state &&
          !a.final_state && !a.state_pass && !a.gate_w && !a.q_strides && !a.k_strides && !a.v_strides &&
-         (long long)a.B * a.H * gla_tile_segments(a.L) <= 0x7fffffffLL;
+         gla_tile_segments(a.L) <= 65535;
 }
 
 int launch_gla_tiles_chain(const GlaArgs& a, const float* states, const float* maxima) {
