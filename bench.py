@@ -420,6 +420,27 @@ def main():
     k_min = durs[0]
     log(f"wall {ms_per_step*1e3:.1f} us/step; event-bracketed launch avg {k_avg*1e3:.1f} us, median {k_med*1e3:.1f}, min {k_min*1e3:.1f}")
 
+    # what this box's memory system gives a plain device-to-device copy that moves the same number of bytes (half read,
+    # half written), timed the same way on rotating buffers: the practical ceiling beside the published 8 TB/s
+    copy_ref = None
+    if not args.exact:
+        half = alg_bytes // 2
+        bufs = [(torch.empty(half, dtype=torch.uint8, device=dev), torch.empty(half, dtype=torch.uint8, device=dev))
+                for _ in range(max(3, int(300e6 // alg_bytes) + 1))]
+        for i in range(10):
+            bufs[i % len(bufs)][1].copy_(bufs[i % len(bufs)][0])
+        cev = [(torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)) for _ in range(50)]
+        for i, (a, b) in enumerate(cev):
+            a.record(stream)
+            bufs[i % len(bufs)][1].copy_(bufs[i % len(bufs)][0])
+            b.record(stream)
+        torch.cuda.synchronize()
+        c_us = sum(a.elapsed_time(b) for a, b in cev) / len(cev) * 1e3
+        copy_ref = {"bytes": 2 * half, "us": c_us, "GBps": 2 * half / (c_us * 1e-6) / 1e9,
+                    "what": "torch copy_ of alg_bytes/2 (read) into alg_bytes/2 (written), event-bracketed, rotating buffers"}
+        log(f"device copy of the same bytes: {c_us:.1f} us ({copy_ref['GBps']:.0f} GB/s)")
+        del bufs
+
     # HBM bytes per launch measured with rocprofv3 --pmc (FETCH_SIZE / WRITE_SIZE, scaled by a copy kernel of known
     # size); the figures live with the profile summaries, keyed by workload, with the commit and date they were taken at
     traffic = _measured_traffic(s.name)
@@ -451,9 +472,11 @@ def main():
         "kernel_us": {"avg": k_avg * 1e3, "median": k_med * 1e3, "min": k_min * 1e3},
         "roofline": {"bound": "hbm", "achieved": achieved_gbps, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                      "frac": achieved_gbps / HBM_PEAK_GBPS, **traffic},
+        "device_copy_same_bytes": copy_ref,
     }
     # the headline run (config 1) also reports the other half of the metric (ViG-S images/s) and the backward
-    want_backward = (args.backward or args.config == 1) and not args.op_only and not args.exact
+    # (--backward --op-only: the forward and the backward of the op, nothing else)
+    want_backward = (args.backward or (args.config == 1 and not args.op_only)) and not args.exact
     want_model = (args.model or args.config == 1) and not args.op_only and not args.exact
     if want_backward:
         out["backward"] = backward_time(lib, sets, s, io_dt, scale, sp, stream, dev)

@@ -14,7 +14,7 @@ import pytest
 
 from vig_amd import build as B
 
-SOURCES = ["gla_mfma.hip", "gla_backward_mfma.hip", "gates.hip", "patch_conv.hip", "linear.hip"]
+SOURCES = ["gla_tiles.hip", "gla_mfma.hip", "gla_backward_mfma.hip", "gates.hip", "patch_conv.hip", "linear.hip"]
 WINDOW = 8  # issue slots behind a 32x32x16 matrix instruction in which its destination must not be read
 
 

@@ -1,6 +1,7 @@
-// Bidirectional GLA forward for whole-sequence slabs (L <= 256) on MFMA tiles (gfx950), Dk in {32, 64}, Dv = 64,
-// bf16 in and out: one workgroup per (batch, head) slab, one wave per 32-token query tile, both directions in the
-// same wave.
+// Bidirectional GLA forward on MFMA tiles (gfx950), Dk in {32, 64}, Dv = 64, bf16 in and out: one workgroup per
+// (batch, head) slab of up to 256 tokens, one wave per 32-token query tile, both directions in the same wave.  A longer
+// sequence is cut into segments of at most seven tiles, each handled like a slab plus the products with the states
+// that enter it from either side (apply_state; the states come from a state pass and a scan, gla_mfma.hip).
 //
 // Wave i owns the queries of tile i.  Along the forward direction they see the keys of tiles j <= i, along the
 // reverse direction those of tiles j >= i, so every wave multiplies against NT + 1 key tiles whatever its position, the
