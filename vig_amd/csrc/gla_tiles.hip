@@ -43,9 +43,6 @@ namespace vig {
 namespace {
 
 #define VIG_PHASE() __builtin_amdgcn_sched_barrier(0)
-#ifndef VIG_GENERAL_INLINE
-#define VIG_GENERAL_INLINE __noinline__
-#endif
 
 constexpr float kTileRange = 10.0f;     // fp16 form: |tile total| * log2(e) per channel
 constexpr float kMaxSquaresQ = 32768.0f;  // rows of q: |q| < 182
@@ -358,22 +355,25 @@ __device__ __forceinline__ void apply_state(const float* slot, const float* top1
   const int shift = __builtin_amdgcn_readfirstlane(max(ex - 13, -30));
   // (directly down to a top of 2^-4: smaller entries keep their weight relative to it in fp16's subnormal range)
   if (shift <= 0 && shift >= -17 && extra == 0) {
+    // (two k-steps' worth of the state in flight at a time: sixteen registers)
 #pragma unroll
-    for (int pv = 0; pv < 2; ++pv) {
-      f32x4_t a[NG], b[NG];
+    for (int pv = 0; pv < 2; ++pv)
 #pragma unroll
-      for (int g = 0; g < NG; ++g) {
-        a[g] = *reinterpret_cast<const f32x4_t*>(slot + (((0 * 2 + pv) * 4 + g) * 64 + lane) * 4);
-        b[g] = *reinterpret_cast<const f32x4_t*>(slot + (((1 * 2 + pv) * 4 + g) * 64 + lane) * 4);
+      for (int g0 = 0; g0 < NG; g0 += 2) {
+        f32x4_t a[2], b[2];
+#pragma unroll
+        for (int g = 0; g < 2; ++g) {
+          a[g] = *reinterpret_cast<const f32x4_t*>(slot + (((0 * 2 + pv) * 4 + g0 + g) * 64 + lane) * 4);
+          b[g] = *reinterpret_cast<const f32x4_t*>(slot + (((1 * 2 + pv) * 4 + g0 + g) * 64 + lane) * 4);
+        }
+#pragma unroll
+        for (int g = 0; g < 2; ++g) {
+          u32x4_t f;
+#pragma unroll
+          for (int m = 0; m < 4; ++m) f[m] = pack_f16x2(a[g][m], b[g][m]);
+          O[pv] = mfma_f16(f, qh[g0 + g], O[pv]);
+        }
       }
-#pragma unroll
-      for (int g = 0; g < NG; ++g) {
-        u32x4_t f;
-#pragma unroll
-        for (int m = 0; m < 4; ++m) f[m] = pack_f16x2(a[g][m], b[g][m]);
-        O[pv] = mfma_f16(f, qh[g], O[pv]);
-      }
-    }
     return;
   }
   const float pre = __builtin_amdgcn_exp2f(-(float)shift), post = __builtin_amdgcn_exp2f((float)(shift + extra));
@@ -736,7 +736,7 @@ struct TileKernArgs {
 // yields null inside a called function): handed over as parameters, the geometry would need a copy in per-lane
 // memory, and the compiler writes that copy at the top of the kernel, for every wave, redo or not.
 template <int NG, bool BIDIR, bool PITCHED, bool GATE, bool CHAIN>
-__device__ VIG_GENERAL_INLINE void tile_pass_general(const TileKernArgs* ka, char* lds) {
+__device__ __noinline__ void tile_pass_general(const TileKernArgs* ka, char* lds) {
   const TileCtx cx = make_tile_ctx<NG, BIDIR, PITCHED, GATE, CHAIN>(ka->q, ka->k, ka->v, ka->gf, ka->gb, ka->o, ka->geo,
                                                                      ka->oscale, ka->gate_w, lds);
   tile_pass<NG, BIDIR, PITCHED, true, GATE, CHAIN>(cx);
