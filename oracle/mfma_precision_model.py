@@ -1,6 +1,8 @@
-"""CPU emulation of the MFMA kernel's arithmetic (which operands are rounded where).
+"""CPU emulation of the MFMA kernels' arithmetic (which operands are rounded where).
 
-TEST INFRASTRUCTURE ONLY.  It rebuilds the chunk algebra of vig_amd/csrc/gla_mfma.hip in numpy with explicit
+TEST INFRASTRUCTURE ONLY.  `emulate_tiles` rebuilds the tile-pair algebra of vig_amd/csrc/gla_tiles.hip (the forward
+that ships: 32-token tiles, q^ = q exp(G), k^ = k exp(T - G), k' = k exp(-G), D = exp(T), everything the matrix cores
+see rounded to fp16), `emulate` the chunk algebra of vig_amd/csrc/gla_mfma.hip, in numpy with explicit
 roundings, so the precision design (which operands are fp16, which carry a bf16 hi + lo pair) can be checked on the
 CPU against the fp64 oracle.  Chunk algebra as in flash-linear-attention/fla/ops/gla/chunk_util.py:9-78 and
 chunk_fuse.py:76-97, here with the anchor at half the chunk total: q~ = q*exp(G - G_end/2), k~ = k*exp(G_end/2 - G),
@@ -121,3 +123,51 @@ def emulate(q, k, v, gf, gb, chunk, splits=SHIPPED):
                 earlier.insert(0, (f16_round(U), f16_round(np.exp(half).astype(np.float32))))
             S = (Sd + U) * sd
     return o
+
+
+def emulate_tiles(q, k, v, gf, gb, tile=32):
+    """The tile-pair kernel's fp16 form.  Same arguments and result as `emulate`.  Per direction and 32-token tile:
+    tile-local cumulative gates G (fp32), total T; a = f16(exp(G)), b = f16(exp(-G)), d = f16(exp(T));
+    q^ = f16(q a), k' = f16(k b), k^ = f16(k' d); own tile: P = mask(k' q^T), rounded to fp16 per direction and the two
+    directions added in fp16; another tile j walked outwards: q^ <- f16(q^ d_m) for every tile m passed, P = k^_j q^T
+    rounded once to fp16; O += P V with fp32 accumulation (chunk_util.py:37-78 with the anchors per tile)."""
+    N, L, Dk = q.shape
+    Dv = v.shape[-1]
+    s = np.float32(Dk ** -0.5)
+    nt = -(-L // tile)
+    T_ = lambda x: x.transpose(0, 2, 1)
+    sl = [slice(i * tile, min(L, (i + 1) * tile)) for i in range(nt)]
+    acc = np.zeros((N, L, Dv), np.float32)
+    diag = [np.zeros((N, sl[i].stop - sl[i].start, sl[i].stop - sl[i].start), np.float32) for i in range(nt)]
+    for direction in (0, 1):
+        g = gf if direction == 0 else gb
+        qh, kc, kh, d = [], [], [], []
+        for i in range(nt):
+            gc = g[:, sl[i]].astype(np.float32)
+            if direction == 0:
+                G = np.cumsum(gc, axis=1, dtype=np.float32)
+                Tt = G[:, -1:, :]
+            else:
+                G = np.flip(np.cumsum(np.flip(gc, 1), axis=1, dtype=np.float32), 1)
+                Tt = G[:, :1, :]
+            a16, b16 = f16_round(np.exp(G)), f16_round(np.exp(-G))
+            d16 = f16_round(np.exp(Tt))
+            qh.append(f16_round(q[:, sl[i]] * a16))
+            kci = f16_round(k[:, sl[i]] * b16)
+            kc.append(kci)
+            kh.append(f16_round(kci * d16))
+            d.append(d16)
+        for i in range(nt):
+            n = qh[i].shape[1]
+            tri = np.tril(np.ones((n, n), np.float32)) if direction == 0 else np.triu(np.ones((n, n), np.float32))
+            # own tile: P[i, j] over the pairs the direction keeps; the two directions meet in fp16
+            diag[i] = f16_round(diag[i] + f16_round(_mm(qh[i], T_(kc[i])) * tri))
+            qw = qh[i]
+            others = range(i - 1, -1, -1) if direction == 0 else range(i + 1, nt)
+            for step, j in enumerate(others):
+                if step > 0:
+                    qw = f16_round(qw * d[j + 1 if direction == 0 else j - 1])
+                acc[:, sl[i]] += _mm(f16_round(_mm(qw, T_(kh[j]))), v[:, sl[j]])
+    for i in range(nt):
+        acc[:, sl[i]] += _mm(diag[i], v[:, sl[i]])
+    return s * acc
