@@ -227,6 +227,29 @@ def test_bf16_long_sequences_segment_edges(L, Dk, both):
     assert np.all(np.abs(got - want) <= BF16_TOL + 2.0 ** -8 * np.abs(want))
 
 
+def _random_shapes(n, seed):
+    rng = np.random.default_rng(seed)
+    out = []
+    for i in range(n):
+        L = int(rng.choice([rng.integers(1, 33), rng.integers(33, 257), rng.integers(257, 900)]))
+        out.append((int(rng.integers(1, 4)), int(rng.integers(1, 4)), L, int(rng.choice([32, 64])),
+                    float(rng.choice([1 / 64, 1 / 16, 1 / 4, 1.0])), bool(rng.integers(0, 2)), 9000 + i))
+    return out
+
+
+@pytest.mark.parametrize("B,H,L,Dk,gate_scale,both,seed", _random_shapes(36, 2024))
+def test_bf16_random_shapes(B, H, L, Dk, gate_scale, both, seed):
+    """Seeded random shapes across the slab / long-sequence boundary, both head widths, one or two directions, gates
+    from mild to strong (the fp16 form, the general form and mixtures of them within one launch)."""
+    announce(f"bf16 random shape B{B} H{H} L{L} Dk{Dk} gates x{gate_scale} both={both} seed={seed}")
+    q, k, v, gf, gb = make_gla_inputs(B, H, L, Dk, 64, seed=seed, dtype=torch.bfloat16, gate_scale=gate_scale)
+    gf, gb = gf.clamp_min(-3), (gb.clamp_min(-3) if both else None)
+    want = oracle_bidir(q, k, v, gf, gb)
+    got = f64(vig_amd.gla_bidir_forward(*dev(q, k, v, gf, gb)))
+    assert np.isfinite(got).all()
+    assert np.all(np.abs(got - want) <= BF16_TOL + 2.0 ** -8 * np.abs(want))
+
+
 @pytest.mark.parametrize("vscale,gate_scale", [(1000.0, 1.0 / 64), (1e-4, 1.0 / 64), (1000.0, 1.0)])
 def test_bf16_long_sequence_state_magnitudes(vscale, gate_scale):
     """States entering the segments far above and far below 1 (they reach the matrix cores as fp16, scaled by a power of
