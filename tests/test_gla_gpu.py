@@ -210,6 +210,21 @@ def test_bf16_strong_gates_one_direction(B, L):
     assert max_abs(got, want) <= BF16_TOL
 
 
+def test_bf16_long_sequences_many_slabs_mixed_gate_strength():
+    """More (sequence, segment) workgroups than the chip holds at once, every 7th sequence with gates too strong for
+    the fp16 form: segments of one launch take different forms, and the states of a strongly gated sequence stay its own."""
+    announce("bf16 long sequences, 240 sequences x 3 segments, mixed gate strength")
+    B, H, L = 40, 6, 500
+    q, k, v, gf, gb = make_gla_inputs(B, H, L, 32, 64, seed=91, dtype=torch.bfloat16)
+    _, _, _, sf, sb = make_gla_inputs(B, H, L, 32, 64, seed=92, dtype=torch.bfloat16, gate_scale=1.0)
+    strong = (torch.arange(B * H).reshape(B, H) % 7 == 3)[:, :, None, None]
+    gf, gb = torch.where(strong, sf.clamp_min(-3), gf), torch.where(strong, sb.clamp_min(-3), gb)
+    want = oracle_bidir(q, k, v, gf, gb)
+    got = f64(vig_amd.gla_bidir_forward(*dev(q, k, v, gf, gb)))
+    assert np.isfinite(got).all()
+    assert np.all(np.abs(got - want) <= BF16_TOL + 2.0 ** -8 * np.abs(want))
+
+
 @pytest.mark.parametrize("L,Dk,both", [(257, 64, True), (449, 64, True), (1569, 64, True), (1000, 32, True),
                                        (480, 64, False), (2049, 32, False)])
 def test_bf16_long_sequences_segment_edges(L, Dk, both):
