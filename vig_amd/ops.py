@@ -77,7 +77,8 @@ def gla_bidir_backward(q, k, v, g_fwd, g_bwd, d_o, scale: float = -1, out_scale:
 
     bf16 tensors and gates with Dk in {32, 64} and Dv = 64 run on the matrix cores, bidirectional or causal, any L (sequences
     longer than 256 tokens as segments chained through their states; bf16 operands,
-    fp32 accumulation); everything else, and `exact=True`, on the fp32-arithmetic token-recurrent kernel.
+    fp32 accumulation); everything else, and `exact=True`, on the fp32-arithmetic token-recurrent kernel.  Head widths
+    of 128 are taken block by block (64 x 64 blocks, summed here).
     """
     lib = _lib.load()
     _check_cuda(q, k, v, g_fwd, g_bwd, d_o)
@@ -90,6 +91,8 @@ def gla_bidir_backward(q, k, v, g_fwd, g_bwd, d_o, scale: float = -1, out_scale:
         raise ValueError("d_o must match the output in shape and dtype")
     if scale == -1 or scale is None:
         scale = Dk ** -0.5
+    if (Dk > 64 or Dv > 64) and Dk % 64 == 0 and Dv % 64 == 0:
+        return _gla_bidir_backward_blocks(q, k, v, g_fwd, g_bwd, d_o, float(scale), out_scale, exact)
     dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
     dgf = torch.empty_like(g_fwd)
     dgb = torch.empty_like(g_bwd) if g_bwd is not None else None
@@ -109,6 +112,33 @@ def gla_bidir_backward(q, k, v, g_fwd, g_bwd, d_o, scale: float = -1, out_scale:
                                    B, H, L, Dk, Dv, float(scale), float(out_scale), _dt(q), _dt(g_fwd), _stream_ptr(q))
     _lib.check(rc, "vig_gla_bidir_bwd")
     return dq, dk, dv, dgf, dgb
+
+
+def _gla_bidir_backward_blocks(q, k, v, g_fwd, g_bwd, d_o, scale, out_scale, exact):
+    """Head widths beyond 64 (the reference's own op tests use Dk = Dv = 128, tests/ops/test_gla.py:10-77): the op is a
+    sum over key channels and acts on every value channel separately, so its backward is the backward of the 64 x 64
+    blocks: dq, dk and the gate gradients of a key block summed over the value blocks, dv of a value block summed over
+    the key blocks (in fp32; each block call rounds to the tensors' dtype once)."""
+    Dk, Dv = q.shape[-1], v.shape[-1]
+    kb = [slice(i, i + 64) for i in range(0, Dk, 64)]
+    vb = [slice(i, i + 64) for i in range(0, Dv, 64)]
+    f32 = lambda t: torch.zeros(t.shape, dtype=torch.float32, device=t.device)
+    dq, dk, dv, dgf = f32(q), f32(k), f32(v), f32(g_fwd)
+    dgb = f32(g_bwd) if g_bwd is not None else None
+    for a in kb:
+        qa, ka, gfa = (t[..., a].contiguous() for t in (q, k, g_fwd))
+        gba = g_bwd[..., a].contiguous() if g_bwd is not None else None
+        for b in vb:
+            r = gla_bidir_backward(qa, ka, v[..., b].contiguous(), gfa, gba, d_o[..., b].contiguous(), scale, out_scale,
+                                   exact)
+            dq[..., a] += r[0].float()
+            dk[..., a] += r[1].float()
+            dv[..., b] += r[2].float()
+            dgf[..., a] += r[3].float()
+            if dgb is not None:
+                dgb[..., a] += r[4].float()
+    return (dq.to(q.dtype), dk.to(k.dtype), dv.to(v.dtype), dgf.to(g_fwd.dtype),
+            dgb.to(g_bwd.dtype) if dgb is not None else None)
 
 
 class _GLABidirFunction(torch.autograd.Function):
