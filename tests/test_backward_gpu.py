@@ -332,3 +332,37 @@ def test_autograd_keeps_the_exact_path():
     for leaf, w in zip(leaves, want):
         assert torch.equal(leaf.grad, w)
     assert any(not torch.equal(a, b) for a, b in zip(want, other))
+
+
+@pytest.mark.parametrize("dtype,L,Dk", [(torch.float32, 70, 32), (torch.float32, 150, 64), (torch.bfloat16, 196, 64),
+                                        (torch.bfloat16, 300, 32)])
+def test_causal_op_gradients_with_initial_state(dtype, L, Dk):
+    """fused_chunk_gla(initial_state=S0, output_final_state=True) while autograd records: outputs, final state and the
+    gradients of q, k, v, g (S0 a constant, as chunk_fuse.py:565-566 detaches it) against torch autograd through a
+    float64 recurrence started from S0 on the same rounded inputs."""
+    announce(f"causal op gradients with an initial state {dtype} L={L} Dk={Dk}")
+    B, H, Dv = 2, 2, 64
+    q, k, v, g, _ = make_gla_inputs(B, H, L, Dk, Dv, seed=71, dtype=dtype)
+    gen = torch.Generator().manual_seed(72)
+    s0 = torch.randn(B, H, Dk, Dv, generator=gen)
+    do = torch.randn(B, H, L, Dv, generator=gen).to(dtype)
+    # float64 reference: S_t = exp(g_t) * S_{t-1} + k_t v_t^T, o_t = scale q_t S_t (naive.py:13-44 with a start state)
+    rq, rk, rv, rg = (t.double().requires_grad_(True) for t in (q, k, v, g))
+    S = s0.double()
+    outs = []
+    for t in range(L):
+        S = torch.exp(rg[:, :, t, :, None]) * S + rk[:, :, t, :, None] * rv[:, :, t, None, :]
+        outs.append(torch.einsum("bhk,bhkv->bhv", rq[:, :, t] * Dk ** -0.5, S))
+    ro = torch.stack(outs, 2)
+    ro.backward(do.double())
+    tq, tk, tv, tg = (t.cuda().requires_grad_(True) for t in (q, k, v, g))
+    o, final = vig_amd.fused_chunk_gla(tq, tk, tv, tg, initial_state=s0.cuda(), output_final_state=True)
+    assert final is not None and not final.requires_grad
+    o.backward(do.cuda())
+    fp32 = dtype == torch.float32
+    scale_of = lambda w: max(1.0, float(w.abs().max()))
+    assert (o.detach().double().cpu() - ro.detach()).abs().max() <= (1e-4 if fp32 else 2e-2) * scale_of(ro.detach())
+    assert (final.double().cpu() - S.detach()).abs().max() <= (1e-4 if fp32 else 1e-2) * scale_of(S.detach())
+    for name, got, want in (("dq", tq.grad, rq.grad), ("dk", tk.grad, rk.grad), ("dv", tv.grad, rv.grad), ("dg", tg.grad, rg.grad)):
+        err = (got.double().cpu() - want).abs().max().item()
+        assert err <= (1e-4 if fp32 else 2e-2) * scale_of(want), f"{name}: {err:.3e} against {scale_of(want):.3e}"

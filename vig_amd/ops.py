@@ -263,12 +263,12 @@ def gla_causal_state_forward(q, k, v, g, initial_state=None, output_final_state:
     """The causal op with a state carried in and / or out: (o, final_state or None).
 
     initial_state [B,H,Dk,Dv] (any float dtype; used as fp32, detached as in chunk_fuse.py:565-566) is the state
-    before the first token; final_state is fp32 [B,H,Dk,Dv] (chunk_fuse.py:353-356).  Forward only: the library's
-    backward kernels start from a zero state, so a call that records a gradient is refused."""
+    before the first token; final_state is fp32 [B,H,Dk,Dv] (chunk_fuse.py:353-356).  A call that records a gradient
+    goes through _causal_state_recording."""
     lib = _lib.load()
     _check_cuda(q, k, v, g, initial_state)
     if torch.is_grad_enabled() and any(t.requires_grad for t in (q, k, v, g)):
-        raise NotImplementedError("initial_state / output_final_state are forward-only in the HIP path")
+        return _causal_state_recording(q, k, v, g, initial_state, output_final_state, scale, exact)
     q, k, v, g = (_dense(t) for t in (q, k, v, g))
     B, H, L, Dk = q.shape
     Dv = v.shape[-1]
@@ -298,6 +298,37 @@ def gla_causal_state_forward(q, k, v, g, initial_state=None, output_final_state:
             rc = lib.vig_gla_causal_state_fwd(*ptrs, ws.data_ptr() if ws is not None else None, ws_bytes, *tail)
     _lib.check(rc, "vig_gla_causal_state_fwd")
     return out, final
+
+
+def _causal_state_recording(q, k, v, g, initial_state, output_final_state, scale, exact):
+    """The causal op with a state in and / or out while autograd records.  As in the reference the initial state is a
+    constant (chunk_fuse.py:565-566 detaches it) and the final state carries no gradient (chunk_fuse.py:413: its
+    cotangent is ignored), so what is needed are the gradients of q, k, v, g with the initial state's share in them.
+    The library's backward kernels start from a zero state; a state S0 is what 2*Dk gate-free tokens in front of the
+    sequence leave behind (keys = unit vectors, values = the rows of S0 as a high and a low part in the tensors' dtype,
+    queries zero), so the plain differentiable op on the lengthened sequence gives outputs and gradients alike."""
+    B, H, L, Dk = q.shape
+    Dv = v.shape[-1]
+    if scale == -1 or scale is None:
+        scale = Dk ** -0.5
+    final = None
+    if output_final_state:
+        with torch.no_grad():
+            final = gla_causal_state_forward(q.detach(), k.detach(), v.detach(), g.detach(), initial_state, True, scale,
+                                             exact)[1]
+    if initial_state is None:
+        return gla_bidir_forward(q, k, v, g, None, scale, 1.0, exact=exact), final
+    if tuple(initial_state.shape) != (B, H, Dk, Dv):
+        raise ValueError(f"initial_state must be [B,H,Dk,Dv] = {(B, H, Dk, Dv)}; got {tuple(initial_state.shape)}")
+    s0 = initial_state.detach().float()
+    hi = s0.to(v.dtype)
+    lo = (s0 - hi.float()).to(v.dtype)
+    eye = torch.eye(Dk, dtype=k.dtype, device=k.device).expand(B, H, Dk, Dk)
+    zq = torch.zeros(B, H, 2 * Dk, Dk, dtype=q.dtype, device=q.device)
+    zg = torch.zeros(B, H, 2 * Dk, Dk, dtype=g.dtype, device=g.device)
+    o = gla_bidir_forward(torch.cat([zq, q], 2), torch.cat([eye, eye, k], 2), torch.cat([hi, lo, v], 2),
+                          torch.cat([zg, g], 2), None, scale, 1.0, exact=exact)
+    return o[:, :, 2 * Dk:], final
 
 
 def fused_chunk_gla(q, k, v, g, scale: int = -1, initial_state=None, output_final_state: bool = False
