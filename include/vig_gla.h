@@ -67,10 +67,13 @@ const char* vig_gla_strerror(int code);
  *   2^10 / 10^8; a sequence outside that is redone by the same workgroup with
  *   power-of-two input scales and split-bf16 diagonal tiles, good for gates down
  *   to about -5 per token (beyond: exponents are clamped, far tokens count as 0).
- *   L > 256 (segments of <= 256 tokens chained through states in the workspace;
- *   refused with VIG_ENOTSUP when B*H*directions > 65535): the sum of |g| over
- *   any 64 consecutive tokens of one channel must stay below about 80 (beyond it
- *   results may be inf / NaN, never silently wrong finite numbers).
+ *   L > 256 (segments of <= 224 tokens, seven tiles each, chained through states
+ *   in the workspace: a state pass, a scan, then the kernel above once more per
+ *   segment with the entering states; refused with VIG_ENOTSUP when
+ *   B*H*directions > 65535): the same per-tile behaviour for the outputs, and for
+ *   the state pass the sum of |g| over any 56 consecutive tokens of one channel
+ *   must stay below about 80 (beyond it results may be inf / NaN, never silently
+ *   wrong finite numbers).
  * HierViG's head shape (bf16, Dk = 16, Dv = 32, both directions) takes the same
  * paths from L = 128 on, zero-padded to Dk 32 / Dv 64 in the workspace
  * (classification/models/vig_h.py:377-385 with EXPAND_K 0.5, EXPAND_V 1.0).
@@ -143,11 +146,12 @@ int vig_gla_causal_state_fwd_exact(const void* q, const void* k, const void* v, 
 
 /*
  * Same contract, workspace and accuracy bar as vig_gla_bidir_fwd, for callers who know their gates to be strong.
- * The matrix-core kernel computes scores on fp16 operands while a chunk's gate total stays within about 8 (natural
- * log units) in every channel, and on split-bf16 operands beyond; it finds out per workgroup, on the first segment
- * that refuses, and walks that segment twice.  This entry point starts with the split variant: about 10 % faster than
- * finding out when every slab refuses and a workgroup has three slabs (nothing to gain at six or more), 25-30 %
- * slower than the fp16 variant when none would have refused.  No counterpart
+ * The matrix-core kernel computes on fp16 operands while every 32-token tile's gate total stays within about 7
+ * (natural log units) in every channel, and in its wider-range form beyond; it finds out per sequence (or segment),
+ * after preparing the fp16 operands in vain, and redoes it at about four times the cost.  This entry point runs the
+ * wider-range form alone, in a kernel of its own with twice the registers: about 1.65 times the fp16 form's time
+ * whatever the gates (60 against 37 us at B128 H6 L196 Dk64), against 3.8 times through the default entry point when
+ * every sequence refuses.  No counterpart
  * in the reference, whose kernels have one arithmetic (fla/ops/gla/chunk_fuse.py:25-101,212-254).
  */
 int vig_gla_bidir_fwd_wide(const void* q, const void* k, const void* v,

@@ -739,10 +739,22 @@ struct TileKernArgs {
 // yields null inside a called function): handed over as parameters, the geometry would need a copy in per-lane
 // memory, and the compiler writes that copy at the top of the kernel, for every wave, redo or not.
 template <int NG, bool BIDIR, bool PITCHED, bool GATE, bool CHAIN>
-__device__ __noinline__ void tile_pass_general(const TileKernArgs* ka, char* lds) {
-  const TileCtx cx = make_tile_ctx<NG, BIDIR, PITCHED, GATE, CHAIN>(ka->q, ka->k, ka->v, ka->gf, ka->gb, ka->o, ka->geo,
+__device__ __noinline__ void tile_pass_general(const TileKernArgs* ka_in) {
+#if defined(__HIP_DEVICE_COMPILE__)  // (the host pass has no constant address space to copy the geometry from)
+  // (a called function gets its arguments in vector registers: back to scalars, or every argument read through the
+  // pointer, and every descriptor built from one, counts as divergent and each load gets a loop around it; the LDS
+  // base is named here again for the same reason: a pointer handed over would be a generic one)
+  extern __shared__ __align__(16) char lds[];
+  const uint64_t kp = reinterpret_cast<uint64_t>(ka_in);
+  // (constant address space: scalar loads)
+  typedef const TileKernArgs __attribute__((address_space(4))) * KernArgPtr;
+  const KernArgPtr ka = (KernArgPtr)(((uint64_t)(uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)(kp >> 32)) << 32) |
+                                     (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)kp));
+  const TileGeo geo = ka->geo;
+  const TileCtx cx = make_tile_ctx<NG, BIDIR, PITCHED, GATE, CHAIN>(ka->q, ka->k, ka->v, ka->gf, ka->gb, ka->o, geo,
                                                                      ka->oscale, ka->gate_w, lds);
   tile_pass<NG, BIDIR, PITCHED, true, GATE, CHAIN>(cx);
+#endif
 }
 
 }  // namespace
@@ -761,7 +773,23 @@ __global__ __launch_bounds__(512, 4) void gla_tile_kernel(const uint16_t* __rest
     redo = tile_pass<NG, BIDIR, PITCHED, false, GATE, CHAIN>(cx);
   }
   if (redo)
-    tile_pass_general<NG, BIDIR, PITCHED, GATE, CHAIN>((const TileKernArgs*)__builtin_amdgcn_kernarg_segment_ptr(), lds);
+    tile_pass_general<NG, BIDIR, PITCHED, GATE, CHAIN>((const TileKernArgs*)__builtin_amdgcn_kernarg_segment_ptr());
+}
+
+// The general form alone, for launches whose caller knows the gates to be strong: with 256 registers per wave (one
+// workgroup per CU) it keeps its unpacked operands in registers, which the function above, bound to the fp16 form's
+// 128, has to send through per-lane memory.
+template <int NG, bool BIDIR, bool PITCHED, bool GATE, bool CHAIN = false>
+__global__ __launch_bounds__(512, 2) void gla_tile_wide_kernel(const uint16_t* __restrict__ q,
+                                                               const uint16_t* __restrict__ k,
+                                                               const uint16_t* __restrict__ v,
+                                                               const uint16_t* __restrict__ gf,
+                                                               const uint16_t* __restrict__ gb, uint16_t* __restrict__ o,
+                                                               TileGeo geo, float oscale,
+                                                               const float* __restrict__ gate_w) {
+  extern __shared__ __align__(16) char lds[];
+  const TileCtx cx = make_tile_ctx<NG, BIDIR, PITCHED, GATE, CHAIN>(q, k, v, gf, gb, o, geo, oscale, gate_w, lds);
+  tile_pass<NG, BIDIR, PITCHED, true, GATE, CHAIN>(cx);
 }
 
 constexpr int kTileMaxLds = 160 * 1024;
@@ -784,16 +812,24 @@ static int launch_tiles_t(const GlaArgs& a, const TileGeo& geo, int dev) {
   constexpr int kMaxDevices = 64;
   static bool attr_done_dev[kMaxDevices] = {};
   const void* kf = reinterpret_cast<const void*>(gla_tile_kernel<NG, BIDIR, PITCHED, GATE, CHAIN>);
+  const void* kw = reinterpret_cast<const void*>(gla_tile_wide_kernel<NG, BIDIR, PITCHED, GATE, CHAIN>);
   if (!attr_done_dev[dev]) {
     if (hipFuncSetAttribute(kf, hipFuncAttributeMaxDynamicSharedMemorySize, kTileMaxLds) != hipSuccess) return -5;
+    if (hipFuncSetAttribute(kw, hipFuncAttributeMaxDynamicSharedMemorySize, kTileMaxLds) != hipSuccess) return -5;
     attr_done_dev[dev] = true;
   }
   const TileLds<NG> lay(geo.NT, GATE ? gate_stage_bytes(geo.gw, geo.gh) : 0);
   if (lay.total > kTileMaxLds) return -95;
-  hipLaunchKernelGGL((gla_tile_kernel<NG, BIDIR, PITCHED, GATE, CHAIN>), dim3(a.B * a.H, CHAIN ? geo.nseg : 1),
-                     dim3(64 * geo.NT), lay.total, a.stream,
-                     (const uint16_t*)a.q, (const uint16_t*)a.k, (const uint16_t*)a.v, (const uint16_t*)a.g_fwd,
-                     (const uint16_t*)a.g_bwd, (uint16_t*)a.o, geo, a.scale * a.out_scale, a.gate_w);
+  if (geo.wide)
+    hipLaunchKernelGGL((gla_tile_wide_kernel<NG, BIDIR, PITCHED, GATE, CHAIN>), dim3(a.B * a.H, CHAIN ? geo.nseg : 1),
+                       dim3(64 * geo.NT), lay.total, a.stream,
+                       (const uint16_t*)a.q, (const uint16_t*)a.k, (const uint16_t*)a.v, (const uint16_t*)a.g_fwd,
+                       (const uint16_t*)a.g_bwd, (uint16_t*)a.o, geo, a.scale * a.out_scale, a.gate_w);
+  else
+    hipLaunchKernelGGL((gla_tile_kernel<NG, BIDIR, PITCHED, GATE, CHAIN>), dim3(a.B * a.H, CHAIN ? geo.nseg : 1),
+                       dim3(64 * geo.NT), lay.total, a.stream,
+                       (const uint16_t*)a.q, (const uint16_t*)a.k, (const uint16_t*)a.v, (const uint16_t*)a.g_fwd,
+                       (const uint16_t*)a.g_bwd, (uint16_t*)a.o, geo, a.scale * a.out_scale, a.gate_w);
   return hipGetLastError() == hipSuccess ? 0 : -5;
 }
 
