@@ -185,6 +185,29 @@ def test_graphed_forward_replays_match_eager():
         torch.cuda.synchronize()
 
 
+def test_calibrate_strong_gates_marks_the_layer_and_keeps_the_logits():
+    """A layer whose gate projection is biased far negative gets `strong_gates` from one sample forward, the others do
+    not; the marked model (that layer on the GLA op's wide-range form, off the fused block operator) gives the logits
+    of the unmarked one within the bf16 bar."""
+    announce("layers.calibrate_strong_gates on a 3-layer ViG with one strongly gated layer")
+    torch.manual_seed(0)
+    model = layers.ViG(img_size=64, depth=3, num_heads=3, embed_dim=96, num_classes=10).eval().cuda().to(torch.bfloat16)
+    with torch.no_grad():
+        model.blocks[1].attn.gk_proj[1].bias.fill_(-24.0)  # logsigmoid(-24) / 16 = -1.5 per token
+    layers.invalidate_caches(model)
+    x = torch.randn(8, 3, 64, 64, generator=torch.Generator().manual_seed(3)).cuda().to(torch.bfloat16)
+    with torch.no_grad():
+        want = model(x).float()
+    shares = layers.calibrate_strong_gates(model, x)
+    flags = [blk.attn.strong_gates for blk in model.blocks]
+    assert flags == [False, True, False], (flags, shares)
+    assert shares["blocks.1.attn"] == 1.0 and shares["blocks.0.attn"] == 0.0
+    with torch.no_grad():
+        got = model(x).float()
+    assert torch.isfinite(got).all()
+    assert (got - want).abs().max().item() <= 2e-2 * max(1.0, want.abs().max().item())
+
+
 # ---- HierViG's GLA2D (classification/models/vig_h.py:338-606): Dk 16, Dv 32 at every stage ----
 def test_gla2d_parameter_names():
     m = layers.GLA2D(d_model=96, expand_k=0.5, expand_v=1.0, num_heads=3, use_act_in_conv=False, channel_first=True)

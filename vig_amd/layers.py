@@ -149,6 +149,9 @@ class GatedLinearAttention(_CacheMixin, nn.Module):
         self.head_v_dim = self.value_dim // num_heads
         self.use_out_gate = use_out_gate  # stored, never read (as in the reference, vig.py:285)
         self.use_out_act = use_out_act
+        # inference switch (not a parameter of the reference): this layer's gates are known to be strong, so the GLA
+        # op starts with its wide-range form (calibrate_strong_gates sets it from a sample batch)
+        self.strong_gates = False
         self.use_act_in_conv = use_act_in_conv
         self.layernorm_eps = layernorm_eps
         self.gate_logit_normalizer = gate_logit_normalizer
@@ -208,7 +211,7 @@ class GatedLinearAttention(_CacheMixin, nn.Module):
         conv = self.in_proj[0]
         ext = _ext.load()
         if (ext is not None and x.is_cuda and x.is_contiguous() and self.gk_proj[0].weight.shape[0] == ops.GATE_RANK
-                and x.dtype == self.qkv_proj.weight.dtype):
+                and x.dtype == self.qkv_proj.weight.dtype and not self.strong_gates):
             # the whole mixer as one operator of the library (csrc/torch_ext.cpp: the same kernel sequence as below)
             w_in, b_in = self._stacked_in()
             up = self.gk_proj[1]
@@ -233,7 +236,9 @@ class GatedLinearAttention(_CacheMixin, nn.Module):
             gates = ops.dirgate_lowrank(gk_low, up.weight, up.bias, H, self.gate_logit_normalizer, self.clamp_min)
         else:
             gates = ops.dirgate(up(gk_low), H, self.gate_logit_normalizer, self.clamp_min)
-        o = ops.gla_bidir_forward(q, k, v, gates[0], gates[1], scale=-1, out_scale=out_scale)
+        self._last_gates = gates if getattr(self, "_keep_gates", False) else None
+        o = ops.gla_bidir_forward(q, k, v, gates[0], gates[1], scale=-1, out_scale=out_scale,
+                                  strong_gates=self.strong_gates)
         if ops.locality_blend_linear_supported(o, self.o_proj.weight):  # ViG-S / ViG-T widths: no blended intermediate
             return ops.locality_blend_linear(o, xs, g_lin, self.g_norm._w32(), self.l_norm._w32(), self.o_proj.weight,
                                              eps=self.layernorm_eps, silu_out=self.use_out_act)
@@ -270,6 +275,47 @@ class GatedLinearAttention(_CacheMixin, nn.Module):
             return self._mix_autograd(x, hw, 0.5)
         with torch.no_grad():
             return self._mix(x, hw, 0.5 if self.training else 0.25)
+
+
+def calibrate_strong_gates(model: nn.Module, *sample_inputs, share: float = 0.25, tile: int = 32,
+                           limit: float = 6.9) -> dict:
+    """Sets `strong_gates` on every GatedLinearAttention of `model` from one eval forward on a sample batch: a layer is
+    marked when more than `share` of its (batch, head) sequences hold a 32-token tile whose summed log-gate falls
+    below -`limit` in some channel (the range of the GLA kernel's fp16 form: such a sequence is computed twice by the
+    default entry point, at about four times the cost, while the wide-range form costs 1.65 times).  Returns
+    {module name: share of such sequences}.  One-off: it synchronises and runs the unfused block path."""
+    mods = {n: m for n, m in model.named_modules() if isinstance(m, GatedLinearAttention)}
+    was_training = model.training
+    model.eval()
+    saved = {}
+    for n, m in mods.items():
+        saved[n] = m.strong_gates
+        m.strong_gates, m._keep_gates = True, True  # (the unfused path, which exposes the gates)
+    out = {}
+    try:
+        with torch.no_grad():
+            model(*sample_inputs)
+        for n, m in mods.items():
+            g = getattr(m, "_last_gates", None)
+            if g is None:
+                out[n] = 0.0
+                continue
+            worst = None
+            for gd in (g[0], g[1]):  # [B, H, L, Dk] natural-log gates of one direction
+                L = gd.shape[2]
+                pad = (-L) % tile
+                t = F.pad(gd.float(), (0, 0, 0, pad)).unflatten(2, (-1, tile)).sum(3)  # [B, H, tiles, Dk]
+                w = t.amin(dim=(2, 3))
+                worst = w if worst is None else torch.minimum(worst, w)
+            out[n] = float((worst < -limit).float().mean().item())
+    finally:
+        for n, m in mods.items():
+            m._keep_gates, m._last_gates = False, None
+            m.strong_gates = saved[n]
+        model.train(was_training)
+    for n, m in mods.items():
+        m.strong_gates = out[n] > share
+    return out
 
 
 class GLA2D(GatedLinearAttention):
@@ -384,6 +430,7 @@ class GLABlock(nn.Module):
         at = self.attn
         if (ext is not None and not _recording(self) and not self.training and branch.is_cuda and branch.is_contiguous()
                 and type(at) is GatedLinearAttention and at.gk_proj[0].weight.shape[0] == ops.GATE_RANK
+                and not at.strong_gates
                 and branch.dtype == at.qkv_proj.weight.dtype and kwargs.get("token_position", None) is None
                 and (residual is None or (residual.is_contiguous() and residual.dtype == branch.dtype))
                 # (the operator takes one eps for both norms and the eval-mode output scale)
