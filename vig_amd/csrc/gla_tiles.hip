@@ -151,7 +151,11 @@ __device__ __forceinline__ void cumulative_gates(const uint32_t (&gD)[2][8], int
 // the tile totals (G at the last token walked) travel from the one lane pair that holds them to a lane per channel:
 // sc[32h + 16p + 4g + m] = total of channel 8*NG*h + 8g + 2m + p
 template <bool FWD>
-__device__ __forceinline__ void park_totals(const f32x16_t (&G)[2], float* sc, int r, int h) {
+__device__ __forceinline__ void park_totals(f32x16_t (&G)[2], float* sc, int r, int h) {
+  // (G comes straight out of the matrix cores and the store below sits behind a branch: the compiler's wait states
+  // cover the path it expects to be taken; these cover the other one as well, where a register of G may be reused
+  // before the matrix instruction has written it.  20 idle clocks per direction.)
+  asm volatile("s_nop 7\n\ts_nop 7\n\ts_nop 3" : "+v"(G[0]), "+v"(G[1]));  // (tied to G: stays behind its producers)
   if (r == (FWD ? 31 : 0)) {
 #pragma unroll
     for (int p = 0; p < 2; ++p)
