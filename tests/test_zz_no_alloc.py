@@ -89,3 +89,39 @@ def test_noalloc_refuses_shapes_beyond_its_array():
     assert rc == _lib.VIG_ENOSPC
     assert lib.vig_gla_bidir_fwd_noalloc(p, p, p, p, p, p, 0, 1, 1, 64, 64, 0.125, 1.0, 1, 1, None) == _lib.VIG_EINVAL
     torch.cuda.synchronize()
+
+
+def test_noalloc_allocates_nothing_and_replays_from_a_graph():
+    """After one warm-up call per device (kernel attributes, the array's address) the entry point neither allocates
+    device memory (free memory as the driver reports it stays put over repeated calls) nor does anything a HIP graph
+    capture refuses: a captured call on a long sequence, replayed with eager calls in between, reproduces the eager
+    output bit for bit."""
+    lib = _lib.load()
+    dev = torch.device("cuda:0")
+    B, H, L, Dk, Dv = 2, 3, 1000, 64, 64
+    announce("noalloc: no device allocation, graph capture and replays")
+    t = [x.to(dev) for x in make_gla_inputs(B, H, L, Dk, Dv, seed=31, dtype=torch.bfloat16)]
+    dims = (B, H, L, Dk, Dv)
+    eager = torch.empty(B, H, L, Dv, dtype=torch.bfloat16, device=dev)
+    got = torch.full_like(eager, float("nan"))
+    assert _call(lib, "vig_gla_bidir_fwd_noalloc", t, eager, dims) == 0  # warm-up, outside any capture
+    torch.cuda.synchronize()
+    free0 = torch.cuda.mem_get_info(dev)[0]
+    for _ in range(3):
+        assert _call(lib, "vig_gla_bidir_fwd_noalloc", t, eager, dims) == 0
+    torch.cuda.synchronize()
+    assert torch.cuda.mem_get_info(dev)[0] == free0
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        rc = _call(lib, "vig_gla_bidir_fwd_noalloc", t, got, dims)
+    assert rc == 0
+    other = [x.to(dev) for x in make_gla_inputs(1, 2, 300, Dk, Dv, seed=32, dtype=torch.bfloat16)]
+    scratch_out = torch.empty(1, 2, 300, Dv, dtype=torch.bfloat16, device=dev)
+    for i in range(3):
+        got.fill_(float("nan"))
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(got.view(torch.int16), eager.view(torch.int16)), f"replay {i}"
+        # eager work on the same array between the replays
+        assert _call(lib, "vig_gla_bidir_fwd_noalloc", other, scratch_out, (1, 2, 300, Dk, Dv)) == 0
+        torch.cuda.synchronize()
