@@ -36,6 +36,7 @@
 #include "common.h"
 #include "launch.h"
 #include "mfma_tiles.h"
+#include <stddef.h>
 #include <stdlib.h>
 
 namespace vig {
@@ -737,6 +738,10 @@ struct TileKernArgs {
   float oscale;
   const float* gate_w;
 };
+
+static_assert(offsetof(TileKernArgs, geo) == 6 * sizeof(void*) && offsetof(TileKernArgs, oscale) == 48 + sizeof(TileGeo) &&
+                  offsetof(TileKernArgs, gate_w) == 48 + sizeof(TileGeo) + 8 && alignof(TileGeo) == 8,
+              "TileKernArgs has to mirror the parameter list of gla_tile_kernel");
 
 // The general form as a function of its own: its register needs stay out of the fp16 form's allocation.  It reads
 // the kernel's arguments from the argument block itself (ka: the kernel's own kernarg segment pointer; the builtin
